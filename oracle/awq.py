@@ -1,0 +1,128 @@
+"""TEST INFRASTRUCTURE ONLY - CPU restatement of the reference's AWQ codec.
+
+Follows, function by function (paths relative to the reference root,
+PE = programming_examples):
+
+  AWQ_PACK_ORDER / AWQ_UNPACK_PERM   PE/llms/llama32_1b_int4/awq_repacker.py:33-38
+                                     (= _AWQ_REORDER_PERM, awq_pack.py:61-63)
+  unpack_awq_int32                   awq_repacker.py:41-54 (= awq_pack.py:66-76)
+  pack_awq_int32                     awq_repacker.py:155-162 (packer inside
+                                     _gen_synthetic_awq)
+  dequant_to_bf16                    awq_repacker.py:57-82 (= awq_dequant_layer,
+                                     awq_pack.py:84-104)
+  repack_hf_awq_linear               awq_repacker.py:85-109
+  l1_unpack_nibbles                  matvec_int4_packed.py:282-283 (byte ->
+                                     even/odd-k nibble)
+  dequant_1d                         PE/dequant_awq/dequant_awq.py:391-396
+
+bf16 tensors are uint16 bit patterns (see oracle/bf16.py).
+
+Pins (tests/test_oracle_awq.py): the hand-computed word 0x76543210, a scalar
+brute-force packer, exhaustive (q, z) x scale-bit-pattern dequant against
+exact rational arithmetic, the self-test identities of awq_repacker.py:166-206.
+"""
+
+import numpy as np
+
+from .bf16 import bf16_bits_to_f32, f32_to_bf16_bits
+
+# Bit position 4*i of each int32 holds output column 8*block + AWQ_PACK_ORDER[i].
+AWQ_PACK_ORDER = np.array([0, 2, 4, 6, 1, 3, 5, 7], dtype=np.int64)
+# AWQ_UNPACK_PERM[j] is the bit-position index holding natural column j.
+AWQ_UNPACK_PERM = np.argsort(AWQ_PACK_ORDER)
+
+
+def unpack_awq_int32(packed):
+    """int32 [..., N/8] -> uint8 nibbles [..., N] in natural column order."""
+    packed64 = np.asarray(packed).astype(np.int64)
+    shifts = np.arange(8, dtype=np.int64) * 4
+    nibs = ((packed64[..., :, None] >> shifts) & 0xF).astype(np.uint8)
+    nibs = nibs[..., AWQ_UNPACK_PERM]
+    return nibs.reshape(*packed64.shape[:-1], packed64.shape[-1] * 8)
+
+
+def pack_awq_int32(nibs):
+    """uint8 nibbles [R, N] (natural order) -> int32 [R, N/8] in AWQ order."""
+    nibs = np.asarray(nibs)
+    rows, n = nibs.shape
+    assert n % 8 == 0
+    out = np.zeros((rows, n // 8), dtype=np.uint32)
+    for i in range(8):
+        col = int(AWQ_PACK_ORDER[i])
+        out |= (nibs[:, col::8].astype(np.uint32) & 0xF) << np.uint32(4 * i)
+    return out.view(np.int32)
+
+
+def dequant_to_bf16(qweight, qzeros, scales_bits, group_size):
+    """AWQ tensors -> dense W[K, N] as bf16 bits.
+
+    W[k, n] = bf16_rne((q[k, n] - z[k // gs, n]) * s[k // gs, n]); the product
+    is formed in float32 exactly as the reference does.
+    """
+    q = unpack_awq_int32(qweight)
+    z = unpack_awq_int32(qzeros)
+    k, n = q.shape
+    n_groups = k // group_size
+    if z.shape != (n_groups, n):
+        raise ValueError(f"qzeros shape {z.shape} vs expected ({n_groups}, {n})")
+    if np.shape(scales_bits) != (n_groups, n):
+        raise ValueError(f"scales shape {np.shape(scales_bits)} vs expected ({n_groups}, {n})")
+    s = bf16_bits_to_f32(scales_bits)
+    z_per_k = np.repeat(z.astype(np.int32), group_size, axis=0)
+    s_per_k = np.repeat(s, group_size, axis=0)
+    w_f32 = ((q.astype(np.int32) - z_per_k).astype(np.float32)) * s_per_k
+    return f32_to_bf16_bits(w_f32)
+
+
+def dequant_unrounded_f32(qweight, qzeros, scales_bits, group_size):
+    """(q - z) * s in float32 without the final bf16 rounding (exact: the
+    product has at most 13 significant bits)."""
+    q = unpack_awq_int32(qweight).astype(np.int32)
+    z = unpack_awq_int32(qzeros).astype(np.int32)
+    s = bf16_bits_to_f32(scales_bits)
+    return (q - np.repeat(z, group_size, axis=0)).astype(np.float32) * np.repeat(s, group_size, axis=0)
+
+
+def repack_hf_awq_linear(qweight, qzeros, scales_bits, group_size):
+    """AWQ tensors -> the examples' kernel-side arrays
+    (A_q u8 [out, K/2], A_s bf16-bits [K/gs, out], A_z u8 [K/gs, out])."""
+    q = unpack_awq_int32(qweight)
+    z = unpack_awq_int32(qzeros)
+    k, n = q.shape
+    n_groups = k // group_size
+    if z.shape != (n_groups, n):
+        raise ValueError(f"qzeros shape {z.shape} vs expected ({n_groups}, {n})")
+    if np.shape(scales_bits) != (n_groups, n):
+        raise ValueError(f"scales shape {np.shape(scales_bits)} vs expected ({n_groups}, {n})")
+    q_mn = np.ascontiguousarray(q.T)
+    a_q = ((q_mn[:, 0::2] & 0x0F) | ((q_mn[:, 1::2] & 0x0F) << 4)).astype(np.uint8)
+    a_s = np.ascontiguousarray(scales_bits).astype(np.uint16)
+    a_z = np.ascontiguousarray(z).astype(np.uint8)
+    return a_q, a_s, a_z
+
+
+def l1_unpack_nibbles(a_q):
+    """A_q u8 [out, K/2] -> nibbles int32 [out, K] (even k = low nibble)."""
+    a = np.asarray(a_q).astype(np.int32)
+    out = np.empty((a.shape[0], a.shape[1] * 2), dtype=np.int32)
+    out[:, 0::2] = a & 0x0F
+    out[:, 1::2] = (a >> 4) & 0x0F
+    return out
+
+
+def l1_to_awq(a_q, a_s_bits, a_z):
+    """Inverse of repack_hf_awq_linear: kernel-side arrays -> AWQ tensors."""
+    nibs_kn = np.ascontiguousarray(l1_unpack_nibbles(a_q).T).astype(np.uint8)
+    qweight = pack_awq_int32(nibs_kn)
+    qzeros = pack_awq_int32(np.asarray(a_z).astype(np.uint8))
+    return qweight, qzeros, np.ascontiguousarray(a_s_bits).astype(np.uint16)
+
+
+def dequant_1d(int4_vals, scales_bits, zeros, group_size):
+    """1-D form of the dequant example: out[i] = bf16((q[i] - z[g]) * s[g])
+    evaluated in double as the reference's Python floats do."""
+    q = np.asarray(int4_vals).astype(np.float64)
+    g = np.arange(q.size) // group_size
+    z = np.asarray(zeros).astype(np.float64)[g]
+    s = bf16_bits_to_f32(scales_bits).astype(np.float64)[g]
+    return f32_to_bf16_bits(((q - z) * s).astype(np.float32))

@@ -1,0 +1,158 @@
+"""Pins oracle/reference.py (GEMV / GEMM / SwiGLU / FFN restatements) with
+closed forms and library routines, chosen so that a dropped term, a swapped
+nibble, a transposed operand or a wrong group index fails at least one."""
+import numpy as np
+import torch
+
+import oracle
+from oracle import awq, reference as ref
+from oracle.bf16 import bf16_bits_to_f32, f32_to_bf16_bits
+
+
+def _l1(M, K, gs, seed, z_lo=0, z_hi=16):
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 16, size=(M, K), dtype=np.uint8)
+    a_q = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)
+    a_s = f32_to_bf16_bits(rng.uniform(0.005, 0.02, size=(K // gs, M)).astype(np.float32))
+    a_z = rng.integers(z_lo, z_hi, size=(K // gs, M), dtype=np.uint8)
+    b = f32_to_bf16_bits(rng.standard_normal(K).astype(np.float32))
+    return q, a_q, a_s, a_z, b
+
+
+def test_integer_matrix_special_case_is_exact():
+    # z = 0, s = 1, small-integer x: the GEMV is an exact integer product
+    M, K, gs = 24, 256, 128
+    q, a_q, _, _, _ = _l1(M, K, gs, 0)
+    a_s = np.full((K // gs, M), 0x3F80, np.uint16)
+    a_z = np.zeros((K // gs, M), np.uint8)
+    xi = np.random.default_rng(1).integers(-2, 3, K)
+    b = f32_to_bf16_bits(xi.astype(np.float32))
+    want = q.astype(np.int64) @ xi
+    assert np.array_equal(ref.matvec_f64(a_q, a_s, a_z, b), want.astype(np.float64))
+    assert np.array_equal(bf16_bits_to_f32(ref.matvec_cpu_reference_loop(a_q, a_s, a_z, b)),
+                          bf16_bits_to_f32(f32_to_bf16_bits(want.astype(np.float32))))
+
+
+def test_one_hot_x_returns_one_dequantised_row_bit_exact():
+    M, K, gs = 16, 256, 128
+    q, a_q, a_s, a_z, _ = _l1(M, K, gs, 2)
+    qweight, qzeros, s = awq.l1_to_awq(a_q, a_s, a_z)
+    w = awq.dequant_to_bf16(qweight, qzeros, s, gs)  # [K, M]
+    for k0 in (0, 1, 127, 128, 255):   # even/odd nibble and both groups
+        b = np.zeros(K, np.uint16)
+        b[k0] = 0x3F80
+        assert np.array_equal(ref.matvec_cpu_reference(a_q, a_s, a_z, b), w[k0])
+        assert np.array_equal(ref.matvec_cpu_reference_loop(a_q, a_s, a_z, b), w[k0])
+
+
+def test_constant_q_per_group_closed_form():
+    # q constant within each group: y[r] = sum_g (c_g - z[g,r]) * s[g,r] * sum_{k in g} x[k]
+    M, K, gs = 8, 384, 128
+    rng = np.random.default_rng(3)
+    cg = rng.integers(0, 16, K // gs)
+    q = np.repeat(cg, gs)[None, :].repeat(M, 0).astype(np.uint8)
+    a_q = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)
+    _, _, a_s, a_z, b = _l1(M, K, gs, 4)
+    x = bf16_bits_to_f32(b).astype(np.float64)
+    xs = x.reshape(K // gs, gs).sum(1)
+    s = bf16_bits_to_f32(a_s).astype(np.float64)
+    want = ((cg[:, None] - a_z.astype(np.float64)) * s * xs[:, None]).sum(0)
+    assert np.allclose(ref.matvec_f64(a_q, a_s, a_z, b), want, rtol=1e-12, atol=1e-12)
+
+
+def test_scalar_loop_python_vs_c_and_vs_f64():
+    M, K, gs = 12, 256, 128
+    _, a_q, a_s, a_z, b = _l1(M, K, gs, 5)
+    py = ref.matvec_cpu_reference_loop(a_q, a_s, a_z, b)
+    lib = oracle.load_c_oracle()
+    out = np.zeros(M, np.uint16)
+    lib.oracle_matvec_loop(a_q.ctypes.data, a_s.ctypes.data, a_z.ctypes.data, b.ctypes.data, M, K, gs, out.ctypes.data)
+    assert np.array_equal(py, out)
+    # sequential float32 accumulation stays within one bf16 ulp of the float64 sum
+    f64 = ref.matvec_f64(a_q, a_s, a_z, b)
+    assert np.all(np.abs(bf16_bits_to_f32(out) - f64) <= np.abs(f64) * 2.0**-8 + 1e-3)
+
+
+def test_residual_and_down_projection_rounding_points():
+    M, K, gs = 8, 256, 128
+    _, a_q, a_s, a_z, b = _l1(M, K, gs, 6)
+    r = f32_to_bf16_bits(np.random.default_rng(7).standard_normal(M).astype(np.float32))
+    f64 = ref.matvec_f64(a_q, a_s, a_z, b)
+    # matvec_add: one rounding after adding R in float32
+    want = f32_to_bf16_bits(f64.astype(np.float32) + bf16_bits_to_f32(r))
+    assert np.array_equal(ref.matvec_add_cpu_reference(a_q, a_s, a_z, b, r), want)
+    # ld: GEMV result is rounded to bf16 BEFORE R is added, then rounded again
+    raw = bf16_bits_to_f32(f32_to_bf16_bits(f64.astype(np.float32)))
+    assert np.array_equal(ref.ld_cpu_reference(a_q, a_s, a_z, b, r), f32_to_bf16_bits(raw + bf16_bits_to_f32(r)))
+    assert np.array_equal(ref.ld_cpu_reference(a_q, a_s, a_z, b, None), ref.matvec_cpu_reference(a_q, a_s, a_z, b))
+
+
+def test_matmul_matches_matvec_rows_and_torch():
+    N, K, gs, M = 32, 256, 128, 5
+    _, w_q, w_s, w_z, _ = _l1(N, K, gs, 8)
+    a = f32_to_bf16_bits(np.random.default_rng(9).standard_normal((M, K)).astype(np.float32))
+    c64 = ref.matmul_cpu_reference(w_q, w_s, w_z, a, accumulate="f64")
+    for m in range(M):
+        assert np.array_equal(c64[m], ref.matvec_cpu_reference(w_q, w_s, w_z, a[m]))
+    # torch float64 matmul of the dense dequantised weights (library routine, [K, N] orientation)
+    qweight, qzeros, s = awq.l1_to_awq(w_q, w_s, w_z)
+    w = awq.dequant_unrounded_f32(qweight, qzeros, s, gs)
+    t = (torch.from_numpy(bf16_bits_to_f32(a)).double() @ torch.from_numpy(w).double()).float().numpy()
+    assert np.array_equal(c64, f32_to_bf16_bits(t))
+    c32 = ref.matmul_cpu_reference(w_q, w_s, w_z, a)
+    assert np.max(np.abs(bf16_bits_to_f32(c32) - bf16_bits_to_f32(c64))) <= 2.0**-7 * np.max(np.abs(bf16_bits_to_f32(c64)))
+    # rounded-weight variant multiplies exactly the dequant kernel's output
+    wr = bf16_bits_to_f32(awq.dequant_to_bf16(qweight, qzeros, s, gs)).astype(np.float64)
+    cr = f32_to_bf16_bits((bf16_bits_to_f32(a).astype(np.float64) @ wr).astype(np.float32))
+    assert np.array_equal(ref.matmul_cpu_reference(w_q, w_s, w_z, a, round_weights=True, accumulate="f64"), cr)
+
+
+def test_silu_identity_and_library_cross_check():
+    g = np.linspace(-12, 12, 4001).astype(np.float32)
+    got = ref.silu_tanh_f32(g)
+    sig = g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64)))
+    assert np.allclose(got, sig, rtol=2e-6, atol=1e-6)
+    t = torch.nn.functional.silu(torch.from_numpy(g)).numpy()
+    assert np.allclose(got, t, rtol=4e-6, atol=1e-6)
+
+
+def test_swiglu_rounding_points_and_interleave():
+    H, K, gs = 16, 256, 128
+    _, gq, gs_, gz, x = _l1(H, K, gs, 10)
+    _, uq, us_, uz, _ = _l1(H, K, gs, 11)
+    a_q, a_s, a_z = ref.interleave_gate_up((gq, gs_, gz), (uq, us_, uz))
+    assert np.array_equal(a_q[0::2], gq) and np.array_equal(a_q[1::2], uq)
+    assert np.array_equal(a_s[:, 1::2], us_) and np.array_equal(a_z[:, 0::2], gz)
+    h = ref.swiglu_rms_cpu_reference(a_q, a_s, a_z, x, None)
+    g = bf16_bits_to_f32(ref.matvec_cpu_reference(gq, gs_, gz, x))       # bf16 after the GEMV
+    u = bf16_bits_to_f32(ref.matvec_cpu_reference(uq, us_, uz, x))
+    want = f32_to_bf16_bits(ref.silu_tanh_f32(g) * u)                     # bf16 after silu * up
+    assert np.array_equal(h, want)
+    # RMSNorm prologue: unit weight and x with mean square 1 leaves x (up to eps) unchanged
+    xn = np.where(np.arange(K) % 2 == 0, 0x3F80, 0xBF80).astype(np.uint16)
+    ones = np.full(K, 0x3F80, np.uint16)
+    assert np.array_equal(f32_to_bf16_bits(ref.rms_norm_bf16(xn, ones)), xn)
+    h2 = ref.swiglu_rms_cpu_reference(a_q, a_s, a_z, xn, ones)
+    assert np.array_equal(h2, ref.swiglu_rms_cpu_reference(a_q, a_s, a_z, xn, None))
+
+
+def test_ffn_chain():
+    H, K, gs = 256, 128, 128
+    _, gq, gs_, gz, x = _l1(H, K, gs, 12)
+    _, uq, us_, uz, _ = _l1(H, K, gs, 13)
+    _, dq, ds, dz, _ = _l1(K, H, gs, 14)
+    h, y = ref.ffn_swiglu_reference((gq, gs_, gz), (uq, us_, uz), (dq, ds, dz), x)
+    assert h.shape == (H,) and y.shape == (K,)
+    assert np.array_equal(y, ref.matvec_cpu_reference(dq, ds, dz, h))
+
+
+def test_check_outputs_semantics():
+    e = np.linspace(1, 2, 1000)
+    a = e.copy()
+    assert ref.check_outputs(a, e, rtol=0.1, atol=0.05, min_correlation=0.999)
+    a[:5] += 1.0
+    assert not ref.check_outputs(a, e, rtol=0.1, atol=0.05)
+    assert ref.check_outputs(a, e, rtol=0.1, atol=0.05, max_mismatch_percentage=0.5)      # int(1000*0.5/100)=5
+    assert not ref.check_outputs(a, e, rtol=0.1, atol=0.05, max_mismatch_percentage=0.49)  # int(4.9)=4
+    # constant actual -> NaN correlation -> fail
+    assert not ref.check_outputs(np.ones(10), np.ones(10), rtol=1, atol=1, min_correlation=0.5)
