@@ -1,0 +1,122 @@
+/*
+ * w4a16.h - C ABI of the MI355X (gfx950) AWQ int4 / W4A16 kernels.
+ *
+ * One shared library (libw4a16_hip.so).  All data pointers are DEVICE pointers owned by
+ * the caller; nothing here allocates or frees device memory.  Every entry point returns
+ * W4A16_OK (0) or a negative W4A16_ERR_* code.  Arguments are validated before the first
+ * HIP call, so every error path below can be exercised on a host without a GPU.
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream); launches are
+ * asynchronous on that stream.
+ *
+ * Tensor conventions (AutoAWQ "gemm" layout, the reference's checkpoint format,
+ * programming_examples/llms/llama32_1b_int4/awq_repacker.py:7-11):
+ *   qweight  int32 [K, N/8]   8 uint4 per word along N; bit position 4*i holds column
+ *                             8*b + {0,2,4,6,1,3,5,7}[i]      (awq_repacker.py:33-38)
+ *   qzeros   int32 [K/group, N/8]  same packing
+ *   scales   bf16  [K/group, N]    (uint16 bit patterns)
+ *   x        bf16  [M, K] row-major,  y  bf16 [M, N] row-major,  y = x . W
+ *   W[k, n] = (q[k, n] - z[k/group, n]) * s[k/group, n]
+ * The examples' D[out] = A[out, K] @ B[K] (matvec_int4_packed.py:4) is the same product
+ * with out = N.
+ *
+ * Constraints: group == 128, K % 128 == 0, N % 8 == 0 for the dequant and N % 32 == 0
+ * for GEMV / GEMM / FFN, 16-byte aligned pointers.
+ */
+#ifndef W4A16_H
+#define W4A16_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define W4A16_OK 0
+#define W4A16_ERR_NULL (-1)        /* a required pointer is NULL */
+#define W4A16_ERR_SHAPE (-2)       /* M/K/N non-positive or not a supported multiple */
+#define W4A16_ERR_GROUP (-3)       /* group size other than 128 */
+#define W4A16_ERR_ALIGN (-4)       /* a pointer is not 16-byte aligned */
+#define W4A16_ERR_WORKSPACE (-5)   /* workspace missing or smaller than *_workspace_bytes */
+#define W4A16_ERR_HIP (-6)         /* a HIP call failed; see w4a16_last_hip_error() */
+#define W4A16_ERR_TUNE (-7)        /* unknown tuning key or value out of range */
+
+#define W4A16_ABI_VERSION 1
+
+int w4a16_abi_version(void);
+
+/* Static description of an error code (never NULL). */
+const char *w4a16_strerror(int code);
+
+/* hipGetErrorString of the last failing HIP call on this thread ("" if none). */
+const char *w4a16_last_hip_error(void);
+
+/*
+ * Dense dequant: out[k, n] = bf16_rne((q - z) * s), bit-exact with the reference's
+ * awq_dequant_layer (programming_examples/llms/llama32_1b_int4/awq_pack.py:84-104) and
+ * dequant_to_bf16 (awq_repacker.py:57-82).  Replaces the device kernel
+ * dequant_int4_bf16(uint8_t *packed, bfloat16 *out)
+ * (programming_examples/dequant_awq/dequant.cc:77-85).
+ */
+int awq_dequant_bf16(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                     uint16_t *out_bf16, int K, int N, int group, void *stream);
+
+/*
+ * Workspace for the split-K GEMV / small-M GEMM and the FFN.  The caller allocates
+ * `*_workspace_bytes` bytes of device memory once, clears it once with
+ * w4a16_workspace_init, and may then reuse it for any number of calls that do not
+ * overlap in time (each call leaves it cleared again).  Calls that run concurrently
+ * (different streams) need separate workspaces.
+ */
+size_t w4a16_gemm_workspace_bytes(int M, int K, int N);
+size_t w4a16_ffn_workspace_bytes(int K, int H);
+int w4a16_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Decode GEMV, M = 1: y[N] = bf16(x[K] . W).  fp32 accumulation, one bf16 rounding.
+ * Replaces matvec_int4_bf16_packed(uint8_t *packed, bfloat16 *b, bfloat16 *c)
+ * (programming_examples/matrix_vector_multiplication/int4_awq/mv_int4_bf16.cc:403-411)
+ * and matches matvec_int4_packed.cpu_reference (matvec_int4_packed.py:272-287).
+ */
+int w4a16_gemv_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
+                    const uint16_t *scales, uint16_t *y, int K, int N, int group,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * GEMM, any M >= 1: y[M, N] = bf16(x[M, K] . W).  M <= 16 streams the weights once
+ * through a split-K MFMA kernel; larger M uses the tiled prefill kernel that dequantises
+ * weight tiles to bf16 in LDS.  Replaces matmul_int4_bf16_packed_f32 + f32_to_bf16_mn
+ * (mv_int4_bf16.cc:430-448) and matches matmul_int4_packed.cpu_reference
+ * (programming_examples/matrix_multiplication/int4_awq/matmul_int4_packed.py:89-105).
+ */
+int w4a16_gemm_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
+                    const uint16_t *scales, uint16_t *y, int M, int K, int N, int group,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Fused decode SwiGLU FFN, batch 1:
+ *   g = bf16(x . Wg), u = bf16(x . Wu), h = bf16(silu(g) * u), y = bf16(h . Wd)
+ * with silu(g) = g * 0.5 * (tanh(g / 2) + 1) in fp32; Wg, Wu are [K, H], Wd is [H, K].
+ * Rounding points follow matvec_int4_swiglu_rms.cpu_reference
+ * (programming_examples/decode_ffn_swiglu/matvec_int4_swiglu_rms.py:512-516) and
+ * ld_cpu_reference (programming_examples/llms/llama32_1b_int4/multi_launch_builder/
+ * o_gemv_ffn_int4_fused.py:1078-1094) with R = 0 and no RMSNorm prologue.
+ * `h_out` (bf16 [H]) may be NULL; when given it receives the intermediate.
+ */
+int w4a16_ffn_swiglu_bf16(const uint16_t *x,
+                          const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                          const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                          const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
+                          uint16_t *y, uint16_t *h_out, int K, int H, int group,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
+ * "gemv_ksteps", "gemv_waves", "gemv_units" (0 = built-in heuristic).  Process-wide.
+ */
+int w4a16_tune(const char *key, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* W4A16_H */

@@ -1,0 +1,133 @@
+"""Host-side AWQ layout tools: the device format of this backend is the AutoAWQ
+"gemm" checkpoint layout itself, so static weights are written once without a
+per-tile repack.
+
+  qweight int32 [K, N/8], qzeros int32 [K/gs, N/8], scales bf16 [K/gs, N];
+  bit position 4*i of a word holds column 8*b + PACK_ORDER[i]
+  (programming_examples/llms/llama32_1b_int4/awq_repacker.py:33-38).
+
+The examples' kernel-side arrays (A_q u8 [out, K/2], A_s bf16 [K/gs, out],
+A_z u8 [K/gs, out]; matvec_int4_packed.py:346-350) convert both ways.
+"""
+
+import numpy as np
+
+from . import bf16
+
+PACK_ORDER = (0, 2, 4, 6, 1, 3, 5, 7)
+UNPACK_POS = (0, 4, 1, 5, 2, 6, 3, 7)   # bit-position index that holds natural column j
+GROUP = 128
+
+
+def pack_int4(nibs):
+    """uint8 [R, N] values 0..15 in natural column order -> int32 [R, N/8]."""
+    nibs = np.asarray(nibs)
+    if nibs.ndim != 2 or nibs.shape[1] % 8:
+        raise ValueError("pack_int4 expects [R, N] with N % 8 == 0")
+    blocks = nibs.reshape(nibs.shape[0], -1, 8).astype(np.uint32) & 0xF
+    word = np.zeros(blocks.shape[:2], dtype=np.uint32)
+    for j in range(8):
+        word |= blocks[:, :, j] << np.uint32(4 * UNPACK_POS[j])
+    return word.view(np.int32)
+
+
+def unpack_int4(packed):
+    """int32 [R, N/8] -> uint8 [R, N] in natural column order."""
+    w = np.ascontiguousarray(np.asarray(packed, dtype=np.int32)).view(np.uint32)
+    out = np.empty(w.shape + (8,), dtype=np.uint8)
+    for j in range(8):
+        out[..., j] = (w >> np.uint32(4 * UNPACK_POS[j])) & np.uint32(0xF)
+    return out.reshape(w.shape[0], -1)
+
+
+def awq_from_l1(A_q, A_s, A_z):
+    """Kernel-side arrays of the examples -> (qweight, qzeros, scales) in AWQ layout."""
+    A_q = np.asarray(A_q, dtype=np.uint8)
+    out, half_k = A_q.shape
+    nib = np.empty((out, 2 * half_k), dtype=np.uint8)
+    nib[:, 0::2] = A_q & 0x0F
+    nib[:, 1::2] = A_q >> 4
+    qweight = pack_int4(np.ascontiguousarray(nib.T))
+    qzeros = pack_int4(np.asarray(A_z, dtype=np.uint8))
+    scales = bf16.from_bits(bf16.bits_of(A_s))
+    if qzeros.shape[0] != scales.shape[0] or scales.shape[1] != out:
+        raise ValueError(f"A_s {scales.shape} / A_z {np.shape(A_z)} do not match A_q {A_q.shape}")
+    return qweight, qzeros, scales
+
+
+def l1_from_awq(qweight, qzeros, scales):
+    """AWQ layout -> (A_q, A_s, A_z) as repack_hf_awq_linear builds them
+    (awq_repacker.py:85-109)."""
+    q = unpack_int4(qweight)
+    z = unpack_int4(qzeros)
+    q_mn = np.ascontiguousarray(q.T)
+    A_q = ((q_mn[:, 0::2] & 0x0F) | ((q_mn[:, 1::2] & 0x0F) << 4)).astype(np.uint8)
+    return A_q, bf16.from_bits(bf16.bits_of(scales)), z
+
+
+def interleave_rows(gate, up):
+    """Row-interleave two kernel-side weight triples (row 2i = gate[i], 2i+1 = up[i]),
+    the layout of the decode FFN front half (llama32_1b_int4_weights.py:173-207)."""
+    def il(a, b, axis):
+        a, b = np.asarray(a), np.asarray(b)
+        shape = list(a.shape)
+        shape[axis] *= 2
+        out = np.empty(shape, dtype=a.dtype)
+        sl0 = [slice(None)] * a.ndim
+        sl1 = [slice(None)] * a.ndim
+        sl0[axis] = slice(0, None, 2)
+        sl1[axis] = slice(1, None, 2)
+        out[tuple(sl0)] = a
+        out[tuple(sl1)] = b
+        return out
+    return il(gate[0], up[0], 0), il(bf16.bits_of(gate[1]), bf16.bits_of(up[1]), 1).view(bf16.BF16Array), il(gate[2], up[2], 1)
+
+
+def deinterleave_rows(A_q, A_s, A_z):
+    """Inverse of interleave_rows -> (gate triple, up triple)."""
+    s = bf16.bits_of(A_s)
+    gate = (np.ascontiguousarray(A_q[0::2]), bf16.from_bits(s[:, 0::2]), np.ascontiguousarray(np.asarray(A_z)[:, 0::2]))
+    up = (np.ascontiguousarray(A_q[1::2]), bf16.from_bits(s[:, 1::2]), np.ascontiguousarray(np.asarray(A_z)[:, 1::2]))
+    return gate, up
+
+
+# --- single packed buffer ("BO") ------------------------------------------------------
+
+def _round256(v):
+    return (v + 255) & ~255
+
+
+def packed_layout(K, N, gs=GROUP):
+    """Byte offsets of the three sections inside one packed weight buffer."""
+    q_bytes = K * (N // 8) * 4
+    z_bytes = (K // gs) * (N // 8) * 4
+    s_bytes = (K // gs) * N * 2
+    z_off = _round256(q_bytes)
+    s_off = z_off + _round256(z_bytes)
+    return {"q_off": 0, "z_off": z_off, "s_off": s_off, "total": s_off + _round256(s_bytes),
+            "q_bytes": q_bytes, "z_bytes": z_bytes, "s_bytes": s_bytes}
+
+
+def pack_buffer(qweight, qzeros, scales):
+    """[qweight | qzeros | scales] in one uint8 buffer, sections 256-byte aligned
+    (the counterpart of the examples' single packed weight BO)."""
+    K, nb = qweight.shape
+    N = nb * 8
+    gs = K // qzeros.shape[0]
+    lay = packed_layout(K, N, gs)
+    buf = np.zeros(lay["total"], dtype=np.uint8)
+    buf[0:lay["q_bytes"]] = np.ascontiguousarray(qweight).view(np.uint8).reshape(-1)
+    buf[lay["z_off"]:lay["z_off"] + lay["z_bytes"]] = np.ascontiguousarray(qzeros).view(np.uint8).reshape(-1)
+    buf[lay["s_off"]:lay["s_off"] + lay["s_bytes"]] = bf16.bits_of(scales).view(np.uint8).reshape(-1)
+    return buf
+
+
+def unpack_buffer(buf, K, N, gs=GROUP):
+    lay = packed_layout(K, N, gs)
+    buf = np.asarray(buf, dtype=np.uint8).reshape(-1)
+    if buf.size != lay["total"]:
+        raise ValueError(f"packed buffer has {buf.size} bytes, expected {lay['total']} for K={K} N={N}")
+    qweight = buf[0:lay["q_bytes"]].view(np.int32).reshape(K, N // 8)
+    qzeros = buf[lay["z_off"]:lay["z_off"] + lay["z_bytes"]].view(np.int32).reshape(K // gs, N // 8)
+    scales = buf[lay["s_off"]:lay["s_off"] + lay["s_bytes"]].view(np.uint16).reshape(K // gs, N).view(bf16.BF16Array)
+    return qweight, qzeros, scales

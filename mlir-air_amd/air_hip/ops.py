@@ -1,0 +1,122 @@
+"""Operator-level wrappers over the C ABI for torch (ROCm) tensors.
+
+torch is used for device memory and streams only.  Every function launches on
+the current torch stream of the tensors' device and returns without
+synchronising.  There is no CPU path: tensors must live on the GPU.
+"""
+
+import torch
+
+from . import _lib
+
+GROUP = 128
+_workspaces = {}
+
+
+def _ptr(t):
+    return t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("air_hip ops need GPU tensors; there is no CPU fallback")
+        if not t.is_contiguous():
+            raise ValueError("air_hip ops need contiguous tensors")
+
+
+def _bits(t):
+    """bf16 tensors are passed as their 16-bit patterns."""
+    if t.dtype == torch.bfloat16:
+        return t
+    if t.dtype in (torch.int16, torch.uint16):
+        return t
+    raise TypeError(f"expected a bf16 tensor (or its int16 bits), got {t.dtype}")
+
+
+def workspace(nbytes, device):
+    """Cleared workspace per (device, stream), grown on demand."""
+    lib = _lib.load_library()
+    key = (device.index, _stream())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+        _lib.check(lib.w4a16_workspace_init(_ptr(ws), ws.numel(), _stream()))
+        _workspaces[key] = ws
+    return ws
+
+
+def awq_dequant(qweight, qzeros, scales, group=GROUP, out=None):
+    """Dense W[K, N] bf16 from AWQ tensors (int32 [K, N/8], int32 [K/g, N/8], bf16 [K/g, N])."""
+    lib = _lib.load_library()
+    _need_cuda(qweight, qzeros, scales)
+    K, nb = qweight.shape
+    N = nb * 8
+    if out is None:
+        out = torch.empty((K, N), dtype=torch.bfloat16, device=qweight.device)
+    _lib.check(lib.awq_dequant_bf16(_ptr(qweight), _ptr(qzeros), _ptr(_bits(scales)), _ptr(out), K, N, group, _stream()))
+    return out
+
+
+def w4a16_gemm(x, qweight, qzeros, scales, group=GROUP, out=None):
+    """y[M, N] = bf16(x[M, K] . W); x may also be a vector [K] (returns [N])."""
+    lib = _lib.load_library()
+    _need_cuda(x, qweight, qzeros, scales)
+    vec = x.dim() == 1
+    x2 = x.unsqueeze(0) if vec else x
+    M, K = x2.shape
+    if qweight.shape[0] != K:
+        raise ValueError(f"x has K={K} but qweight has {qweight.shape[0]} rows")
+    N = qweight.shape[1] * 8
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    nbytes = lib.w4a16_gemm_workspace_bytes(M, K, N)
+    ws = workspace(nbytes, x.device)
+    _lib.check(lib.w4a16_gemm_bf16(_ptr(_bits(x2)), _ptr(qweight), _ptr(qzeros), _ptr(_bits(scales)), _ptr(out),
+                                   M, K, N, group, _ptr(ws), ws.numel(), _stream()))
+    return out.squeeze(0) if vec else out
+
+
+def w4a16_gemv(x, qweight, qzeros, scales, group=GROUP, out=None):
+    """Decode GEMV: y[N] = bf16(x[K] . W)."""
+    lib = _lib.load_library()
+    _need_cuda(x, qweight, qzeros, scales)
+    K = x.numel()
+    if qweight.shape[0] != K:
+        raise ValueError(f"x has K={K} but qweight has {qweight.shape[0]} rows")
+    N = qweight.shape[1] * 8
+    if out is None:
+        out = torch.empty((N,), dtype=torch.bfloat16, device=x.device)
+    ws = workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
+    _lib.check(lib.w4a16_gemv_bf16(_ptr(_bits(x)), _ptr(qweight), _ptr(qzeros), _ptr(_bits(scales)), _ptr(out),
+                                   K, N, group, _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def ffn_swiglu(x, gate, up, down, group=GROUP, return_h=False):
+    """Decode FFN: y = Wd(silu(x Wg) * (x Wu)); gate/up/down are (qweight, qzeros, scales)."""
+    lib = _lib.load_library()
+    _need_cuda(x, *gate, *up, *down)
+    K = x.numel()
+    H = gate[0].shape[1] * 8
+    if gate[0].shape[0] != K or up[0].shape != gate[0].shape or down[0].shape[0] != H or down[0].shape[1] * 8 != K:
+        raise ValueError("ffn_swiglu: gate/up must be [K, H/8] and down [H, K/8]")
+    y = torch.empty((K,), dtype=torch.bfloat16, device=x.device)
+    h = torch.empty((H,), dtype=torch.bfloat16, device=x.device) if return_h else None
+    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device)
+    _lib.check(lib.w4a16_ffn_swiglu_bf16(
+        _ptr(_bits(x)),
+        _ptr(gate[0]), _ptr(gate[1]), _ptr(_bits(gate[2])),
+        _ptr(up[0]), _ptr(up[1]), _ptr(_bits(up[2])),
+        _ptr(down[0]), _ptr(down[1]), _ptr(_bits(down[2])),
+        _ptr(y), _ptr(h) if h is not None else None, K, H, group, _ptr(ws), ws.numel(), _stream()))
+    return (y, h) if return_h else y
+
+
+def tune(key, value):
+    lib = _lib.load_library()
+    _lib.check(lib.w4a16_tune(key.encode(), int(value)))

@@ -1,0 +1,155 @@
+// C ABI of libw4a16_hip.so: argument validation (before any HIP call) and dispatch.
+#include <string.h>
+
+#include "../../include/w4a16.h"
+#include "common.h"
+#include "kernels.h"
+
+using namespace w4a16;
+
+namespace {
+
+thread_local char t_hip_error[256] = "";
+
+int hip_fail(hipError_t e) {
+    strncpy(t_hip_error, hipGetErrorString(e), sizeof(t_hip_error) - 1);
+    t_hip_error[sizeof(t_hip_error) - 1] = 0;
+    return W4A16_ERR_HIP;
+}
+
+inline bool misaligned(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+int check_quant(const void *qweight, const void *qzeros, const void *scales, int K, int N, int group, int n_mult) {
+    if (!qweight || !qzeros || !scales) return W4A16_ERR_NULL;
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    if (K <= 0 || N <= 0 || K % kGroup != 0 || N % n_mult != 0) return W4A16_ERR_SHAPE;
+    if (N / 32 > 16 * kCounterWords) return W4A16_ERR_SHAPE;
+    if (misaligned(qweight) || misaligned(qzeros) || misaligned(scales)) return W4A16_ERR_ALIGN;
+    return W4A16_OK;
+}
+
+size_t round256(size_t v) { return (v + 255) & ~size_t(255); }
+
+size_t stream_partial_bytes(int M, int N, int nmat) {
+    return round256((size_t)nmat * kMaxKSplit * (size_t)(M < 16 ? M : 16) * (size_t)N * sizeof(float));
+}
+
+}  // namespace
+
+extern "C" {
+
+int w4a16_abi_version(void) { return W4A16_ABI_VERSION; }
+
+const char *w4a16_strerror(int code) {
+    switch (code) {
+        case W4A16_OK: return "ok";
+        case W4A16_ERR_NULL: return "required pointer is NULL";
+        case W4A16_ERR_SHAPE: return "unsupported shape (need K % 128 == 0, N % 32 == 0 (dequant: N % 8 == 0), M >= 1)";
+        case W4A16_ERR_GROUP: return "unsupported group size (only 128)";
+        case W4A16_ERR_ALIGN: return "pointer is not 16-byte aligned";
+        case W4A16_ERR_WORKSPACE: return "workspace is NULL or too small";
+        case W4A16_ERR_HIP: return "HIP call failed";
+        case W4A16_ERR_TUNE: return "unknown tuning key or value out of range";
+        default: return "unknown error code";
+    }
+}
+
+const char *w4a16_last_hip_error(void) { return t_hip_error; }
+
+int awq_dequant_bf16(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, uint16_t *out_bf16,
+                     int K, int N, int group, void *stream) {
+    if (!out_bf16) return W4A16_ERR_NULL;
+    int rc = check_quant(qweight, qzeros, scales, K, N, group, 8);
+    if (rc) return rc;
+    if (misaligned(out_bf16)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_dequant(qweight, qzeros, scales, out_bf16, K, N, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+size_t w4a16_gemm_workspace_bytes(int M, int K, int N) {
+    if (M <= 0 || K <= 0 || N <= 0) return 0;
+    return kCounterBytes + stream_partial_bytes(M, N, 1);
+}
+
+size_t w4a16_ffn_workspace_bytes(int K, int H) {
+    if (K <= 0 || H <= 0) return 0;
+    const size_t a = stream_partial_bytes(1, H, 2), b = stream_partial_bytes(1, K, 1);
+    return kCounterBytes + (a > b ? a : b) + round256((size_t)H * sizeof(uint16_t));
+}
+
+int w4a16_workspace_init(void *workspace, size_t workspace_bytes, void *stream) {
+    if (!workspace) return W4A16_ERR_NULL;
+    if (workspace_bytes < kCounterBytes) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_fill_zero(workspace, kCounterBytes, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_gemm_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                    uint16_t *y, int M, int K, int N, int group, void *workspace, size_t workspace_bytes,
+                    void *stream) {
+    if (!x || !y) return W4A16_ERR_NULL;
+    int rc = check_quant(qweight, qzeros, scales, K, N, group, 32);
+    if (rc) return rc;
+    if (M <= 0) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(y)) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_gemm_workspace_bytes(M, K, N)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (M <= 16)
+        e = launch_stream(x, qweight, qzeros, scales, nullptr, nullptr, nullptr, y, M, K, N, workspace, st);
+    else
+        e = launch_gemm_prefill(x, qweight, qzeros, scales, y, M, K, N, st);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_gemv_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                    uint16_t *y, int K, int N, int group, void *workspace, size_t workspace_bytes, void *stream) {
+    return w4a16_gemm_bf16(x, qweight, qzeros, scales, y, 1, K, N, group, workspace, workspace_bytes, stream);
+}
+
+int w4a16_ffn_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
+                          const uint16_t *gate_scales, const int32_t *up_qweight, const int32_t *up_qzeros,
+                          const uint16_t *up_scales, const int32_t *down_qweight, const int32_t *down_qzeros,
+                          const uint16_t *down_scales, uint16_t *y, uint16_t *h_out, int K, int H, int group,
+                          void *workspace, size_t workspace_bytes, void *stream) {
+    if (!x || !y) return W4A16_ERR_NULL;
+    int rc = check_quant(gate_qweight, gate_qzeros, gate_scales, K, H, group, 32);
+    if (rc) return rc;
+    rc = check_quant(up_qweight, up_qzeros, up_scales, K, H, group, 32);
+    if (rc) return rc;
+    rc = check_quant(down_qweight, down_qzeros, down_scales, H, K, group, 32);
+    if (rc) return rc;
+    if (misaligned(x) || misaligned(y) || (h_out && misaligned(h_out))) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_ffn_workspace_bytes(K, H)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint16_t *h = h_out;
+    if (!h) h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + w4a16_ffn_workspace_bytes(K, H) -
+                                             round256((size_t)H * sizeof(uint16_t)));
+    hipError_t e = launch_stream(x, gate_qweight, gate_qzeros, gate_scales, up_qweight, up_qzeros, up_scales, h, 1, K,
+                                 H, workspace, st);
+    if (e != hipSuccess) return hip_fail(e);
+    e = launch_stream(h, down_qweight, down_qzeros, down_scales, nullptr, nullptr, nullptr, y, 1, H, K, workspace, st);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_tune(const char *key, int value) {
+    if (!key || value < 0) return W4A16_ERR_TUNE;
+    if (!strcmp(key, "gemv_ksteps")) {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return W4A16_ERR_TUNE;
+        g_stream_tune.ksteps = value;
+    } else if (!strcmp(key, "gemv_waves")) {
+        if (value != 0 && value != 4 && value != 8) return W4A16_ERR_TUNE;
+        g_stream_tune.waves = value;
+    } else if (!strcmp(key, "gemv_units")) {
+        if (value > 64) return W4A16_ERR_TUNE;
+        g_stream_tune.units = value;
+    } else {
+        return W4A16_ERR_TUNE;
+    }
+    return W4A16_OK;
+}
+
+}  // extern "C"

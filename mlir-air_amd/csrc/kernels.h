@@ -1,0 +1,45 @@
+// Internal launch interface between the C ABI (capi.hip) and the kernel files.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace w4a16 {
+
+// Layout of the caller-provided workspace: [kCounterWords uint32 arrival counters]
+// [fp32 split-K partials].  Counters are zero between calls.
+constexpr int kCounterWords = 4096;
+constexpr size_t kCounterBytes = kCounterWords * sizeof(uint32_t);
+constexpr int kMaxKSplit = 32;
+
+struct StreamTune {
+    int ksteps = 0;   // K-steps (32 rows) a wave loads per unit: 1, 2 or 4 (0 = heuristic)
+    int waves = 0;    // waves per workgroup: 4 or 8
+    int units = 0;    // units each wave processes back to back
+};
+extern StreamTune g_stream_tune;
+
+struct StreamPlan {
+    int ksteps, waves, units, ksplit, ntiles, mi;
+};
+StreamPlan plan_stream(int M, int K, int N);
+
+// Epilogue selector for the streaming kernel.
+enum StreamEpilogue { kEpiStore = 0, kEpiSwiGLU = 1 };
+
+hipError_t launch_dequant(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, uint16_t *out,
+                          int K, int N, hipStream_t stream);
+
+// y[M, N] = bf16(x[M, K] . W), M <= 16.  With `up_*` given (SwiGLU epilogue, M == 1) the
+// kernel streams both weight sets and writes y = bf16(silu(bf16(x.Wg)) * bf16(x.Wu)).
+hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                         const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                         uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream);
+
+hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
+                               const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream);
+
+hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
+
+}  // namespace w4a16
