@@ -1,0 +1,307 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn]
+
+Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
+A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
+To measure HBM rather than the 256 MB Infinity Cache, the steps rotate over enough
+independent copies of the weights to exceed it ("cold"); the same-buffer ("hot") rate is
+reported beside it.  The timed region is a HIP graph of exactly K launches bracketed by
+events on the launching stream and by device synchronisation.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "mlir-air_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+MALL_BYTES = 256 << 20
+
+CONFIGS = {
+    # name: (M, K, N, bound, description)
+    "dequant": dict(M=0, K=4096, N=4096, cfg=0, desc="AWQ dequant K=4096 N=4096 -> bf16"),
+    "gemv": dict(M=1, K=4096, N=11008, cfg=1, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128"),
+    "gemm16": dict(M=16, K=4096, N=14336, cfg=2, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128"),
+    "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128"),
+    "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128"),
+}
+
+
+def weight_bytes(K, N):
+    return K * N // 2 + (K // 128) * (N // 8) * 4 + (K // 128) * N * 2
+
+
+def algorithmic_bytes(name):
+    c = CONFIGS[name]
+    M, K, N = c["M"], c["K"], c["N"]
+    if name == "dequant":
+        return weight_bytes(K, N) + K * N * 2
+    if name == "ffn":
+        return 3 * weight_bytes(K, N) + K * 2 + K * 2
+    return weight_bytes(K, N) + M * K * 2 + M * N * 2
+
+
+def algorithmic_flops(name):
+    c = CONFIGS[name]
+    if name == "ffn":
+        return 2 * 3 * c["K"] * c["N"]
+    return 2 * max(c["M"], 0) * c["K"] * c["N"]
+
+
+def make_weights(torch, K, N, seed):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    # uniform random words = uniform uint4 nibbles in every position
+    qweight = torch.randint(-2**31, 2**31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    qzeros = torch.randint(-2**31, 2**31 - 1, (K // 128, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    scales = (torch.randn((K // 128, N), device="cuda", generator=g).abs() * 0.02 + 1e-3).to(torch.bfloat16)
+    return qweight, qzeros, scales
+
+
+def run_workload(name, steps, warmup, with_cpu_baseline):
+    import torch
+
+    from air_hip import _lib
+
+    lib = _lib.load_library()
+    c = CONFIGS[name]
+    M, K, N = c["M"], c["K"], c["N"]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream()
+
+    per_copy = weight_bytes(K, N) * (3 if name == "ffn" else 1)
+    if name == "prefill":
+        ncopies = 1
+    else:
+        ncopies = max(2, -(-(MALL_BYTES + MALL_BYTES // 2) // per_copy))
+    copies = []
+    for i in range(ncopies):
+        if name == "ffn":
+            copies.append((make_weights(torch, K, N, 100 + 3 * i), make_weights(torch, K, N, 101 + 3 * i),
+                           make_weights(torch, N, K, 102 + 3 * i)))
+        else:
+            copies.append(make_weights(torch, K, N, 100 + i))
+    gx = torch.Generator(device="cuda")
+    gx.manual_seed(7)
+    x = torch.randn((max(M, 1), K), device="cuda", generator=gx).to(torch.bfloat16)
+    if name == "dequant":
+        outs = [torch.empty((K, N), dtype=torch.bfloat16, device=dev) for _ in range(min(ncopies, 8))]
+    elif name == "ffn":
+        outs = [torch.empty((K,), dtype=torch.bfloat16, device=dev)]
+    else:
+        outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev)]
+
+    if name == "ffn":
+        ws_bytes = lib.w4a16_ffn_workspace_bytes(K, N)
+    else:
+        ws_bytes = max(lib.w4a16_gemm_workspace_bytes(max(M, 1), K, N), 16384)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    _lib.check(lib.w4a16_workspace_init(ws.data_ptr(), ws.numel(), stream.cuda_stream))
+
+    def launch(i, st):
+        w = copies[i % ncopies]
+        if name == "dequant":
+            o = outs[i % len(outs)]
+            rc = lib.awq_dequant_bf16(w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), o.data_ptr(), K, N, 128, st)
+        elif name == "ffn":
+            g, u, d = w
+            rc = lib.w4a16_ffn_swiglu_bf16(x.data_ptr(), g[0].data_ptr(), g[1].data_ptr(), g[2].data_ptr(),
+                                           u[0].data_ptr(), u[1].data_ptr(), u[2].data_ptr(),
+                                           d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(),
+                                           outs[0].data_ptr(), None, K, N, 128, ws.data_ptr(), ws.numel(), st)
+        else:
+            rc = lib.w4a16_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
+                                     outs[0].data_ptr(), M, K, N, 128, ws.data_ptr(), ws.numel(), st)
+        _lib.check(rc)
+
+    def timed_graph(indices):
+        """Capture len(indices) launches into one HIP graph, replay it once between events."""
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(graph, stream=stream):
+                for i in indices:
+                    launch(i, stream.cuda_stream)
+            graph.replay()          # untimed replay: instantiation / first-touch effects
+            stream.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            e0.record(stream)
+            graph.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
+        return e0.elapsed_time(e1) * 1e-3, wall
+
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            launch(i, stream.cuda_stream)
+        stream.synchronize()
+
+    cold_s, cold_wall = timed_graph(list(range(steps)))
+    hot_s, _ = timed_graph([0] * steps)
+
+    res = {
+        "name": name,
+        "cold_us": cold_s / steps * 1e6,
+        "hot_us": hot_s / steps * 1e6,
+        "wall_s": cold_wall,
+        "bytes": algorithmic_bytes(name),
+        "flops": algorithmic_flops(name),
+        "ncopies": ncopies,
+    }
+
+    if with_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(name, torch, copies[0], x, outs, launch, stream)
+    return res
+
+
+def cpu_baseline(name, torch, w, x, outs, launch, stream):
+    """The reference's NumPy path (restated in oracle/baseline.py) timed on this host's cores,
+    on the same inputs as GPU launch 0; also used to sanity-check the GPU result."""
+    import numpy as np
+
+    from oracle import baseline
+    from oracle.bf16 import bf16_bits_to_f32
+
+    try:
+        from threadpoolctl import threadpool_info
+        blas_threads = max([p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"] or [1])
+    except Exception:
+        blas_threads = 1
+
+    def host(t):
+        if t.dtype == torch.bfloat16:
+            return t.view(torch.int16).cpu().numpy().view(np.uint16)
+        return t.cpu().numpy()
+
+    c = CONFIGS[name]
+    with torch.cuda.stream(stream):
+        launch(0, stream.cuda_stream)
+        stream.synchronize()
+    got = bf16_bits_to_f32(host(outs[0]))
+
+    if name == "dequant":
+        args = tuple(host(t) for t in w)
+        fn = lambda: baseline.dequant_numpy(*args)
+        sample = "full config 0 (K=4096, N=4096), vectorised NumPy unpack + dequant, median of 3"
+    elif name == "ffn":
+        g, u, d = (tuple(host(t) for t in m) for m in w)
+        xb = host(x)[0]
+        fn = lambda: baseline.ffn_numpy(xb, g, u, d)
+        sample = "full config 4, vectorised NumPy dequant + float32 BLAS products, median of 3"
+    elif name == "prefill":
+        # bounded sample: the first 128 rows of x against the full weight matrix
+        args = tuple(host(t) for t in w)
+        xb = host(x)[:128]
+        fn = lambda: baseline.gemm_numpy(xb, *args)
+        sample = "rows 0..127 of config 3 (M=128 of 2048) incl. the full dequant, scaled by M; median of 3"
+    else:
+        args = tuple(host(t) for t in w)
+        xb = host(x)
+        fn = lambda: baseline.gemm_numpy(xb, *args)
+        sample = f"full config {c['cfg']}, vectorised NumPy dequant + float32 BLAS product, median of 3"
+
+    ref = fn()   # warm-up, and the reference output
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[1]
+    ref_f = bf16_bits_to_f32(ref)
+    n = ref_f.size
+    err = float(np.max(np.abs(got.reshape(-1)[:n] - ref_f.reshape(-1))))
+    if name == "prefill":
+        value = algorithmic_flops(name) * (128 / c["M"]) / t / 1e12
+        unit = "TFLOP/s"
+    else:
+        value = algorithmic_bytes(name) / t / 1e9
+        unit = "GB/s"
+    return {"value": value, "unit": unit, "cores": int(blas_threads), "kind": "port", "sample": sample,
+            "seconds": t, "host_cpus": len(os.sched_getaffinity(0)), "max_abs_diff_vs_gpu": err}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configs")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures the single-GPU W4A16 kernels; --gpus must be 1 "
+              "(this build has no multi-GPU path and every box has one GPU)", file=sys.stderr)
+        sys.exit(2)
+
+    main_res = run_workload(a.workload, a.steps, a.warmup, not a.no_cpu_baseline)
+    name = a.workload
+    sec = main_res["cold_us"] * 1e-6
+    if name == "prefill":
+        metric, unit = "W4A16 prefill GEMM TFLOP/s", "TFLOP/s"
+        value = main_res["flops"] / sec / 1e12
+        roof = {"bound": "mfma", "achieved": value, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": value / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
+    else:
+        metric, unit = "int4 GEMV HBM GB/s at M=1" if name == "gemv" else f"{name} HBM GB/s", "GB/s"
+        value = main_res["bytes"] / sec / 1e9
+        roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": value / HBM_PEAK_GBS, "traffic": None}
+    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel"}.get(name, "stream_kernel")
+    roof["algorithmic_per_launch"] = main_res["flops"] if name == "prefill" else main_res["bytes"]
+    roof["avg_launch_us"] = main_res["cold_us"]
+
+    out = {
+        "metric": metric,
+        "value": value,
+        "unit": unit,
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": main_res["cold_us"] * 1e-3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int4 weights, bf16 activations, fp32 accumulate",
+        "data": "synthetic (uniform uint4 q/z, scales |N(0,1)|*0.02+1e-3, x ~ N(0,1)), random weights",
+        "config": {"workload": CONFIGS[name]["desc"], "group": 128,
+                   "weight_copies_rotated": main_res["ncopies"], "timing": "HIP graph of K launches, events on the launch stream"},
+        "roofline": roof,
+        "hot_cache": {"us_per_step": main_res["hot_us"],
+                      "value": (main_res["flops"] / 1e12 if name == "prefill" else main_res["bytes"] / 1e9) / (main_res["hot_us"] * 1e-6),
+                      "note": "same buffers every step (Infinity Cache resident for the decode shapes)"},
+    }
+    if "cpu_baseline" in main_res:
+        out["cpu_baseline"] = main_res["cpu_baseline"]
+
+    if not a.no_extra:
+        extra = {}
+        for other in CONFIGS:
+            if other == name:
+                continue
+            r = run_workload(other, 20 if other == "prefill" else 100, 5, False)
+            s = r["cold_us"] * 1e-6
+            if other == "prefill":
+                extra[other] = {"us": r["cold_us"], "TFLOP/s": r["flops"] / s / 1e12,
+                                "frac_mfma_peak": r["flops"] / s / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+            else:
+                extra[other] = {"us": r["cold_us"], "GB/s": r["bytes"] / s / 1e9,
+                                "frac_hbm_peak": r["bytes"] / s / 1e9 / HBM_PEAK_GBS, "hot_us": r["hot_us"]}
+        out["other_workloads"] = extra
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -242,12 +242,14 @@ StreamPlan plan_stream(int M, int K, int N) {
     pl.mi = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     pl.ntiles = (N / 32 + 15) / 16;
     const int nksteps = K / 32;
-    pl.ksteps = M <= 4 ? 2 : 4;
+    pl.ksteps = M <= 4 ? 1 : 4;
     pl.waves = 8;
     pl.units = 1;
     if (g_stream_tune.ksteps) pl.ksteps = g_stream_tune.ksteps;
     if (g_stream_tune.waves) pl.waves = g_stream_tune.waves;
     if (g_stream_tune.units) pl.units = g_stream_tune.units;
+    // 512-thread workgroups cap a wave at 256 VGPRs; the wide variants need more.
+    if (pl.waves == 8 && (pl.ksteps == 4 || pl.mi == 4)) pl.waves = 4;
     auto split = [&]() { return (nksteps + pl.ksteps * pl.waves * pl.units - 1) / (pl.ksteps * pl.waves * pl.units); };
     pl.ksplit = split();
     while (pl.ksplit > kMaxKSplit) {

@@ -177,7 +177,7 @@ def _ffn_case(ops, K, H, seed):
 
 def test_ffn_small(ops):
     _ffn_case(ops, 256, 512, seed=20)
-    _ffn_case(ops, 1024, 2048 + 32, seed=30)
+    _ffn_case(ops, 1024, 2048 + 128, seed=30)
 
 
 def test_ffn_config4(ops):
