@@ -40,6 +40,7 @@ extern "C" {
 #define W4A16_ERR_WORKSPACE (-5)   /* workspace missing or smaller than *_workspace_bytes */
 #define W4A16_ERR_HIP (-6)         /* a HIP call failed; see w4a16_last_hip_error() */
 #define W4A16_ERR_TUNE (-7)        /* unknown tuning key or value out of range */
+#define W4A16_ERR_TIMEOUT (-8)     /* w4a16_workspace_check: a split-K reducer timed out */
 
 #define W4A16_ABI_VERSION 1
 
@@ -63,14 +64,21 @@ int awq_dequant_bf16(const int32_t *qweight, const int32_t *qzeros, const uint16
 
 /*
  * Workspace for the split-K GEMV / small-M GEMM and the FFN.  The caller allocates
- * `*_workspace_bytes` bytes of device memory once, clears it once with
+ * `*_workspace_bytes` bytes of device memory once, prepares it once with
  * w4a16_workspace_init, and may then reuse it for any number of calls that do not
- * overlap in time (each call leaves it cleared again).  Calls that run concurrently
+ * overlap in time (each call leaves it prepared again).  Calls that run concurrently
  * (different streams) need separate workspaces.
  */
 size_t w4a16_gemm_workspace_bytes(int M, int K, int N);
 size_t w4a16_ffn_workspace_bytes(int K, int H);
 int w4a16_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Health check (synchronises `stream`): W4A16_ERR_TIMEOUT if any split-K reducer of an
+ * earlier call on this workspace gave up waiting for a partial result (its bounded poll ran
+ * out; that call's output is invalid and the workspace must be re-initialised), else W4A16_OK.
+ */
+int w4a16_workspace_check(const void *workspace, void *stream);
 
 /*
  * Decode GEMV, M = 1: y[N] = bf16(x[K] . W).  fp32 accumulation, one bf16 rounding.
@@ -112,7 +120,8 @@ int w4a16_ffn_swiglu_bf16(const uint16_t *x,
 
 /*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
- * "gemv_ksteps", "gemv_waves", "gemv_units" (0 = built-in heuristic).  Process-wide.
+ * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units" (0 = built-in heuristic) and
+ * "gemv_spin_limit" (reducer poll bound).  Process-wide.
  */
 int w4a16_tune(const char *key, int value);
 

@@ -7,7 +7,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libw4a16_hip.so")
 
 OK = 0
-ERR_NULL, ERR_SHAPE, ERR_GROUP, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_TUNE = -1, -2, -3, -4, -5, -6, -7
+ERR_NULL, ERR_SHAPE, ERR_GROUP, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_TUNE, ERR_TIMEOUT = -1, -2, -3, -4, -5, -6, -7, -8
 
 # every symbol include/w4a16.h declares: name -> (restype, argtypes)
 _vp, _ci, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -19,6 +19,7 @@ SYMBOLS = {
     "w4a16_gemm_workspace_bytes": (_sz, [_ci, _ci, _ci]),
     "w4a16_ffn_workspace_bytes": (_sz, [_ci, _ci]),
     "w4a16_workspace_init": (_ci, [_vp, _sz, _vp]),
+    "w4a16_workspace_check": (_ci, [_vp, _vp]),
     "w4a16_gemv_bf16": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_gemm_bf16": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_ffn_swiglu_bf16": (_ci, [_vp] * 12 + [_ci, _ci, _ci, _vp, _sz, _vp]),

@@ -20,6 +20,7 @@ SOURCES = ["capi.hip", "dequant.hip", "stream.hip", "gemm.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
+    *os.environ.get("W4A16_EXTRA", "").split(),
     "--offload-arch=gfx950",
     "-O3",
     "-std=c++17",

@@ -23,7 +23,6 @@ int check_quant(const void *qweight, const void *qzeros, const void *scales, int
     if (!qweight || !qzeros || !scales) return W4A16_ERR_NULL;
     if (group != kGroup) return W4A16_ERR_GROUP;
     if (K <= 0 || N <= 0 || K % kGroup != 0 || N % n_mult != 0) return W4A16_ERR_SHAPE;
-    if (N / 32 > 16 * kCounterWords) return W4A16_ERR_SHAPE;
     if (misaligned(qweight) || misaligned(qzeros) || misaligned(scales)) return W4A16_ERR_ALIGN;
     return W4A16_OK;
 }
@@ -31,7 +30,8 @@ int check_quant(const void *qweight, const void *qzeros, const void *scales, int
 size_t round256(size_t v) { return (v + 255) & ~size_t(255); }
 
 size_t stream_partial_bytes(int M, int N, int nmat) {
-    return round256((size_t)nmat * kMaxKSplit * (size_t)(M < 16 ? M : 16) * (size_t)N * sizeof(float));
+    // tiles are at most 512 columns wide; a ragged last tile is stored in full
+    return round256((size_t)nmat * kMaxKSplit * (size_t)(M < 16 ? M : 16) * ((size_t)N + 512) * sizeof(float));
 }
 
 }  // namespace
@@ -50,6 +50,7 @@ const char *w4a16_strerror(int code) {
         case W4A16_ERR_WORKSPACE: return "workspace is NULL or too small";
         case W4A16_ERR_HIP: return "HIP call failed";
         case W4A16_ERR_TUNE: return "unknown tuning key or value out of range";
+        case W4A16_ERR_TIMEOUT: return "a split-K reducer gave up waiting for a partial result; the output is invalid";
         default: return "unknown error code";
     }
 }
@@ -68,21 +69,31 @@ int awq_dequant_bf16(const int32_t *qweight, const int32_t *qzeros, const uint16
 
 size_t w4a16_gemm_workspace_bytes(int M, int K, int N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
-    return kCounterBytes + stream_partial_bytes(M, N, 1);
+    return kHeaderBytes + stream_partial_bytes(M, N, 1);
 }
 
 size_t w4a16_ffn_workspace_bytes(int K, int H) {
     if (K <= 0 || H <= 0) return 0;
     const size_t a = stream_partial_bytes(1, H, 2), b = stream_partial_bytes(1, K, 1);
-    return kCounterBytes + (a > b ? a : b) + round256((size_t)H * sizeof(uint16_t));
+    return kHeaderBytes + (a > b ? a : b) + round256((size_t)H * sizeof(uint16_t));
 }
 
 int w4a16_workspace_init(void *workspace, size_t workspace_bytes, void *stream) {
     if (!workspace) return W4A16_ERR_NULL;
-    if (workspace_bytes < kCounterBytes) return W4A16_ERR_WORKSPACE;
+    if (workspace_bytes < kHeaderBytes) return W4A16_ERR_WORKSPACE;
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
-    hipError_t e = launch_fill_zero(workspace, kCounterBytes, static_cast<hipStream_t>(stream));
+    hipError_t e = launch_fill_workspace(workspace, workspace_bytes & ~size_t(3), static_cast<hipStream_t>(stream));
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_workspace_check(const void *workspace, void *stream) {
+    if (!workspace) return W4A16_ERR_NULL;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint32_t flag = 0;
+    hipError_t e = hipMemcpyAsync(&flag, workspace, sizeof(flag), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return hip_fail(e);
+    return flag ? W4A16_ERR_TIMEOUT : W4A16_OK;
 }
 
 int w4a16_gemm_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
@@ -137,12 +148,17 @@ int w4a16_ffn_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const 
 
 int w4a16_tune(const char *key, int value) {
     if (!key || value < 0) return W4A16_ERR_TUNE;
-    if (!strcmp(key, "gemv_ksteps")) {
+    if (!strcmp(key, "gemv_lw")) {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return W4A16_ERR_TUNE;
+        g_stream_tune.lw = value;
+    } else if (!strcmp(key, "gemv_ksteps")) {
         if (value != 0 && value != 1 && value != 2 && value != 4) return W4A16_ERR_TUNE;
         g_stream_tune.ksteps = value;
     } else if (!strcmp(key, "gemv_waves")) {
         if (value != 0 && value != 4 && value != 8) return W4A16_ERR_TUNE;
         g_stream_tune.waves = value;
+    } else if (!strcmp(key, "gemv_spin_limit")) {
+        g_stream_tune.spin_limit = value;
     } else if (!strcmp(key, "gemv_units")) {
         if (value > 64) return W4A16_ERR_TUNE;
         g_stream_tune.units = value;

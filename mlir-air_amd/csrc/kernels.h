@@ -7,26 +7,24 @@
 
 namespace w4a16 {
 
-// Layout of the caller-provided workspace: [kCounterWords uint32 arrival counters]
-// [fp32 split-K partials].  Counters are zero between calls.
-constexpr int kCounterWords = 4096;
-constexpr size_t kCounterBytes = kCounterWords * sizeof(uint32_t);
+// Layout of the caller-provided workspace: [kHeaderBytes header: word 0 counts poll
+// timeouts][fp32 split-K partial slots].  Between calls every slot holds 0xFFFFFFFF.
+constexpr size_t kHeaderBytes = 256;
 constexpr int kMaxKSplit = 32;
 
 struct StreamTune {
+    int lw = 0;       // packed words per lane per row: 1, 2 or 4 (tile = 128 * lw columns)
     int ksteps = 0;   // K-steps (32 rows) a wave loads per unit: 1, 2 or 4 (0 = heuristic)
     int waves = 0;    // waves per workgroup: 4 or 8
     int units = 0;    // units each wave processes back to back
+    int spin_limit = 0;   // reducer poll bound (0 = default); tiny values force the timeout path in tests
 };
 extern StreamTune g_stream_tune;
 
 struct StreamPlan {
-    int ksteps, waves, units, ksplit, ntiles, mi;
+    int lw, ksteps, waves, units, ksplit, ntiles, mi;
 };
 StreamPlan plan_stream(int M, int K, int N);
-
-// Epilogue selector for the streaming kernel.
-enum StreamEpilogue { kEpiStore = 0, kEpiSwiGLU = 1 };
 
 hipError_t launch_dequant(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, uint16_t *out,
                           int K, int N, hipStream_t stream);
@@ -40,6 +38,6 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
 hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
                                const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream);
 
-hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
+hipError_t launch_fill_workspace(void *ptr, size_t bytes, hipStream_t stream);
 
 }  // namespace w4a16

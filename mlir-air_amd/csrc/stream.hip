@@ -1,18 +1,19 @@
 // Split-K streaming W4A16 kernel for M <= 16 (decode GEMV, batched decode, SwiGLU front half).
 //
-// HBM-bound: every packed weight byte is read exactly once with 16-byte loads.  The
-// arithmetic runs on the matrix cores even at M = 1, because the fp32 VALU cannot keep
-// up with HBM: at 8 TB/s the chip has ~2.5 VALU lane-ops per weight, and a convert + FMA
-// path needs ~2.4.  Building MFMA operands costs ~1 op per weight and the MACs are free.
+// HBM-bound: every packed weight byte is read exactly once.  The arithmetic runs on the
+// matrix cores even at M = 1, because the fp32 VALU cannot keep up with HBM: at 8 TB/s the
+// chip has ~2.5 VALU lane-ops per weight and a convert + FMA path needs ~2.4.  Building MFMA
+// operands costs 1 op per weight and the MACs are free.
 //
 // Work decomposition
-//   tile   = 512 output columns = 16 lanes x one 16-byte chunk (32 columns) per lane
+//   tile   = 128 * LW output columns = 16 lanes x LW packed words (8 * LW columns) per lane
 //   K-step = 32 rows = one v_mfma_f32_16x16x32_bf16; lane (lg, ln) = (lane / 16, lane % 16)
 //            loads rows 8*lg .. 8*lg+7 of chunk ln, i.e. exactly the K-slice the MFMA B
-//            operand wants from that lane.  One load instruction covers 4 x 256 B segments.
-//   unit   = KSTEPS consecutive K-steps inside one quantisation group, loaded up front
+//            operand wants from that lane
+//   unit   = KSTEPS consecutive K-steps inside one quantisation group, all loads issued up
+//            front and consumed K-step by K-step as they land
 //   wave   = `units` units; workgroup = WAVES waves on one (tile, K-slice); the grid is
-//            (tiles x ksplit) with all K-slices of a tile on the same XCD.
+//            (tiles x ksplit) with all K-slices of a tile on the same XCD
 //
 // Operand construction.  For rows (k, k+1) and byte p of a packed word, v_perm_b32 builds
 // [0, byte_p(row k+1), 0, byte_p(row k)]; `& 0x000F000F | 0x43004300` turns the low nibbles
@@ -25,9 +26,17 @@
 // The M rows of x sit in MFMA rows 4*i + lg' (row m -> lane group m % 4, register m / 4) so
 // that for M <= 4 only accumulator register 0 is live in the group flush.
 //
-// Cross-wave combine goes through LDS, the cross-workgroup combine through fp32 partials in
-// the workspace; the last workgroup to arrive at a tile (arrival counter) sums the partials
-// in fixed order (deterministic), applies the epilogue and resets the counter.
+// Cross-wave combine goes through LDS.  Cross-workgroup combine: every workgroup of a tile
+// except the one with the highest block id stores its fp32 partial to the workspace and
+// exits; the highest one (the reducer) polls for those partials, adds them in fixed order
+// (deterministic), applies the epilogue and writes y.  A partial slot holds the sentinel
+// 0xFFFFFFFF ("empty") until its producer overwrites it, and the reducer puts the sentinel
+// back after reading, so the workspace is clean again when the kernel ends.  All slot
+// traffic uses agent-scope atomic loads/stores (served at the device coherence point, never
+// stale in an XCD's L2) and needs no fences: validity travels with each 32-bit value.  The
+// reducer is dispatched after its producers (workgroups are dispatched in block-id order), so
+// the producers never wait on anything and the poll terminates; it is bounded all the same
+// and reports a timeout through the workspace header instead of hanging.
 #include "common.h"
 #include "kernels.h"
 
@@ -37,30 +46,69 @@ StreamTune g_stream_tune;
 
 struct StreamParams {
     const uint16_t *x;
-    const u32x4 *qw[2];
-    const u32x4 *qz[2];
+    const uint32_t *qw[2];
+    const uint32_t *qz[2];
     const uint16_t *sc[2];
     uint16_t *y;
-    float *partial;
-    uint32_t *counters;
+    uint32_t *header;   // workspace header: word 0 = poll timeouts seen
+    float *partial;     // [nmat * ksplit][ntiles][M * tile columns]
     int M, K, N;
-    int nchunks;   // N / 32
-    int ntiles;    // ceil(nchunks / 16)
+    int nb;        // N / 8 packed words per row
+    int ntiles;    // ceil(N / tile columns)
     int ksplit;    // workgroups along K per tile
     int units;     // units per wave
     int nmat;      // 1, or 2 for gate/up with the SwiGLU epilogue
-    int slots;     // LDS combine slots (power of two, divides WAVES)
+    int spin_limit;
 };
 
-constexpr int kTileCols = 512;
-constexpr int kRowStride = 32 * 17;   // LDS floats per output row: [j (32)][ln (16) + 1 pad]
+constexpr uint32_t kEmpty = 0xFFFFFFFFu;
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// 16-byte slot access as two 8-byte atomics.
+#ifndef SLOT_ST_SCOPE
+#define SLOT_ST_SCOPE __HIP_MEMORY_SCOPE_AGENT
+#endif
+#ifndef SLOT_LD_SCOPE
+#define SLOT_LD_SCOPE __HIP_MEMORY_SCOPE_AGENT
+#endif
+__device__ __forceinline__ void slot_store(float *p, u32x4 v) {
+    uint64_t *q = reinterpret_cast<uint64_t *>(p);
+    __hip_atomic_store(q, (uint64_t)v[0] | ((uint64_t)v[1] << 32), __ATOMIC_RELAXED, SLOT_ST_SCOPE);
+    __hip_atomic_store(q + 1, (uint64_t)v[2] | ((uint64_t)v[3] << 32), __ATOMIC_RELAXED, SLOT_ST_SCOPE);
+}
+__device__ __forceinline__ u32x4 slot_load(const float *p) {
+    const uint64_t *q = reinterpret_cast<const uint64_t *>(p);
+    const uint64_t a = __hip_atomic_load(q, __ATOMIC_RELAXED, SLOT_LD_SCOPE);
+    const uint64_t b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, SLOT_LD_SCOPE);
+    return u32x4{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
+}
+__device__ __forceinline__ bool slot_full(u32x4 v) {
+    return v[0] != kEmpty && v[1] != kEmpty && v[2] != kEmpty && v[3] != kEmpty;
+}
 
 __device__ __forceinline__ float silu_tanh(float g) { return g * 0.5f * (tanhf(g * 0.5f) + 1.0f); }
 
-template <int KSTEPS, int WAVES, int MI>
-__global__ void __launch_bounds__(WAVES * 64) stream_kernel(const StreamParams p) {
+template <int LW>
+struct Words;
+template <>
+struct Words<4> { typedef u32x4 type; };
+template <>
+struct Words<2> { typedef u32x2 type; };
+template <>
+struct Words<1> { typedef uint32_t type __attribute__((ext_vector_type(1))); };
+
+// LW     packed words per lane per row: the tile is 16 lanes x 8*LW columns = 128*LW columns
+// KSTEPS K-steps per unit, WAVES waves per workgroup, MI live accumulator registers (M <= 4*MI)
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT>
+__global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParams p) {
+    constexpr int SLOTS = MI == 1 ? WAVES : (MI == 2 ? WAVES / 2 : WAVES / 4);   // LDS combine slots
+    typedef typename Words<LW>::type wvec;
+    constexpr int TC = 128 * LW;            // tile columns
+    constexpr int LC = 8 * LW;              // columns per lane
+    constexpr int ROWF = LC * 17;           // LDS floats per output row: [j (LC)][ln (16) + 1 pad]
+    constexpr int QPR = TC / 4;             // 4-column quads per output row
     extern __shared__ float red[];
-    __shared__ int s_last;
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -68,7 +116,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(const StreamParams p
     const int ln = lane & 15;
 
     // blockIdx -> (tile, matrix, K-slice); consecutive block ids go to consecutive XCDs, so
-    // the workgroups that share a tile (and its counter and partials) share one L2.
+    // the workgroups of one tile share an XCD and the reducer has the highest id of its tile.
     const int per_tile = p.nmat * p.ksplit;
     const int xcd = blockIdx.x & 7;
     const int local = blockIdx.x >> 3;
@@ -78,11 +126,12 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(const StreamParams p
     const int mat = sub / p.ksplit;
     const int kslice = sub % p.ksplit;
 
+    const int nchunks = p.nb / LW;
     const int chunk = tile * 16 + ln;
-    const int chunk_c = chunk < p.nchunks ? chunk : p.nchunks - 1;   // ragged tile: load in range, never written
-    const u32x4 *__restrict__ qw = p.qw[mat];
-    const u32x4 *__restrict__ qz = p.qz[mat];
-    const uint16_t *__restrict__ sc = p.sc[mat];
+    const int chunk_c = chunk < nchunks ? chunk : nchunks - 1;   // ragged tile: load in range, never written
+    const uint32_t *__restrict__ qw = p.qw[mat] + (size_t)chunk_c * LW;
+    const uint32_t *__restrict__ qz = p.qz[mat] + (size_t)chunk_c * LW;
+    const uint16_t *__restrict__ sc = p.sc[mat] + (size_t)chunk_c * LC;
 
     // x row held by this lane in the MFMA A operand (A row = ln): m = ln / 4 + 4 * (ln % 4).
     const int am = (ln >> 2) + 4 * (ln & 3);
@@ -92,10 +141,15 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(const StreamParams p
     const uint32_t ones_w = 0x3F803F80u;
     const u32x4 ones4 = {ones_w, ones_w, ones_w, ones_w};
     const bf16x8 ones = __builtin_bit_cast(bf16x8, ones4);
+    // Kept opaque so the compiler holds them in registers and fuses (v & mask) | magic into
+    // one v_and_or_b32 instead of two literal-operand instructions.
+    uint32_t nib_mask = 0x000F000Fu, magic = 0x43004300u;
+    asm volatile("" : "+s"(nib_mask));
+    asm volatile("" : "+v"(magic));
 
-    floatx4 yacc[32];
+    floatx4 yacc[LC];
 #pragma unroll
-    for (int t = 0; t < 32; ++t) yacc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < LC; ++t) yacc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const int nksteps = p.K >> 5;
     for (int u = 0; u < p.units; ++u) {
@@ -103,82 +157,95 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(const StreamParams p
         if (kstep0 >= nksteps) break;   // wave-uniform
         const int g = kstep0 >> 2;
 
-        u32x4 w[KSTEPS][8];
+        wvec w[KSTEPS][8];
         u32x4 av[KSTEPS];
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
             const size_t row0 = (size_t)(kstep0 + s) * 32 + 8 * lg;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) w[s][i] = __builtin_nontemporal_load(qw + (row0 + i) * p.nchunks + chunk_c);
             av[s] = *reinterpret_cast<const u32x4 *>(xrow + (size_t)(kstep0 + s) * 32);
-            if (!a_valid) av[s] = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                w[s][i] = __builtin_nontemporal_load(reinterpret_cast<const wvec *>(qw + (row0 + i) * p.nb));
         }
-        const u32x4 zw = qz[(size_t)g * p.nchunks + chunk_c];
-        u32x4 sv[4];
+        const wvec zw = *reinterpret_cast<const wvec *>(qz + (size_t)g * p.nb);
+        u32x4 sv[LW];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-            sv[q] = *reinterpret_cast<const u32x4 *>(sc + (size_t)g * p.N + (size_t)chunk_c * 32 + 8 * q);
+        for (int c = 0; c < LW; ++c) sv[c] = *reinterpret_cast<const u32x4 *>(sc + (size_t)g * p.N + 8 * c);
 
-        floatx4 acc[32];
 #pragma unroll
-        for (int t = 0; t < 32; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < KSTEPS; ++s)
+            if (!a_valid) av[s] = u32x4{0u, 0u, 0u, 0u};
         floatx4 xs = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+            xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av[s]), ones, xs, 0, 0, 0);
 
+        // WB packed words (8 * WB MFMA tiles) at a time: K-steps outer so that work starts as
+        // soon as a K-step's loads have landed, then the group flush of those words.
+        // acc[cc * 8 + pos]: word cb + cc, nibble position pos (= 2 * byte + nibble-in-byte).
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) {
-            const bf16x8 a = __builtin_bit_cast(bf16x8, av[s]);
-            xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ones, xs, 0, 0, 0);
+        for (int cb = 0; cb < LW; cb += WB) {
+            floatx4 acc[8 * WB];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+            for (int t = 0; t < 8 * WB; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    const uint32_t sel = 0x0C000C00u | ((4u + b) << 16) | (uint32_t)b;
-                    u32x4 lo, hi;
+            for (int s = 0; s < KSTEPS; ++s) {
+                const bf16x8 a = __builtin_bit_cast(bf16x8, av[s]);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const uint32_t pr = __builtin_amdgcn_perm(w[s][2 * v + 1][c], w[s][2 * v][c], sel);
-                        lo[v] = (pr & 0x000F000Fu) | 0x43004300u;
-                        hi[v] = ((pr >> 4) & 0x000F000Fu) | 0x43004300u;
+                for (int cc = 0; cc < WB; ++cc) {
+                    const int c = cb + cc;
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const uint32_t sel = 0x0C000C00u | ((4u + b) << 16) | (uint32_t)b;
+                        u32x4 lo, hi;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            const uint32_t pr = __builtin_amdgcn_perm(w[s][2 * v + 1][c], w[s][2 * v][c], sel);
+                            lo[v] = (pr & nib_mask) | magic;
+                            hi[v] = ((pr >> 4) & nib_mask) | magic;
+                        }
+                        const int t = cc * 8 + 2 * b;
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, lo), acc[t], 0, 0, 0);
+                        acc[t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, hi), acc[t + 1], 0, 0, 0);
                     }
-                    const int t = (c * 4 + b) * 2;
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, lo), acc[t], 0, 0, 0);
-                    acc[t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, hi), acc[t + 1], 0, 0, 0);
                 }
             }
-        }
-
-        // Group flush: tile t = (word c, nibble position pos = 2b + h) is natural column
-        // j = 8c + pack_order(pos) of this lane's chunk.
+            // Group flush.  Nibble positions (q, q + 4) of a word are natural columns (2q, 2q + 1),
+            // i.e. the two halves of scale word q; (zw >> 4q) & 0x000F000F | 0x43004300 is the bf16
+            // pair (128 + z) of the same two columns.  yacc[c * 8 + j] is natural column 8c + j.
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+            for (int cc = 0; cc < WB; ++cc) {
+                const int c = cb + cc;
 #pragma unroll
-            for (int pos = 0; pos < 8; ++pos) {
-                const int t = c * 8 + pos;
-                const int j = 8 * c + pack_order(pos);
-                const float zc = 128.0f + static_cast<float>((zw[c] >> (4 * pos)) & 0xFu);
-                const uint32_t sw = sv[j >> 3][(j & 7) >> 1];
-                const float sj = bf16_bits_to_float((j & 1) ? (sw >> 16) : (sw & 0xFFFFu));
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t zp = ((zw[c] >> (4 * q)) & nib_mask) | magic;
+                    const uint32_t sw = sv[c][q];
+                    const float z_lo = __builtin_bit_cast(float, zp << 16), z_hi = __builtin_bit_cast(float, zp & 0xFFFF0000u);
+                    const float s_lo = __builtin_bit_cast(float, sw << 16), s_hi = __builtin_bit_cast(float, sw & 0xFFFF0000u);
 #pragma unroll
-                for (int i = 0; i < MI; ++i) yacc[t][i] = fmaf(sj, fmaf(-zc, xs[i], acc[t][i]), yacc[t][i]);
+                    for (int i = 0; i < MI; ++i) {
+                        yacc[c * 8 + 2 * q][i] = fmaf(s_lo, fmaf(-z_lo, xs[i], acc[cc * 8 + q][i]), yacc[c * 8 + 2 * q][i]);
+                        yacc[c * 8 + 2 * q + 1][i] = fmaf(s_hi, fmaf(-z_hi, xs[i], acc[cc * 8 + q + 4][i]), yacc[c * 8 + 2 * q + 1][i]);
+                    }
+                }
             }
         }
     }
 
-    // ---- cross-wave combine in LDS: red[slot][m][j * 17 + ln] ----
-    const int slot_stride = p.M * kRowStride;
-    const int rounds = WAVES / p.slots;
-    for (int r = 0; r < rounds; ++r) {
-        if (wave / p.slots == r) {
-            float *dst = red + (wave % p.slots) * slot_stride;
+    // ---- cross-wave combine in LDS: red[slot][m][j * 17 + ln], j = natural column in the lane's chunk ----
+    const int slot_stride = p.M * ROWF;
 #pragma unroll
-            for (int t = 0; t < 32; ++t) {
-                const int j = 8 * (t >> 3) + pack_order(t & 7);
+    for (int r = 0; r < WAVES / SLOTS; ++r) {
+        if (wave / SLOTS == r) {
+            float *dst = red + (wave % SLOTS) * slot_stride;
+#pragma unroll
+            for (int j = 0; j < LC; ++j) {
 #pragma unroll
                 for (int i = 0; i < MI; ++i) {
                     const int m = lg + 4 * i;
                     if (m < p.M) {
-                        float *q = dst + m * kRowStride + j * 17 + ln;
-                        *q = (r == 0) ? yacc[t][i] : (*q + yacc[t][i]);
+                        float *q = dst + m * ROWF + j * 17 + ln;
+                        *q = (r == 0) ? yacc[j][i] : (*q + yacc[j][i]);
                     }
                 }
             }
@@ -186,71 +253,107 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(const StreamParams p
         __syncthreads();
     }
 
-    const bool direct = (per_tile == 1);
-    const int nelem = p.M * kTileCols;
-    const int col0 = tile * kTileCols;
-    for (int e = threadIdx.x; e < nelem; e += WAVES * 64) {
-        const int m = e >> 9;
-        const int col = e & (kTileCols - 1);
-        const int gcol = col0 + col;
-        if (gcol >= p.N) continue;
-        const float *src = red + m * kRowStride + (col & 31) * 17 + (col >> 5);
-        float v = 0.f;
-        for (int s = 0; s < p.slots; ++s) v += src[s * slot_stride];
-        if (direct)
-            p.y[(size_t)m * p.N + gcol] = float_to_bf16_bits(v);
-        else
-            store_agent(p.partial + ((size_t)(mat * p.ksplit + kslice) * p.M + m) * p.N + gcol, v);
-    }
-    if (direct) return;
-
-    // ---- cross-workgroup combine: last arrival at this tile reduces the partials ----
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(p.counters + tile, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (old == (uint32_t)per_tile - 1u);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    for (int e = threadIdx.x; e < nelem; e += WAVES * 64) {
-        const int m = e >> 9;
-        const int gcol = col0 + (e & (kTileCols - 1));
-        if (gcol >= p.N) continue;
-        float v0 = 0.f;
-        for (int ks = 0; ks < p.ksplit; ++ks) v0 += load_agent(p.partial + ((size_t)ks * p.M + m) * p.N + gcol);
-        if (p.nmat == 1) {
-            p.y[(size_t)m * p.N + gcol] = float_to_bf16_bits(v0);
+    // ---- workgroup result in 4-column quads; producers publish, the reducer gathers ----
+    const int nprod = per_tile - 1;
+    const bool reducer = (sub == nprod);
+    const int nquads = p.M * QPR;
+    const int col0 = tile * TC;
+    const size_t slice_stride = (size_t)p.ntiles * nquads * 4;                 // floats per (mat, kslice)
+    float *tile_partial = p.partial + (size_t)tile * nquads * 4;
+    for (int e = threadIdx.x; e < nquads; e += WAVES * 64) {
+        const int m = e / QPR;
+        const int col = (e % QPR) * 4;
+        floatx4 own = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float *src = red + m * ROWF + ((col + q) % LC) * 17 + ((col + q) / LC);
+#pragma unroll
+            for (int s = 0; s < SLOTS; ++s) own[q] += src[s * slot_stride];
+        }
+        float *slot0 = tile_partial + (size_t)e * 4;
+        if (!reducer) {
+            u32x4 bits = __builtin_bit_cast(u32x4, own);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) bits[q] = bits[q] == kEmpty ? 0x7FC00000u : bits[q];   // keep the sentinel unique
+            slot_store(slot0 + sub * slice_stride, bits);
+            continue;
+        }
+        // Reducer: fetch the producers' slots eight at a time (all loads of a round in flight
+        // together), repeat a round until its slots are all filled, then hand the slots back.
+        floatx4 sum0 = floatx4{0.f, 0.f, 0.f, 0.f}, sum1 = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int s0 = 0; s0 < nprod; s0 += 8) {
+            u32x4 v[8];
+            int spins = 0;
+            bool ok;
+            do {
+                ok = true;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (s0 + j < nprod) {
+                        v[j] = slot_load(slot0 + (s0 + j) * slice_stride);
+                        ok = ok && slot_full(v[j]);
+                    }
+                }
+                if (!ok && ++spins > p.spin_limit) {
+                    __hip_atomic_store(p.header, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+            } while (!ok);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                if (s0 + j < nprod) {
+                    slot_store(slot0 + (s0 + j) * slice_stride, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
+                    if (NMAT == 2 && s0 + j >= p.ksplit)
+                        sum1 += __builtin_bit_cast(floatx4, v[j]);
+                    else
+                        sum0 += __builtin_bit_cast(floatx4, v[j]);
+                }
+            }
+        }
+        floatx4 out;
+        if (NMAT == 2) {
+            sum1 += own;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float gate = bf16_bits_to_float(float_to_bf16_bits(sum0[q]));
+                const float up = bf16_bits_to_float(float_to_bf16_bits(sum1[q]));
+                out[q] = silu_tanh(gate) * up;
+            }
         } else {
-            float v1 = 0.f;
-            for (int ks = 0; ks < p.ksplit; ++ks)
-                v1 += load_agent(p.partial + ((size_t)(p.ksplit + ks) * p.M + m) * p.N + gcol);
-            const float gate = bf16_bits_to_float(float_to_bf16_bits(v0));
-            const float up = bf16_bits_to_float(float_to_bf16_bits(v1));
-            p.y[(size_t)m * p.N + gcol] = float_to_bf16_bits(silu_tanh(gate) * up);
+            out = sum0 + own;
+        }
+        if (col0 + col < p.N) {
+            uint2 o;
+            o.x = pack_bf16x2(out[0], out[1]);
+            o.y = pack_bf16x2(out[2], out[3]);
+            *reinterpret_cast<uint2 *>(p.y + (size_t)m * p.N + col0 + col) = o;
         }
     }
-    if (threadIdx.x == 0) __hip_atomic_store(p.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Launch shape: enough workgroups to cover 256 CUs a few times over, with every wave's
-// loads issued up front; K-split bounded so the fp32 partials stay a small fraction of
-// the weight bytes.
+// Launch shape.  Measured on MI355X (K = 4096, N = 11008): 256-column tiles (8-byte loads),
+// 8 waves per workgroup and a K-split of 4 are the fastest; a reducer fetches up to 8
+// producers' slots in one polling round, so the split is kept at or below 8 (4 for M > 4,
+// where the fp32 partials are M times larger) by giving each wave more units instead.
 StreamPlan plan_stream(int M, int K, int N) {
     StreamPlan pl;
     pl.mi = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
-    pl.ntiles = (N / 32 + 15) / 16;
     const int nksteps = K / 32;
-    pl.ksteps = M <= 4 ? 1 : 4;
+    pl.lw = M <= 4 ? 2 : 1;
+    pl.ksteps = 4;
     pl.waves = 8;
     pl.units = 1;
-    if (g_stream_tune.ksteps) pl.ksteps = g_stream_tune.ksteps;
-    if (g_stream_tune.waves) pl.waves = g_stream_tune.waves;
-    if (g_stream_tune.units) pl.units = g_stream_tune.units;
-    // 512-thread workgroups cap a wave at 256 VGPRs; the wide variants need more.
-    if (pl.waves == 8 && (pl.ksteps == 4 || pl.mi == 4)) pl.waves = 4;
+    if (g_stream_tune.lw) pl.lw = g_stream_tune.lw == 1 ? 1 : 2;
+    if (g_stream_tune.ksteps) pl.ksteps = g_stream_tune.ksteps == 2 ? 2 : 4;
+    if (g_stream_tune.waves) pl.waves = g_stream_tune.waves == 4 ? 4 : 8;
+    pl.ntiles = (N + 128 * pl.lw - 1) / (128 * pl.lw);
     auto split = [&]() { return (nksteps + pl.ksteps * pl.waves * pl.units - 1) / (pl.ksteps * pl.waves * pl.units); };
+    if (g_stream_tune.units) {
+        pl.units = g_stream_tune.units;
+    } else {
+        const int max_split = M <= 4 ? 8 : 4;
+        while (split() > max_split) ++pl.units;
+    }
     pl.ksplit = split();
     while (pl.ksplit > kMaxKSplit) {
         pl.units *= 2;
@@ -259,24 +362,32 @@ StreamPlan plan_stream(int M, int K, int N) {
     return pl;
 }
 
-template <int KSTEPS, int WAVES, int MI>
-static hipError_t launch_one(const StreamParams &p, int grid, size_t lds, hipStream_t stream) {
-    hipLaunchKernelGGL((stream_kernel<KSTEPS, WAVES, MI>), dim3(grid), dim3(WAVES * 64), lds, stream, p);
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT>
+static hipError_t launch_one(const StreamParams &p, int grid, hipStream_t stream) {
+    constexpr int SLOTS = MI == 1 ? WAVES : (MI == 2 ? WAVES / 2 : WAVES / 4);
+    const size_t lds = (size_t)SLOTS * p.M * 8 * LW * 17 * sizeof(float);
+    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT>), dim3(grid), dim3(WAVES * 64), lds, stream, p);
     return hipGetLastError();
 }
 
-template <int KSTEPS, int WAVES>
-static hipError_t launch_mi(int mi, const StreamParams &p, int grid, size_t lds, hipStream_t stream) {
+template <int LW, int WB, int KSTEPS, int WAVES>
+static hipError_t launch_mi(int mi, const StreamParams &p, int grid, hipStream_t stream) {
+    if (p.nmat == 2) return launch_one<LW, WB, KSTEPS, WAVES, 1, 2>(p, grid, stream);
     switch (mi) {
-        case 1: return launch_one<KSTEPS, WAVES, 1>(p, grid, lds, stream);
-        case 2: return launch_one<KSTEPS, WAVES, 2>(p, grid, lds, stream);
-        default: return launch_one<KSTEPS, WAVES, 4>(p, grid, lds, stream);
+        case 1: return launch_one<LW, WB, KSTEPS, WAVES, 1, 1>(p, grid, stream);
+        case 2: return launch_one<LW, WB, KSTEPS, WAVES, 2, 1>(p, grid, stream);
+        default: return launch_one<LW, WB, KSTEPS, WAVES, 4, 1>(p, grid, stream);
     }
 }
 
-template <int KSTEPS>
-static hipError_t launch_waves(int waves, int mi, const StreamParams &p, int grid, size_t lds, hipStream_t stream) {
-    return waves == 4 ? launch_mi<KSTEPS, 4>(mi, p, grid, lds, stream) : launch_mi<KSTEPS, 8>(mi, p, grid, lds, stream);
+template <int LW, int WB, int KSTEPS>
+static hipError_t launch_waves(int waves, int mi, const StreamParams &p, int grid, hipStream_t stream) {
+    return waves == 4 ? launch_mi<LW, WB, KSTEPS, 4>(mi, p, grid, stream) : launch_mi<LW, WB, KSTEPS, 8>(mi, p, grid, stream);
+}
+
+template <int LW, int WB>
+static hipError_t launch_ksteps(int ksteps, int waves, int mi, const StreamParams &p, int grid, hipStream_t stream) {
+    return ksteps == 2 ? launch_waves<LW, WB, 2>(waves, mi, p, grid, stream) : launch_waves<LW, WB, 4>(waves, mi, p, grid, stream);
 }
 
 hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
@@ -285,46 +396,42 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     const StreamPlan pl = plan_stream(M, K, N);
     StreamParams p;
     p.x = x;
-    p.qw[0] = reinterpret_cast<const u32x4 *>(qweight);
-    p.qz[0] = reinterpret_cast<const u32x4 *>(qzeros);
+    p.qw[0] = reinterpret_cast<const uint32_t *>(qweight);
+    p.qz[0] = reinterpret_cast<const uint32_t *>(qzeros);
     p.sc[0] = scales;
     p.nmat = up_qweight ? 2 : 1;
-    p.qw[1] = reinterpret_cast<const u32x4 *>(up_qweight ? up_qweight : qweight);
-    p.qz[1] = reinterpret_cast<const u32x4 *>(up_qzeros ? up_qzeros : qzeros);
+    p.qw[1] = reinterpret_cast<const uint32_t *>(up_qweight ? up_qweight : qweight);
+    p.qz[1] = reinterpret_cast<const uint32_t *>(up_qzeros ? up_qzeros : qzeros);
     p.sc[1] = up_scales ? up_scales : scales;
     p.y = y;
-    p.counters = reinterpret_cast<uint32_t *>(workspace);
-    p.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + kCounterBytes);
+    p.header = reinterpret_cast<uint32_t *>(workspace);
+    p.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + kHeaderBytes);
     p.M = M;
     p.K = K;
     p.N = N;
-    p.nchunks = N / 32;
+    p.nb = N / 8;
     p.ntiles = pl.ntiles;
     p.ksplit = pl.ksplit;
     p.units = pl.units;
-    // LDS slots: as many as fit in 64 KiB, power of two, at most one per wave.
-    int slots = pl.waves;
-    while (slots > 1 && (size_t)slots * M * kRowStride * sizeof(float) > 65536) slots >>= 1;
-    p.slots = slots;
-    const size_t lds = (size_t)slots * M * kRowStride * sizeof(float);
+    p.spin_limit = g_stream_tune.spin_limit > 0 ? g_stream_tune.spin_limit : (1 << 18);
     const int grid = ((pl.ntiles + 7) / 8) * 8 * p.nmat * pl.ksplit;
-    switch (pl.ksteps) {
-        case 1: return launch_waves<1>(pl.waves, pl.mi, p, grid, lds, stream);
-        case 2: return launch_waves<2>(pl.waves, pl.mi, p, grid, lds, stream);
-        default: return launch_waves<4>(pl.waves, pl.mi, p, grid, lds, stream);
-    }
+    return pl.lw == 1 ? launch_ksteps<1, 1>(pl.ksteps, pl.waves, pl.mi, p, grid, stream)
+                      : launch_ksteps<2, 2>(pl.ksteps, pl.waves, pl.mi, p, grid, stream);
 }
 
-__global__ void fill_zero_kernel(uint32_t *p, size_t nwords) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nwords; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
+// Workspace reset: header words zero, every partial slot "empty".
+__global__ void fill_workspace_kernel(uint32_t *p, size_t nwords, size_t header_words) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nwords; i += (size_t)gridDim.x * blockDim.x)
+        p[i] = i < header_words ? 0u : kEmpty;
 }
 
-hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream) {
+hipError_t launch_fill_workspace(void *ptr, size_t bytes, hipStream_t stream) {
     const size_t nwords = bytes / 4;
     int grid = (int)((nwords + 255) / 256);
-    if (grid > 2048) grid = 2048;
+    if (grid > 4096) grid = 4096;
     if (grid < 1) grid = 1;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, stream, reinterpret_cast<uint32_t *>(ptr), nwords);
+    hipLaunchKernelGGL(fill_workspace_kernel, dim3(grid), dim3(256), 0, stream, reinterpret_cast<uint32_t *>(ptr), nwords,
+                       kHeaderBytes / 4);
     return hipGetLastError();
 }
 
