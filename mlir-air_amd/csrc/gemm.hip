@@ -1,13 +1,23 @@
 // Prefill W4A16 GEMM for gfx950: y[M, N] = bf16(x[M, K] . W), M > 16.
 //
-// Compute-bound.  Each workgroup owns a BM x BN output tile and walks K in steps of BK.
-// Per step the x tile is copied to LDS and the packed weight tile is dequantised ONCE to
-// bf16 - bit-identical to the dense dequant kernel, W = bf16_rne((q - z) * s) - and written
-// to LDS in [n][k] order, so both MFMA operands are 16-byte ds_read_b128 of 8 consecutive k.
-// v_mfma_f32_32x32x16_bf16 accumulates in fp32; one bf16 rounding at the end.
+// Compute-bound.  A workgroup (4 waves) owns a 256 x 256 output tile and walks K in steps of
+// 64; each wave owns 128 x 128 of it as 4 x 4 v_mfma_f32_32x32x16_bf16 tiles (256 fp32
+// accumulators per lane, one wave per SIMD).  Per K step the x tile is copied to LDS and the
+// packed weight tile is dequantised ONCE per workgroup to bf16 - the same values the dense
+// dequant produces, W = bf16_rne((q - z) * s) - and stored [n][k], so both MFMA operands are
+// 16-byte LDS reads of 8 consecutive k.  LDS is double buffered (2 x 72 KiB of the 160 KiB):
+// while the MFMAs run on one buffer the next tile is dequantised into the other, and the
+// global loads for the tile after that are already in flight; one barrier per K step.
 //
-// Dequant work is shared by the whole M-tile: a thread takes the same packed word from 4
-// consecutive rows (same 8 columns), so each column's 4 k-values leave as one ds_write_b64.
+// LDS layout: rows of 64 bf16 padded to 144 B keep the 16-byte operand reads of 8
+// consecutive rows on distinct banks; the weight tile additionally XORs the 16-byte chunk
+// index with (n / 8) % 8 so that the dequant's 16-byte stores (one column, 8 k, from lanes
+// that differ in n / 8) spread over the banks as well.
+//
+// blockIdx -> tile: each XCD (blockIdx % 8) takes a contiguous range of tiles with N
+// fastest, so one XCD's L2 keeps an x panel resident while the weight panels stream by.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -15,9 +25,14 @@ namespace w4a16 {
 
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 64;
-constexpr int LDK = BK + 8;   // padded LDS row (bf16 elements): 144 B keeps ds_read_b128 conflict-free
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int LDK = BK + 8;                      // padded LDS row, bf16 elements (144 B)
 constexpr int kThreads = 256;
+#ifndef VALU_SLOTS
+#define VALU_SLOTS 5
+#endif
+constexpr int kStageElems = (BM + BN) * LDK;     // bf16 elements per stage
+constexpr size_t kLdsBytes = 2 * kStageElems * sizeof(uint16_t);
 
 struct GemmParams {
     const uint16_t *x;
@@ -29,118 +44,201 @@ struct GemmParams {
     int tiles_m, tiles_n;
 };
 
-__global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) uint16_t sA[BM * LDK];
-    __shared__ __attribute__((aligned(16))) uint16_t sB[BN * LDK];
+__global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;   // 2 x 2 waves, 64 x 64 each
+    const int wm = wave >> 1, wn = wave & 1;
 
-    // Each XCD (blockIdx % 8) walks a contiguous range of tiles, M fastest, so the
-    // workgroups sharing an L2 reuse the same weight tile across their M tiles.
     const int total = p.tiles_m * p.tiles_n;
     const int per_xcd = (total + 7) / 8;
     const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (tile >= total) return;
-    const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
+    const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
     const int m0 = tm * BM, n0 = tn * BN;
     const int nb = p.N >> 3;
 
-    // ---- global -> register staging assignments ----
-    // A: 128 rows x 64 k = 1024 x 16 B; thread takes 4 pieces: row = tid / 8 + 32 * i, kseg = tid % 8.
-    const int a_row = tid >> 3, a_seg = tid & 7;
-    // B: item = (octet of rows, word column); two threads per item (4 rows each).
-    const int b_col = tid & 15;          // word column inside the tile (8 columns)
-    const int b_quad = tid >> 4;         // 0..15: rows 4 * b_quad .. +3 of the K tile
+    // ---- staging assignments ----
+    // A: 256 rows x 8 chunks of 16 B; thread takes chunk tid % 8 of rows tid / 8 + 32 i.
+    const int a_chunk = tid & 7, a_row = tid >> 3;
+    const uint16_t *a_src[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        int row = m0 + a_row + 32 * i;
+        if (row >= p.M) row = p.M - 1;              // ragged M: load in range, never stored
+        a_src[i] = p.x + (size_t)row * p.K + 8 * a_chunk;
+    }
+    // B: thread takes packed word column tid % 32 (8 columns) for the 8 rows of octet tid / 32.
+    const int b_col = tid & 31, b_oct = tid >> 5;
     int b_word = (n0 >> 3) + b_col;
-    if (b_word >= nb) b_word = nb - 1;   // ragged N: load in range, never stored
+    if (b_word >= nb) b_word = nb - 1;              // ragged N
+    const uint32_t *b_src = p.qw + (size_t)(8 * b_oct) * nb + b_word;
+    const int b_chunk = b_oct ^ (b_col & 7);        // swizzled 16-byte chunk inside the LDS row
 
-    u32x4 ra[4];
-    uint32_t rb[4];
-    uint32_t rz;
+    u32x4 ra[8];
+    uint32_t rb[2][8];                              // two register sets: tiles kt + 1 and kt + 2
+    float zs[8], sf[8];                             // -z * s and s of this thread's 8 columns
+
+    auto load_a = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(a_src[i] + k0);
+    };
+    auto load_b = [&](int k0, uint32_t (&dst)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dst[i] = __builtin_nontemporal_load(b_src + (size_t)(k0 + i) * nb);
+    };
+    uint32_t raw_z;
     u32x4 rs;
-
-    auto load_tile = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int row = m0 + a_row + 32 * i;
-            if (row >= p.M) row = p.M - 1;
-            ra[i] = *reinterpret_cast<const u32x4 *>(p.x + (size_t)row * p.K + k0 + 8 * a_seg);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) rb[i] = p.qw[(size_t)(k0 + 4 * b_quad + i) * nb + b_word];
+    auto fetch_group = [&](int k0) {                // issue the loads; convert_group() consumes them later
         const int g = k0 / kGroup;
-        rz = p.qz[(size_t)g * nb + b_word];
+        raw_z = p.qz[(size_t)g * nb + b_word];
         rs = *reinterpret_cast<const u32x4 *>(p.sc + (size_t)g * p.N + 8 * (size_t)b_word);
     };
-
-    auto store_tile = [&]() {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<u32x4 *>(&sA[(a_row + 32 * i) * LDK + 8 * a_seg]) = ra[i];
-        float z[8], s[8], q[4][8];
-        unpack8_f32(rz, z);
+    auto convert_group = [&]() {
+        float z[8];
+        unpack8_f32(raw_z, z);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            s[2 * j] = bf16_bits_to_float(rs[j] & 0xFFFFu);
-            s[2 * j + 1] = bf16_bits_to_float(rs[j] >> 16);
+            sf[2 * j] = bf16_bits_to_float(rs[j] & 0xFFFFu);
+            sf[2 * j + 1] = bf16_bits_to_float(rs[j] >> 16);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) unpack8_f32(rb[i], q[i]);
+        for (int j = 0; j < 8; ++j) zs[j] = -z[j] * sf[j];   // exact: 4 x 8 significant bits
+    };
+    // x chunks [i0, i1) of the staged tile -> LDS
+    auto store_a = [&](uint16_t *st, int i0, int i1) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            uint2 v;
-            v.x = pack_bf16x2((q[0][j] - z[j]) * s[j], (q[1][j] - z[j]) * s[j]);
-            v.y = pack_bf16x2((q[2][j] - z[j]) * s[j], (q[3][j] - z[j]) * s[j]);
-            *reinterpret_cast<uint2 *>(&sB[(8 * b_col + j) * LDK + 4 * b_quad]) = v;
+        for (int i = i0; i < i1; ++i)
+            *reinterpret_cast<u32x4 *>(&st[(a_row + 32 * i) * LDK + 8 * a_chunk]) = ra[i];
+    };
+    // weight columns 2 * part, 2 * part + 1 (all 8 k of each) -> LDS.  q * s - z * s equals (q - z) * s exactly.
+    auto store_b = [&](uint16_t *st, const uint32_t (&src)[8], int part) {
+        uint16_t *sB = st + BM * LDK;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int j = 2 * part + h;              // natural column inside the packed word
+            const int sh = 4 * unpack_pos(j);
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = fmaf(static_cast<float>((src[i] >> sh) & 0xFu), sf[j], zs[j]);
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+            *reinterpret_cast<u32x4 *>(&sB[(8 * b_col + j) * LDK + 8 * b_chunk]) = o;
         }
     };
 
-    floatx16 acc[2][2];
+    floatx16 acc[4][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int frag_row = lane & 31;        // row (A) / column (B) inside a 32-wide MFMA tile
-    const int frag_k = 8 * (lane >> 5);    // k offset inside a 16-wide MFMA step
+    const int fr = lane & 31;          // row (A) / column (B) inside a 32-wide MFMA tile
+    const int fk = lane >> 5;          // which 8-k half of a 16-k MFMA step
+    // per-lane LDS offsets of the operand fragments (elements), without the k term
+    int a_off[4], b_off[4], b_sw[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a_off[i] = (wm * 128 + i * 32 + fr) * LDK;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = wn * 128 + j * 32 + fr;
+        b_off[j] = n * LDK;
+        b_sw[j] = (n >> 3) & 7;
+    }
 
-    load_tile(0);
-    for (int k0 = 0; k0 < p.K; k0 += BK) {
-        store_tile();
-        __syncthreads();
-        if (k0 + BK < p.K) load_tile(k0 + BK);
+    const int KT = p.K / BK;                        // even: K % 128 == 0
+    uint16_t *stage0 = lds, *stage1 = lds + kStageElems;
+
+    // Pipeline (stage = kt % 2, one barrier per K step).  While the MFMAs of tile kt run:
+    //   - x of tile kt + 1 is loaded (L2-resident panel) at the top of the step and stored to
+    //     the other stage in its last quarter;
+    //   - the packed weights of tile kt + 1, loaded during the previous step, are dequantised
+    //     into the other stage, a quarter per MFMA group;
+    //   - the packed weights of tile kt + 2 are loaded into the other register set.
+    // A step is one basic block (the flags are compile-time), and sched_group_barrier pins the
+    // interleaving: one wave per SIMD issues in order, so VALU / LDS / global instructions only
+    // overlap with the matrix pipe when they sit between MFMAs in program order.
+    load_a(0);
+    load_b(0, rb[0]);
+    fetch_group(0);
+    convert_group();
+    store_a(stage0, 0, 8);
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 16) {
-            bf16x8 a[2], b[2];
+    for (int part = 0; part < 4; ++part) store_b(stage0, rb[0], part);
+    load_b(BK, rb[1]);
+    __syncthreads();
+
+    auto read_frags = [&](const uint16_t *st, int kk, bf16x8 (&a)[4], bf16x8 (&b)[4]) {
+        const uint16_t *sA = st, *sB = st + BM * LDK;
+        const int chunk = 2 * kk + fk;
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                a[i] = *reinterpret_cast<const bf16x8 *>(&sA[(wm * 64 + i * 32 + frag_row) * LDK + kk + frag_k]);
+        for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const bf16x8 *>(&sA[a_off[i] + 8 * chunk]);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                b[j] = *reinterpret_cast<const bf16x8 *>(&sB[(wn * 64 + j * 32 + frag_row) * LDK + kk + frag_k]);
+        for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const bf16x8 *>(&sB[b_off[j] + 8 * (chunk ^ b_sw[j])]);
+    };
+
+    // NEXT: tile kt + 1 exists; AFTER: tile kt + 2 exists; ODD: kt is odd.  With BK = 64 a new
+    // quantisation group opens at every even tile: on odd kt tile kt + 1 opens one (convert the
+    // registers fetched a step ago), on even kt tile kt + 2 does (fetch them now).
+    auto step = [&](int kt, uint16_t *cur, uint16_t *nxt, uint32_t (&rb_next)[8], uint32_t (&rb_after)[8],
+                    auto NEXT, auto AFTER, auto ODD) {
+        bf16x8 fa[2][4], fb[2][4];
+        if (NEXT) load_a((kt + 1) * BK);
+        if (AFTER) {
+            load_b((kt + 2) * BK, rb_after);
+            if (!ODD) fetch_group((kt + 2) * BK);
+        }
+        if (NEXT && ODD) convert_group();
+        read_frags(cur, 0, fa[0], fb[0]);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+        for (int kk = 0; kk < 4; ++kk) {
+            if (kk < 3) read_frags(cur, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+            if (NEXT) {
+                store_b(nxt, rb_next, kk);
+                if (kk == 3) store_a(nxt, 0, 8);
+            }
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][i], fb[kk & 1][j], acc[i][j], 0, 0, 0);
+            // 16 MFMAs, each followed by a slice of the other work of this quarter
+#pragma unroll
+            for (int m = 0; m < 16; ++m) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // DS read
+                __builtin_amdgcn_sched_group_barrier(0x002, VALU_SLOTS, 0);   // VALU
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // DS write
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // VMEM read
+            }
         }
         __syncthreads();
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    int kt = 0;
+    for (; kt + 3 < KT; kt += 2) {
+        step(kt, stage0, stage1, rb[1], rb[0], T{}, T{}, F{});
+        step(kt + 1, stage1, stage0, rb[0], rb[1], T{}, T{}, T{});
     }
+    // KT is even: two steps remain
+    step(kt, stage0, stage1, rb[1], rb[0], T{}, F{}, F{});
+    step(kt + 1, stage1, stage0, rb[0], rb[1], F{}, F{}, T{});
 
     // D layout of the 32x32 MFMA: register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+        for (int j = 0; j < 4; ++j) {
+            const int col = n0 + wn * 128 + j * 32 + fr;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * fk + (r & 3);
                 if (row < p.M && col < p.N) p.y[(size_t)row * p.N + col] = float_to_bf16_bits(acc[i][j][r]);
             }
         }
@@ -150,6 +248,13 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmParams p) {
 
 hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
                                const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
     GemmParams p;
     p.x = x;
     p.qw = reinterpret_cast<const uint32_t *>(qweight);
@@ -163,7 +268,7 @@ hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const 
     p.tiles_n = (N + BN - 1) / BN;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL(gemm_kernel, dim3(grid), dim3(kThreads), 0, stream, p);
+    hipLaunchKernelGGL(gemm_kernel, dim3(grid), dim3(kThreads), kLdsBytes, stream, p);
     return hipGetLastError();
 }
 
