@@ -102,6 +102,19 @@ int w4a16_gemm_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qz
                     void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Decode FFN front half, batch 1: h[H] = bf16(silu(bf16(x . Wg)) * bf16(x . Wu)), both weight
+ * matrices streamed by one kernel.  Matches matvec_int4_swiglu_rms.cpu_reference
+ * (programming_examples/decode_ffn_swiglu/matvec_int4_swiglu_rms.py:501-516) without the
+ * RMSNorm prologue; the reference's interleaved gate/up rows are passed as two matrices.
+ * Workspace: w4a16_ffn_workspace_bytes(K, H).
+ */
+int w4a16_gemv_swiglu_bf16(const uint16_t *x,
+                           const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                           const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                           uint16_t *h, int K, int H, int group,
+                           void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Fused decode SwiGLU FFN, batch 1:
  *   g = bf16(x . Wg), u = bf16(x . Wu), h = bf16(silu(g) * u), y = bf16(h . Wd)
  * with silu(g) = g * 0.5 * (tanh(g / 2) + 1) in fp32; Wg, Wu are [K, H], Wd is [H, K].
@@ -121,7 +134,8 @@ int w4a16_ffn_swiglu_bf16(const uint16_t *x,
 /*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units" (0 = built-in heuristic) and
- * "gemv_spin_limit" (reducer poll bound).  Process-wide.
+ * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the
+ * timeout test: split-K producers do not publish).  Process-wide.
  */
 int w4a16_tune(const char *key, int value);
 

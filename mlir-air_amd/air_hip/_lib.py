@@ -22,6 +22,7 @@ SYMBOLS = {
     "w4a16_workspace_check": (_ci, [_vp, _vp]),
     "w4a16_gemv_bf16": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_gemm_bf16": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a16_gemv_swiglu_bf16": (_ci, [_vp] * 8 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_ffn_swiglu_bf16": (_ci, [_vp] * 12 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_tune": (_ci, [ctypes.c_char_p, _ci]),
 }

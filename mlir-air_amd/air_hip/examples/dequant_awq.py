@@ -1,0 +1,62 @@
+"""AWQ int4 -> bf16 dequant of a 1-D vector: out[i] = (q[i] - z[i // gs]) * s[i // gs]
+(counterpart of programming_examples/dequant_awq/dequant_awq.py).
+
+The GPU kernel dequantises AWQ matrices W[K, N]; the 1-D example maps onto it with K = n and
+one packed word (8 columns) per row that repeats the element, of which column 0 is returned."""
+
+import argparse
+
+import numpy as np
+
+from .. import awq, bf16
+from ..backend import HIPBackend, HIPRunner, HipModule
+
+
+def build_module(n, group_size=128, herd_n=4, **ignored):
+    if n % group_size:
+        raise ValueError("N must be divisible by group_size")
+    return HipModule("dequant_awq", K=n, N=8, gs=group_size)
+
+
+def pack_inputs(int4_vals, scales, zeros, n, group_size, herd_n=4):
+    q = np.repeat(np.asarray(int4_vals, dtype=np.uint8)[:, None], 8, axis=1)
+    z = np.repeat(np.asarray(zeros, dtype=np.uint8)[:, None], 8, axis=1)
+    s = np.repeat(bf16.bits_of(scales)[:, None], 8, axis=1)
+    return awq.pack_buffer(awq.pack_int4(q), awq.pack_int4(z), bf16.from_bits(s))
+
+
+def parse_args(argv=None):
+    p = argparse.ArgumentParser(prog="dequant_awq.py", description="AWQ-style int4 to bf16 dequantization example")
+    p.add_argument("-v", "--verbose", action="store_true")
+    p.add_argument("--n", type=int, default=1024)
+    p.add_argument("--group-size", type=int, default=128)
+    p.add_argument("--herd-n", type=int, default=4, dest="herd_n")
+    return p.parse_args(argv)
+
+
+def draw_inputs(args):
+    np.random.seed(0)
+    n_groups = args.n // args.group_size
+    int4_vals = np.random.randint(0, 16, args.n).astype(np.uint8)
+    scales = bf16.from_f32(np.random.uniform(0.01, 0.1, n_groups))
+    zeros = np.random.randint(7, 10, n_groups).astype(np.uint8)
+    return int4_vals, scales, zeros
+
+
+def dequant(int4_vals, scales, zeros, group_size):
+    """Run the 1-D dequant on the GPU and return bf16 bits [n]."""
+    n = len(int4_vals)
+    backend = HIPBackend()
+    invoker = backend.compile_and_load(build_module(n, group_size))
+    out = invoker(pack_inputs(int4_vals, scales, zeros, n, group_size), np.zeros((n, 8), np.uint16).view(bf16.BF16Array))[-1]
+    backend.unload()
+    return np.ascontiguousarray(bf16.bits_of(out)[:, 0]).view(bf16.BF16Array)
+
+
+def run(args, cpu_reference):
+    int4_vals, scales, zeros = draw_inputs(args)
+    ref = bf16.from_bits(cpu_reference(int4_vals, bf16.bits_of(scales), zeros, args.group_size))
+    got = dequant(int4_vals, scales, zeros, args.group_size)
+    ok = HIPRunner(verbose=args.verbose)._check_outputs([got], [ref], rtol=1e-1, atol=5e-2)
+    print("PASS!" if ok else "failed.")
+    return 0 if ok else -1

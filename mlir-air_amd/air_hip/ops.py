@@ -97,6 +97,22 @@ def w4a16_gemv(x, qweight, qzeros, scales, group=GROUP, out=None):
     return out
 
 
+def w4a16_swiglu(x, gate, up, group=GROUP):
+    """Decode FFN front half: h[H] = bf16(silu(bf16(x Wg)) * bf16(x Wu)); gate/up are (qweight, qzeros, scales)."""
+    lib = _lib.load_library()
+    _need_cuda(x, *gate, *up)
+    K = x.numel()
+    H = gate[0].shape[1] * 8
+    if gate[0].shape[0] != K or up[0].shape != gate[0].shape:
+        raise ValueError("w4a16_swiglu: gate and up must both be [K, H/8]")
+    h = torch.empty((H,), dtype=torch.bfloat16, device=x.device)
+    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device)
+    _lib.check(lib.w4a16_gemv_swiglu_bf16(
+        _ptr(_bits(x)), _ptr(gate[0]), _ptr(gate[1]), _ptr(_bits(gate[2])),
+        _ptr(up[0]), _ptr(up[1]), _ptr(_bits(up[2])), _ptr(h), K, H, group, _ptr(ws), ws.numel(), _stream()))
+    return h
+
+
 def ffn_swiglu(x, gate, up, down, group=GROUP, return_h=False):
     """Decode FFN: y = Wd(silu(x Wg) * (x Wu)); gate/up/down are (qweight, qzeros, scales)."""
     lib = _lib.load_library()

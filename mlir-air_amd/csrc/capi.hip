@@ -120,6 +120,23 @@ int w4a16_gemv_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qz
     return w4a16_gemm_bf16(x, qweight, qzeros, scales, y, 1, K, N, group, workspace, workspace_bytes, stream);
 }
 
+int w4a16_gemv_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
+                           const uint16_t *gate_scales, const int32_t *up_qweight, const int32_t *up_qzeros,
+                           const uint16_t *up_scales, uint16_t *h, int K, int H, int group, void *workspace,
+                           size_t workspace_bytes, void *stream) {
+    if (!x || !h) return W4A16_ERR_NULL;
+    int rc = check_quant(gate_qweight, gate_qzeros, gate_scales, K, H, group, 32);
+    if (rc) return rc;
+    rc = check_quant(up_qweight, up_qzeros, up_scales, K, H, group, 32);
+    if (rc) return rc;
+    if (misaligned(x) || misaligned(h)) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_ffn_workspace_bytes(K, H)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_stream(x, gate_qweight, gate_qzeros, gate_scales, up_qweight, up_qzeros, up_scales, h, 1, K, H,
+                                 workspace, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_ffn_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
                           const uint16_t *gate_scales, const int32_t *up_qweight, const int32_t *up_qzeros,
                           const uint16_t *up_scales, const int32_t *down_qweight, const int32_t *down_qzeros,
@@ -157,6 +174,8 @@ int w4a16_tune(const char *key, int value) {
     } else if (!strcmp(key, "gemv_waves")) {
         if (value != 0 && value != 4 && value != 8) return W4A16_ERR_TUNE;
         g_stream_tune.waves = value;
+    } else if (!strcmp(key, "gemv_skip_publish")) {
+        g_stream_tune.skip_publish = value ? 1 : 0;
     } else if (!strcmp(key, "gemv_spin_limit")) {
         g_stream_tune.spin_limit = value;
     } else if (!strcmp(key, "gemv_units")) {

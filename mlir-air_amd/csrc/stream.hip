@@ -59,6 +59,7 @@ struct StreamParams {
     int units;     // units per wave
     int nmat;      // 1, or 2 for gate/up with the SwiGLU epilogue
     int spin_limit;
+    int skip_publish;   // fault injection for tests: producers keep their partials to themselves
 };
 
 constexpr uint32_t kEmpty = 0xFFFFFFFFu;
@@ -275,7 +276,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             u32x4 bits = __builtin_bit_cast(u32x4, own);
 #pragma unroll
             for (int q = 0; q < 4; ++q) bits[q] = bits[q] == kEmpty ? 0x7FC00000u : bits[q];   // keep the sentinel unique
-            slot_store(slot0 + sub * slice_stride, bits);
+            if (!p.skip_publish) slot_store(slot0 + sub * slice_stride, bits);
             continue;
         }
         // Reducer: fetch the producers' slots eight at a time (all loads of a round in flight
@@ -413,6 +414,7 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.ntiles = pl.ntiles;
     p.ksplit = pl.ksplit;
     p.units = pl.units;
+    p.skip_publish = g_stream_tune.skip_publish;
     p.spin_limit = g_stream_tune.spin_limit > 0 ? g_stream_tune.spin_limit : (1 << 18);
     const int grid = ((pl.ntiles + 7) / 8) * 8 * p.nmat * pl.ksplit;
     return pl.lw == 1 ? launch_ksteps<1, 1>(pl.ksteps, pl.waves, pl.mi, p, grid, stream)

@@ -1,0 +1,178 @@
+"""GPU: the example entry points end to end (PASS! harness), the golden fixtures, full-size
+properties, and the host-forced failure path of the split-K reducer."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import make_awq, make_x
+from oracle import awq as oawq, reference as oref
+from oracle.bf16 import bf16_bits_to_f32
+
+pytestmark = pytest.mark.gpu
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def dev(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(a).cuda()
+
+
+def bits(t):
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def test_example_matvec_int4_packed(capsys):
+    from air_hip.examples import matvec_int4_packed as ex
+    for argv in (["--m", "256", "--k", "256"], ["--m", "2048", "--k", "2048"]):
+        print("example matvec", argv, flush=True)
+        assert ex.run(ex.parse_args(argv), oref.matvec_cpu_reference) == 0
+    assert "PASS!" in capsys.readouterr().out
+
+
+def test_example_matvec_small_vs_scalar_loop_reference(capsys):
+    from air_hip.examples import matvec_int4_packed as ex
+    print("example matvec scalar-loop reference", flush=True)
+    assert ex.run(ex.parse_args(["--m", "64", "--k", "256"]), oref.matvec_cpu_reference_loop) == 0
+    assert "PASS!" in capsys.readouterr().out
+
+
+def test_example_matvec_add(capsys):
+    from air_hip.examples import matvec_int4_packed_add as ex
+    print("example matvec add", flush=True)
+    assert ex.run(ex.parse_args(["--m", "2048", "--k", "2048"]), oref.matvec_add_cpu_reference) == 0
+    assert "PASS!" in capsys.readouterr().out
+
+
+def test_example_matmul(capsys):
+    from air_hip.examples import matmul_int4_packed as ex
+    for argv in (["--m", "64", "--k", "128", "--n", "128"], ["--m", "32", "--k", "2048", "--n", "2048"]):
+        print("example matmul", argv, flush=True)
+        assert ex.run(ex.parse_args(argv), oref.matmul_cpu_reference) == 0
+    assert "PASS!" in capsys.readouterr().out
+
+
+def test_example_swiglu_rms(capsys):
+    from air_hip.examples import matvec_int4_swiglu_rms as ex
+    print("example swiglu", flush=True)
+
+    def reference(a_q, a_s, a_z, rms_in):
+        return oref.swiglu_rms_cpu_reference(a_q, a_s, a_z, rms_in[0], rms_in[1])
+
+    assert ex.run(ex.parse_args(["--m", "4096", "--k", "2048"]), reference) == 0
+    assert "PASS!" in capsys.readouterr().out
+
+
+def test_example_dequant_1d_bit_exact(capsys):
+    from air_hip.examples import dequant_awq as ex
+    print("example dequant", flush=True)
+    args = ex.parse_args([])
+    assert ex.run(args, oawq.dequant_1d) == 0
+    q, s, z = ex.draw_inputs(args)
+    got = ex.dequant(q, s, z, args.group_size)
+    assert np.array_equal(np.asarray(got), oawq.dequant_1d(q, np.asarray(s), z, 128))
+    assert np.array_equal(np.asarray(got), np.load(os.path.join(G, "dequant1d_n1024_seed0.npz"))["out"])
+    capsys.readouterr()
+
+
+def test_kernels_against_golden_fixtures():
+    from air_hip import ops
+    print("golden fixtures", flush=True)
+    f = np.load(os.path.join(G, "gemv_m64_k256_seed42.npz"))
+    w = [dev(f["qweight"]), dev(f["qzeros"]), dev(f["scales"])]
+    assert np.array_equal(bits(ops.awq_dequant(*w)), f["W_bf16"])
+    y = bits(ops.w4a16_gemv(dev(f["B"]), *w)).astype(np.int32)
+    assert np.max(np.abs(y - f["D_f64"].astype(np.int32))) <= 1          # one bf16 ulp, no sign flips near zero here
+    f = np.load(os.path.join(G, "gemm_m32_k256_n64_seed42.npz"))
+    c = bits(ops.w4a16_gemm(dev(f["A"]), dev(f["qweight"]), dev(f["qzeros"]), dev(f["scales"])))
+    ok = oref.check_outputs(bf16_bits_to_f32(c), bf16_bits_to_f32(f["C_f64_rounded_w"]), rtol=2.0**-7, atol=2e-3)
+    assert ok
+    f = np.load(os.path.join(G, "ffn_k256_h128_seed7.npz"))
+    trip = lambda n: tuple(dev(a) for a in oawq.l1_to_awq(f[f"{n}_q"], f[f"{n}_s"], f[f"{n}_z"]))
+    yy, hh = ops.ffn_swiglu(dev(f["x"]), trip("gate"), trip("up"), trip("down"), return_h=True)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(hh)), bf16_bits_to_f32(f["h"]), rtol=0.15, atol=0.5, min_correlation=0.99)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(yy)), bf16_bits_to_f32(f["y"]), rtol=0.2, atol=2.0, min_correlation=0.99)
+    assert np.mean(bits(hh) != f["h"]) < 0.05
+
+
+def test_full_size_properties_one_hot_rows_reproduce_the_dequant():
+    """Config 1 and config 3 sizes: x = e_k makes every output row a dequantised weight row, so the
+    GEMV and the prefill GEMM must reproduce the dequant kernel's rows bit for bit."""
+    from air_hip import ops
+    print("full-size one-hot property", flush=True)
+    K, N = 4096, 11008
+    qw, qz, s = make_awq(K, N, seed=11)
+    w = [dev(qw), dev(qz), dev(s)]
+    dense = ops.awq_dequant(*w)
+    for k0 in (0, 127, 128, 2049, 4095):
+        x = torch.zeros(K, dtype=torch.bfloat16, device="cuda")
+        x[k0] = 1.0
+        assert torch.equal(ops.w4a16_gemv(x, *w).view(torch.int16), dense[k0].view(torch.int16)), k0
+    K, N, M = 4096, 14336, 2048
+    qw, qz, s = make_awq(K, N, seed=12)
+    w = [dev(qw), dev(qz), dev(s)]
+    dense = ops.awq_dequant(*w)
+    rows = torch.randperm(K, device="cuda")[:M]
+    x = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda")
+    x[torch.arange(M, device="cuda"), rows] = 1.0
+    y = ops.w4a16_gemm(x, *w)
+    assert torch.equal(y.view(torch.int16), dense[rows].view(torch.int16))
+    # scaling x by a power of two scales y exactly (no rounding changes)
+    xr = torch.from_numpy(make_x((16, K), seed=5).view(np.int16)).cuda().view(torch.bfloat16)
+    y1 = ops.w4a16_gemm(xr, *w)
+    y2 = ops.w4a16_gemm(xr * 4, *w)
+    assert torch.equal((y1.float() * 4).to(torch.bfloat16).view(torch.int16), y2.view(torch.int16))
+
+
+def test_reducer_timeout_is_reported_and_workspace_recovers():
+    """Fault injection from the host: split-K producers do not publish, so every reducer runs into its
+    (tiny) poll bound, gives up and flags the workspace; all waves exit normally."""
+    from air_hip import _lib, ops
+    print("reducer timeout path", flush=True)
+    lib = _lib.load_library()
+    K, N = 4096, 1024
+    qw, qz, s = make_awq(K, N, seed=21)
+    x = dev(make_x((K,), seed=22))
+    w = [dev(qw), dev(qz), dev(s)]
+    good = ops.w4a16_gemv(x, *w)
+    ws = ops.workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.w4a16_workspace_check(ws.data_ptr(), stream) == 0
+    try:
+        ops.tune("gemv_skip_publish", 1)
+        ops.tune("gemv_spin_limit", 8)
+        ops.w4a16_gemv(x, *w)
+        assert lib.w4a16_workspace_check(ws.data_ptr(), stream) == _lib.ERR_TIMEOUT
+    finally:
+        ops.tune("gemv_skip_publish", 0)
+        ops.tune("gemv_spin_limit", 0)
+    _lib.check(lib.w4a16_workspace_init(ws.data_ptr(), ws.numel(), stream))
+    assert lib.w4a16_workspace_check(ws.data_ptr(), stream) == 0
+    assert torch.equal(ops.w4a16_gemv(x, *w).view(torch.int16), good.view(torch.int16))
+
+
+def test_hip_graph_replay_matches_eager():
+    from air_hip import ops
+    print("graph replay", flush=True)
+    K, N = 4096, 11008
+    qw, qz, s = make_awq(K, N, seed=31)
+    w = [dev(qw), dev(qz), dev(s)]
+    xs = [dev(make_x((K,), seed=40 + i)) for i in range(3)]
+    x = xs[0].clone()
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        y = ops.w4a16_gemv(x, *w)          # warm-up on this stream (allocates its workspace)
+        st.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            ops.w4a16_gemv(x, *w, out=y)
+        for xi in xs:
+            x.copy_(xi)
+            g.replay()
+            st.synchronize()
+            want = ops.w4a16_gemv(xi, *w)
+            st.synchronize()
+            assert torch.equal(y.view(torch.int16), want.view(torch.int16))

@@ -1,0 +1,173 @@
+"""Host logic of the product package (no GPU): layout tools against the oracle, the runner's
+comparator, backend argument checks, and the C ABI's symbols and error paths."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from air_hip import _lib, awq, bf16
+from air_hip.backend import AirBackendError, HIPBackend, HIPRunner, HipModule
+from air_hip.examples import dequant_awq, matmul_int4_packed, matvec_int4_packed, matvec_int4_swiglu_rms
+from oracle import awq as oawq, reference as oref
+from oracle.bf16 import f32_to_bf16_bits
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_bf16_helpers_match_oracle():
+    rng = np.random.default_rng(0)
+    a = np.concatenate([rng.standard_normal(50000).astype(np.float32) * 3, np.array([3.0234375, 0.0, -0.0, np.inf], np.float32)])
+    assert np.array_equal(np.asarray(bf16.from_f32(a)), f32_to_bf16_bits(a))
+    assert np.array_equal(bf16.to_f32(bf16.from_f32(a)), oawq.bf16_bits_to_f32(f32_to_bf16_bits(a)))
+    assert bf16.is_bf16(bf16.from_f32(a)) and not bf16.is_bf16(a)
+
+
+def test_pack_unpack_and_layout_converters_match_oracle():
+    rng = np.random.default_rng(1)
+    nib = rng.integers(0, 16, size=(256, 64), dtype=np.uint8)
+    assert np.array_equal(awq.pack_int4(nib), oawq.pack_awq_int32(nib))
+    assert np.array_equal(awq.unpack_int4(awq.pack_int4(nib)), nib)
+    z = rng.integers(0, 16, size=(2, 64), dtype=np.uint8)
+    s = f32_to_bf16_bits(rng.uniform(0.005, 0.02, size=(2, 64)).astype(np.float32))
+    qw, qz = awq.pack_int4(nib), awq.pack_int4(z)
+    a_q, a_s, a_z = awq.l1_from_awq(qw, qz, s)
+    o_q, o_s, o_z = oawq.repack_hf_awq_linear(qw, qz, s, 128)
+    assert np.array_equal(a_q, o_q) and np.array_equal(np.asarray(a_s), o_s) and np.array_equal(a_z, o_z)
+    qw2, qz2, s2 = awq.awq_from_l1(a_q, a_s, a_z)
+    assert np.array_equal(qw2, qw) and np.array_equal(qz2, qz) and np.array_equal(np.asarray(s2), s)
+    with pytest.raises(ValueError):
+        awq.pack_int4(nib[:, :60])
+
+
+def test_packed_buffer_round_trip_and_alignment():
+    rng = np.random.default_rng(2)
+    K, N = 256, 96
+    qw = awq.pack_int4(rng.integers(0, 16, size=(K, N), dtype=np.uint8))
+    qz = awq.pack_int4(rng.integers(0, 16, size=(K // 128, N), dtype=np.uint8))
+    s = f32_to_bf16_bits(rng.uniform(0.005, 0.02, size=(K // 128, N)).astype(np.float32))
+    buf = awq.pack_buffer(qw, qz, s)
+    lay = awq.packed_layout(K, N)
+    assert buf.size == lay["total"] and lay["z_off"] % 256 == 0 and lay["s_off"] % 256 == 0
+    q2, z2, s2 = awq.unpack_buffer(buf, K, N)
+    assert np.array_equal(q2, qw) and np.array_equal(z2, qz) and np.array_equal(np.asarray(s2), s)
+    with pytest.raises(ValueError):
+        awq.unpack_buffer(buf[:-1], K, N)
+
+
+def test_interleave_round_trip_matches_oracle():
+    rng = np.random.default_rng(3)
+    def l1(rows):
+        q = rng.integers(0, 256, size=(rows, 64), dtype=np.uint8)
+        return q, bf16.from_bits(rng.integers(0, 2**15, size=(1, rows)).astype(np.uint16)), rng.integers(0, 16, size=(1, rows), dtype=np.uint8)
+    g, u = l1(8), l1(8)
+    a_q, a_s, a_z = awq.interleave_rows(g, u)
+    o_q, o_s, o_z = oref.interleave_gate_up((g[0], np.asarray(g[1]), g[2]), (u[0], np.asarray(u[1]), u[2]))
+    assert np.array_equal(a_q, o_q) and np.array_equal(np.asarray(a_s), o_s) and np.array_equal(a_z, o_z)
+    g2, u2 = awq.deinterleave_rows(a_q, a_s, a_z)
+    assert np.array_equal(g2[0], g[0]) and np.array_equal(np.asarray(u2[1]), np.asarray(u[1])) and np.array_equal(u2[2], u[2])
+
+
+def test_examples_draw_order_and_packing():
+    a = matvec_int4_packed.parse_args(["--m", "64", "--k", "256"])
+    A_q, A_s, A_z, B = matvec_int4_packed.draw_inputs(a)
+    f = np.load(os.path.join(ROOT, "tests", "golden", "gemv_m64_k256_seed42.npz"))
+    assert np.array_equal(A_q, f["A_q"]) and np.array_equal(np.asarray(A_s), f["A_s"]) and np.array_equal(A_z, f["A_z"])
+    assert np.array_equal(np.asarray(B), f["B"])
+    buf = matvec_int4_packed.pack_inputs(A_q, A_s, A_z, 64, 256, 128)
+    qw, qz, s = awq.unpack_buffer(buf, 256, 64)
+    assert np.array_equal(qw, f["qweight"]) and np.array_equal(qz, f["qzeros"])
+    assert str(matvec_int4_packed.build_module(64, 256)) == "hip.module @matvec_int4 {M = 1, K = 256, N = 64, gs = 128}"
+    assert matmul_int4_packed.build_module(32, 256, 64, 128, 16, 128, 128, 16, 2, 4) == HipModule("matmul_int4", K=256, N=64, M=32)
+    assert matvec_int4_swiglu_rms.build_module(128, 256).N == 64
+    d = dequant_awq.parse_args([])
+    q, sc, z = dequant_awq.draw_inputs(d)
+    g = np.load(os.path.join(ROOT, "tests", "golden", "dequant1d_n1024_seed0.npz"))
+    assert np.array_equal(q, g["int4_vals"]) and np.array_equal(np.asarray(sc), g["scales"]) and np.array_equal(z, g["zeros"])
+    # RMSNorm prologue on the host equals the oracle's
+    args = matvec_int4_swiglu_rms.parse_args(["--m", "32", "--k", "256"])
+    *_, RMS_in = matvec_int4_swiglu_rms.draw_inputs(args)
+    bits = bf16.bits_of(RMS_in)
+    assert np.array_equal(np.asarray(matvec_int4_swiglu_rms.rms_norm(RMS_in)), f32_to_bf16_bits(oref.rms_norm_bf16(bits[0], bits[1])))
+
+
+def test_runner_comparator_semantics_match_reference_restatement(capsys):
+    r = HIPRunner()
+    e = np.linspace(1, 2, 1000)
+    a = e.copy()
+    a[:5] += 1.0
+    for kw in (dict(rtol=0.1, atol=0.05), dict(rtol=0.1, atol=0.05, max_mismatch_percentage=0.5),
+               dict(rtol=0.1, atol=0.05, max_mismatch_percentage=0.49), dict(rtol=0.1, atol=0.05, min_correlation=0.999)):
+        assert r._check_outputs([a], [e], **kw) == oref.check_outputs(a, e, **kw), kw
+    assert not r._check_outputs([np.ones(10)], [np.ones(10)], rtol=1, atol=1, min_correlation=0.5)   # NaN correlation
+    # bf16 outputs are compared as floats, integers exactly
+    eb = bf16.from_f32(np.array([1.0, 2.0, 3.0], np.float32))
+    ab = bf16.from_f32(np.array([1.0, 2.0, 3.02], np.float32))
+    assert r._check_outputs([ab], [eb], rtol=0.1, atol=0.05)
+    assert not r._check_outputs([np.array([1, 2, 3])], [np.array([1, 2, 4])])
+    capsys.readouterr()
+
+
+def test_backend_compile_rejects_bad_modules_and_load_needs_gpu():
+    b = HIPBackend()
+    for bad in (HipModule("matvec_int4", K=100, N=64), HipModule("matvec_int4", K=128, N=40),
+                HipModule("matvec_int4", K=128, N=64, gs=64), HipModule("nope", K=128, N=64),
+                HipModule("matmul_int4", K=128, N=64, M=0)):
+        with pytest.raises(AirBackendError):
+            b.compile(bad)
+    with pytest.raises(AirBackendError):
+        b.compile("not a module")
+    art = b.compile(HipModule("dequant_awq", K=128, N=40))
+    import torch
+    if not torch.cuda.is_available():
+        with pytest.raises(AirBackendError):
+            b.load(art)
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "w4a16.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(?:int|size_t|const char \*)\s*\*?(\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load_library()
+    names = _declared_functions()
+    assert "w4a16_gemv_bf16" in names and "awq_dequant_bf16" in names and len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/w4a16.h but not exported"
+        assert n in _lib.SYMBOLS, f"{n} has no ctypes prototype"
+    assert lib.w4a16_abi_version() == 1
+    assert lib.w4a16_strerror(0) == b"ok" and b"128" in lib.w4a16_strerror(_lib.ERR_GROUP)
+
+
+def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
+    lib = _lib.load_library()
+    P = 0x10000   # fake, aligned, never dereferenced: validation fails first
+    assert lib.awq_dequant_bf16(None, P, P, P, 128, 8, 128, None) == _lib.ERR_NULL
+    assert lib.awq_dequant_bf16(P, P, P, None, 128, 8, 128, None) == _lib.ERR_NULL
+    assert lib.awq_dequant_bf16(P, P, P, P, 100, 8, 128, None) == _lib.ERR_SHAPE
+    assert lib.awq_dequant_bf16(P, P, P, P, 128, 12, 128, None) == _lib.ERR_SHAPE
+    assert lib.awq_dequant_bf16(P, P, P, P, 128, 8, 64, None) == _lib.ERR_GROUP
+    assert lib.awq_dequant_bf16(P + 4, P, P, P, 128, 8, 128, None) == _lib.ERR_ALIGN
+    ws = lib.w4a16_gemm_workspace_bytes(1, 128, 32)
+    assert ws > 0 and lib.w4a16_gemm_workspace_bytes(0, 128, 32) == 0
+    assert lib.w4a16_gemv_bf16(P, P, P, P, P, 128, 8, 128, P, ws, None) == _lib.ERR_SHAPE      # GEMV needs N % 32 == 0
+    assert lib.w4a16_gemv_bf16(P, P, P, P, P, 128, 32, 128, None, ws, None) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_gemv_bf16(P, P, P, P, P, 128, 32, 128, P, ws - 1, None) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_gemm_bf16(P, P, P, P, P, 0, 128, 32, 128, P, ws, None) == _lib.ERR_SHAPE
+    assert lib.w4a16_gemm_bf16(None, P, P, P, P, 4, 128, 32, 128, P, ws, None) == _lib.ERR_NULL
+    fws = lib.w4a16_ffn_workspace_bytes(128, 256)
+    args = [P] * 10 + [P, None, 128, 256, 128, P, fws, None]
+    bad = list(args)
+    bad[13] = 200                                                                              # H not a multiple of 128
+    assert lib.w4a16_ffn_swiglu_bf16(*bad) == _lib.ERR_SHAPE
+    bad = list(args)
+    bad[16] = fws - 1
+    assert lib.w4a16_ffn_swiglu_bf16(*bad) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_workspace_init(None, 1024, None) == _lib.ERR_NULL
+    assert lib.w4a16_workspace_init(P, 16, None) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_tune(b"no_such_key", 1) == _lib.ERR_TUNE and lib.w4a16_tune(b"gemv_waves", 0) == 0
+    with pytest.raises(_lib.W4A16Error):
+        _lib.check(_lib.ERR_ALIGN)
