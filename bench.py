@@ -240,12 +240,23 @@ def main():
     ap.add_argument("--workload", default="gemv", choices=list(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configs")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch one device copy of 256 MiB (a dispatch of known traffic that calibrates "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures the single-GPU W4A16 kernels; --gpus must be 1 "
               "(this build has no multi-GPU path and every box has one GPU)", file=sys.stderr)
         sys.exit(2)
 
+    if a.copy_probe:
+        import torch
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     main_res = run_workload(a.workload, a.steps, a.warmup, not a.no_cpu_baseline)
     name = a.workload
     sec = main_res["cold_us"] * 1e-6
