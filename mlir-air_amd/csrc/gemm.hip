@@ -9,10 +9,16 @@
 // while the MFMAs run on one buffer the next tile is dequantised into the other, and the
 // global loads for the tile after that are already in flight; one barrier per K step.
 //
-// LDS layout: rows of 64 bf16 padded to 144 B keep the 16-byte operand reads of 8
-// consecutive rows on distinct banks; the weight tile additionally XORs the 16-byte chunk
-// index with (n / 8) % 8 so that the dequant's 16-byte stores (one column, 8 k, from lanes
-// that differ in n / 8) spread over the banks as well.
+// LDS layout (checked with a ds_read_b128 / ds_write_b128 timing probe and SQ_LDS_BANK_CONFLICT;
+// the LDS behaves as 64 banks of 4 B: a read pass is 16 lanes x 16 B, a write pass 8 lanes x 16 B).
+// x tile: rows of 64 bf16 padded to 144 B: operand reads of 16 consecutive rows and the copy's
+// row-contiguous stores are conflict-free.  Weight tile [n][k]: rows padded to 160 B and the
+// 16-byte chunk index XORed with (n / 8) % 8.  Reads (lanes = 16 consecutive n, same chunk): 160 n
+// covers the even 16-byte slots of a 256-byte window for n = 0..7 and the XOR flips bit 0 for
+// n = 8..15, which takes the odd slots.  Dequant stores (lanes = same column j of consecutive
+// packed words, n = 8 * word + j): 1280 * word is 0 mod 128, so the slot is chunk ^ word % 8,
+// distinct over 8 lanes; and the 8 columns of a lane are one base address plus j * 160 B.
+// With 144-byte rows the same XOR cost 512 conflict cycles per K step on the weight operand reads.
 //
 // blockIdx -> tile: each XCD (blockIdx % 8) takes a contiguous range of tiles with N
 // fastest, so one XCD's L2 keeps an x panel resident while the weight panels stream by.
@@ -26,12 +32,13 @@ namespace w4a16 {
 namespace {
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int LDK = BK + 8;                      // padded LDS row, bf16 elements (144 B)
+constexpr int LDA = BK;                          // x tile rows are unpadded (128 B), chunks XOR-swizzled
+constexpr int LDB = BK + 16;                     // padded LDS row of the weight tile (160 B), chunks XOR-swizzled
 constexpr int kThreads = 256;
 #ifndef VALU_SLOTS
 #define VALU_SLOTS 5
 #endif
-constexpr int kStageElems = (BM + BN) * LDK;     // bf16 elements per stage
+constexpr int kStageElems = BM * LDA + BN * LDB; // bf16 elements per stage
 constexpr size_t kLdsBytes = 2 * kStageElems * sizeof(uint16_t);
 
 struct GemmParams {
@@ -61,33 +68,44 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
     const int nb = p.N >> 3;
 
     // ---- staging assignments ----
-    // A: 256 rows x 8 chunks of 16 B; thread takes chunk tid % 8 of rows tid / 8 + 32 i.
-    const int a_chunk = tid & 7, a_row = tid >> 3;
-    const uint16_t *a_src[8];
+    // x tile: copied global -> LDS without passing through registers (global_load_lds_dwordx4).
+    // One wave instruction fills 1 KiB of LDS linearly with lane l's 16 bytes at 16 * l, i.e. 8
+    // rows of 128 B; lane l = (row l / 8, slot l % 8) fetches chunk slot ^ row % 8 of its row, so
+    // that chunk c of row r sits at slot c ^ r % 8 (the operand reads of consecutive rows are then
+    // conflict-free without padding).  Wave w, instruction i covers rows 32 i + 8 w .. + 7.
+    const int a_slot = lane & 7, a_sub = lane >> 3;
+    uint32_t a_voff[8];                             // byte offsets from x + m0 * K + k0
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        int row = m0 + a_row + 32 * i;
-        if (row >= p.M) row = p.M - 1;              // ragged M: load in range, never stored
-        a_src[i] = p.x + (size_t)row * p.K + 8 * a_chunk;
+        int row = 32 * i + 8 * wave + a_sub;
+        if (m0 + row >= p.M) row = p.M - 1 - m0;    // ragged M: load in range, never stored
+        a_voff[i] = (uint32_t)(((size_t)row * p.K + 8 * (a_slot ^ a_sub)) * sizeof(uint16_t));
     }
-    // B: thread takes packed word column tid % 32 (8 columns) for the 8 rows of octet tid / 32.
+    const char *a_base = reinterpret_cast<const char *>(p.x + (size_t)m0 * p.K);
+    // weight tile: thread takes packed word column tid % 32 (8 columns) for the 8 rows of octet tid / 32.
     const int b_col = tid & 31, b_oct = tid >> 5;
     int b_word = (n0 >> 3) + b_col;
     if (b_word >= nb) b_word = nb - 1;              // ragged N
-    const uint32_t *b_src = p.qw + (size_t)(8 * b_oct) * nb + b_word;
-    const int b_chunk = b_oct ^ (b_col & 7);        // swizzled 16-byte chunk inside the LDS row
+    const uint32_t b_voff = (uint32_t)(((size_t)(8 * b_oct) * nb + b_word - (n0 >> 3)) * sizeof(uint32_t));
+    const char *b_base = reinterpret_cast<const char *>(p.qw + (n0 >> 3));
+    const int b_chunk = b_oct ^ (b_col & 7);        // swizzled 16-byte chunk inside the LDS row: oct ^ (n / 8) % 8
 
-    u32x4 ra[8];
     uint32_t rb[2][8];                              // two register sets: tiles kt + 1 and kt + 2
     float zs[8], sf[8];                             // -z * s and s of this thread's 8 columns
 
-    auto load_a = [&](int k0) {
+    auto dma_a = [&](uint16_t *st, int k0) {
+        const char *src = a_base + (size_t)k0 * sizeof(uint16_t);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(a_src[i] + k0);
+        for (int i = 0; i < 8; ++i)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(src + a_voff[i]),
+                (__attribute__((address_space(3))) void *)(st + (32 * i + 8 * wave) * LDA), 16, 0, 0);
     };
     auto load_b = [&](int k0, uint32_t (&dst)[8]) {
+        const char *src = b_base + (size_t)k0 * nb * sizeof(uint32_t);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) dst[i] = __builtin_nontemporal_load(b_src + (size_t)(k0 + i) * nb);
+        for (int i = 0; i < 8; ++i)
+            dst[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(src + (size_t)i * nb * sizeof(uint32_t) + b_voff));
     };
     uint32_t raw_z;
     u32x4 rs;
@@ -107,15 +125,9 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) zs[j] = -z[j] * sf[j];   // exact: 4 x 8 significant bits
     };
-    // x chunks [i0, i1) of the staged tile -> LDS
-    auto store_a = [&](uint16_t *st, int i0, int i1) {
-#pragma unroll
-        for (int i = i0; i < i1; ++i)
-            *reinterpret_cast<u32x4 *>(&st[(a_row + 32 * i) * LDK + 8 * a_chunk]) = ra[i];
-    };
     // weight columns 2 * part, 2 * part + 1 (all 8 k of each) -> LDS.  q * s - z * s equals (q - z) * s exactly.
     auto store_b = [&](uint16_t *st, const uint32_t (&src)[8], int part) {
-        uint16_t *sB = st + BM * LDK;
+        uint16_t *sB = st + BM * LDA;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int j = 2 * part + h;              // natural column inside the packed word
@@ -126,7 +138,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
             u32x4 o;
 #pragma unroll
             for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
-            *reinterpret_cast<u32x4 *>(&sB[(8 * b_col + j) * LDK + 8 * b_chunk]) = o;
+            *reinterpret_cast<u32x4 *>(&sB[(8 * b_col + j) * LDB + 8 * b_chunk]) = o;
         }
     };
 
@@ -142,12 +154,13 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
     const int fk = lane >> 5;          // which 8-k half of a 16-k MFMA step
     // per-lane LDS offsets of the operand fragments (elements), without the k term
     int a_off[4], b_off[4], b_sw[4];
+    const int a_sw = fr & 7;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a_off[i] = (wm * 128 + i * 32 + fr) * LDK;
+    for (int i = 0; i < 4; ++i) a_off[i] = (wm * 128 + i * 32 + fr) * LDA;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int n = wn * 128 + j * 32 + fr;
-        b_off[j] = n * LDK;
+        b_off[j] = n * LDB;
         b_sw[j] = (n >> 3) & 7;
     }
 
@@ -163,21 +176,21 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
     // A step is one basic block (the flags are compile-time), and sched_group_barrier pins the
     // interleaving: one wave per SIMD issues in order, so VALU / LDS / global instructions only
     // overlap with the matrix pipe when they sit between MFMAs in program order.
-    load_a(0);
+    dma_a(stage0, 0);
     load_b(0, rb[0]);
     fetch_group(0);
     convert_group();
-    store_a(stage0, 0, 8);
 #pragma unroll
     for (int part = 0; part < 4; ++part) store_b(stage0, rb[0], part);
     load_b(BK, rb[1]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the x tile copy writes LDS behind the compiler's back
     __syncthreads();
 
     auto read_frags = [&](const uint16_t *st, int kk, bf16x8 (&a)[4], bf16x8 (&b)[4]) {
-        const uint16_t *sA = st, *sB = st + BM * LDK;
+        const uint16_t *sA = st, *sB = st + BM * LDA;
         const int chunk = 2 * kk + fk;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const bf16x8 *>(&sA[a_off[i] + 8 * chunk]);
+        for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const bf16x8 *>(&sA[a_off[i] + 8 * (chunk ^ a_sw)]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const bf16x8 *>(&sB[b_off[j] + 8 * (chunk ^ b_sw[j])]);
     };
@@ -188,7 +201,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
     auto step = [&](int kt, uint16_t *cur, uint16_t *nxt, uint32_t (&rb_next)[8], uint32_t (&rb_after)[8],
                     auto NEXT, auto AFTER, auto ODD) {
         bf16x8 fa[2][4], fb[2][4];
-        if (NEXT) load_a((kt + 1) * BK);
+        if (NEXT) dma_a(nxt, (kt + 1) * BK);
         if (AFTER) {
             load_b((kt + 2) * BK, rb_after);
             if (!ODD) fetch_group((kt + 2) * BK);
@@ -198,10 +211,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             if (kk < 3) read_frags(cur, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
-            if (NEXT) {
-                store_b(nxt, rb_next, kk);
-                if (kk == 3) store_a(nxt, 0, 8);
-            }
+            if (NEXT) store_b(nxt, rb_next, kk);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -217,6 +227,7 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
                 __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // VMEM read
             }
         }
+        if (NEXT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // x tile copy of kt + 1 has landed in LDS
         __syncthreads();
     };
     using T = std::true_type;
