@@ -233,6 +233,23 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         }
     }
 
+    const int nprod = per_tile - 1;
+    const bool reducer = (sub == nprod);
+    const int nquads = p.M * QPR;
+    const int col0 = tile * TC;
+    const size_t slice_stride = (size_t)p.ntiles * nquads * 4;                 // floats per (mat, kslice)
+    float *tile_partial = p.partial + (size_t)tile * nquads * 4;
+
+    // The reducer's first polling round is issued before the LDS combine, so that its latency
+    // (one trip to L2 per slot) is hidden behind the combine and its barriers.
+    u32x4 pre[8];
+    const bool prefetched = reducer && (int)threadIdx.x < nquads;
+    if (prefetched) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (j < nprod) pre[j] = slot_load(tile_partial + (size_t)threadIdx.x * 4 + j * slice_stride);
+    }
+
     // ---- cross-wave combine in LDS: red[slot][m][j * 17 + ln], j = natural column in the lane's chunk ----
     const int slot_stride = p.M * ROWF;
 #pragma unroll
@@ -255,12 +272,6 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     }
 
     // ---- workgroup result in 4-column quads; producers publish, the reducer gathers ----
-    const int nprod = per_tile - 1;
-    const bool reducer = (sub == nprod);
-    const int nquads = p.M * QPR;
-    const int col0 = tile * TC;
-    const size_t slice_stride = (size_t)p.ntiles * nquads * 4;                 // floats per (mat, kslice)
-    float *tile_partial = p.partial + (size_t)tile * nquads * 4;
     for (int e = threadIdx.x; e < nquads; e += WAVES * 64) {
         const int m = e / QPR;
         const int col = (e % QPR) * 4;
@@ -286,15 +297,17 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             u32x4 v[8];
             int spins = 0;
             bool ok;
+            bool use_pre = prefetched && s0 == 0 && e == (int)threadIdx.x;
             do {
                 ok = true;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     if (s0 + j < nprod) {
-                        v[j] = slot_load(slot0 + (s0 + j) * slice_stride);
+                        v[j] = use_pre ? pre[j] : slot_load(slot0 + (s0 + j) * slice_stride);
                         ok = ok && slot_full(v[j]);
                     }
                 }
+                use_pre = false;
                 if (!ok && ++spins > p.spin_limit) {
                     __hip_atomic_store(p.header, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     break;
