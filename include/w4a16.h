@@ -132,6 +132,64 @@ int w4a16_ffn_swiglu_bf16(const uint16_t *x,
                           void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Decode GEMV with residual, batch 1: y[N] = bf16(x . W + R), the residual joining the fp32
+ * sum before the single rounding.  Replaces matvec_int4_packed_add.cpu_reference
+ * (programming_examples/matrix_vector_multiplication/int4_awq/matvec_int4_packed_add.py:302-319)
+ * and its device kernel matvec_int4_bf16_packed_add.  `residual` is bf16 [N]; y may alias it.
+ * Workspace: w4a16_gemm_workspace_bytes(1, K, N).
+ */
+int w4a16_gemv_add_bf16(const uint16_t *x,
+                        const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                        const uint16_t *residual, uint16_t *y, int K, int N, int group,
+                        void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * RMSNorm prologue + decode GEMV, batch 1:
+ *   rstd = 1 / sqrt(mean(x^2) + eps),  n = bf16((x * rstd) * norm_weight),  y = bf16(n . W)
+ * The normalisation of matvec_int4_swiglu_rms.cpu_reference
+ * (programming_examples/decode_ffn_swiglu/matvec_int4_swiglu_rms.py:496-500) in front of a
+ * plain GEMV (the shape of the Q/K/V projections of rms_qkv_int4_rope_multi.py:4-30).
+ * `norm_weight` is bf16 [K].  Workspace: w4a16_gemm_workspace_bytes(1, K, N).
+ */
+int w4a16_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps,
+                        const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                        uint16_t *y, int K, int N, int group,
+                        void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * RMSNorm + gate/up GEMV + SwiGLU, batch 1: the whole of matvec_int4_swiglu_rms.cpu_reference
+ * (programming_examples/decode_ffn_swiglu/matvec_int4_swiglu_rms.py:490-516) =
+ * lgu_cpu_reference (programming_examples/llms/llama32_1b_int4/multi_launch_builder/
+ * o_gemv_ffn_int4_fused.py:127-151) in one kernel.  Workspace: w4a16_ffn_workspace_bytes(K, H).
+ */
+int w4a16_rms_gemv_swiglu_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps,
+                               const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                               const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                               uint16_t *h, int K, int H, int group,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Decode block "O projection + FFN", batch 1 — the three stages of o_gemv_ffn_int4
+ * (programming_examples/llms/llama32_1b_int4/multi_launch_builder/o_gemv_ffn_int4_multi.py:4-37):
+ *   res1 = bf16(attn_out . Wo + x_residual)
+ *   h    = bf16(silu(bf16(n . Wg)) * bf16(n . Wu)),  n = bf16((res1 * rstd) * ffn_norm_weight)
+ *   y    = bf16(h . Wd + res1)
+ * Wo is [E, E], Wg and Wu are [E, H], Wd is [H, E]; attn_out, x_residual, ffn_norm_weight, y
+ * are bf16 [E].  `res1_out` (bf16 [E]) and `h_out` (bf16 [H]) may be NULL; when given they
+ * receive the intermediates.  Three kernel launches on `stream`.
+ * Workspace: w4a16_block_workspace_bytes(E, H).
+ */
+size_t w4a16_block_workspace_bytes(int E, int H);
+int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual,
+                          const uint16_t *ffn_norm_weight, float eps,
+                          const int32_t *o_qweight, const int32_t *o_qzeros, const uint16_t *o_scales,
+                          const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                          const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                          const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
+                          uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int E, int H, int group,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units" (0 = built-in heuristic) and
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the

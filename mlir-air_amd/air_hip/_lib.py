@@ -10,7 +10,7 @@ OK = 0
 ERR_NULL, ERR_SHAPE, ERR_GROUP, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_TUNE, ERR_TIMEOUT = -1, -2, -3, -4, -5, -6, -7, -8
 
 # every symbol include/w4a16.h declares: name -> (restype, argtypes)
-_vp, _ci, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+_vp, _ci, _sz, _cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_float
 SYMBOLS = {
     "w4a16_abi_version": (_ci, []),
     "w4a16_strerror": (ctypes.c_char_p, [_ci]),
@@ -24,6 +24,11 @@ SYMBOLS = {
     "w4a16_gemm_bf16": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_gemv_swiglu_bf16": (_ci, [_vp] * 8 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_ffn_swiglu_bf16": (_ci, [_vp] * 12 + [_ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a16_gemv_add_bf16": (_ci, [_vp] * 6 + [_ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a16_rms_gemv_bf16": (_ci, [_vp, _vp, _cf] + [_vp] * 4 + [_ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a16_rms_gemv_swiglu_bf16": (_ci, [_vp, _vp, _cf] + [_vp] * 7 + [_ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a16_block_workspace_bytes": (_sz, [_ci, _ci]),
+    "w4a16_o_gemv_ffn_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 15 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_tune": (_ci, [ctypes.c_char_p, _ci]),
 }
 

@@ -19,7 +19,10 @@ import numpy as np
 from .. import awq, bf16
 from .abc import AirBackend, AirBackendError
 
-OPS = ("dequant_awq", "matvec_int4", "matvec_int4_add", "matmul_int4", "matvec_int4_swiglu", "ffn_swiglu_int4")
+OPS = ("dequant_awq", "matvec_int4", "matvec_int4_add", "matmul_int4", "matvec_int4_swiglu",
+       "matvec_int4_swiglu_rms", "ffn_swiglu_int4", "o_gemv_ffn_int4")
+# ops whose N is a hidden size that is also the K of a following projection
+_HIDDEN_OPS = ("ffn_swiglu_int4", "o_gemv_ffn_int4")
 
 
 @dataclasses.dataclass(frozen=True)
@@ -32,6 +35,7 @@ class HipModule:
     N: int
     M: int = 1
     gs: int = 128
+    eps: float = 1e-5
 
     def __str__(self):
         return f"hip.module @{self.op} {{M = {self.M}, K = {self.K}, N = {self.N}, gs = {self.gs}}}"
@@ -62,7 +66,7 @@ class HIPBackend(AirBackend):
         n_mult = 8 if module.op == "dequant_awq" else 32
         if module.N <= 0 or module.N % n_mult:
             raise AirBackendError(f"N = {module.N} must be a positive multiple of {n_mult}")
-        if module.op in ("ffn_swiglu_int4",) and module.N % awq.GROUP:
+        if module.op in _HIDDEN_OPS and module.N % awq.GROUP:
             raise AirBackendError(f"hidden size {module.N} must be a multiple of {awq.GROUP}")
         if module.M <= 0:
             raise AirBackendError(f"M = {module.M} must be positive")
@@ -103,15 +107,18 @@ class HIPBackend(AirBackend):
             if mod.op == "matvec_int4":
                 return [ops.w4a16_gemv(dev_in[1], *dev_in[0])]
             if mod.op == "matvec_int4_add":
-                y = ops.w4a16_gemv(dev_in[1], *dev_in[0])
-                # the residual joins in fp32 on the host side of the boundary for now
-                return [(y.float() + dev_in[2].float()).to(torch.bfloat16)]
+                return [ops.w4a16_gemv_add(dev_in[1], *dev_in[0], dev_in[2])]
             if mod.op == "matmul_int4":
                 return [ops.w4a16_gemm(dev_in[0], *dev_in[1])]
             if mod.op == "matvec_int4_swiglu":
                 return [ops.w4a16_swiglu(dev_in[2], dev_in[0], dev_in[1])]
+            if mod.op == "matvec_int4_swiglu_rms":
+                return [ops.w4a16_rms_swiglu(dev_in[2][0], dev_in[2][1], dev_in[0], dev_in[1], eps=mod.eps)]
             if mod.op == "ffn_swiglu_int4":
                 return [ops.ffn_swiglu(dev_in[3], dev_in[0], dev_in[1], dev_in[2])]
+            if mod.op == "o_gemv_ffn_int4":
+                wo, attn_out, x_res, norm_w, gate, up, down = dev_in
+                return [ops.o_gemv_ffn(attn_out, x_res, norm_w, wo, gate, up, down, eps=mod.eps)]
             raise AirBackendError(f"unknown op {mod.op}")
 
         def invoker(*args):
@@ -162,6 +169,14 @@ class HIPBackend(AirBackend):
         if mod.op == "matvec_int4_swiglu":
             need(3)
             return [weights(inputs[0], K, N), weights(inputs[1], K, N), to_dev(bf16.bits_of(inputs[2]).reshape(K))]
+        if mod.op == "matvec_int4_swiglu_rms":
+            need(3)   # gate buffer, up buffer, RMS_in [2, K]: row 0 = x, row 1 = norm weight
+            return [weights(inputs[0], K, N), weights(inputs[1], K, N), to_dev(bf16.bits_of(inputs[2]).reshape(2, K))]
+        if mod.op == "o_gemv_ffn_int4":
+            need(7)   # wo buffer, attn_out, x_residual, ffn_norm_w, gate, up, down buffers; K = emb, N = hidden
+            return [weights(inputs[0], K, K), to_dev(bf16.bits_of(inputs[1]).reshape(K)),
+                    to_dev(bf16.bits_of(inputs[2]).reshape(K)), to_dev(bf16.bits_of(inputs[3]).reshape(K)),
+                    weights(inputs[4], K, N), weights(inputs[5], K, N), weights(inputs[6], N, K)]
         if mod.op == "ffn_swiglu_int4":
             need(4)
             return [weights(inputs[0], K, N), weights(inputs[1], K, N), weights(inputs[2], N, K),

@@ -133,6 +133,87 @@ def ffn_swiglu(x, gate, up, down, group=GROUP, return_h=False):
     return (y, h) if return_h else y
 
 
+def _wptrs(w):
+    return [_ptr(w[0]), _ptr(w[1]), _ptr(_bits(w[2]))]
+
+
+def w4a16_gemv_add(x, qweight, qzeros, scales, residual, group=GROUP, out=None):
+    """Decode GEMV with residual: y[N] = bf16(x[K] . W + R[N]) (one rounding)."""
+    lib = _lib.load_library()
+    _need_cuda(x, qweight, qzeros, scales, residual)
+    K = x.numel()
+    if qweight.shape[0] != K:
+        raise ValueError(f"x has K={K} but qweight has {qweight.shape[0]} rows")
+    N = qweight.shape[1] * 8
+    if residual.numel() != N:
+        raise ValueError(f"residual has {residual.numel()} elements, expected N={N}")
+    if out is None:
+        out = torch.empty((N,), dtype=torch.bfloat16, device=x.device)
+    ws = workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
+    _lib.check(lib.w4a16_gemv_add_bf16(_ptr(_bits(x)), *_wptrs((qweight, qzeros, scales)), _ptr(_bits(residual)),
+                                       _ptr(out), K, N, group, _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def w4a16_rms_gemv(x, norm_weight, qweight, qzeros, scales, eps=1e-5, group=GROUP):
+    """y[N] = bf16(rms_norm(x, norm_weight) . W), the normalised vector rounded to bf16 first."""
+    lib = _lib.load_library()
+    _need_cuda(x, norm_weight, qweight, qzeros, scales)
+    K = x.numel()
+    if qweight.shape[0] != K or norm_weight.numel() != K:
+        raise ValueError("w4a16_rms_gemv: x, norm_weight must have K elements and qweight K rows")
+    N = qweight.shape[1] * 8
+    out = torch.empty((N,), dtype=torch.bfloat16, device=x.device)
+    ws = workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
+    _lib.check(lib.w4a16_rms_gemv_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
+                                       *_wptrs((qweight, qzeros, scales)), _ptr(out), K, N, group,
+                                       _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def w4a16_rms_swiglu(x, norm_weight, gate, up, eps=1e-5, group=GROUP):
+    """h[H] = bf16(silu(bf16(n Wg)) * bf16(n Wu)) with n = bf16((x * rstd) * norm_weight)."""
+    lib = _lib.load_library()
+    _need_cuda(x, norm_weight, *gate, *up)
+    K = x.numel()
+    H = gate[0].shape[1] * 8
+    if gate[0].shape[0] != K or up[0].shape != gate[0].shape or norm_weight.numel() != K:
+        raise ValueError("w4a16_rms_swiglu: gate and up must both be [K, H/8], norm_weight [K]")
+    h = torch.empty((H,), dtype=torch.bfloat16, device=x.device)
+    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device)
+    _lib.check(lib.w4a16_rms_gemv_swiglu_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
+                                              *_wptrs(gate), *_wptrs(up), _ptr(h), K, H, group,
+                                              _ptr(ws), ws.numel(), _stream()))
+    return h
+
+
+def o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, group=GROUP,
+               return_intermediates=False):
+    """Decode block: res1 = Wo(attn_out) + x_residual; y = Wd(swiglu(rms_norm(res1))) + res1.
+
+    wo/gate/up/down are (qweight, qzeros, scales).  Returns y, or (y, res1, h).
+    """
+    lib = _lib.load_library()
+    _need_cuda(attn_out, x_residual, ffn_norm_weight, *wo, *gate, *up, *down)
+    E = attn_out.numel()
+    H = gate[0].shape[1] * 8
+    if (wo[0].shape[0] != E or wo[0].shape[1] * 8 != E or gate[0].shape[0] != E or up[0].shape != gate[0].shape
+            or down[0].shape[0] != H or down[0].shape[1] * 8 != E or x_residual.numel() != E
+            or ffn_norm_weight.numel() != E):
+        raise ValueError("o_gemv_ffn: wo must be [E, E/8], gate/up [E, H/8], down [H, E/8], vectors [E]")
+    dev = attn_out.device
+    y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
+    res1 = torch.empty((E,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
+    h = torch.empty((H,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
+    ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev)
+    _lib.check(lib.w4a16_o_gemv_ffn_bf16(
+        _ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
+        *_wptrs(wo), *_wptrs(gate), *_wptrs(up), *_wptrs(down), _ptr(y),
+        _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
+        E, H, group, _ptr(ws), ws.numel(), _stream()))
+    return (y, res1, h) if return_intermediates else y
+
+
 def tune(key, value):
     lib = _lib.load_library()
     _lib.check(lib.w4a16_tune(key.encode(), int(value)))

@@ -163,6 +163,116 @@ int w4a16_ffn_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const 
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+int w4a16_gemv_add_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                        const uint16_t *residual, uint16_t *y, int K, int N, int group, void *workspace,
+                        size_t workspace_bytes, void *stream) {
+    if (!x || !y || !residual) return W4A16_ERR_NULL;
+    int rc = check_quant(qweight, qzeros, scales, K, N, group, 32);
+    if (rc) return rc;
+    if (misaligned(x) || misaligned(y) || misaligned(residual)) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_gemm_workspace_bytes(1, K, N)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    StreamExtras ex;
+    ex.residual = residual;
+    hipError_t e = launch_stream(x, qweight, qzeros, scales, nullptr, nullptr, nullptr, y, 1, K, N, workspace,
+                                 static_cast<hipStream_t>(stream), ex);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const int32_t *qweight,
+                        const int32_t *qzeros, const uint16_t *scales, uint16_t *y, int K, int N, int group,
+                        void *workspace, size_t workspace_bytes, void *stream) {
+    if (!x || !y || !norm_weight) return W4A16_ERR_NULL;
+    int rc = check_quant(qweight, qzeros, scales, K, N, group, 32);
+    if (rc) return rc;
+    if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(y) || misaligned(norm_weight)) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_gemm_workspace_bytes(1, K, N)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    StreamExtras ex;
+    ex.norm_w = norm_weight;
+    ex.eps = eps;
+    hipError_t e = launch_stream(x, qweight, qzeros, scales, nullptr, nullptr, nullptr, y, 1, K, N, workspace,
+                                 static_cast<hipStream_t>(stream), ex);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_rms_gemv_swiglu_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps,
+                               const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                               const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                               uint16_t *h, int K, int H, int group, void *workspace, size_t workspace_bytes,
+                               void *stream) {
+    if (!x || !h || !norm_weight) return W4A16_ERR_NULL;
+    int rc = check_quant(gate_qweight, gate_qzeros, gate_scales, K, H, group, 32);
+    if (rc) return rc;
+    rc = check_quant(up_qweight, up_qzeros, up_scales, K, H, group, 32);
+    if (rc) return rc;
+    if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(h) || misaligned(norm_weight)) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_ffn_workspace_bytes(K, H)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    StreamExtras ex;
+    ex.norm_w = norm_weight;
+    ex.eps = eps;
+    hipError_t e = launch_stream(x, gate_qweight, gate_qzeros, gate_scales, up_qweight, up_qzeros, up_scales, h, 1, K, H,
+                                 workspace, static_cast<hipStream_t>(stream), ex);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+size_t w4a16_block_workspace_bytes(int E, int H) {
+    if (E <= 0 || H <= 0) return 0;
+    const size_t a = stream_partial_bytes(1, H, 2), b = stream_partial_bytes(1, E, 1);
+    return kHeaderBytes + (a > b ? a : b) + round256((size_t)H * sizeof(uint16_t)) + round256((size_t)E * sizeof(uint16_t));
+}
+
+int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                          float eps, const int32_t *o_qweight, const int32_t *o_qzeros, const uint16_t *o_scales,
+                          const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                          const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                          const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
+                          uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int E, int H, int group, void *workspace,
+                          size_t workspace_bytes, void *stream) {
+    if (!attn_out || !x_residual || !ffn_norm_weight || !y) return W4A16_ERR_NULL;
+    int rc = check_quant(o_qweight, o_qzeros, o_scales, E, E, group, 32);
+    if (rc) return rc;
+    rc = check_quant(gate_qweight, gate_qzeros, gate_scales, E, H, group, 32);
+    if (rc) return rc;
+    rc = check_quant(up_qweight, up_qzeros, up_scales, E, H, group, 32);
+    if (rc) return rc;
+    rc = check_quant(down_qweight, down_qzeros, down_scales, H, E, group, 32);
+    if (rc) return rc;
+    if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(attn_out) || misaligned(x_residual) || misaligned(ffn_norm_weight) || misaligned(y) ||
+        (res1_out && misaligned(res1_out)) || (h_out && misaligned(h_out)))
+        return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_block_workspace_bytes(E, H)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    char *tail = static_cast<char *>(workspace) + w4a16_block_workspace_bytes(E, H);
+    uint16_t *res1 = res1_out ? res1_out : reinterpret_cast<uint16_t *>(tail - round256((size_t)E * sizeof(uint16_t)));
+    uint16_t *h = h_out ? h_out
+                        : reinterpret_cast<uint16_t *>(tail - round256((size_t)E * sizeof(uint16_t)) -
+                                                       round256((size_t)H * sizeof(uint16_t)));
+    // stage 1: res1 = bf16(attn_out . Wo + x_residual)
+    StreamExtras add;
+    add.residual = x_residual;
+    hipError_t e = launch_stream(attn_out, o_qweight, o_qzeros, o_scales, nullptr, nullptr, nullptr, res1, 1, E, E,
+                                 workspace, st, add);
+    if (e != hipSuccess) return hip_fail(e);
+    // stage 2: h = swiglu(rms_norm(res1) . Wgate, rms_norm(res1) . Wup)
+    StreamExtras rms;
+    rms.norm_w = ffn_norm_weight;
+    rms.eps = eps;
+    e = launch_stream(res1, gate_qweight, gate_qzeros, gate_scales, up_qweight, up_qzeros, up_scales, h, 1, E, H,
+                      workspace, st, rms);
+    if (e != hipSuccess) return hip_fail(e);
+    // stage 3: y = bf16(h . Wdown + res1)
+    add.residual = res1;
+    e = launch_stream(h, down_qweight, down_qzeros, down_scales, nullptr, nullptr, nullptr, y, 1, H, E, workspace, st,
+                      add);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_tune(const char *key, int value) {
     if (!key || value < 0) return W4A16_ERR_TUNE;
     if (!strcmp(key, "gemv_lw")) {

@@ -30,11 +30,20 @@ StreamPlan plan_stream(int M, int K, int N);
 hipError_t launch_dequant(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, uint16_t *out,
                           int K, int N, hipStream_t stream);
 
+// Optional stages fused into the streaming kernel.
+struct StreamExtras {
+    const uint16_t *residual = nullptr;   // [M, N] bf16 added to the result before the final rounding
+    int round_before_add = 0;             // 1: y = bf16(bf16(x.W) + R) instead of bf16(x.W + R)
+    const uint16_t *norm_w = nullptr;     // [K] bf16: x is replaced by bf16((x * rstd) * norm_w), M <= 4
+    float eps = 1e-5f;
+};
+
 // y[M, N] = bf16(x[M, K] . W), M <= 16.  With `up_*` given (SwiGLU epilogue, M == 1) the
 // kernel streams both weight sets and writes y = bf16(silu(bf16(x.Wg)) * bf16(x.Wu)).
 hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
                          const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
-                         uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream);
+                         uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream,
+                         const StreamExtras &extras = StreamExtras());
 
 hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
                                const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream);

@@ -58,6 +58,10 @@ struct StreamParams {
     int ksplit;    // workgroups along K per tile
     int units;     // units per wave
     int nmat;      // 1, or 2 for gate/up with the SwiGLU epilogue
+    const uint16_t *residual;   // [M, N] bf16 added in the epilogue, or null
+    int round_before_add;       // 1: y = bf16(bf16(acc) + R); 0: y = bf16(acc + R)
+    const uint16_t *norm_w;     // [K] bf16 RMSNorm weight (RMS kernels only)
+    float eps;
     int spin_limit;
     int skip_publish;   // fault injection for tests: producers keep their partials to themselves
 };
@@ -101,7 +105,10 @@ struct Words<1> { typedef uint32_t type __attribute__((ext_vector_type(1))); };
 
 // LW     packed words per lane per row: the tile is 16 lanes x 8*LW columns = 128*LW columns
 // KSTEPS K-steps per unit, WAVES waves per workgroup, MI live accumulator registers (M <= 4*MI)
-template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT>
+// RMS    x is RMS-normalised on the fly: every wave computes 1/sqrt(mean(x^2) + eps) of its
+//        rows itself (x is K bf16 values, L2-resident) while its weight loads are in
+//        flight, and feeds bf16((x * rstd) * norm_w) to the matrix cores.  M <= 4.
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS>
 __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParams p) {
     constexpr int SLOTS = MI == 1 ? WAVES : (MI == 2 ? WAVES / 2 : WAVES / 4);   // LDS combine slots
     typedef typename Words<LW>::type wvec;
@@ -153,6 +160,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     for (int t = 0; t < LC; ++t) yacc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const int nksteps = p.K >> 5;
+    float rstd = 0.f;
     for (int u = 0; u < p.units; ++u) {
         const int kstep0 = ((kslice * p.units + u) * WAVES + wave) * KSTEPS;
         if (kstep0 >= nksteps) break;   // wave-uniform
@@ -173,6 +181,52 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 #pragma unroll
         for (int c = 0; c < LW; ++c) sv[c] = *reinterpret_cast<const u32x4 *>(sc + (size_t)g * p.N + 8 * c);
 
+        if constexpr (RMS) {
+            u32x4 nw[KSTEPS];
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s)
+                nw[s] = *reinterpret_cast<const u32x4 *>(p.norm_w + (size_t)(kstep0 + s) * 32 + 8 * lg);
+            if (u == 0) {
+                float ss[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (r < p.M) {
+                        const u32x4 *row = reinterpret_cast<const u32x4 *>(p.x + (size_t)r * p.K);
+                        float a0 = 0.f, a1 = 0.f;
+                        for (int c = lane; c < (p.K >> 3); c += 64) {
+                            const u32x4 v = row[c];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                const float lo = __builtin_bit_cast(float, v[j] << 16);
+                                const float hi = __builtin_bit_cast(float, v[j] & 0xFFFF0000u);
+                                a0 = fmaf(lo, lo, a0);
+                                a1 = fmaf(hi, hi, a1);
+                            }
+                        }
+                        float a = a0 + a1;
+#pragma unroll
+                        for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off);
+                        ss[r] = a;
+                    }
+                }
+                float mine = ss[0];
+                if (am == 1) mine = ss[1];
+                if (am == 2) mine = ss[2];
+                if (am == 3) mine = ss[3];
+                rstd = 1.0f / sqrtf(mine / (float)p.K + p.eps);
+            }
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float x_lo = __builtin_bit_cast(float, av[s][j] << 16);
+                    const float x_hi = __builtin_bit_cast(float, av[s][j] & 0xFFFF0000u);
+                    const float w_lo = __builtin_bit_cast(float, nw[s][j] << 16);
+                    const float w_hi = __builtin_bit_cast(float, nw[s][j] & 0xFFFF0000u);
+                    av[s][j] = pack_bf16x2((x_lo * rstd) * w_lo, (x_hi * rstd) * w_hi);
+                }
+            }
+        }
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s)
             if (!a_valid) av[s] = u32x4{0u, 0u, 0u, 0u};
@@ -336,6 +390,17 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         } else {
             out = sum0 + own;
         }
+        if (p.residual && col0 + col < p.N) {
+            const uint2 r = *reinterpret_cast<const uint2 *>(p.residual + (size_t)m * p.N + col0 + col);
+            if (p.round_before_add) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) out[q] = bf16_bits_to_float(float_to_bf16_bits(out[q]));
+            }
+            out[0] += __builtin_bit_cast(float, r.x << 16);
+            out[1] += __builtin_bit_cast(float, r.x & 0xFFFF0000u);
+            out[2] += __builtin_bit_cast(float, r.y << 16);
+            out[3] += __builtin_bit_cast(float, r.y & 0xFFFF0000u);
+        }
         if (col0 + col < p.N) {
             uint2 o;
             o.x = pack_bf16x2(out[0], out[1]);
@@ -376,16 +441,19 @@ StreamPlan plan_stream(int M, int K, int N) {
     return pl;
 }
 
-template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT>
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false>
 static hipError_t launch_one(const StreamParams &p, int grid, hipStream_t stream) {
     constexpr int SLOTS = MI == 1 ? WAVES : (MI == 2 ? WAVES / 2 : WAVES / 4);
     const size_t lds = (size_t)SLOTS * p.M * 8 * LW * 17 * sizeof(float);
-    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT>), dim3(grid), dim3(WAVES * 64), lds, stream, p);
+    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>), dim3(grid), dim3(WAVES * 64), lds, stream, p);
     return hipGetLastError();
 }
 
 template <int LW, int WB, int KSTEPS, int WAVES>
 static hipError_t launch_mi(int mi, const StreamParams &p, int grid, hipStream_t stream) {
+    if (p.norm_w)   // M <= 4 checked by the caller
+        return p.nmat == 2 ? launch_one<LW, WB, KSTEPS, WAVES, 1, 2, true>(p, grid, stream)
+                           : launch_one<LW, WB, KSTEPS, WAVES, 1, 1, true>(p, grid, stream);
     if (p.nmat == 2) return launch_one<LW, WB, KSTEPS, WAVES, 1, 2>(p, grid, stream);
     switch (mi) {
         case 1: return launch_one<LW, WB, KSTEPS, WAVES, 1, 1>(p, grid, stream);
@@ -406,7 +474,8 @@ static hipError_t launch_ksteps(int ksteps, int waves, int mi, const StreamParam
 
 hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
                          const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
-                         uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream) {
+                         uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream,
+                         const StreamExtras &extras) {
     const StreamPlan pl = plan_stream(M, K, N);
     StreamParams p;
     p.x = x;
@@ -427,6 +496,10 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.ntiles = pl.ntiles;
     p.ksplit = pl.ksplit;
     p.units = pl.units;
+    p.residual = extras.residual;
+    p.round_before_add = extras.round_before_add;
+    p.norm_w = extras.norm_w;
+    p.eps = extras.eps;
     p.skip_publish = g_stream_tune.skip_publish;
     p.spin_limit = g_stream_tune.spin_limit > 0 ? g_stream_tune.spin_limit : (1 << 18);
     const int grid = ((pl.ntiles + 7) / 8) * 8 * p.nmat * pl.ksplit;

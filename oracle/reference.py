@@ -18,6 +18,13 @@ Follows (PE = programming_examples, INT4 = PE/llms/llama32_1b_int4):
   ld_cpu_reference           o_gemv_ffn_int4_fused.py:1078-1094
   ffn_swiglu_reference       the chain at o_gemv_ffn_int4_fused.py:1187-1191
                              without the RMSNorm prologue and with R = 0
+  o_gemv_ffn_int4_reference  INT4/multi_launch_builder/o_gemv_ffn_int4_multi.py:273-288
+                             (float32 throughout on bf16-dequantised weights; res1
+                             and gate/up are NOT rounded to bf16)
+  o_gemv_ffn_staged_reference  the three device stages of the same block
+                             (o_gemv_ffn_int4_multi.py:4-37) chained with the
+                             per-stage references above, i.e. with the bf16
+                             rounding points the stages have on the device
   check_outputs              python/air/backend/xrt_runner.py:394-523
 
 Arrays named A_q/A_s/A_z use the examples' kernel-side layout
@@ -169,6 +176,33 @@ def ffn_swiglu_reference(gate_l1, up_l1, down_l1, x_bits):
     h = swiglu_rms_cpu_reference(a_q, a_s, a_z, x_bits, None)
     y = ld_cpu_reference(down_l1[0], down_l1[1], down_l1[2], h, None)
     return h, y
+
+
+def o_gemv_ffn_int4_reference(wo_bits, attn_out_bits, x_residual_bits, ffn_norm_w_bits, wgate_bits, wup_bits,
+                              wdown_bits, eps=1e-5):
+    """Whole O + FFN block on bf16-dequantised weights ([out, in] bf16 bits), float32
+    arithmetic; returns bf16 bits [emb]."""
+    f = bf16_bits_to_f32
+    res1 = f(wo_bits) @ f(attn_out_bits) + f(x_residual_bits)
+    rstd = 1.0 / np.sqrt((res1 * res1).mean() + eps)
+    normed = (res1 * rstd) * f(ffn_norm_w_bits)
+    normed_bf16 = f(f32_to_bf16_bits(normed.astype(np.float32)))
+    gate = f(wgate_bits) @ normed_bf16
+    up = f(wup_bits) @ normed_bf16
+    swiglu = (gate * 0.5 * (np.tanh(gate / 2.0) + 1.0)) * up
+    swiglu_bf16 = f(f32_to_bf16_bits(swiglu.astype(np.float32)))
+    return f32_to_bf16_bits((f(wdown_bits) @ swiglu_bf16 + res1).astype(np.float32))
+
+
+def o_gemv_ffn_staged_reference(wo_l1, gate_l1, up_l1, down_l1, attn_out_bits, x_residual_bits, ffn_norm_w_bits,
+                                eps=1e-5):
+    """Stage 1 matvec_add, stage 2 RMSNorm + gate/up + SwiGLU, stage 3 matvec_add with
+    res1 as the residual.  Returns (res1 bits [emb], h bits [hidden], y bits [emb])."""
+    res1 = matvec_add_cpu_reference(wo_l1[0], wo_l1[1], wo_l1[2], attn_out_bits, x_residual_bits)
+    a_q, a_s, a_z = interleave_gate_up(gate_l1, up_l1)
+    h = swiglu_rms_cpu_reference(a_q, a_s, a_z, res1, ffn_norm_w_bits, eps)
+    y = matvec_add_cpu_reference(down_l1[0], down_l1[1], down_l1[2], h, res1)
+    return res1, h, y
 
 
 def check_outputs(actual, expected, rtol=1e-3, atol=1e-8, max_mismatch_percentage=0, min_correlation=None):

@@ -8,7 +8,7 @@ import torch
 
 from helpers import make_awq, make_x
 from oracle import awq as oawq, reference as oref
-from oracle.bf16 import bf16_bits_to_f32
+from oracle.bf16 import bf16_bits_to_f32, f32_to_bf16_bits
 
 pytestmark = pytest.mark.gpu
 G = os.path.join(os.path.dirname(__file__), "golden")
@@ -63,6 +63,18 @@ def test_example_swiglu_rms(capsys):
         return oref.swiglu_rms_cpu_reference(a_q, a_s, a_z, rms_in[0], rms_in[1])
 
     assert ex.run(ex.parse_args(["--m", "4096", "--k", "2048"]), reference) == 0
+    assert "PASS!" in capsys.readouterr().out
+
+
+def test_example_o_gemv_ffn_block(capsys):
+    from air_hip.examples import o_gemv_ffn_int4 as ex
+    print("example o_gemv_ffn", flush=True)
+
+    def reference(wo, gate, up, wd, attn_out, x_residual, ffn_norm_w):
+        dq = lambda t: f32_to_bf16_bits(oref._dequant_l1_f64(t[0], t[1], t[2], t[0].shape[1] * 2).astype(np.float32))
+        return oref.o_gemv_ffn_int4_reference(dq(wo), attn_out, x_residual, ffn_norm_w, dq(gate), dq(up), dq(wd))
+
+    assert ex.run(ex.parse_args(["--emb-dim", "1024", "--hidden-dim", "4096"]), reference) == 0
     assert "PASS!" in capsys.readouterr().out
 
 

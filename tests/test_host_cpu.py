@@ -9,7 +9,7 @@ import pytest
 
 from air_hip import _lib, awq, bf16
 from air_hip.backend import AirBackendError, HIPBackend, HIPRunner, HipModule
-from air_hip.examples import dequant_awq, matmul_int4_packed, matvec_int4_packed, matvec_int4_swiglu_rms
+from air_hip.examples import dequant_awq, matmul_int4_packed, matvec_int4_packed, matvec_int4_swiglu_rms, o_gemv_ffn_int4
 from oracle import awq as oawq, reference as oref
 from oracle.bf16 import f32_to_bf16_bits
 
@@ -85,11 +85,20 @@ def test_examples_draw_order_and_packing():
     q, sc, z = dequant_awq.draw_inputs(d)
     g = np.load(os.path.join(ROOT, "tests", "golden", "dequant1d_n1024_seed0.npz"))
     assert np.array_equal(q, g["int4_vals"]) and np.array_equal(np.asarray(sc), g["scales"]) and np.array_equal(z, g["zeros"])
-    # RMSNorm prologue on the host equals the oracle's
+    # the fused RMSNorm example hands RMS_in (x row, weight row) to the kernel unchanged
+    assert matvec_int4_swiglu_rms.build_module(128, 256).op == "matvec_int4_swiglu_rms"
     args = matvec_int4_swiglu_rms.parse_args(["--m", "32", "--k", "256"])
     *_, RMS_in = matvec_int4_swiglu_rms.draw_inputs(args)
-    bits = bf16.bits_of(RMS_in)
-    assert np.array_equal(np.asarray(matvec_int4_swiglu_rms.rms_norm(RMS_in)), f32_to_bf16_bits(oref.rms_norm_bf16(bits[0], bits[1])))
+    assert bf16.bits_of(RMS_in).shape == (2, 256)
+    # block example: reference argument names, weight generator seeds and shapes
+    a = o_gemv_ffn_int4.parse_args(["--emb-dim", "256", "--hidden-dim", "512"])
+    wo, gu, wd, attn_out, x_residual, ffn_norm_w = o_gemv_ffn_int4.draw_inputs(a)
+    assert wo[0].shape == (256, 128) and gu[0].shape == (1024, 128) and wd[0].shape == (256, 256)
+    assert wd[1].shape == (4, 256) and set(np.unique(wo[2])) <= {7, 8}
+    assert o_gemv_ffn_int4.build_module(256, 512) == HipModule("o_gemv_ffn_int4", K=256, N=512)
+    rng = np.random.default_rng(100)
+    q = rng.integers(0, 16, size=(256, 256), dtype=np.uint8)
+    assert np.array_equal(wo[0], q[:, 0::2] | (q[:, 1::2] << 4))
 
 
 def test_runner_comparator_semantics_match_reference_restatement(capsys):

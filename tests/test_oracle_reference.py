@@ -136,6 +136,63 @@ def test_swiglu_rounding_points_and_interleave():
     assert np.array_equal(h2, ref.swiglu_rms_cpu_reference(a_q, a_s, a_z, xn, None))
 
 
+def test_rms_norm_against_library_and_closed_forms():
+    K = 512
+    rng = np.random.default_rng(40)
+    x = f32_to_bf16_bits(rng.standard_normal(K).astype(np.float32))
+    w = f32_to_bf16_bits((rng.standard_normal(K) * 0.1 + 1.0).astype(np.float32))
+    got = ref.rms_norm_bf16(x, w, eps=1e-5)
+    # library routine (float64 so that its own rounding cannot matter), then one bf16 rounding
+    t = torch.nn.functional.rms_norm(torch.from_numpy(bf16_bits_to_f32(x)).double(), (K,),
+                                     torch.from_numpy(bf16_bits_to_f32(w)).double(), eps=1e-5)
+    want = bf16_bits_to_f32(f32_to_bf16_bits(t.float().numpy()))
+    assert np.mean(got != want) <= 0.01 and np.max(np.abs(got - want) / np.abs(want)) <= 2.0**-7
+    # constant x = c: rstd = 1 / sqrt(c^2 + eps), n = bf16(c * rstd * w); eps matters for small c
+    c = np.float32(0.0078125)
+    xc = f32_to_bf16_bits(np.full(K, c, np.float32))
+    n = ref.rms_norm_bf16(xc, w, eps=1e-5)
+    closed = float(c) / np.sqrt(float(c) ** 2 + 1e-5) * bf16_bits_to_f32(w).astype(np.float64)
+    assert np.max(np.abs(n - closed) / np.abs(closed)) <= 2.0**-8 * 1.001
+    # a dropped eps or a sum instead of a mean would give 1.0 * w and w / sqrt(K)
+    assert not np.allclose(n, bf16_bits_to_f32(w), rtol=1e-2)
+
+
+def test_block_references_agree_and_reduce_to_their_stages():
+    E, H, gs = 256, 512, 128
+    _, oq, os_, oz, attn = _l1(E, E, gs, 50)
+    _, gq, gs_, gz, xres = _l1(H, E, gs, 51)
+    _, uq, us_, uz, _ = _l1(H, E, gs, 52)
+    _, dq, ds, dz, _ = _l1(E, H, gs, 53)
+    rng = np.random.default_rng(54)
+    w = f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32))
+    res1, h, y = ref.o_gemv_ffn_staged_reference((oq, os_, oz), (gq, gs_, gz), (uq, us_, uz), (dq, ds, dz), attn, xres, w)
+    # stage identities
+    assert np.array_equal(res1, ref.matvec_add_cpu_reference(oq, os_, oz, attn, xres))
+    a_q, a_s, a_z = ref.interleave_gate_up((gq, gs_, gz), (uq, us_, uz))
+    assert np.array_equal(h, ref.swiglu_rms_cpu_reference(a_q, a_s, a_z, res1, w))
+    # residual: sum + R in float64, one rounding
+    want_y = ref.matvec_f64(dq, ds, dz, h) + bf16_bits_to_f32(res1)
+    assert np.max(np.abs(bf16_bits_to_f32(y) - want_y)) <= np.max(np.abs(want_y)) * 2.0**-8
+    # W = 0 (q == z): matvec_add returns R bit for bit
+    zq = np.repeat(oz.T, gs, axis=1)                      # [out, K] nibbles equal to the zero points
+    zero_q = (zq[:, 0::2] | (zq[:, 1::2] << 4)).astype(np.uint8)
+    assert np.array_equal(ref.matvec_add_cpu_reference(zero_q, os_, oz, attn, xres), xres)
+    # the float32 whole-block reference on bf16-dequantised weights lands on the same values
+    # within the block's gate (its rounding points differ: res1 and gate/up stay float32)
+    deq = lambda q, s, z: f32_to_bf16_bits(ref._dequant_l1_f64(q, s, z, q.shape[1] * 2).astype(np.float32))
+    whole = ref.o_gemv_ffn_int4_reference(deq(oq, os_, oz), attn, xres, w, deq(gq, gs_, gz), deq(uq, us_, uz), deq(dq, ds, dz))
+    assert ref.check_outputs(bf16_bits_to_f32(y), bf16_bits_to_f32(whole), rtol=0.05, atol=0.05, min_correlation=0.9999)
+    # and against an independent float64 evaluation of the block formula
+    f = lambda b: bf16_bits_to_f32(b).astype(np.float64)
+    r64 = f(deq(oq, os_, oz)) @ f(attn) + f(xres)
+    n64 = f(f32_to_bf16_bits((r64 / np.sqrt(np.mean(r64 * r64) + 1e-5) * f(w)).astype(np.float32)))
+    g64 = f(deq(gq, gs_, gz)) @ n64
+    u64 = f(deq(uq, us_, uz)) @ n64
+    s64 = f(f32_to_bf16_bits((g64 / (1 + np.exp(-g64)) * u64).astype(np.float32)))
+    y64 = f(deq(dq, ds, dz)) @ s64 + r64
+    assert np.max(np.abs(f(whole) - y64)) <= 2.0**-7 * np.max(np.abs(y64))
+
+
 def test_ffn_chain():
     H, K, gs = 256, 128, 128
     _, gq, gs_, gz, x = _l1(H, K, gs, 12)
