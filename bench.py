@@ -32,7 +32,14 @@ CONFIGS = {
     "gemm16": dict(M=16, K=4096, N=14336, cfg=2, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128"),
     "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128"),
     "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128"),
+    # not a BASELINE config: the O projection + RMSNorm + FFN decode block with residuals (3 launches)
+    "block": dict(M=1, K=4096, N=14336, cfg=None, desc="decode block O-proj + RMSNorm + SwiGLU FFN W4A16 E=4096 H=14336 g128"),
 }
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
+# scaled by the same counter's reading for a 256 MiB device copy: x2.000 and x1.000); the
+# summaries under profiles/ hold the commands and the raw readings.
+MEASURED_TRAFFIC_BYTES = {"gemv": 24.36e6, "prefill": 366.2e6}
 
 
 def weight_bytes(K, N):
@@ -46,6 +53,8 @@ def algorithmic_bytes(name):
         return weight_bytes(K, N) + K * N * 2
     if name == "ffn":
         return 3 * weight_bytes(K, N) + K * 2 + K * 2
+    if name == "block":   # wo + gate + up + down; attn_out, x_residual, norm weight in, y out
+        return weight_bytes(K, K) + 3 * weight_bytes(K, N) + 4 * K * 2
     return weight_bytes(K, N) + M * K * 2 + M * N * 2
 
 
@@ -53,6 +62,8 @@ def algorithmic_flops(name):
     c = CONFIGS[name]
     if name == "ffn":
         return 2 * 3 * c["K"] * c["N"]
+    if name == "block":
+        return 2 * (3 * c["K"] * c["N"] + c["K"] * c["K"])
     return 2 * max(c["M"], 0) * c["K"] * c["N"]
 
 
@@ -78,7 +89,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     torch.cuda.set_device(dev)
     stream = torch.cuda.Stream()
 
-    per_copy = weight_bytes(K, N) * (3 if name == "ffn" else 1)
+    per_copy = weight_bytes(K, N) * (3 if name in ("ffn", "block") else 1) + (weight_bytes(K, K) if name == "block" else 0)
     if name == "prefill":
         ncopies = 1
     else:
@@ -88,6 +99,9 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         if name == "ffn":
             copies.append((make_weights(torch, K, N, 100 + 3 * i), make_weights(torch, K, N, 101 + 3 * i),
                            make_weights(torch, N, K, 102 + 3 * i)))
+        elif name == "block":
+            copies.append((make_weights(torch, K, N, 100 + 4 * i), make_weights(torch, K, N, 101 + 4 * i),
+                           make_weights(torch, N, K, 102 + 4 * i), make_weights(torch, K, K, 103 + 4 * i)))
         else:
             copies.append(make_weights(torch, K, N, 100 + i))
     gx = torch.Generator(device="cuda")
@@ -95,13 +109,18 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     x = torch.randn((max(M, 1), K), device="cuda", generator=gx).to(torch.bfloat16)
     if name == "dequant":
         outs = [torch.empty((K, N), dtype=torch.bfloat16, device=dev) for _ in range(min(ncopies, 8))]
-    elif name == "ffn":
+    elif name in ("ffn", "block"):
         outs = [torch.empty((K,), dtype=torch.bfloat16, device=dev)]
     else:
         outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev)]
+    if name == "block":
+        x_residual = torch.randn((K,), device="cuda", generator=gx).to(torch.bfloat16)
+        norm_w = (torch.randn((K,), device="cuda", generator=gx) * 0.1 + 1.0).to(torch.bfloat16)
 
     if name == "ffn":
         ws_bytes = lib.w4a16_ffn_workspace_bytes(K, N)
+    elif name == "block":
+        ws_bytes = lib.w4a16_block_workspace_bytes(K, N)
     else:
         ws_bytes = max(lib.w4a16_gemm_workspace_bytes(max(M, 1), K, N), 16384)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
@@ -118,6 +137,11 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                            u[0].data_ptr(), u[1].data_ptr(), u[2].data_ptr(),
                                            d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(),
                                            outs[0].data_ptr(), None, K, N, 128, ws.data_ptr(), ws.numel(), st)
+        elif name == "block":
+            g, u, d, o = w
+            ptrs = [t.data_ptr() for m in (o, g, u, d) for t in m]
+            rc = lib.w4a16_o_gemv_ffn_bf16(x.data_ptr(), x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, *ptrs,
+                                           outs[0].data_ptr(), None, None, K, N, 128, ws.data_ptr(), ws.numel(), st)
         else:
             rc = lib.w4a16_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
                                      outs[0].data_ptr(), M, K, N, 128, ws.data_ptr(), ws.numel(), st)
@@ -161,7 +185,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         "ncopies": ncopies,
     }
 
-    if with_cpu_baseline:
+    if with_cpu_baseline and name != "block":
         res["cpu_baseline"] = cpu_baseline(name, torch, copies[0], x, outs, launch, stream)
     return res
 
@@ -270,6 +294,7 @@ def main():
         value = main_res["bytes"] / sec / 1e9
         roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": value / HBM_PEAK_GBS, "traffic": None}
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
     roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel"}.get(name, "stream_kernel")
     roof["algorithmic_per_launch"] = main_res["flops"] if name == "prefill" else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]

@@ -110,7 +110,7 @@ struct Words<1> { typedef uint32_t type __attribute__((ext_vector_type(1))); };
 //        flight, and feeds bf16((x * rstd) * norm_w) to the matrix cores.  M <= 4.
 template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS>
 __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParams p) {
-    constexpr int SLOTS = MI == 1 ? WAVES : (MI == 2 ? WAVES / 2 : WAVES / 4);   // LDS combine slots
+    constexpr int SLOTS = WAVES;   // one LDS slot per wave: a single write round, no read-modify-write
     typedef typename Words<LW>::type wvec;
     constexpr int TC = 128 * LW;            // tile columns
     constexpr int LC = 8 * LW;              // columns per lane
@@ -187,32 +187,25 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             for (int s = 0; s < KSTEPS; ++s)
                 nw[s] = *reinterpret_cast<const u32x4 *>(p.norm_w + (size_t)(kstep0 + s) * 32 + 8 * lg);
             if (u == 0) {
-                float ss[4] = {0.f, 0.f, 0.f, 0.f};
+                float mine = 0.f;
+                for (int r = 0; r < p.M; ++r) {   // M <= 4: every lane walks row r, the lanes of row r keep it
+                    const u32x4 *row = reinterpret_cast<const u32x4 *>(p.x + (size_t)r * p.K);
+                    float a0 = 0.f, a1 = 0.f;
+                    for (int c = lane; c < (p.K >> 3); c += 64) {
+                        const u32x4 v = row[c];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if (r < p.M) {
-                        const u32x4 *row = reinterpret_cast<const u32x4 *>(p.x + (size_t)r * p.K);
-                        float a0 = 0.f, a1 = 0.f;
-                        for (int c = lane; c < (p.K >> 3); c += 64) {
-                            const u32x4 v = row[c];
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                const float lo = __builtin_bit_cast(float, v[j] << 16);
-                                const float hi = __builtin_bit_cast(float, v[j] & 0xFFFF0000u);
-                                a0 = fmaf(lo, lo, a0);
-                                a1 = fmaf(hi, hi, a1);
-                            }
+                        for (int j = 0; j < 4; ++j) {
+                            const float lo = __builtin_bit_cast(float, v[j] << 16);
+                            const float hi = __builtin_bit_cast(float, v[j] & 0xFFFF0000u);
+                            a0 = fmaf(lo, lo, a0);
+                            a1 = fmaf(hi, hi, a1);
                         }
-                        float a = a0 + a1;
-#pragma unroll
-                        for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off);
-                        ss[r] = a;
                     }
+                    float a = a0 + a1;
+#pragma unroll
+                    for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off);
+                    if (am == r) mine = a;
                 }
-                float mine = ss[0];
-                if (am == 1) mine = ss[1];
-                if (am == 2) mine = ss[2];
-                if (am == 3) mine = ss[3];
                 rstd = 1.0f / sqrtf(mine / (float)p.K + p.eps);
             }
 #pragma unroll
@@ -306,24 +299,18 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 
     // ---- cross-wave combine in LDS: red[slot][m][j * 17 + ln], j = natural column in the lane's chunk ----
     const int slot_stride = p.M * ROWF;
+    {
+        float *dst = red + wave * slot_stride;
 #pragma unroll
-    for (int r = 0; r < WAVES / SLOTS; ++r) {
-        if (wave / SLOTS == r) {
-            float *dst = red + (wave % SLOTS) * slot_stride;
+        for (int j = 0; j < LC; ++j) {
 #pragma unroll
-            for (int j = 0; j < LC; ++j) {
-#pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    const int m = lg + 4 * i;
-                    if (m < p.M) {
-                        float *q = dst + m * ROWF + j * 17 + ln;
-                        *q = (r == 0) ? yacc[j][i] : (*q + yacc[j][i]);
-                    }
-                }
+            for (int i = 0; i < MI; ++i) {
+                const int m = lg + 4 * i;
+                if (m < p.M) dst[m * ROWF + j * 17 + ln] = yacc[j][i];
             }
         }
-        __syncthreads();
     }
+    __syncthreads();
 
     // ---- workgroup result in 4-column quads; producers publish, the reducer gathers ----
     for (int e = threadIdx.x; e < nquads; e += WAVES * 64) {
@@ -411,14 +398,17 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 }
 
 // Launch shape.  Measured on MI355X (K = 4096, N = 11008): 256-column tiles (8-byte loads),
-// 8 waves per workgroup and a K-split of 4 are the fastest; a reducer fetches up to 8
-// producers' slots in one polling round, so the split is kept at or below 8 (4 for M > 4,
-// where the fp32 partials are M times larger) by giving each wave more units instead.
+// 8 waves per workgroup and one unit per wave are the fastest, which makes the K-split
+// K / 1024.  A long K with few tiles (the FFN down projection, K = 14336, N = 4096: 16 tiles)
+// needs the deep split to put a workgroup on most CUs: split 14 (224 workgroups) beats split 7
+// by 9 %, so the split is only capped at 16 (two polling rounds of the reducer) for M <= 4.
+// For M > 4 the fp32 partials are M times larger and the cap is 4 (M = 16: split 4 16.3 us,
+// split 8 32.6 us, split 2 19.4 us), more units per wave instead.
 StreamPlan plan_stream(int M, int K, int N) {
     StreamPlan pl;
     pl.mi = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     const int nksteps = K / 32;
-    pl.lw = M <= 4 ? 2 : 1;
+    pl.lw = 2;
     pl.ksteps = 4;
     pl.waves = 8;
     pl.units = 1;
@@ -430,7 +420,7 @@ StreamPlan plan_stream(int M, int K, int N) {
     if (g_stream_tune.units) {
         pl.units = g_stream_tune.units;
     } else {
-        const int max_split = M <= 4 ? 8 : 4;
+        const int max_split = M <= 4 ? 16 : 4;
         while (split() > max_split) ++pl.units;
     }
     pl.ksplit = split();
@@ -443,8 +433,14 @@ StreamPlan plan_stream(int M, int K, int N) {
 
 template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false>
 static hipError_t launch_one(const StreamParams &p, int grid, hipStream_t stream) {
-    constexpr int SLOTS = MI == 1 ? WAVES : (MI == 2 ? WAVES / 2 : WAVES / 4);
-    const size_t lds = (size_t)SLOTS * p.M * 8 * LW * 17 * sizeof(float);
+    const size_t lds = (size_t)WAVES * p.M * 8 * LW * 17 * sizeof(float);   // <= 136 KB at M = 16, LW = 2, 8 waves
+    static bool lds_opt_in = false;   // more than 64 KB of dynamic LDS needs the attribute once per kernel
+    if (!lds_opt_in && lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        lds_opt_in = true;
+    }
     hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>), dim3(grid), dim3(WAVES * 64), lds, stream, p);
     return hipGetLastError();
 }
