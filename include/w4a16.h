@@ -191,7 +191,7 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual,
 
 /*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
- * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units" (0 = built-in heuristic) and
+ * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic) and
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the
  * timeout test: split-K producers do not publish).  Process-wide.
  */

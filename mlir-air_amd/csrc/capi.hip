@@ -288,6 +288,9 @@ int w4a16_tune(const char *key, int value) {
         g_stream_tune.skip_publish = value ? 1 : 0;
     } else if (!strcmp(key, "gemv_spin_limit")) {
         g_stream_tune.spin_limit = value;
+    } else if (!strcmp(key, "gemv_ksplit")) {
+        if (value > kMaxKSplit) return W4A16_ERR_TUNE;
+        g_stream_tune.ksplit = value;
     } else if (!strcmp(key, "gemv_units")) {
         if (value > 64) return W4A16_ERR_TUNE;
         g_stream_tune.units = value;

@@ -17,6 +17,7 @@ struct StreamTune {
     int ksteps = 0;   // K-steps (32 rows) a wave loads per unit: 1, 2 or 4 (0 = heuristic)
     int waves = 0;    // waves per workgroup: 4 or 8
     int units = 0;    // units each wave processes back to back
+    int ksplit = 0;   // workgroups along K per tile (overrides units)
     int skip_publish = 0; // tests only: producers do not publish, so reducers run into their poll bound
     int spin_limit = 0;   // reducer poll bound (0 = default); tiny values force the timeout path in tests
 };

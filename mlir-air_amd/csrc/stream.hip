@@ -56,7 +56,8 @@ struct StreamParams {
     int nb;        // N / 8 packed words per row
     int ntiles;    // ceil(N / tile columns)
     int ksplit;    // workgroups along K per tile
-    int units;     // units per wave
+    int units;     // units per wave (of the largest slice)
+    int slice_units, slice_extra;   // units per K-slice: slice_units, +1 for the first slice_extra slices
     int nmat;      // 1, or 2 for gate/up with the SwiGLU epilogue
     const uint16_t *residual;   // [M, N] bf16 added in the epilogue, or null
     int round_before_add;       // 1: y = bf16(bf16(acc) + R); 0: y = bf16(acc + R)
@@ -161,9 +162,14 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 
     const int nksteps = p.K >> 5;
     float rstd = 0.f;
+    // K-slice `kslice` owns units [ulo, uhi) of the K / (32 * KSTEPS) units: slice_units each, the
+    // first slice_extra slices one more; its waves take them round-robin.
+    const int ulo = kslice * p.slice_units + (kslice < p.slice_extra ? kslice : p.slice_extra);
+    const int uhi = ulo + p.slice_units + (kslice < p.slice_extra ? 1 : 0);
     for (int u = 0; u < p.units; ++u) {
-        const int kstep0 = ((kslice * p.units + u) * WAVES + wave) * KSTEPS;
-        if (kstep0 >= nksteps) break;   // wave-uniform
+        const int unit = ulo + u * WAVES + wave;
+        if (unit >= uhi) break;   // wave-uniform
+        const int kstep0 = unit * KSTEPS;
         const int g = kstep0 >> 2;
 
         wvec w[KSTEPS][8];
@@ -399,7 +405,10 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 
 // Launch shape.  Measured on MI355X (K = 4096, N = 11008): 256-column tiles (8-byte loads),
 // 8 waves per workgroup and one unit per wave are the fastest, which makes the K-split
-// K / 1024.  A long K with few tiles (the FFN down projection, K = 14336, N = 4096: 16 tiles)
+// K / 1024.  All workgroups must be resident at once (one 8-wave workgroup per CU at these
+// register counts): a grid beyond 256 workgroups runs in two rounds and takes 17 us instead of
+// 10.7 us, and a deeper split within 256 (5 instead of 4) is slower too, because every extra
+// producer adds partial traffic to the reducer's critical path.  A long K with few tiles (the FFN down projection, K = 14336, N = 4096: 16 tiles)
 // needs the deep split to put a workgroup on most CUs: split 14 (224 workgroups) beats split 7
 // by 9 %, so the split is only capped at 16 (two polling rounds of the reducer) for M <= 4.
 // For M > 4 the fp32 partials are M times larger and the cap is 4 (M = 16: split 4 16.3 us,
@@ -416,18 +425,25 @@ StreamPlan plan_stream(int M, int K, int N) {
     if (g_stream_tune.ksteps) pl.ksteps = g_stream_tune.ksteps == 2 ? 2 : 4;
     if (g_stream_tune.waves) pl.waves = g_stream_tune.waves == 4 ? 4 : 8;
     pl.ntiles = (N + 128 * pl.lw - 1) / (128 * pl.lw);
-    auto split = [&]() { return (nksteps + pl.ksteps * pl.waves * pl.units - 1) / (pl.ksteps * pl.waves * pl.units); };
-    if (g_stream_tune.units) {
-        pl.units = g_stream_tune.units;
+    // Few tiles and a short K (e.g. a 4096 x 4096 projection: 16 tiles, 64 workgroups): halve the
+    // unit so that twice as many workgroups share the stream (9.1 us instead of 10.1 us there).
+    if (!g_stream_tune.ksteps && M <= 4 && pl.ntiles * ((nksteps / 4 + pl.waves - 1) / pl.waves) < 128) pl.ksteps = 2;
+    const int nunits = nksteps / pl.ksteps;   // K % 128 == 0, so this is exact for 2 and 4 K-steps per unit
+    if (g_stream_tune.ksplit) {
+        pl.ksplit = g_stream_tune.ksplit;
+    } else if (g_stream_tune.units) {
+        pl.ksplit = (nunits + pl.waves * g_stream_tune.units - 1) / (pl.waves * g_stream_tune.units);
     } else {
+        // one unit per wave while the split stays under its cap
         const int max_split = M <= 4 ? 16 : 4;
-        while (split() > max_split) ++pl.units;
+        pl.ksplit = (nunits + pl.waves - 1) / pl.waves;
+        if (pl.ksplit > max_split) pl.ksplit = max_split;
     }
-    pl.ksplit = split();
-    while (pl.ksplit > kMaxKSplit) {
-        pl.units *= 2;
-        pl.ksplit = split();
-    }
+    if (pl.ksplit > kMaxKSplit) pl.ksplit = kMaxKSplit;
+    if (pl.ksplit > nunits) pl.ksplit = nunits;
+    if (pl.ksplit < 1) pl.ksplit = 1;
+    const int per_slice = (nunits + pl.ksplit - 1) / pl.ksplit;   // largest slice
+    pl.units = (per_slice + pl.waves - 1) / pl.waves;
     return pl;
 }
 
@@ -492,6 +508,8 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.ntiles = pl.ntiles;
     p.ksplit = pl.ksplit;
     p.units = pl.units;
+    p.slice_units = (K / 32 / pl.ksteps) / pl.ksplit;
+    p.slice_extra = (K / 32 / pl.ksteps) % pl.ksplit;
     p.residual = extras.residual;
     p.round_before_add = extras.round_before_add;
     p.norm_w = extras.norm_w;

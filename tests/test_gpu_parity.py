@@ -100,6 +100,17 @@ def test_gemv_one_hot_x_is_a_dequantised_row(ops):
         assert np.array_equal(bits(y), w[k0]), k0
 
 
+@pytest.mark.parametrize("ksplit", [1, 3, 5, 7])
+def test_gemv_uneven_k_slices(ops, ksplit):
+    """K-slices whose sizes differ by one unit (K = 1024 + 128: 9 units over `ksplit` workgroups)."""
+    ops.tune("gemv_ksplit", ksplit)
+    try:
+        _gemm_case(ops, 1, 1152, 544, seed=60 + ksplit)
+        _gemm_case(ops, 7, 1152, 544, seed=70 + ksplit)
+    finally:
+        ops.tune("gemv_ksplit", 0)
+
+
 def test_gemv_repeat_calls_are_deterministic_and_workspace_is_reusable(ops):
     print("gemv repeat", flush=True)
     K, N = 4096, 11008
