@@ -91,6 +91,59 @@ def deinterleave_rows(A_q, A_s, A_z):
     return gate, up
 
 
+# --- the reference's tiled decode buffers -----------------------------------------------
+
+def bo_tile_bytes(GS, M_TILE, K_CHUNK):
+    """Bytes of one tile [Q: M_TILE * K_CHUNK / 2][S: K_CHUNK / GS * M_TILE bf16][Z: K_CHUNK / GS * M_TILE u8]
+    (matvec_int4_packed.py:63-67)."""
+    n_gpc = K_CHUNK // GS
+    return M_TILE * (K_CHUNK // 2), n_gpc * M_TILE * 2, n_gpc * M_TILE
+
+
+def _check_bo_shape(M, K, GS, M_TILE, K_CHUNK, N_CORES, M_PER_LAUNCH):
+    if M_PER_LAUNCH is None:
+        M_PER_LAUNCH = M
+    if K % K_CHUNK or K_CHUNK % GS or M % M_PER_LAUNCH or M_PER_LAUNCH % (N_CORES * M_TILE):
+        raise ValueError(f"tiling does not divide the matrix: M={M} K={K} GS={GS} M_TILE={M_TILE} "
+                         f"K_CHUNK={K_CHUNK} N_CORES={N_CORES} M_PER_LAUNCH={M_PER_LAUNCH}")
+    return M_PER_LAUNCH
+
+
+def pack_bo_tiles(A_q, A_s, A_z, M, K, GS=GROUP, M_TILE=8, K_CHUNK=2048, N_CORES=8, M_PER_LAUNCH=None):
+    """Kernel-side arrays -> uint8 [tiles, tile_bytes] in the reference's decode buffer layout
+    (matvec_int4_packed.pack_inputs, matvec_int4_packed.py:57-103).  Tiles are ordered launch ->
+    core -> M block -> K chunk; since launches, cores and M blocks each cover consecutive rows,
+    that is row-block-major: tile = (row / M_TILE) * (K / K_CHUNK) + k / K_CHUNK."""
+    _check_bo_shape(M, K, GS, M_TILE, K_CHUNK, N_CORES, M_PER_LAUNCH)
+    A_q = np.ascontiguousarray(A_q, dtype=np.uint8)
+    s_bits = np.ascontiguousarray(bf16.bits_of(A_s))
+    A_z = np.ascontiguousarray(A_z, dtype=np.uint8)
+    if A_q.shape != (M, K // 2) or s_bits.shape != (K // GS, M) or A_z.shape != (K // GS, M):
+        raise ValueError("pack_bo_tiles: array shapes do not match M, K, GS")
+    rb, kd, gpc = M // M_TILE, K // K_CHUNK, K_CHUNK // GS
+    q = A_q.reshape(rb, M_TILE, kd, K_CHUNK // 2).transpose(0, 2, 1, 3).reshape(rb * kd, -1)
+    sc = s_bits.reshape(kd, gpc, rb, M_TILE).transpose(2, 0, 1, 3).reshape(rb * kd, -1)
+    z = A_z.reshape(kd, gpc, rb, M_TILE).transpose(2, 0, 1, 3).reshape(rb * kd, -1)
+    return np.concatenate([q, np.ascontiguousarray(sc).view(np.uint8), z], axis=1)
+
+
+def unpack_bo_tiles(packed, M, K, GS=GROUP, M_TILE=8, K_CHUNK=2048, N_CORES=8, M_PER_LAUNCH=None):
+    """Inverse of pack_bo_tiles: a buffer packed by the reference -> (A_q, A_s, A_z); feed the
+    result to awq_from_l1 to obtain this backend's device tensors."""
+    _check_bo_shape(M, K, GS, M_TILE, K_CHUNK, N_CORES, M_PER_LAUNCH)
+    q_b, s_b, z_b = bo_tile_bytes(GS, M_TILE, K_CHUNK)
+    rb, kd, gpc = M // M_TILE, K // K_CHUNK, K_CHUNK // GS
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    if packed.size != rb * kd * (q_b + s_b + z_b):
+        raise ValueError(f"buffer has {packed.size} bytes, expected {rb * kd * (q_b + s_b + z_b)}")
+    packed = packed.reshape(rb * kd, q_b + s_b + z_b)
+    A_q = packed[:, :q_b].reshape(rb, kd, M_TILE, K_CHUNK // 2).transpose(0, 2, 1, 3).reshape(M, K // 2)
+    sc = np.ascontiguousarray(packed[:, q_b:q_b + s_b]).view(np.uint16).reshape(rb, kd, gpc, M_TILE)
+    A_s = sc.transpose(1, 2, 0, 3).reshape(K // GS, M)
+    A_z = packed[:, q_b + s_b:].reshape(rb, kd, gpc, M_TILE).transpose(1, 2, 0, 3).reshape(K // GS, M)
+    return np.ascontiguousarray(A_q), bf16.from_bits(np.ascontiguousarray(A_s)), np.ascontiguousarray(A_z)
+
+
 # --- single packed buffer ("BO") ------------------------------------------------------
 
 def _round256(v):

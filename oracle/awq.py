@@ -14,6 +14,9 @@ PE = programming_examples):
   l1_unpack_nibbles                  matvec_int4_packed.py:282-283 (byte ->
                                      even/odd-k nibble)
   dequant_1d                         PE/dequant_awq/dequant_awq.py:391-396
+  pack_inputs_loop                   PE/matrix_vector_multiplication/int4_awq/
+                                     matvec_int4_packed.py:57-103 (decode buffer tiling;
+                                     pinned by a hand-computed tile and its byte offsets)
 
 bf16 tensors are uint16 bit patterns (see oracle/bf16.py).
 
@@ -126,3 +129,31 @@ def dequant_1d(int4_vals, scales_bits, zeros, group_size):
     z = np.asarray(zeros).astype(np.float64)[g]
     s = bf16_bits_to_f32(scales_bits).astype(np.float64)[g]
     return f32_to_bf16_bits(((q - z) * s).astype(np.float32))
+
+
+def pack_inputs_loop(a_q, a_s_bits, a_z, M, K, GS, M_TILE, K_CHUNK, N_CORES, M_PER_LAUNCH):
+    """Scalar restatement of the decode buffer tiling (matvec_int4_packed.py:57-103): one tile per
+    (launch, core, M block, K chunk) in that nesting order, each tile
+    [Q rows x K_CHUNK/2 bytes][S groups x rows bf16][Z groups x rows u8].  Pure Python loops over
+    bytes: small shapes only."""
+    n_gpc = K_CHUNK // GS
+    q_bytes, s_bytes, z_bytes = M_TILE * (K_CHUNK // 2), n_gpc * M_TILE * 2, n_gpc * M_TILE
+    m_core = M_PER_LAUNCH // N_CORES
+    tiles = []
+    for launch in range(M // M_PER_LAUNCH):
+        for core in range(N_CORES):
+            for outer in range(m_core // M_TILE):
+                row0 = launch * M_PER_LAUNCH + core * m_core + outer * M_TILE
+                for kc in range(K // K_CHUNK):
+                    t = np.zeros(q_bytes + s_bytes + z_bytes, dtype=np.uint8)
+                    for r in range(M_TILE):
+                        for b in range(K_CHUNK // 2):
+                            t[r * (K_CHUNK // 2) + b] = a_q[row0 + r, kc * (K_CHUNK // 2) + b]
+                    for g in range(n_gpc):
+                        for r in range(M_TILE):
+                            v = int(a_s_bits[kc * n_gpc + g, row0 + r])
+                            o = q_bytes + 2 * (g * M_TILE + r)
+                            t[o], t[o + 1] = v & 0xFF, v >> 8            # little-endian bf16
+                            t[q_bytes + s_bytes + g * M_TILE + r] = a_z[kc * n_gpc + g, row0 + r]
+                    tiles.append(t)
+    return np.stack(tiles)
