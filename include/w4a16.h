@@ -190,6 +190,29 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual,
                           void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Decode attention for one new token with the RoPE of Q and K and the KV-cache append fused in.
+ * `qkv` is the token's fresh projection [Q (n_heads * head_dim) | K (n_kv_heads * head_dim) |
+ * V (n_kv_heads * head_dim)] bf16, e.g. the output of w4a16_rms_gemv_bf16 on the concatenated
+ * Q|K|V weights; `rope_lut_row` is row `pos` of the RoPE table, bf16 [head_dim] = cos then sin
+ * (generate_rope_lut, programming_examples/llms/llama32_1b/llama32_1b_weights.py:395-444).
+ * The kernel rotates Q and K half-split (rope_halfsplit, _cpu_rope in
+ * programming_examples/llms/llama32_1b_int4/llama32_1b_int4_prefill.py:508-524), writes the
+ * rotated K and V into k_cache / v_cache [n_kv_heads, max_seq, head_dim] at `pos`, and computes
+ * single-query grouped-query attention over positions 0..pos (decode_attention_cpu,
+ * programming_examples/llms/llama32_1b_int4/llama32_1b_int4_decode.py:135-168, which the
+ * reference runs on the host CPU) into attn_out bf16 [n_heads * head_dim].
+ * Replaces launches L5, L6 of rms_qkv_int4_rope (rms_qkv_int4_rope_multi.py:4-30), the cache
+ * update and the attention of run_decode_block (llama32_1b_int4_decode.py:270-285).
+ * head_dim 64 or 128; n_heads / n_kv_heads in {1, 2, 4, 8}; 0 <= pos < max_seq.
+ * The workspace is plain scratch (no initialisation), w4a16_attention_workspace_bytes().
+ */
+size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim);
+int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_row,
+                                uint16_t *k_cache, uint16_t *v_cache, uint16_t *attn_out,
+                                int pos, int max_seq, int n_heads, int n_kv_heads, int head_dim,
+                                void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic) and
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the

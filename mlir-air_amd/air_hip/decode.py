@@ -1,0 +1,84 @@
+"""One int4 decode step on the GPU: the counterpart of run_decode_block
+(programming_examples/llms/llama32_1b_int4/llama32_1b_int4_decode.py:176-313).
+
+The reference issues two NPU calls per layer (rms_qkv_int4_rope: 6 launches; o_gemv_ffn_int4:
+3 launches) with the KV-cache update and the attention on the host CPU in between.  Here a layer
+is five kernel launches, all on the device:
+
+  1. RMSNorm + fused Q|K|V int4 GEMV (one matrix, concatenated along the output axis)
+  2. RoPE(Q, K) + cache append + grouped-query attention (+ 3. the chunk combine for long contexts)
+  4-6. O projection + residual, RMSNorm + gate/up + SwiGLU, down projection + residual
+"""
+
+import dataclasses
+
+import numpy as np
+import torch
+
+from . import ops, weights as wmod
+
+
+def generate_rope_lut(config, seq_len=2048, device="cuda"):
+    """bf16 [seq_len, head_dim]: cos(pos * f_i) for i < head_dim / 2, then sin(pos * f_i), with
+    f_i = rope_base^(-2i / head_dim) evaluated in float64 and rounded once
+    (programming_examples/llms/llama32_1b/llama32_1b_weights.py:395-444)."""
+    hd = config.head_dim
+    inv_freq = 1.0 / (config.rope_base ** (np.arange(0, hd, 2, dtype=np.float64) / hd))
+    angles = np.outer(np.arange(seq_len, dtype=np.float64), inv_freq)
+    lut = np.concatenate([np.cos(angles), np.sin(angles)], axis=1).astype(np.float32)
+    return torch.from_numpy(lut).to(torch.bfloat16).to(device)
+
+
+@dataclasses.dataclass
+class DecodeLayer:
+    """Device tensors of one layer in the form the kernels read."""
+
+    attn_norm: torch.Tensor
+    ffn_norm: torch.Tensor
+    wqkv: tuple       # fused (qweight, qzeros, scales), N = (n_heads + 2 n_kv) * head_dim
+    wo: tuple
+    w_gate: tuple
+    w_up: tuple
+    w_down: tuple
+
+
+def prepare_layer(layer: wmod.LayerWeights, device="cuda") -> DecodeLayer:
+    """Host LayerWeights (numpy) -> DecodeLayer: Q, K, V concatenated, everything in HBM."""
+    def dev(a):
+        a = np.ascontiguousarray(a)
+        if a.dtype == np.uint16:
+            return torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+        return torch.from_numpy(a).to(device)
+
+    lin = lambda l: tuple(dev(t) for t in l)
+    return DecodeLayer(attn_norm=dev(layer.attn_norm), ffn_norm=dev(layer.ffn_norm),
+                       wqkv=lin(wmod.concat_linears(layer.wq, layer.wk, layer.wv)), wo=lin(layer.wo),
+                       w_gate=lin(layer.w_gate), w_up=lin(layer.w_up), w_down=lin(layer.w_down))
+
+
+def new_kv_cache(config, max_seq, device="cuda"):
+    """Per-layer caches [n_kv_heads, max_seq, head_dim] bf16 (the reference's layout)."""
+    shape = (config.n_kv_heads, max_seq, config.head_dim)
+    return [(torch.zeros(shape, dtype=torch.bfloat16, device=device), torch.zeros(shape, dtype=torch.bfloat16, device=device))
+            for _ in range(config.n_layers)]
+
+
+def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer, current_pos, rope_lut):
+    """One transformer block for one decode token; x bf16 [emb] -> bf16 [emb].  The caches are
+    updated in place at current_pos."""
+    qkv = ops.w4a16_rms_gemv(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps)
+    attn_out = ops.decode_attention(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads)
+    return ops.o_gemv_ffn(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
+
+
+def decode_token(token_id, layers, embed_table, final_norm, lm_head, config, kv_cache, current_pos, rope_lut):
+    """Full model step: embedding row -> blocks -> final RMSNorm -> logits (fp32 [vocab]).
+    The embedding lookup, the final norm and the bf16 lm_head product are plain torch calls;
+    the reference runs the same three pieces outside its int4 kernels
+    (llama32_1b_int4_inference.py: lm_head_gemv is a bf16 GEMV)."""
+    x = embed_table[token_id].contiguous()
+    for layer, (kc, vc) in zip(layers, kv_cache):
+        x = run_decode_block(x, layer, config, kc, vc, current_pos, rope_lut)
+    xf = x.float()
+    normed = ((xf * torch.rsqrt((xf * xf).mean() + config.rms_eps)) * final_norm.float()).to(torch.bfloat16)
+    return (lm_head @ normed).float()

@@ -214,6 +214,32 @@ def o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e
     return (y, res1, h) if return_intermediates else y
 
 
+_attn_ws = {}
+
+
+def decode_attention(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, out=None):
+    """RoPE on Q and K of the new token, KV-cache append at `pos`, single-query GQA attention.
+
+    qkv bf16 [n_heads * hd + 2 * n_kv * hd]; rope_lut_row bf16 [hd]; caches bf16 [n_kv, max_seq, hd]
+    (updated in place).  Returns attn_out bf16 [n_heads * hd]."""
+    lib = _lib.load_library()
+    _need_cuda(qkv, rope_lut_row, k_cache, v_cache)
+    n_kv, max_seq, hd = k_cache.shape
+    if v_cache.shape != k_cache.shape or qkv.numel() != (n_heads + 2 * n_kv) * hd or rope_lut_row.numel() != hd:
+        raise ValueError("decode_attention: qkv must be [(n_heads + 2 n_kv) * hd], caches [n_kv, max_seq, hd], lut row [hd]")
+    if out is None:
+        out = torch.empty((n_heads * hd,), dtype=torch.bfloat16, device=qkv.device)
+    key = (qkv.device.index, _stream(), n_heads, hd)
+    ws = _attn_ws.get(key)
+    if ws is None:
+        ws = torch.empty(int(lib.w4a16_attention_workspace_bytes(n_heads, hd)), dtype=torch.uint8, device=qkv.device)
+        _attn_ws[key] = ws
+    _lib.check(lib.w4a16_decode_attention_bf16(_ptr(_bits(qkv)), _ptr(_bits(rope_lut_row)), _ptr(_bits(k_cache)),
+                                               _ptr(_bits(v_cache)), _ptr(out), int(pos), max_seq, n_heads, n_kv, hd,
+                                               _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
 def tune(key, value):
     lib = _lib.load_library()
     _lib.check(lib.w4a16_tune(key.encode(), int(value)))

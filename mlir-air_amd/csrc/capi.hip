@@ -273,6 +273,29 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, 
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim) {
+    if (n_heads <= 0 || head_dim <= 0) return 0;
+    return round256(attention_workspace_bytes(n_heads, head_dim));
+}
+
+int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_row, uint16_t *k_cache,
+                                uint16_t *v_cache, uint16_t *attn_out, int pos, int max_seq, int n_heads,
+                                int n_kv_heads, int head_dim, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!qkv || !rope_lut_row || !k_cache || !v_cache || !attn_out) return W4A16_ERR_NULL;
+    if (head_dim != 64 && head_dim != 128) return W4A16_ERR_SHAPE;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads) return W4A16_ERR_SHAPE;
+    const int g = n_heads / n_kv_heads;
+    if (g != 1 && g != 2 && g != 4 && g != 8) return W4A16_ERR_SHAPE;
+    if (max_seq <= 0 || pos < 0 || pos >= max_seq) return W4A16_ERR_SHAPE;
+    if (misaligned(qkv) || misaligned(rope_lut_row) || misaligned(k_cache) || misaligned(v_cache) || misaligned(attn_out))
+        return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_attention_workspace_bytes(n_heads, head_dim)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_decode_attention(qkv, rope_lut_row, k_cache, v_cache, attn_out, pos, max_seq, n_heads,
+                                           n_kv_heads, head_dim, workspace, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_tune(const char *key, int value) {
     if (!key || value < 0) return W4A16_ERR_TUNE;
     if (!strcmp(key, "gemv_lw")) {

@@ -51,4 +51,13 @@ hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const 
 
 hipError_t launch_fill_workspace(void *ptr, size_t bytes, hipStream_t stream);
 
+// Decode attention (attention.hip).  The scratch buffer holds per-chunk softmax partials and
+// needs no initialisation.
+constexpr int kMaxAttnSplit = 32;
+int attention_nsplit(int seq_len);
+size_t attention_workspace_bytes(int n_heads, int head_dim);
+hipError_t launch_decode_attention(const uint16_t *qkv, const uint16_t *lut_row, uint16_t *k_cache, uint16_t *v_cache,
+                                   uint16_t *out, int pos, int max_seq, int n_heads, int n_kv, int head_dim,
+                                   void *workspace, hipStream_t stream);
+
 }  // namespace w4a16

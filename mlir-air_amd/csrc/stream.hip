@@ -160,7 +160,6 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 #pragma unroll
     for (int t = 0; t < LC; ++t) yacc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    const int nksteps = p.K >> 5;
     float rstd = 0.f;
     // K-slice `kslice` owns units [ulo, uhi) of the K / (32 * KSTEPS) units: slice_units each, the
     // first slice_extra slices one more; its waves take them round-robin.

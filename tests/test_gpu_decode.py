@@ -1,0 +1,135 @@
+"""GPU parity of the decode attention kernel and of a whole decode block against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_bf16_close, bf16_ulp, make_awq, make_x
+from oracle import awq as oawq, decode as odec, reference as oref
+from oracle.bf16 import bf16_bits_to_f32, f32_to_bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(a).cuda()
+
+
+def bits(t):
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from air_hip import ops
+    return ops
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,max_seq,positions", [
+    (8, 2, 64, 64, [0, 1, 7, 31, 63]),            # one chunk
+    (32, 8, 64, 2048, [0, 127, 128, 500, 2047]),  # Llama-3.2-1B heads, up to 16 chunks
+    (8, 8, 128, 700, [5, 300, 699]),              # no grouping, head_dim 128, ragged chunks
+    (16, 2, 128, 4500, [4499]),                   # group 8, chunk count capped at 32
+    (4, 2, 64, 300, [299]),                       # group 2
+])
+def test_decode_attention(ops, n_heads, n_kv, hd, max_seq, positions):
+    rng = np.random.default_rng(n_heads * 1000 + hd)
+    lut = odec.generate_rope_lut(hd, 500000.0, max_seq)
+    k_cache = f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32))
+    v_cache = f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32))
+    dk, dv, dlut = dev(k_cache), dev(v_cache), dev(lut)
+    for pos in positions:
+        print(f"attention heads={n_heads}/{n_kv} hd={hd} pos={pos}", flush=True)
+        qkv = f32_to_bf16_bits(rng.standard_normal((n_heads + 2 * n_kv) * hd).astype(np.float32))
+        out = ops.decode_attention(dev(qkv), dlut[pos], dk, dv, pos, n_heads)
+        torch.cuda.synchronize()
+        nq, nkv = n_heads * hd, n_kv * hd
+        q_r = odec.rope_halfsplit(qkv[:nq].reshape(n_heads, hd), lut[pos]).reshape(-1)
+        k_r = odec.rope_halfsplit(qkv[nq:nq + nkv].reshape(n_kv, hd), lut[pos])
+        k_cache[:, pos, :] = k_r
+        v_cache[:, pos, :] = qkv[nq + nkv:].reshape(n_kv, hd)
+        # the append is bit-exact (RoPE is two exact products and one add in fp32, one rounding)
+        assert np.array_equal(bits(dk)[:, pos, :], k_cache[:, pos, :])
+        assert np.array_equal(bits(dv)[:, pos, :], v_cache[:, pos, :])
+        assert np.array_equal(bits(dk), k_cache) and np.array_equal(bits(dv), v_cache)   # nothing else touched
+        want = bf16_bits_to_f32(odec.decode_attention_cpu(q_r, k_cache, v_cache, pos, n_heads, n_kv, hd)).astype(np.float64)
+        # fp32 softmax in a different summation order and exp2 instead of exp: 1 bf16 ulp + 2e-3
+        assert_bf16_close(bits(out), want, ulps=1.0, atol=2e-3, what=f"attention pos={pos}")
+
+
+def _layer(E, H, n_heads, n_kv, hd, seed):
+    t = {"wq": make_awq(E, n_heads * hd, seed=seed), "wk": make_awq(E, n_kv * hd, seed=seed + 1),
+         "wv": make_awq(E, n_kv * hd, seed=seed + 2), "wo": make_awq(n_heads * hd, E, seed=seed + 3),
+         "w_gate": make_awq(E, H, seed=seed + 4), "w_up": make_awq(E, H, seed=seed + 5),
+         "w_down": make_awq(H, E, seed=seed + 6)}
+    rng = np.random.default_rng(seed + 7)
+    norm = lambda: f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32))
+    return t, norm(), norm()
+
+
+def test_decode_block_matches_the_oracle_over_several_tokens(ops):
+    from air_hip import decode, weights
+
+    cfg = weights.LlamaConfig(n_layers=1, emb_dim=512, n_heads=8, head_dim=64, n_kv_heads=2, hidden_dim=1024, vocab_size=32)
+    max_seq = 160
+    t, attn_norm, ffn_norm = _layer(cfg.emb_dim, cfg.hidden_dim, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, seed=300)
+    # scale the projections down so that activations stay O(1) through the block
+    small = lambda w: (w[0], w[1], f32_to_bf16_bits(bf16_bits_to_f32(w[2]) * 0.05))
+    t = {k: small(v) for k, v in t.items()}
+    host = weights.LayerWeights(attn_norm=attn_norm, ffn_norm=ffn_norm, **t)
+    layer = decode.prepare_layer(host)
+    l1 = {k: oawq.repack_hf_awq_linear(*v, 128) for k, v in t.items()}
+    l1.update(attn_norm=attn_norm, ffn_norm=ffn_norm)
+    lut_bits = odec.generate_rope_lut(cfg.head_dim, cfg.rope_base, max_seq)
+    lut = decode.generate_rope_lut(cfg, max_seq)
+    assert np.array_equal(bits(lut), lut_bits)
+    (kc, vc), = decode.new_kv_cache(cfg, max_seq)
+    kc_ref = np.zeros((cfg.n_kv_heads, max_seq, cfg.head_dim), np.uint16)
+    vc_ref = np.zeros_like(kc_ref)
+    rng = np.random.default_rng(9)
+    for pos in list(range(6)) + [130]:
+        print(f"decode block pos={pos}", flush=True)
+        if pos == 130:   # jump ahead: fill the gap identically on both sides
+            fill = f32_to_bf16_bits(rng.standard_normal((2, cfg.n_kv_heads, 124, cfg.head_dim)).astype(np.float32))
+            kc_ref[:, 6:130], vc_ref[:, 6:130] = fill[0], fill[1]
+            kc[:, 6:130] = dev(fill[0])
+            vc[:, 6:130] = dev(fill[1])
+        x = make_x((cfg.emb_dim,), seed=400 + pos)
+        y = decode.run_decode_block(dev(x), layer, cfg, kc, vc, pos, lut)
+        torch.cuda.synchronize()
+        want = odec.decode_block_reference(x, l1, kc_ref, vc_ref, pos, lut_bits, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim)
+        got_f, want_f = bf16_bits_to_f32(bits(y)), bf16_bits_to_f32(want)
+        # the reference's own block gate, then a tighter bound: a few bf16 ulps of the output scale
+        assert oref.check_outputs(got_f, want_f, rtol=0.2, atol=2.0, min_correlation=0.99)
+        assert np.max(np.abs(got_f - want_f)) <= 8 * 2.0**-8 * np.max(np.abs(want_f)), np.max(np.abs(got_f - want_f))
+        # caches agree up to one-ulp flips that the RMSNorm prologue's rounding may cause in K/V
+        kd = np.abs(bf16_bits_to_f32(bits(kc)[:, pos]) - bf16_bits_to_f32(kc_ref[:, pos]))
+        assert np.all(kd <= 2 * bf16_ulp(bf16_bits_to_f32(kc_ref[:, pos])) + 2e-2), kd.max()
+        # keep both sides in lock step for the following positions
+        kc[:, pos] = dev(kc_ref[:, pos])
+        vc[:, pos] = dev(vc_ref[:, pos])
+
+
+def test_decode_token_runs_a_two_layer_model(ops):
+    from air_hip import decode, weights
+
+    cfg = weights.LlamaConfig(n_layers=2, emb_dim=256, n_heads=4, head_dim=64, n_kv_heads=2, hidden_dim=512, vocab_size=64)
+    layers = []
+    for i in range(cfg.n_layers):
+        t, an, fn = _layer(cfg.emb_dim, cfg.hidden_dim, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, seed=500 + 10 * i)
+        t = {k: (v[0], v[1], f32_to_bf16_bits(bf16_bits_to_f32(v[2]) * 0.05)) for k, v in t.items()}
+        layers.append(decode.prepare_layer(weights.LayerWeights(attn_norm=an, ffn_norm=fn, **t)))
+    g = torch.Generator(device="cuda").manual_seed(1)
+    embed = torch.randn((cfg.vocab_size, cfg.emb_dim), device="cuda", generator=g).to(torch.bfloat16)
+    final_norm = torch.ones(cfg.emb_dim, device="cuda", dtype=torch.bfloat16)
+    lut = decode.generate_rope_lut(cfg, 32)
+    cache = decode.new_kv_cache(cfg, 32)
+    tok = 3
+    for pos in range(4):
+        print(f"decode token pos={pos}", flush=True)
+        logits = decode.decode_token(tok, layers, embed, final_norm, embed, cfg, cache, pos, lut)
+        assert logits.shape == (cfg.vocab_size,) and torch.isfinite(logits).all()
+        tok = int(torch.argmax(logits))
+    assert float(cache[1][0][:, :4].float().abs().sum()) > 0 and float(cache[1][0][:, 4:].float().abs().sum()) == 0

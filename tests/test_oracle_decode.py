@@ -1,0 +1,62 @@
+"""Pins for the decode-block oracle: each check fails for a plausible slip (swapped sin/cos,
+wrong sign, interleaved instead of half-split pairing, missing scale, wrong head grouping)."""
+import numpy as np
+import torch
+
+from oracle import decode as dec
+from oracle.bf16 import bf16_bits_to_f32, f32_to_bf16_bits
+
+
+def test_rope_lut_closed_forms():
+    lut = bf16_bits_to_f32(dec.generate_rope_lut(64, 500000.0, 33))
+    assert lut.shape == (33, 64)
+    assert np.all(lut[0, :32] == 1.0) and np.all(lut[0, 32:] == 0.0)          # position 0: cos 1, sin 0
+    r = lambda v: bf16_bits_to_f32(f32_to_bf16_bits(np.float32(v)))
+    assert lut[1, 0] == r(np.cos(1.0)) and lut[1, 32] == r(np.sin(1.0))       # index 0: frequency 1
+    assert lut[5, 16] == r(np.cos(5.0 * 500000.0 ** -0.5))                     # i = 16: base^(-32/64)
+    assert lut[7, 32 + 31] == r(np.sin(7.0 * 500000.0 ** (-62.0 / 64.0)))
+
+
+def test_rope_is_the_complex_rotation_of_half_split_pairs():
+    rng = np.random.default_rng(0)
+    x = f32_to_bf16_bits(rng.standard_normal((5, 64)).astype(np.float32))
+    lut = dec.generate_rope_lut(64, 10000.0, 40)
+    got = bf16_bits_to_f32(dec.rope_halfsplit(x, lut[17]))
+    xf = bf16_bits_to_f32(x).astype(np.float64)
+    l = bf16_bits_to_f32(lut[17]).astype(np.float64)
+    z = (xf[:, :32] + 1j * xf[:, 32:]) * (l[:32] + 1j * l[32:])               # pair (i, i + 32)
+    want = np.concatenate([z.real, z.imag], axis=1)
+    assert np.max(np.abs(got - want)) <= 2.0**-8 * np.max(np.abs(want)) + 1e-6
+    # position 0 is the identity, bit for bit
+    assert np.array_equal(dec.rope_halfsplit(x, lut[0]), x)
+    # an interleaved pairing (2i, 2i + 1) would differ
+    zi = (xf[:, 0::2] + 1j * xf[:, 1::2]) * (l[:32] + 1j * l[32:])
+    assert np.max(np.abs(got[:, :32] - zi.real)) > 0.1
+
+
+def test_attention_against_library_and_closed_forms():
+    n_heads, n_kv, hd, max_seq, pos = 8, 2, 64, 48, 36
+    rng = np.random.default_rng(1)
+    q = f32_to_bf16_bits(rng.standard_normal(n_heads * hd).astype(np.float32))
+    k = f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32))
+    v = f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32))
+    got = bf16_bits_to_f32(dec.decode_attention_cpu(q, k, v, pos, n_heads, n_kv, hd)).reshape(n_heads, hd)
+    tq = torch.from_numpy(bf16_bits_to_f32(q)).double().reshape(1, n_heads, 1, hd)
+    tk = torch.from_numpy(bf16_bits_to_f32(k[:, :pos + 1])).double().repeat_interleave(n_heads // n_kv, dim=0)[None]
+    tv = torch.from_numpy(bf16_bits_to_f32(v[:, :pos + 1])).double().repeat_interleave(n_heads // n_kv, dim=0)[None]
+    want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv)[0, :, 0].numpy()
+    assert np.max(np.abs(got - want)) <= 2.0**-8 * np.max(np.abs(want)) + 1e-5
+    # positions beyond current_pos are ignored
+    k2, v2 = k.copy(), v.copy()
+    k2[:, pos + 1:] = 0x7F80
+    v2[:, pos + 1:] = 0x7F80
+    assert np.array_equal(dec.decode_attention_cpu(q, k2, v2, pos, n_heads, n_kv, hd), f32_to_bf16_bits(got.reshape(-1)))
+    # seq_len 1: the output is v[kv head of h][0] for every head
+    one = dec.decode_attention_cpu(q, k, v, 0, n_heads, n_kv, hd).reshape(n_heads, hd)
+    for h in range(n_heads):
+        assert np.array_equal(one[h], v[h // 4, 0])
+    # equal keys: uniform softmax, the output is the mean of the values
+    ke = np.broadcast_to(k[:, :1], k.shape).copy()
+    me = bf16_bits_to_f32(dec.decode_attention_cpu(q, ke, v, pos, n_heads, n_kv, hd)).reshape(n_heads, hd)
+    mean = bf16_bits_to_f32(v[:, :pos + 1]).astype(np.float64).mean(axis=1)
+    assert np.max(np.abs(me - mean[np.arange(n_heads) // 4])) <= 2.0**-8 * np.abs(mean).max() + 1e-4
