@@ -34,7 +34,11 @@ CONFIGS = {
     "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128"),
     # not a BASELINE config: the O projection + RMSNorm + FFN decode block with residuals (3 launches)
     "block": dict(M=1, K=4096, N=14336, cfg=None, desc="decode block O-proj + RMSNorm + SwiGLU FFN W4A16 E=4096 H=14336 g128"),
+    # one whole decode layer: RMSNorm + fused QKV GEMV, RoPE + KV append + GQA attention over 2048 cached
+    # positions (32 heads, 8 KV heads, head_dim 128), then the block above
+    "layer": dict(M=1, K=4096, N=14336, cfg=None, desc="decode layer W4A16 E=4096 H=14336 32/8 heads hd=128 pos=2047 g128"),
 }
+LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 2048
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
 # scaled by the same counter's reading for a 256 MiB device copy: x2.000 and x1.000); the
@@ -55,6 +59,10 @@ def algorithmic_bytes(name):
         return 3 * weight_bytes(K, N) + K * 2 + K * 2
     if name == "block":   # wo + gate + up + down; attn_out, x_residual, norm weight in, y out
         return weight_bytes(K, K) + 3 * weight_bytes(K, N) + 4 * K * 2
+    if name == "layer":   # + fused QKV weights and the K and V caches up to pos
+        nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
+        return (weight_bytes(K, nqkv) + 2 * LAYER_KV * (LAYER_POS + 1) * LAYER_HD * 2
+                + weight_bytes(K, K) + 3 * weight_bytes(K, N) + 5 * K * 2)
     return weight_bytes(K, N) + M * K * 2 + M * N * 2
 
 
@@ -62,7 +70,7 @@ def algorithmic_flops(name):
     c = CONFIGS[name]
     if name == "ffn":
         return 2 * 3 * c["K"] * c["N"]
-    if name == "block":
+    if name in ("block", "layer"):
         return 2 * (3 * c["K"] * c["N"] + c["K"] * c["K"])
     return 2 * max(c["M"], 0) * c["K"] * c["N"]
 
@@ -89,7 +97,10 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     torch.cuda.set_device(dev)
     stream = torch.cuda.Stream()
 
-    per_copy = weight_bytes(K, N) * (3 if name in ("ffn", "block") else 1) + (weight_bytes(K, K) if name == "block" else 0)
+    per_copy = weight_bytes(K, N) * (3 if name in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if name in ("block", "layer") else 0)
+    nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
+    if name == "layer":
+        per_copy += weight_bytes(K, nqkv)
     if name == "prefill":
         ncopies = 1
     else:
@@ -99,9 +110,10 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         if name == "ffn":
             copies.append((make_weights(torch, K, N, 100 + 3 * i), make_weights(torch, K, N, 101 + 3 * i),
                            make_weights(torch, N, K, 102 + 3 * i)))
-        elif name == "block":
-            copies.append((make_weights(torch, K, N, 100 + 4 * i), make_weights(torch, K, N, 101 + 4 * i),
-                           make_weights(torch, N, K, 102 + 4 * i), make_weights(torch, K, K, 103 + 4 * i)))
+        elif name in ("block", "layer"):
+            c4 = (make_weights(torch, K, N, 100 + 5 * i), make_weights(torch, K, N, 101 + 5 * i),
+                  make_weights(torch, N, K, 102 + 5 * i), make_weights(torch, K, K, 103 + 5 * i))
+            copies.append(c4 + ((make_weights(torch, K, nqkv, 104 + 5 * i),) if name == "layer" else ()))
         else:
             copies.append(make_weights(torch, K, N, 100 + i))
     gx = torch.Generator(device="cuda")
@@ -109,18 +121,26 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     x = torch.randn((max(M, 1), K), device="cuda", generator=gx).to(torch.bfloat16)
     if name == "dequant":
         outs = [torch.empty((K, N), dtype=torch.bfloat16, device=dev) for _ in range(min(ncopies, 8))]
-    elif name in ("ffn", "block"):
+    elif name in ("ffn", "block", "layer"):
         outs = [torch.empty((K,), dtype=torch.bfloat16, device=dev)]
     else:
         outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev)]
-    if name == "block":
+    if name in ("block", "layer"):
         x_residual = torch.randn((K,), device="cuda", generator=gx).to(torch.bfloat16)
         norm_w = (torch.randn((K,), device="cuda", generator=gx) * 0.1 + 1.0).to(torch.bfloat16)
+    if name == "layer":
+        kv_shape = (LAYER_KV, LAYER_MAXSEQ, LAYER_HD)
+        k_cache = torch.randn(kv_shape, device="cuda", generator=gx).to(torch.bfloat16)
+        v_cache = torch.randn(kv_shape, device="cuda", generator=gx).to(torch.bfloat16)
+        lut_row = torch.rand((LAYER_HD,), device="cuda", generator=gx).to(torch.bfloat16)
+        qkv = torch.empty((nqkv,), dtype=torch.bfloat16, device=dev)
+        attn_out = torch.empty((K,), dtype=torch.bfloat16, device=dev)
+        attn_ws = torch.empty(int(lib.w4a16_attention_workspace_bytes(LAYER_HEADS, LAYER_HD)), dtype=torch.uint8, device=dev)
 
     if name == "ffn":
         ws_bytes = lib.w4a16_ffn_workspace_bytes(K, N)
-    elif name == "block":
-        ws_bytes = lib.w4a16_block_workspace_bytes(K, N)
+    elif name in ("block", "layer"):
+        ws_bytes = max(lib.w4a16_block_workspace_bytes(K, N), lib.w4a16_gemm_workspace_bytes(1, K, nqkv))
     else:
         ws_bytes = max(lib.w4a16_gemm_workspace_bytes(max(M, 1), K, N), 16384)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
@@ -137,10 +157,21 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                            u[0].data_ptr(), u[1].data_ptr(), u[2].data_ptr(),
                                            d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(),
                                            outs[0].data_ptr(), None, K, N, 128, ws.data_ptr(), ws.numel(), st)
-        elif name == "block":
-            g, u, d, o = w
+        elif name in ("block", "layer"):
+            g, u, d, o = w[:4]
             ptrs = [t.data_ptr() for m in (o, g, u, d) for t in m]
-            rc = lib.w4a16_o_gemv_ffn_bf16(x.data_ptr(), x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, *ptrs,
+            a_in = x
+            if name == "layer":
+                qw = w[4]
+                _lib.check(lib.w4a16_rms_gemv_bf16(x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, qw[0].data_ptr(),
+                                                   qw[1].data_ptr(), qw[2].data_ptr(), qkv.data_ptr(), K, nqkv, 128,
+                                                   ws.data_ptr(), ws.numel(), st))
+                _lib.check(lib.w4a16_decode_attention_bf16(qkv.data_ptr(), lut_row.data_ptr(), k_cache.data_ptr(),
+                                                           v_cache.data_ptr(), attn_out.data_ptr(), LAYER_POS, LAYER_MAXSEQ,
+                                                           LAYER_HEADS, LAYER_KV, LAYER_HD, attn_ws.data_ptr(),
+                                                           attn_ws.numel(), st))
+                a_in = attn_out
+            rc = lib.w4a16_o_gemv_ffn_bf16(a_in.data_ptr(), x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, *ptrs,
                                            outs[0].data_ptr(), None, None, K, N, 128, ws.data_ptr(), ws.numel(), st)
         else:
             rc = lib.w4a16_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
@@ -185,7 +216,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         "ncopies": ncopies,
     }
 
-    if with_cpu_baseline and name != "block":
+    if with_cpu_baseline and name not in ("block", "layer"):
         res["cpu_baseline"] = cpu_baseline(name, torch, copies[0], x, outs, launch, stream)
     return res
 
