@@ -116,24 +116,39 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const AttnParams p) {
         for (int j = 0; j < 8; ++j) acc[h][j] = 0.f;
     }
 
-    for (int t = t0 + wave * PPW + slot; t < t1; t += 4 * PPW) {
-        float k[8], v[8];
-        unpack8(*reinterpret_cast<const u32x4 *>(kc + (size_t)t * HD + 8 * sub), k);
-        unpack8(*reinterpret_cast<const u32x4 *>(vc + (size_t)t * HD + 8 * sub), v);
+    // UN positions per lane are requested together, so that a chunk costs one or two memory
+    // round trips instead of one per position
+    constexpr int UN = G == 8 ? 2 : 4;
+    for (int tb = t0 + wave * PPW + slot; tb < t1; tb += UN * 4 * PPW) {
+        u32x4 kraw[UN], vraw[UN];
 #pragma unroll
-        for (int h = 0; h < G; ++h) {
-            float s = 0.f;
+        for (int i = 0; i < UN; ++i) {
+            const int t = tb + i * 4 * PPW;
+            const int tc = t < t1 ? t : t0;   // in range; the result of a clamped slot is discarded
+            kraw[i] = *reinterpret_cast<const u32x4 *>(kc + (size_t)tc * HD + 8 * sub);
+            vraw[i] = *reinterpret_cast<const u32x4 *>(vc + (size_t)tc * HD + 8 * sub);
+        }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) s = fmaf(q[h][j], k[j], s);
+        for (int i = 0; i < UN; ++i) {
+            if (tb + i * 4 * PPW >= t1) break;   // uniform within a lane group
+            float k[8], v[8];
+            unpack8(kraw[i], k);
+            unpack8(vraw[i], v);
 #pragma unroll
-            for (int off = 1; off < LPP; off <<= 1) s += __shfl_xor(s, off);
-            const float mn = fmaxf(m[h], s);
-            const float corr = exp2f(m[h] - mn);
-            const float pr = exp2f(s - mn);
-            m[h] = mn;
-            l[h] = l[h] * corr + pr;
+            for (int h = 0; h < G; ++h) {
+                float s = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[h][j] = fmaf(pr, v[j], acc[h][j] * corr);
+                for (int j = 0; j < 8; ++j) s = fmaf(q[h][j], k[j], s);
+#pragma unroll
+                for (int off = 1; off < LPP; off <<= 1) s += __shfl_xor(s, off);
+                const float mn = fmaxf(m[h], s);
+                const float corr = exp2f(m[h] - mn);
+                const float pr = exp2f(s - mn);
+                m[h] = mn;
+                l[h] = l[h] * corr + pr;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[h][j] = fmaf(pr, v[j], acc[h][j] * corr);
+            }
         }
     }
 
@@ -193,19 +208,32 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const AttnParams p) {
     }
 }
 
-// out[head] = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M); grid = n_heads, block = HD threads
+// out[head] = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M); grid = n_heads, block = HD threads.
+// The chunk weights are computed once by the first wave (lane s owns chunk s, nsplit <= 32).
 __global__ void attn_combine_kernel(const float *part_ml, const float *part_acc, uint16_t *out, int nsplit, int hd) {
+    __shared__ float wgt[kMaxAttnSplit];
+    __shared__ float inv_l;
     const int head = blockIdx.x, e = threadIdx.x;
-    float mn = kNegBig;
-    for (int s = 0; s < nsplit; ++s) mn = fmaxf(mn, part_ml[2 * ((size_t)head * nsplit + s)]);
-    float ls = 0.f, as = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-        const size_t i = (size_t)head * nsplit + s;
-        const float c = exp2f(part_ml[2 * i] - mn);
-        ls += part_ml[2 * i + 1] * c;
-        as += part_acc[i * hd + e] * c;
+    if (e < 64) {
+        const bool live = e < nsplit;
+        const float m = live ? part_ml[2 * ((size_t)head * nsplit + e)] : kNegBig;
+        const float l = live ? part_ml[2 * ((size_t)head * nsplit + e) + 1] : 0.f;
+        float mn = m;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) mn = fmaxf(mn, __shfl_xor(mn, off));
+        const float c = exp2f(m - mn);
+        float ls = l * c;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) ls += __shfl_xor(ls, off);
+        if (live) wgt[e] = c;
+        if (e == 0) inv_l = 1.0f / ls;
     }
-    out[(size_t)head * hd + e] = float_to_bf16_bits(as / ls);
+    __syncthreads();
+    const float *src = part_acc + (size_t)head * nsplit * hd + e;
+    float as = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < nsplit; ++s) as = fmaf(src[(size_t)s * hd], wgt[s], as);
+    out[(size_t)head * hd + e] = float_to_bf16_bits(as * inv_l);
 }
 
 template <int HD>
@@ -223,7 +251,7 @@ hipError_t launch_g(int g, const AttnParams &p, dim3 grid, hipStream_t stream) {
 }  // namespace
 
 int attention_nsplit(int seq_len) {
-    int n = (seq_len + 127) / 128;   // >= 128 positions per chunk
+    int n = (seq_len + 63) / 64;   // >= 64 positions per chunk
     if (n > kMaxAttnSplit) n = kMaxAttnSplit;
     return n < 1 ? 1 : n;
 }

@@ -93,6 +93,17 @@ __device__ __forceinline__ bool slot_full(u32x4 v) {
     return v[0] != kEmpty && v[1] != kEmpty && v[2] != kEmpty && v[3] != kEmpty;
 }
 
+// a0 += sum of squares of the low bf16 halves of v, a1 += of the high halves
+__device__ __forceinline__ void sumsq8(const u32x4 v, float &a0, float &a1) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = __builtin_bit_cast(float, v[j] << 16);
+        const float hi = __builtin_bit_cast(float, v[j] & 0xFFFF0000u);
+        a0 = fmaf(lo, lo, a0);
+        a1 = fmaf(hi, hi, a1);
+    }
+}
+
 __device__ __forceinline__ float silu_tanh(float g) { return g * 0.5f * (tanhf(g * 0.5f) + 1.0f); }
 
 template <int LW>
@@ -160,7 +171,39 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 #pragma unroll
     for (int t = 0; t < LC; ++t) yacc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+    // RMSNorm prologue.  Loads of one wave return in order, so x is requested before the weights:
+    // for M == 1 the lane's chunks of x are held in registers and reduced once the weight loads
+    // are in flight; for M = 2..4 the row sums are finished up front.
     float rstd = 0.f;
+    u32x4 xpre[RMS ? 8 : 1];
+    if constexpr (RMS) {
+        if (p.M == 1) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = lane + 64 * i;
+                xpre[i] = c < (p.K >> 3) ? reinterpret_cast<const u32x4 *>(p.x)[c] : u32x4{0u, 0u, 0u, 0u};
+            }
+        } else {
+            float mine = 0.f;
+            for (int r = 0; r < p.M; ++r) {   // every lane walks row r, the lanes that feed row r keep its sum
+                const u32x4 *row = reinterpret_cast<const u32x4 *>(p.x + (size_t)r * p.K);
+                float a0 = 0.f, a1 = 0.f;
+                for (int c0 = lane; c0 < (p.K >> 3); c0 += 256) {
+                    u32x4 v[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        v[i] = c0 + 64 * i < (p.K >> 3) ? row[c0 + 64 * i] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) sumsq8(v[i], a0, a1);
+                }
+                float a = a0 + a1;
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off);
+                if (am == r) mine = a;
+            }
+            rstd = 1.0f / sqrtf(mine / (float)p.K + p.eps);
+        }
+    }
     // K-slice `kslice` owns units [ulo, uhi) of the K / (32 * KSTEPS) units: slice_units each, the
     // first slice_extra slices one more; its waves take them round-robin.
     const int ulo = kslice * p.slice_units + (kslice < p.slice_extra ? kslice : p.slice_extra);
@@ -173,6 +216,12 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 
         wvec w[KSTEPS][8];
         u32x4 av[KSTEPS];
+        u32x4 nw[RMS ? KSTEPS : 1];   // norm weights: requested before the packed weights, like x
+        if constexpr (RMS) {
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s)
+                nw[s] = *reinterpret_cast<const u32x4 *>(p.norm_w + (size_t)(kstep0 + s) * 32 + 8 * lg);
+        }
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
             const size_t row0 = (size_t)(kstep0 + s) * 32 + 8 * lg;
@@ -187,31 +236,16 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         for (int c = 0; c < LW; ++c) sv[c] = *reinterpret_cast<const u32x4 *>(sc + (size_t)g * p.N + 8 * c);
 
         if constexpr (RMS) {
-            u32x4 nw[KSTEPS];
+            if (u == 0 && p.M == 1) {
+                // sum of squares from the preloaded chunks (plus a tail for K > 4096), then across the wave
+                float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-            for (int s = 0; s < KSTEPS; ++s)
-                nw[s] = *reinterpret_cast<const u32x4 *>(p.norm_w + (size_t)(kstep0 + s) * 32 + 8 * lg);
-            if (u == 0) {
-                float mine = 0.f;
-                for (int r = 0; r < p.M; ++r) {   // M <= 4: every lane walks row r, the lanes of row r keep it
-                    const u32x4 *row = reinterpret_cast<const u32x4 *>(p.x + (size_t)r * p.K);
-                    float a0 = 0.f, a1 = 0.f;
-                    for (int c = lane; c < (p.K >> 3); c += 64) {
-                        const u32x4 v = row[c];
+                for (int i = 0; i < 8; ++i) sumsq8(xpre[i], a0, a1);
+                for (int c = lane + 512; c < (p.K >> 3); c += 64) sumsq8(reinterpret_cast<const u32x4 *>(p.x)[c], a0, a1);
+                float a = a0 + a1;
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const float lo = __builtin_bit_cast(float, v[j] << 16);
-                            const float hi = __builtin_bit_cast(float, v[j] & 0xFFFF0000u);
-                            a0 = fmaf(lo, lo, a0);
-                            a1 = fmaf(hi, hi, a1);
-                        }
-                    }
-                    float a = a0 + a1;
-#pragma unroll
-                    for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off);
-                    if (am == r) mine = a;
-                }
-                rstd = 1.0f / sqrtf(mine / (float)p.K + p.eps);
+                for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off);
+                rstd = 1.0f / sqrtf(a / (float)p.K + p.eps);
             }
 #pragma unroll
             for (int s = 0; s < KSTEPS; ++s) {
