@@ -11,14 +11,15 @@
 //
 // LDS layout (checked with a ds_read_b128 / ds_write_b128 timing probe and SQ_LDS_BANK_CONFLICT;
 // the LDS behaves as 64 banks of 4 B: a read pass is 16 lanes x 16 B, a write pass 8 lanes x 16 B).
-// x tile: rows of 64 bf16 padded to 144 B: operand reads of 16 consecutive rows and the copy's
-// row-contiguous stores are conflict-free.  Weight tile [n][k]: rows padded to 160 B and the
-// 16-byte chunk index XORed with (n / 8) % 8.  Reads (lanes = 16 consecutive n, same chunk): 160 n
-// covers the even 16-byte slots of a 256-byte window for n = 0..7 and the XOR flips bit 0 for
-// n = 8..15, which takes the odd slots.  Dequant stores (lanes = same column j of consecutive
-// packed words, n = 8 * word + j): 1280 * word is 0 mod 128, so the slot is chunk ^ word % 8,
-// distinct over 8 lanes; and the 8 columns of a lane are one base address plus j * 160 B.
-// With 144-byte rows the same XOR cost 512 conflict cycles per K step on the weight operand reads.
+// x tile: unpadded rows of 64 bf16 (128 B) filled by global_load_lds_dwordx4, 16-byte chunk c of
+// row r at slot c ^ r % 8 (the lanes of a copy choose their global chunk accordingly), so the
+// operand reads of 16 consecutive rows touch 16 distinct slots of a 256-byte window.
+// Weight tile [n][k]: rows padded to 160 B and the chunk index XORed with (n / 8) % 8.  Reads
+// (lanes = 16 consecutive n, same chunk): 160 n covers the even 16-byte slots of a 256-byte
+// window for n = 0..7 and the XOR flips bit 0 for n = 8..15, which takes the odd slots.  Dequant
+// stores (lanes = same column j of consecutive packed words, n = 8 * word + j): 1280 * word is
+// 0 mod 128, so the slot is chunk ^ word % 8, distinct over 8 lanes; and the 8 columns of a lane
+// are one base address plus j * 160 B.
 //
 // blockIdx -> tile: each XCD (blockIdx % 8) takes a contiguous range of tiles with N
 // fastest, so one XCD's L2 keeps an x panel resident while the weight panels stream by.
