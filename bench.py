@@ -206,6 +206,19 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     cold_s, cold_wall = timed_graph(list(range(steps)))
     hot_s, _ = timed_graph([0] * steps)
 
+    # one event pair per launch, outside a graph (the reference's harness style,
+    # programming_examples/matrix_vector_multiplication/int4_awq/test_packed.cpp:114-150): each figure
+    # carries the full eager launch overhead, so these are a distribution, not the throughput claim
+    per_launch = []
+    with torch.cuda.stream(stream):
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i, (a, b) in enumerate(evs):
+            a.record(stream)
+            launch(i, stream.cuda_stream)
+            b.record(stream)
+        stream.synchronize()
+        per_launch = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
+
     res = {
         "name": name,
         "cold_us": cold_s / steps * 1e6,
@@ -214,6 +227,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         "bytes": algorithmic_bytes(name),
         "flops": algorithmic_flops(name),
         "ncopies": ncopies,
+        "per_launch_events_us": {"min": per_launch[0], "median": per_launch[len(per_launch) // 2],
+                                 "avg": sum(per_launch) / len(per_launch), "max": per_launch[-1]},
     }
 
     if with_cpu_baseline and name not in ("block", "layer"):
@@ -267,6 +282,31 @@ def cpu_baseline(name, torch, w, x, outs, launch, stream):
         fn = lambda: baseline.gemm_numpy(xb, *args)
         sample = f"full config {c['cfg']}, vectorised NumPy dequant + float32 BLAS product, median of 3"
 
+    extra = {}
+    if name in ("gemv", "gemm16", "prefill", "dequant"):
+        wargs = tuple(host(t) for t in w)
+        baseline.dequant_numpy(*wargs)                             # warm-up
+        t0 = time.perf_counter()
+        baseline.dequant_numpy(*wargs)
+        extra["dequant_seconds"] = time.perf_counter() - t0      # the unpack + dequant part alone
+    if name == "gemv":
+        # the reference's own cpu_reference is a scalar double loop (matvec_int4_packed.py:281-286);
+        # its C restatement runs at full size on one core
+        import ctypes
+
+        import oracle
+        from oracle import awq as oawq
+        a_q, a_s, a_z = oawq.repack_hf_awq_linear(*wargs, 128)
+        a_q, a_s, a_z = (np.ascontiguousarray(t) for t in (a_q, a_s, a_z))
+        xb0 = np.ascontiguousarray(host(x)[0])
+        out = np.zeros(c["N"], np.uint16)
+        clib = oracle.load_c_oracle()
+        ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+        t0 = time.perf_counter()
+        clib.oracle_matvec_loop(ptr(a_q), ptr(a_s), ptr(a_z), ptr(xb0), c["N"], c["K"], 128, ptr(out))
+        extra["scalar_loop_c_seconds"] = time.perf_counter() - t0
+        extra["scalar_loop_c_max_abs_diff_vs_gpu"] = float(np.max(np.abs(bf16_bits_to_f32(out) - got.reshape(-1))))
+
     ref = fn()   # warm-up, and the reference output
     times = []
     for _ in range(3):
@@ -284,7 +324,7 @@ def cpu_baseline(name, torch, w, x, outs, launch, stream):
         value = algorithmic_bytes(name) / t / 1e9
         unit = "GB/s"
     return {"value": value, "unit": unit, "cores": int(blas_threads), "kind": "port", "sample": sample,
-            "seconds": t, "host_cpus": len(os.sched_getaffinity(0)), "max_abs_diff_vs_gpu": err}
+            "seconds": t, "host_cpus": len(os.sched_getaffinity(0)), "max_abs_diff_vs_gpu": err, **extra}
 
 
 def main():
@@ -346,6 +386,7 @@ def main():
         "config": {"workload": CONFIGS[name]["desc"], "group": 128,
                    "weight_copies_rotated": main_res["ncopies"], "timing": "HIP graph of K launches, events on the launch stream"},
         "roofline": roof,
+        "per_launch_events_us": main_res["per_launch_events_us"],
         "hot_cache": {"us_per_step": main_res["hot_us"],
                       "value": (main_res["flops"] / 1e12 if name == "prefill" else main_res["bytes"] / 1e9) / (main_res["hot_us"] * 1e-6),
                       "note": "same buffers every step (Infinity Cache resident for the decode shapes)"},
