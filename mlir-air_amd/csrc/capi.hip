@@ -222,7 +222,9 @@ int w4a16_rms_gemv_swiglu_bf16(const uint16_t *x, const uint16_t *norm_weight, f
 size_t w4a16_block_workspace_bytes(int E, int H) {
     if (E <= 0 || H <= 0) return 0;
     const size_t a = stream_partial_bytes(1, H, 2), b = stream_partial_bytes(1, E, 1);
-    return kHeaderBytes + (a > b ? a : b) + round256((size_t)H * sizeof(uint16_t)) + round256((size_t)E * sizeof(uint16_t));
+    // [header][partial slots][h bf16 H][res1 bf16 E][sum of squares of res1, one float per column tile, <= 64]
+    return kHeaderBytes + (a > b ? a : b) + round256((size_t)H * sizeof(uint16_t)) +
+           round256((size_t)E * sizeof(uint16_t)) + 256;
 }
 
 int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
@@ -248,14 +250,19 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, 
     if (!workspace || workspace_bytes < w4a16_block_workspace_bytes(E, H)) return W4A16_ERR_WORKSPACE;
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    char *tail = static_cast<char *>(workspace) + w4a16_block_workspace_bytes(E, H);
+    char *tail = static_cast<char *>(workspace) + w4a16_block_workspace_bytes(E, H) - 256;
+    float *res1_sumsq = reinterpret_cast<float *>(tail);
     uint16_t *res1 = res1_out ? res1_out : reinterpret_cast<uint16_t *>(tail - round256((size_t)E * sizeof(uint16_t)));
     uint16_t *h = h_out ? h_out
                         : reinterpret_cast<uint16_t *>(tail - round256((size_t)E * sizeof(uint16_t)) -
                                                        round256((size_t)H * sizeof(uint16_t)));
-    // stage 1: res1 = bf16(attn_out . Wo + x_residual)
+    // stage 1: res1 = bf16(attn_out . Wo + x_residual); its reducers also leave sum(res1^2) per column
+    // tile, so that stage 2 does not have to read res1 again for the norm
+    const int res1_tiles = plan_stream(1, E, E).ntiles;
+    const bool chain_norm = res1_tiles <= 64;
     StreamExtras add;
     add.residual = x_residual;
+    if (chain_norm) add.sumsq_out = res1_sumsq;
     hipError_t e = launch_stream(attn_out, o_qweight, o_qzeros, o_scales, nullptr, nullptr, nullptr, res1, 1, E, E,
                                  workspace, st, add);
     if (e != hipSuccess) return hip_fail(e);
@@ -263,6 +270,11 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, 
     StreamExtras rms;
     rms.norm_w = ffn_norm_weight;
     rms.eps = eps;
+    if (chain_norm) {
+        rms.sumsq_in = res1_sumsq;
+        rms.sumsq_n = res1_tiles;
+    }
+    add.sumsq_out = nullptr;
     e = launch_stream(res1, gate_qweight, gate_qzeros, gate_scales, up_qweight, up_qzeros, up_scales, h, 1, E, H,
                       workspace, st, rms);
     if (e != hipSuccess) return hip_fail(e);

@@ -37,6 +37,12 @@ struct StreamExtras {
     int round_before_add = 0;             // 1: y = bf16(bf16(x.W) + R) instead of bf16(x.W + R)
     const uint16_t *norm_w = nullptr;     // [K] bf16: x is replaced by bf16((x * rstd) * norm_w), M <= 4
     float eps = 1e-5f;
+    // M == 1 only.  A launch with `sumsq_out` leaves the sum of squares of its (rounded) outputs there,
+    // one float per 256-column tile; a following RMS launch on that vector passes it as `sumsq_in`
+    // (`sumsq_n` <= 64 pieces) and skips reading x for the norm.
+    const float *sumsq_in = nullptr;
+    int sumsq_n = 0;
+    float *sumsq_out = nullptr;
 };
 
 // y[M, N] = bf16(x[M, K] . W), M <= 16.  With `up_*` given (SwiGLU epilogue, M == 1) the

@@ -63,6 +63,9 @@ struct StreamParams {
     int round_before_add;       // 1: y = bf16(bf16(acc) + R); 0: y = bf16(acc + R)
     const uint16_t *norm_w;     // [K] bf16 RMSNorm weight (RMS kernels only)
     float eps;
+    const float *sumsq_in;      // RMS, M == 1: partial sums of x^2 written by the kernel that produced x, or null
+    int sumsq_n;
+    float *sumsq_out;           // M == 1: sum of squares of this launch's bf16 outputs, one float per column tile, or null
     int spin_limit;
     int skip_publish;   // fault injection for tests: producers keep their partials to themselves
 };
@@ -171,18 +174,16 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 #pragma unroll
     for (int t = 0; t < LC; ++t) yacc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // RMSNorm prologue.  Loads of one wave return in order, so x is requested before the weights:
-    // for M == 1 the lane's chunks of x are held in registers and reduced once the weight loads
-    // are in flight; for M = 2..4 the row sums are finished up front.
+    // RMSNorm prologue: rstd = 1 / sqrt(mean(x^2) + eps) of the lane's row of x, computed by every
+    // wave for itself.  When the kernel that produced x left its sum of squares behind (M == 1,
+    // at most 64 pieces) that is one 4-byte load per lane, requested ahead of the weights (loads
+    // of one wave return in order) and reduced while they are in flight; otherwise the wave walks
+    // x (K bf16 values per row, L2-resident) before it requests its weights.
     float rstd = 0.f;
-    u32x4 xpre[RMS ? 8 : 1];
+    float piece = 0.f;
     if constexpr (RMS) {
-        if (p.M == 1) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int c = lane + 64 * i;
-                xpre[i] = c < (p.K >> 3) ? reinterpret_cast<const u32x4 *>(p.x)[c] : u32x4{0u, 0u, 0u, 0u};
-            }
+        if (p.M == 1 && p.sumsq_in) {
+            piece = lane < p.sumsq_n ? p.sumsq_in[lane] : 0.f;
         } else {
             float mine = 0.f;
             for (int r = 0; r < p.M; ++r) {   // every lane walks row r, the lanes that feed row r keep its sum
@@ -204,6 +205,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             rstd = 1.0f / sqrtf(mine / (float)p.K + p.eps);
         }
     }
+
     // K-slice `kslice` owns units [ulo, uhi) of the K / (32 * KSTEPS) units: slice_units each, the
     // first slice_extra slices one more; its waves take them round-robin.
     const int ulo = kslice * p.slice_units + (kslice < p.slice_extra ? kslice : p.slice_extra);
@@ -236,13 +238,8 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         for (int c = 0; c < LW; ++c) sv[c] = *reinterpret_cast<const u32x4 *>(sc + (size_t)g * p.N + 8 * c);
 
         if constexpr (RMS) {
-            if (u == 0 && p.M == 1) {
-                // sum of squares from the preloaded chunks (plus a tail for K > 4096), then across the wave
-                float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) sumsq8(xpre[i], a0, a1);
-                for (int c = lane + 512; c < (p.K >> 3); c += 64) sumsq8(reinterpret_cast<const u32x4 *>(p.x)[c], a0, a1);
-                float a = a0 + a1;
+            if (u == 0 && p.M == 1 && p.sumsq_in) {
+                float a = piece;
 #pragma unroll
                 for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off);
                 rstd = 1.0f / sqrtf(a / (float)p.K + p.eps);
@@ -427,11 +424,22 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             out[2] += __builtin_bit_cast(float, r.y << 16);
             out[3] += __builtin_bit_cast(float, r.y & 0xFFFF0000u);
         }
-        if (col0 + col < p.N) {
-            uint2 o;
-            o.x = pack_bf16x2(out[0], out[1]);
-            o.y = pack_bf16x2(out[2], out[3]);
-            *reinterpret_cast<uint2 *>(p.y + (size_t)m * p.N + col0 + col) = o;
+        uint2 o;
+        o.x = pack_bf16x2(out[0], out[1]);
+        o.y = pack_bf16x2(out[2], out[3]);
+        const bool in_range = col0 + col < p.N;
+        if (in_range) *reinterpret_cast<uint2 *>(p.y + (size_t)m * p.N + col0 + col) = o;
+        if (p.sumsq_out && p.M == 1) {
+            // M == 1: the tile's quads are exactly the lanes of wave 0 (one trip through this loop)
+            float sq = 0.f;
+            if (in_range) {
+                const float r0 = __builtin_bit_cast(float, o.x << 16), r1 = __builtin_bit_cast(float, o.x & 0xFFFF0000u);
+                const float r2 = __builtin_bit_cast(float, o.y << 16), r3 = __builtin_bit_cast(float, o.y & 0xFFFF0000u);
+                sq = fmaf(r0, r0, fmaf(r1, r1, fmaf(r2, r2, r3 * r3)));
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+            if (threadIdx.x == 0) p.sumsq_out[tile] = sq;
         }
     }
 }
@@ -547,6 +555,9 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.round_before_add = extras.round_before_add;
     p.norm_w = extras.norm_w;
     p.eps = extras.eps;
+    p.sumsq_in = extras.sumsq_in;
+    p.sumsq_n = extras.sumsq_n;
+    p.sumsq_out = extras.sumsq_out;
     p.skip_publish = g_stream_tune.skip_publish;
     p.spin_limit = g_stream_tune.spin_limit > 0 ? g_stream_tune.spin_limit : (1 << 18);
     const int grid = ((pl.ntiles + 7) / 8) * 8 * p.nmat * pl.ksplit;
