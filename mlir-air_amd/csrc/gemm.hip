@@ -260,13 +260,10 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
 
 hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
                                const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    // 144 KiB of dynamic LDS needs the attribute; it is per device, so it is set on every launch
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+    if (e != hipSuccess) return e;
     GemmParams p;
     p.x = x;
     p.qw = reinterpret_cast<const uint32_t *>(qweight);

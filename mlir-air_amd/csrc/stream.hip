@@ -491,12 +491,10 @@ StreamPlan plan_stream(int M, int K, int N) {
 template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false>
 static hipError_t launch_one(const StreamParams &p, int grid, hipStream_t stream) {
     const size_t lds = (size_t)WAVES * p.M * 8 * LW * 17 * sizeof(float);   // <= 136 KB at M = 16, LW = 2, 8 waves
-    static bool lds_opt_in = false;   // more than 64 KB of dynamic LDS needs the attribute once per kernel
-    if (!lds_opt_in && lds > 64 * 1024) {
+    if (lds > 64 * 1024) {   // more than 64 KB of dynamic LDS needs the attribute (per device, so set it every time)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
-        lds_opt_in = true;
     }
     hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>), dim3(grid), dim3(WAVES * 64), lds, stream, p);
     return hipGetLastError();

@@ -111,6 +111,12 @@ def test_gemv_uneven_k_slices(ops, ksplit):
         ops.tune("gemv_ksplit", 0)
 
 
+def test_gemv_grid_larger_than_the_chip(ops):
+    """2052 workgroups (513 column tiles x 4 K-slices, ragged last tile) on 256 CUs: reducers are
+    dispatched after their producers, so a grid of several rounds still completes."""
+    _gemm_case(ops, 1, 4096, 131072 + 96, seed=77)
+
+
 def test_gemv_repeat_calls_are_deterministic_and_workspace_is_reusable(ops):
     print("gemv repeat", flush=True)
     K, N = 4096, 11008
