@@ -92,8 +92,9 @@ int w4a16_gemv_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qz
 
 /*
  * GEMM, any M >= 1: y[M, N] = bf16(x[M, K] . W).  M <= 16 streams the weights once
- * through a split-K MFMA kernel; larger M uses the tiled prefill kernel that dequantises
- * weight tiles to bf16 in LDS.  Replaces matmul_int4_bf16_packed_f32 + f32_to_bf16_mn
+ * through a split-K MFMA kernel; M <= 96 does the same in launches of 16 rows (the weights
+ * stay cache-resident between them); larger M uses the tiled prefill kernel that dequantises
+ * weight tiles to bf16 in LDS (and therefore multiplies bf16-rounded weights).  Replaces matmul_int4_bf16_packed_f32 + f32_to_bf16_mn
  * (mv_int4_bf16.cc:430-448) and matches matmul_int4_packed.cpu_reference
  * (programming_examples/matrix_multiplication/int4_awq/matmul_int4_packed.py:89-105).
  */
@@ -214,7 +215,8 @@ int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_ro
 
 /*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
- * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic) and
+ * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic),
+ * "gemm_stream_max_m" (largest M given to the streaming kernel, 0 = default 96, otherwise >= 16) and
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the
  * timeout test: split-K producers do not publish).  Process-wide.
  */

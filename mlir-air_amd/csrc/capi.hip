@@ -108,10 +108,19 @@ int w4a16_gemm_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qz
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e;
-    if (M <= 16)
-        e = launch_stream(x, qweight, qzeros, scales, nullptr, nullptr, nullptr, y, M, K, N, workspace, st);
-    else
+    const int stream_max_m = g_stream_tune.stream_max_m >= 16 ? g_stream_tune.stream_max_m : kStreamMaxM;
+    if (M <= stream_max_m) {
+        // the streaming kernel takes up to 16 rows per launch; a few more launches over the same
+        // (cache-resident) weights still beat one 256-row MFMA tile that is mostly padding
+        e = hipSuccess;
+        for (int m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
+            const int rows = M - m0 < 16 ? M - m0 : 16;
+            e = launch_stream(x + (size_t)m0 * K, qweight, qzeros, scales, nullptr, nullptr, nullptr,
+                              y + (size_t)m0 * N, rows, K, N, workspace, st);
+        }
+    } else {
         e = launch_gemm_prefill(x, qweight, qzeros, scales, y, M, K, N, st);
+    }
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
@@ -323,6 +332,8 @@ int w4a16_tune(const char *key, int value) {
         g_stream_tune.skip_publish = value ? 1 : 0;
     } else if (!strcmp(key, "gemv_spin_limit")) {
         g_stream_tune.spin_limit = value;
+    } else if (!strcmp(key, "gemm_stream_max_m")) {
+        g_stream_tune.stream_max_m = value;
     } else if (!strcmp(key, "gemv_ksplit")) {
         if (value > kMaxKSplit) return W4A16_ERR_TUNE;
         g_stream_tune.ksplit = value;

@@ -11,6 +11,7 @@ namespace w4a16 {
 // timeouts][fp32 split-K partial slots].  Between calls every slot holds 0xFFFFFFFF.
 constexpr size_t kHeaderBytes = 256;
 constexpr int kMaxKSplit = 32;
+constexpr int kStreamMaxM = 96;   // up to here w4a16_gemm_bf16 runs the streaming kernel in 16-row launches
 
 struct StreamTune {
     int lw = 0;       // packed words per lane per row: 1, 2 or 4 (tile = 128 * lw columns)
@@ -18,6 +19,7 @@ struct StreamTune {
     int waves = 0;    // waves per workgroup: 4 or 8
     int units = 0;    // units each wave processes back to back
     int ksplit = 0;   // workgroups along K per tile (overrides units)
+    int stream_max_m = 0;   // largest M that w4a16_gemm_bf16 gives to the streaming kernel (0 = kStreamMaxM; at least 16)
     int skip_publish = 0; // tests only: producers do not publish, so reducers run into their poll bound
     int spin_limit = 0;   // reducer poll bound (0 = default); tiny values force the timeout path in tests
 };

@@ -71,7 +71,7 @@ def _gemm_case(ops, M, K, N, seed, ulps=1.0, atol=2e-3):
     torch.cuda.synchronize()
     got = bits(y)
     xf = bf16_bits_to_f32(x).astype(np.float64)
-    want = xf @ dense_f64(qw, qz, s, rounded=(M > 16))
+    want = xf @ dense_f64(qw, qz, s, rounded=(M > 96))   # M <= 96 streams exact weights, larger M multiplies bf16-rounded ones
     assert_bf16_close(got, want, ulps=ulps, atol=atol, what=f"gemm M={M} K={K} N={N}")
     assert oref.check_outputs(bf16_bits_to_f32(got), bf16_bits_to_f32(f32_to_bf16_bits(want.astype(np.float32))),
                               rtol=0.1, atol=0.05, min_correlation=0.999 if want.size > 8 else None)
@@ -128,7 +128,7 @@ def test_gemv_repeat_calls_are_deterministic_and_workspace_is_reusable(ops):
         assert np.array_equal(bits(ops.w4a16_gemv(dx, dq, dz, ds)), first)
 
 
-@pytest.mark.parametrize("M", [2, 3, 4, 5, 8, 13, 16])
+@pytest.mark.parametrize("M", [2, 3, 4, 5, 8, 13, 16, 17, 40, 96])
 def test_small_m_gemm(ops, M):
     _gemm_case(ops, M, 1024, 1056, seed=M)
 
@@ -137,9 +137,26 @@ def test_gemm_config2(ops):
     _gemm_case(ops, 16, 4096, 14336, seed=2)
 
 
-@pytest.mark.parametrize("M,K,N", [(17, 128, 32), (64, 256, 128), (130, 512, 544), (200, 1024, 1056), (256, 4096, 512)])
+@pytest.mark.parametrize("M,K,N", [(97, 128, 32), (100, 256, 128), (130, 512, 544), (200, 1024, 1056), (256, 4096, 512)])
 def test_prefill_gemm_small(ops, M, K, N):
     _gemm_case(ops, M, K, N, seed=M + K + N)
+
+
+@pytest.mark.parametrize("M,K,N", [(17, 128, 32), (64, 256, 128)])
+def test_prefill_kernel_at_small_m(ops, M, K, N):
+    """The tiled kernel itself on tiles that are mostly padding (the boundary to the streaming
+    kernel lowered to 16)."""
+    ops.tune("gemm_stream_max_m", 16)
+    try:
+        print(f"prefill kernel M={M} K={K} N={N}", flush=True)
+        qw, qz, s = make_awq(K, N, seed=M + K)
+        x = make_x((M, K), seed=M)
+        y = ops.w4a16_gemm(dev(x), dev(qw), dev(qz), dev(s))
+        torch.cuda.synchronize()
+        want = bf16_bits_to_f32(x).astype(np.float64) @ dense_f64(qw, qz, s, rounded=True)
+        assert_bf16_close(bits(y), want, ulps=1.0, atol=2e-3, what="prefill kernel at small M")
+    finally:
+        ops.tune("gemm_stream_max_m", 0)
 
 
 def test_prefill_gemm_config3(ops):
