@@ -32,7 +32,7 @@ CONFIGS = {
     "gemm16": dict(M=16, K=4096, N=14336, cfg=2, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128"),
     "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128"),
     "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128"),
-    # not a BASELINE config: the O projection + RMSNorm + FFN decode block with residuals (3 launches)
+    # beyond the five headline configs: the O projection + RMSNorm + FFN decode block with residuals (3 launches)
     "block": dict(M=1, K=4096, N=14336, cfg=None, desc="decode block O-proj + RMSNorm + SwiGLU FFN W4A16 E=4096 H=14336 g128"),
     # one whole decode layer: RMSNorm + fused QKV GEMV, RoPE + KV append + GQA attention over 2048 cached
     # positions (32 heads, 8 KV heads, head_dim 128), then the block above

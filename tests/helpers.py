@@ -6,7 +6,7 @@ from oracle.bf16 import bf16_bits_to_f32, f32_to_bf16_bits
 
 
 def make_awq(K, N, gs=128, seed=0, z_range=(0, 16)):
-    """BASELINE-style synthetic AWQ tensors: q, z uniform uint4, scales = bf16(|N(0,1)|*0.02 + 1e-3)."""
+    """Synthetic AWQ tensors in the benchmark distribution: q, z uniform uint4, scales = bf16(|N(0,1)|*0.02 + 1e-3)."""
     rng = np.random.default_rng(seed)
     q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
     z = rng.integers(z_range[0], z_range[1], size=(K // gs, N), dtype=np.uint8)
