@@ -117,6 +117,25 @@ def test_gemv_grid_larger_than_the_chip(ops):
     _gemm_case(ops, 1, 4096, 131072 + 96, seed=77)
 
 
+def test_one_workspace_serves_interleaved_shapes(ops):
+    """Every launch leaves the partial slots it used empty again, so launches of different shapes
+    (different slot maps) can alternate on one workspace without re-initialising it."""
+    print("interleaved shapes on one workspace", flush=True)
+    cases = []
+    for M, K, N, seed in [(1, 4096, 11008, 1), (16, 1024, 4128, 2), (1, 14336, 4096, 3), (5, 512, 32, 4), (1, 2048, 2048, 5)]:
+        qw, qz, s = make_awq(K, N, seed=seed)
+        args = (dev(make_x((M, K), seed=seed + 10)), dev(qw), dev(qz), dev(s))
+        cases.append((args, bits(ops.w4a16_gemm(*args))))
+    g = make_awq(1024, 2048, seed=6), make_awq(1024, 2048, seed=7), make_awq(2048, 1024, seed=8)
+    gd = [tuple(map(dev, t)) for t in g]
+    xf = dev(make_x((1024,), seed=9))
+    ffn_first = bits(ops.ffn_swiglu(xf, *gd))
+    for it in range(40):
+        for args, first in cases:
+            assert np.array_equal(bits(ops.w4a16_gemm(*args)), first), it
+        assert np.array_equal(bits(ops.ffn_swiglu(xf, *gd)), ffn_first), it
+
+
 def test_gemv_repeat_calls_are_deterministic_and_workspace_is_reusable(ops):
     print("gemv repeat", flush=True)
     K, N = 4096, 11008
