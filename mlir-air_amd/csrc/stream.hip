@@ -71,6 +71,9 @@ struct StreamParams {
 };
 
 constexpr uint32_t kEmpty = 0xFFFFFFFFu;
+#ifndef POLL_SLEEP
+#define POLL_SLEEP 1   // s_sleep units of 64 cycles between issuing the two polling rounds (0..2 measure the same, 8 and 16 slower)
+#endif
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -325,12 +328,12 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 
     // The reducer's first polling round is issued before the LDS combine, so that its latency
     // (one trip to L2 per slot) is hidden behind the combine and its barriers.
-    u32x4 pre[8];
+    u32x4 va[8], vb[8];   // the two polling rounds a reducer thread keeps in flight
     const bool prefetched = reducer && (int)threadIdx.x < nquads;
     if (prefetched) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            if (j < nprod) pre[j] = slot_load(tile_partial + (size_t)threadIdx.x * 4 + j * slice_stride);
+            if (j < nprod) va[j] = slot_load(tile_partial + (size_t)threadIdx.x * 4 + j * slice_stride);
     }
 
     // ---- cross-wave combine in LDS: red[slot][m][j * 17 + ln], j = natural column in the lane's chunk ----
@@ -368,38 +371,49 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             continue;
         }
         // Reducer: fetch the producers' slots eight at a time (all loads of a round in flight
-        // together), repeat a round until its slots are all filled, then hand the slots back.
+        // together) until they are all filled, then hand the slots back.  Two rounds are kept in
+        // flight, half a round trip apart, so that a partial is noticed about one round trip after
+        // it was published instead of up to two.
         floatx4 sum0 = floatx4{0.f, 0.f, 0.f, 0.f}, sum1 = floatx4{0.f, 0.f, 0.f, 0.f};
         for (int s0 = 0; s0 < nprod; s0 += 8) {
-            u32x4 v[8];
+#define W4A16_POLL_ISSUE(dst)                                                                 \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < nprod) dst[j] = slot_load(slot0 + (s0 + j) * slice_stride)
+#define W4A16_POLL_FULL(src, ok)                                                              \
+    ok = true;                                                                                \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < nprod) ok = ok && slot_full(src[j])
+#define W4A16_POLL_TAKE(src)                                                                  \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < nprod) {                       \
+        if (NMAT == 2 && s0 + j >= p.ksplit) sum1 += __builtin_bit_cast(floatx4, src[j]);     \
+        else sum0 += __builtin_bit_cast(floatx4, src[j]);                                     \
+    }
+            if (!(prefetched && s0 == 0 && e == (int)threadIdx.x)) {   // else: va holds the early first round
+                W4A16_POLL_ISSUE(va);
+            }
             int spins = 0;
             bool ok;
-            bool use_pre = prefetched && s0 == 0 && e == (int)threadIdx.x;
-            do {
-                ok = true;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    if (s0 + j < nprod) {
-                        v[j] = use_pre ? pre[j] : slot_load(slot0 + (s0 + j) * slice_stride);
-                        ok = ok && slot_full(v[j]);
-                    }
-                }
-                use_pre = false;
-                if (!ok && ++spins > p.spin_limit) {
-                    __hip_atomic_store(p.header, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (;;) {
+                W4A16_POLL_ISSUE(vb);
+                W4A16_POLL_FULL(va, ok);
+                if (ok || ++spins > p.spin_limit) {
+                    W4A16_POLL_TAKE(va);
                     break;
                 }
-            } while (!ok);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                if (s0 + j < nprod) {
-                    slot_store(slot0 + (s0 + j) * slice_stride, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
-                    if (NMAT == 2 && s0 + j >= p.ksplit)
-                        sum1 += __builtin_bit_cast(floatx4, v[j]);
-                    else
-                        sum0 += __builtin_bit_cast(floatx4, v[j]);
+                __builtin_amdgcn_s_sleep(POLL_SLEEP);
+                W4A16_POLL_ISSUE(va);
+                W4A16_POLL_FULL(vb, ok);
+                if (ok) {
+                    W4A16_POLL_TAKE(vb);
+                    break;
                 }
+                __builtin_amdgcn_s_sleep(POLL_SLEEP);
             }
+            if (!ok) __hip_atomic_store(p.header, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#undef W4A16_POLL_ISSUE
+#undef W4A16_POLL_FULL
+#undef W4A16_POLL_TAKE
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (s0 + j < nprod) slot_store(slot0 + (s0 + j) * slice_stride, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
         }
         floatx4 out;
         if (NMAT == 2) {
