@@ -239,6 +239,11 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         u32x4 sv[LW];
 #pragma unroll
         for (int c = 0; c < LW; ++c) sv[c] = *reinterpret_cast<const u32x4 *>(sc + (size_t)g * p.N + 8 * c);
+        // Keep every load of the unit above this point: left alone, the scheduler sinks half of
+        // them below the first MFMAs to save registers, and a wave then waits for memory twice
+        // (GEMV 10.55 -> 10.25 us).  It costs ~27 registers, i.e. the third wave per SIMD, which the
+        // plain two-matrix kernel needs more (its grid runs in two rounds), so that one is left alone.
+        if constexpr (NMAT == 1 || RMS) __builtin_amdgcn_sched_barrier(0);
 
         if constexpr (RMS) {
             if (u == 0 && p.M == 1 && p.sumsq_in) {
