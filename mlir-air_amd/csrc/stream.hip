@@ -137,7 +137,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     extern __shared__ float red[];
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses built from it stay on the SALU
     const int lg = lane >> 4;
     const int ln = lane & 15;
 
@@ -155,14 +155,21 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     const int nchunks = p.nb / LW;
     const int chunk = tile * 16 + ln;
     const int chunk_c = chunk < nchunks ? chunk : nchunks - 1;   // ragged tile: load in range, never written
-    const uint32_t *__restrict__ qw = p.qw[mat] + (size_t)chunk_c * LW;
-    const uint32_t *__restrict__ qz = p.qz[mat] + (size_t)chunk_c * LW;
-    const uint16_t *__restrict__ sc = p.sc[mat] + (size_t)chunk_c * LC;
+    // Every load address is a scalar part (matrix base + K-step row offset, SALU) plus one 32-bit
+    // per-lane byte offset, so that issuing a unit's 39 loads costs no vector address arithmetic.
+    const char *qw_s = reinterpret_cast<const char *>(p.qw[mat]);
+    const char *qz_s = reinterpret_cast<const char *>(p.qz[mat]);
+    const char *sc_s = reinterpret_cast<const char *>(p.sc[mat]);
+    const uint32_t qw_lane = (uint32_t)(((size_t)chunk_c * LW + (size_t)(8 * lg) * p.nb) * sizeof(uint32_t));
+    const uint32_t qz_lane = (uint32_t)((size_t)chunk_c * LW * sizeof(uint32_t));
+    const uint32_t sc_lane = (uint32_t)((size_t)chunk_c * LC * sizeof(uint16_t));
+    const size_t row_bytes = (size_t)p.nb * sizeof(uint32_t);
 
     // x row held by this lane in the MFMA A operand (A row = ln): m = ln / 4 + 4 * (ln % 4).
     const int am = (ln >> 2) + 4 * (ln & 3);
     const bool a_valid = ((ln & 3) < MI) && (am < p.M);
-    const uint16_t *xrow = p.x + (size_t)(a_valid ? am : 0) * p.K + 8 * lg;
+    const char *x_s = reinterpret_cast<const char *>(p.x);
+    const uint32_t x_lane = (uint32_t)(((size_t)(a_valid ? am : 0) * p.K + 8 * lg) * sizeof(uint16_t));
 
     const uint32_t ones_w = 0x3F803F80u;
     const u32x4 ones4 = {ones_w, ones_w, ones_w, ones_w};
@@ -229,16 +236,17 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         }
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
-            const size_t row0 = (size_t)(kstep0 + s) * 32 + 8 * lg;
-            av[s] = *reinterpret_cast<const u32x4 *>(xrow + (size_t)(kstep0 + s) * 32);
+            const size_t krow = (size_t)(kstep0 + s) * 32;          // scalar
+            av[s] = *reinterpret_cast<const u32x4 *>(x_s + krow * sizeof(uint16_t) + x_lane);
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                w[s][i] = __builtin_nontemporal_load(reinterpret_cast<const wvec *>(qw + (row0 + i) * p.nb));
+                w[s][i] = __builtin_nontemporal_load(reinterpret_cast<const wvec *>(qw_s + (krow + i) * row_bytes + qw_lane));
         }
-        const wvec zw = *reinterpret_cast<const wvec *>(qz + (size_t)g * p.nb);
+        const wvec zw = *reinterpret_cast<const wvec *>(qz_s + (size_t)g * row_bytes + qz_lane);
         u32x4 sv[LW];
 #pragma unroll
-        for (int c = 0; c < LW; ++c) sv[c] = *reinterpret_cast<const u32x4 *>(sc + (size_t)g * p.N + 8 * c);
+        for (int c = 0; c < LW; ++c)
+            sv[c] = *reinterpret_cast<const u32x4 *>(sc_s + ((size_t)g * p.N + 8 * c) * sizeof(uint16_t) + sc_lane);
         // Keep every load of the unit above this point: left alone, the scheduler sinks half of
         // them below the first MFMAs to save registers, and a wave then waits for memory twice
         // (GEMV 10.55 -> 10.25 us).  It costs ~27 registers, i.e. the third wave per SIMD, which the
