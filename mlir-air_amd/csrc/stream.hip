@@ -141,16 +141,16 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     const int lg = lane >> 4;
     const int ln = lane & 15;
 
-    // blockIdx -> (tile, matrix, K-slice); consecutive block ids go to consecutive XCDs, so
-    // the workgroups of one tile share an XCD and the reducer has the highest id of its tile.
+    // grid = (tiles rounded up to 8, K-slices, matrices).  Workgroups are numbered x fastest and
+    // consecutive numbers go to consecutive XCDs, so with gridDim.x a multiple of 8 all workgroups
+    // of a tile share an XCD (tile % 8); they are dispatched in that order too, so the reducer,
+    // the last K-slice of the last matrix, starts after all of its producers.
     const int per_tile = p.nmat * p.ksplit;
-    const int xcd = blockIdx.x & 7;
-    const int local = blockIdx.x >> 3;
-    const int tile = (local / per_tile) * 8 + xcd;
+    const int tile = blockIdx.x;
     if (tile >= p.ntiles) return;
-    const int sub = local % per_tile;
-    const int mat = sub / p.ksplit;
-    const int kslice = sub % p.ksplit;
+    const int kslice = blockIdx.y;
+    const int mat = blockIdx.z;
+    const int sub = mat * p.ksplit + kslice;
 
     const int nchunks = p.nb / LW;
     const int chunk = tile * 16 + ln;
@@ -516,19 +516,19 @@ StreamPlan plan_stream(int M, int K, int N) {
 }
 
 template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false>
-static hipError_t launch_one(const StreamParams &p, int grid, hipStream_t stream) {
+static hipError_t launch_one(const StreamParams &p, dim3 grid, hipStream_t stream) {
     const size_t lds = (size_t)WAVES * p.M * 8 * LW * 17 * sizeof(float);   // <= 136 KB at M = 16, LW = 2, 8 waves
     if (lds > 64 * 1024) {   // more than 64 KB of dynamic LDS needs the attribute (per device, so set it every time)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>), dim3(grid), dim3(WAVES * 64), lds, stream, p);
+    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>), grid, dim3(WAVES * 64), lds, stream, p);
     return hipGetLastError();
 }
 
 template <int LW, int WB, int KSTEPS, int WAVES>
-static hipError_t launch_mi(int mi, const StreamParams &p, int grid, hipStream_t stream) {
+static hipError_t launch_mi(int mi, const StreamParams &p, dim3 grid, hipStream_t stream) {
     if (p.norm_w)   // M <= 4 checked by the caller
         return p.nmat == 2 ? launch_one<LW, WB, KSTEPS, WAVES, 1, 2, true>(p, grid, stream)
                            : launch_one<LW, WB, KSTEPS, WAVES, 1, 1, true>(p, grid, stream);
@@ -541,12 +541,12 @@ static hipError_t launch_mi(int mi, const StreamParams &p, int grid, hipStream_t
 }
 
 template <int LW, int WB, int KSTEPS>
-static hipError_t launch_waves(int waves, int mi, const StreamParams &p, int grid, hipStream_t stream) {
+static hipError_t launch_waves(int waves, int mi, const StreamParams &p, dim3 grid, hipStream_t stream) {
     return waves == 4 ? launch_mi<LW, WB, KSTEPS, 4>(mi, p, grid, stream) : launch_mi<LW, WB, KSTEPS, 8>(mi, p, grid, stream);
 }
 
 template <int LW, int WB>
-static hipError_t launch_ksteps(int ksteps, int waves, int mi, const StreamParams &p, int grid, hipStream_t stream) {
+static hipError_t launch_ksteps(int ksteps, int waves, int mi, const StreamParams &p, dim3 grid, hipStream_t stream) {
     return ksteps == 2 ? launch_waves<LW, WB, 2>(waves, mi, p, grid, stream) : launch_waves<LW, WB, 4>(waves, mi, p, grid, stream);
 }
 
@@ -585,7 +585,7 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.sumsq_out = extras.sumsq_out;
     p.skip_publish = g_stream_tune.skip_publish;
     p.spin_limit = g_stream_tune.spin_limit > 0 ? g_stream_tune.spin_limit : (1 << 18);
-    const int grid = ((pl.ntiles + 7) / 8) * 8 * p.nmat * pl.ksplit;
+    const dim3 grid(((pl.ntiles + 7) / 8) * 8, pl.ksplit, p.nmat);
     return pl.lw == 1 ? launch_ksteps<1, 1>(pl.ksteps, pl.waves, pl.mi, p, grid, stream)
                       : launch_ksteps<2, 2>(pl.ksteps, pl.waves, pl.mi, p, grid, stream);
 }
