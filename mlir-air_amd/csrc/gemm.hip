@@ -202,17 +202,30 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
     auto step = [&](int kt, uint16_t *cur, uint16_t *nxt, uint32_t (&rb_next)[8], uint32_t (&rb_after)[8],
                     auto NEXT, auto AFTER, auto ODD) {
         bf16x8 fa[2][4], fb[2][4];
-        if (NEXT) dma_a(nxt, (kt + 1) * BK);
+        // Everything that was loaded into registers earlier is taken over before the x tile copy is
+        // issued: with a copy to LDS pending the compiler waits for vmcnt(0) at the first use of
+        // any loaded register, which would expose the copy's latency in every step.
+        uint32_t rbn[8];
+        if (NEXT) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                rbn[i] = rb_next[i];
+                asm volatile("" : "+v"(rbn[i]));
+            }
+            if (ODD) convert_group();
+#pragma unroll
+            for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(zs[j]), "+v"(sf[j]));
+            dma_a(nxt, (kt + 1) * BK);
+        }
         if (AFTER) {
             load_b((kt + 2) * BK, rb_after);
             if (!ODD) fetch_group((kt + 2) * BK);
         }
-        if (NEXT && ODD) convert_group();
         read_frags(cur, 0, fa[0], fb[0]);
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             if (kk < 3) read_frags(cur, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
-            if (NEXT) store_b(nxt, rb_next, kk);
+            if (NEXT) store_b(nxt, rbn, kk);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
