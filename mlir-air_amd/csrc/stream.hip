@@ -10,10 +10,10 @@
 //   K-step = 32 rows = one v_mfma_f32_16x16x32_bf16; lane (lg, ln) = (lane / 16, lane % 16)
 //            loads rows 8*lg .. 8*lg+7 of chunk ln, i.e. exactly the K-slice the MFMA B
 //            operand wants from that lane
-//   unit   = KSTEPS consecutive K-steps inside one quantisation group, all loads issued up
-//            front and consumed K-step by K-step as they land
-//   wave   = `units` units; workgroup = WAVES waves on one (tile, K-slice); the grid is
-//            (tiles x ksplit) with all K-slices of a tile on the same XCD
+//   unit   = KSTEPS consecutive K-steps inside one quantisation group, all of its loads issued
+//            before any of it is consumed
+//   wave   = `units` units; workgroup = WAVES waves on one (tile, K-slice, matrix); the grid is
+//            (tiles, K-slices, matrices) with all workgroups of a tile on the same XCD
 //
 // Operand construction.  For rows (k, k+1) and byte p of a packed word, v_perm_b32 builds
 // [0, byte_p(row k+1), 0, byte_p(row k)]; `& 0x000F000F | 0x43004300` turns the low nibbles
@@ -27,14 +27,15 @@
 // that for M <= 4 only accumulator register 0 is live in the group flush.
 //
 // Cross-wave combine goes through LDS.  Cross-workgroup combine: every workgroup of a tile
-// except the one with the highest block id stores its fp32 partial to the workspace and
-// exits; the highest one (the reducer) polls for those partials, adds them in fixed order
+// except the last one in dispatch order (last K-slice of the last matrix) stores its fp32
+// partial to the workspace and exits; the last one (the reducer) polls for those partials,
+// two polling rounds in flight at a time, adds them in fixed order
 // (deterministic), applies the epilogue and writes y.  A partial slot holds the sentinel
 // 0xFFFFFFFF ("empty") until its producer overwrites it, and the reducer puts the sentinel
 // back after reading, so the workspace is clean again when the kernel ends.  All slot
 // traffic uses agent-scope atomic loads/stores (served at the device coherence point, never
 // stale in an XCD's L2) and needs no fences: validity travels with each 32-bit value.  The
-// reducer is dispatched after its producers (workgroups are dispatched in block-id order), so
+// reducer is dispatched after its producers (workgroups are dispatched in linear id order, x fastest), so
 // the producers never wait on anything and the poll terminates; it is bounded all the same
 // and reports a timeout through the workspace header instead of hanging.
 #include "common.h"
