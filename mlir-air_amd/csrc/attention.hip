@@ -214,6 +214,11 @@ __global__ void attn_combine_kernel(const float *part_ml, const float *part_acc,
     __shared__ float wgt[kMaxAttnSplit];
     __shared__ float inv_l;
     const int head = blockIdx.x, e = threadIdx.x;
+    // every load of the kernel is requested up front: one memory round trip in total
+    const float *src = part_acc + (size_t)head * nsplit * hd + e;
+    float a[kMaxAttnSplit];
+#pragma unroll
+    for (int s = 0; s < kMaxAttnSplit; ++s) a[s] = s < nsplit ? src[(size_t)s * hd] : 0.f;
     if (e < 64) {
         const bool live = e < nsplit;
         const float m = live ? part_ml[2 * ((size_t)head * nsplit + e)] : kNegBig;
@@ -225,14 +230,13 @@ __global__ void attn_combine_kernel(const float *part_ml, const float *part_acc,
         float ls = l * c;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) ls += __shfl_xor(ls, off);
-        if (live) wgt[e] = c;
+        if (e < kMaxAttnSplit) wgt[e] = live ? c : 0.f;
         if (e == 0) inv_l = 1.0f / ls;
     }
     __syncthreads();
-    const float *src = part_acc + (size_t)head * nsplit * hd + e;
     float as = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < nsplit; ++s) as = fmaf(src[(size_t)s * hd], wgt[s], as);
+#pragma unroll
+    for (int s = 0; s < kMaxAttnSplit; ++s) as = fmaf(a[s], wgt[s], as);
     out[(size_t)head * hd + e] = float_to_bf16_bits(as * inv_l);
 }
 
