@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -37,6 +37,10 @@ CONFIGS = {
     # one whole decode layer: RMSNorm + fused QKV GEMV, RoPE + KV append + GQA attention over 2048 cached
     # positions (32 heads, 8 KV heads, head_dim 128), then the block above
     "layer": dict(M=1, K=4096, N=14336, cfg=None, desc="decode layer W4A16 E=4096 H=14336 32/8 heads hd=128 pos=2047 g128"),
+    # the Q4NX codec (w = q * s + m, 32-column groups) through the same streaming kernel: the gate / up
+    # projection shape of Llama-3.1-8B (programming_examples/llms/llama31_8b_q4nx)
+    "q4nx_gemv": dict(M=1, K=4096, N=14336, cfg=None, desc="decode GEMV Q4NX M=1 K=4096 N=14336 g32"),
+    "q4nx_gemm16": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM Q4NX M=16 K=4096 N=14336 g32"),
 }
 LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 2048
 
@@ -50,9 +54,15 @@ def weight_bytes(K, N):
     return K * N // 2 + (K // 128) * (N // 8) * 4 + (K // 128) * N * 2
 
 
+def q4nx_weight_bytes(K, N):
+    return K * N // 2 + 2 * (K // 32) * N * 2
+
+
 def algorithmic_bytes(name):
     c = CONFIGS[name]
     M, K, N = c["M"], c["K"], c["N"]
+    if name.startswith("q4nx"):
+        return q4nx_weight_bytes(K, N) + M * K * 2 + M * N * 2
     if name == "dequant":
         return weight_bytes(K, N) + K * N * 2
     if name == "ffn":
@@ -85,6 +95,15 @@ def make_weights(torch, K, N, seed):
     return qweight, qzeros, scales
 
 
+def make_q4nx_weights(torch, K, N, seed):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    qweight = torch.randint(-2**31, 2**31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    scales = (torch.randn((K // 32, N), device="cuda", generator=g).abs() * 0.003 + 1e-3).to(torch.bfloat16)
+    mins = (-torch.randn((K // 32, N), device="cuda", generator=g).abs() * 0.02 - 0.01).to(torch.bfloat16)
+    return qweight, scales, mins
+
+
 def run_workload(name, steps, warmup, with_cpu_baseline):
     import torch
 
@@ -97,7 +116,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     torch.cuda.set_device(dev)
     stream = torch.cuda.Stream()
 
-    per_copy = weight_bytes(K, N) * (3 if name in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if name in ("block", "layer") else 0)
+    q4nx = name.startswith("q4nx")
+    per_copy = q4nx_weight_bytes(K, N) if q4nx else weight_bytes(K, N) * (3 if name in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if name in ("block", "layer") else 0)
     nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
     if name == "layer":
         per_copy += weight_bytes(K, nqkv)
@@ -114,6 +134,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             c4 = (make_weights(torch, K, N, 100 + 5 * i), make_weights(torch, K, N, 101 + 5 * i),
                   make_weights(torch, N, K, 102 + 5 * i), make_weights(torch, K, K, 103 + 5 * i))
             copies.append(c4 + ((make_weights(torch, K, nqkv, 104 + 5 * i),) if name == "layer" else ()))
+        elif q4nx:
+            copies.append(make_q4nx_weights(torch, K, N, 100 + i))
         else:
             copies.append(make_weights(torch, K, N, 100 + i))
     gx = torch.Generator(device="cuda")
@@ -173,6 +195,9 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                 a_in = attn_out
             rc = lib.w4a16_o_gemv_ffn_bf16(a_in.data_ptr(), x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, *ptrs,
                                            outs[0].data_ptr(), None, None, K, N, 128, ws.data_ptr(), ws.numel(), st)
+        elif q4nx:
+            rc = lib.w4a16_q4nx_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), None,
+                                          outs[0].data_ptr(), M, K, N, ws.data_ptr(), ws.numel(), st)
         else:
             rc = lib.w4a16_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
                                      outs[0].data_ptr(), M, K, N, 128, ws.data_ptr(), ws.numel(), st)
@@ -231,7 +256,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                  "avg": sum(per_launch) / len(per_launch), "max": per_launch[-1]},
     }
 
-    if with_cpu_baseline and name not in ("block", "layer"):
+    if with_cpu_baseline and name not in ("block", "layer") and not q4nx:
         res["cpu_baseline"] = cpu_baseline(name, torch, copies[0], x, outs, launch, stream)
     return res
 
@@ -383,7 +408,7 @@ def main():
         "vs_baseline": None,
         "dtype": "int4 weights, bf16 activations, fp32 accumulate",
         "data": "synthetic (uniform uint4 q/z, scales |N(0,1)|*0.02+1e-3, x ~ N(0,1)), random weights",
-        "config": {"workload": CONFIGS[name]["desc"], "group": 128,
+        "config": {"workload": CONFIGS[name]["desc"], "group": 32 if name.startswith("q4nx") else 128,
                    "weight_copies_rotated": main_res["ncopies"], "timing": "HIP graph of K launches, events on the launch stream"},
         "roofline": roof,
         "per_launch_events_us": main_res["per_launch_events_us"],

@@ -214,6 +214,55 @@ int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_ro
                                 void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Q4NX / Q4_0 block codec (the 4-bit formats of the fused decode examples).  W[M, K] (M output
+ * features, K input features) is stored as (M / 32) x (K / 256) blocks of 5120 bytes, row-block
+ * major, each holding bf16 scales[8][32], bf16 mins[8][32] (one per row and 32-column group) and
+ * the nibbles qs[2][256][8] with byte kk of (rg, col) = (q[16 rg + 2 kk + 1][col] << 4) |
+ * q[16 rg + 2 kk][col] (pack_q4k_block, programming_examples/fused_decode/proj_qmm_pack.py:4-58;
+ * q4k_block_t, programming_examples/fused_decode/kernels/model_spec.h:86-103).
+ * `mode` selects the value convention:
+ *   W4A16_Q4NX_ADDITIVE     w = s * q + m, q unsigned: what the proj_qmm kernel computes
+ *                           (programming_examples/fused_decode/kernels/q4_k.h:9-17) and what bundles
+ *                           with an "I8" header hold (Q4nxModel.dequant,
+ *                           programming_examples/llms/llama32_1b_q4nx/llama32_1b_q4nx_weights.py:205-266)
+ *   W4A16_Q4NX_SUBTRACTIVE  w = s * (q - m): bundles with a "Q4NX" header (same function, :255-261)
+ *   W4A16_Q4_0              w = s * q, q signed two's complement, mins ignored
+ *                           (programming_examples/fused_decode/qwen25_3b_requant.py:13-17, 116-134)
+ *
+ * q4nx_dequant_bf16 writes the dense matrix out[M, K] = bf16(w) (fp32 arithmetic in the order
+ * written above, one rounding to bf16), replacing Q4nxModel.dequant / dequant_q4_0
+ * (programming_examples/llms/qwen25_3b_q4/qwen25_3b_q4_weights.py:86-95) followed by the cast to bf16.
+ *
+ * q4nx_repack turns the blocks into the operands of w4a16_q4nx_gemm_bf16, once at load time (the
+ * reference re-packs the same blocks into its own device stream order, pack_q4k_cascade,
+ * proj_qmm_pack.py:61-140): qweight int32 [K, M / 8] (word (k, j) = rows 8 j .. 8 j + 7 of
+ * column k, unsigned nibbles in the AutoAWQ order), scales and mins bf16 [K / 32, M] with
+ * w = q * scale + min.  W4A16_Q4_0 is exact (q ^ 8, min = -8 s); W4A16_Q4NX_SUBTRACTIVE stores
+ * min = bf16(-s * m), one extra rounding of the constant term.
+ * M % 32 == 0, K % 256 == 0, all pointers 16-byte aligned.
+ */
+#define W4A16_Q4NX_ADDITIVE 0
+#define W4A16_Q4NX_SUBTRACTIVE 1
+#define W4A16_Q4_0 2
+int q4nx_dequant_bf16(const void *blocks, uint16_t *out_bf16, int M, int K, int mode, void *stream);
+int q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t *mins,
+                int M, int K, int mode, void *stream);
+
+/*
+ * y[M, N] = bf16(x[M, K] . W + residual) for the affine 32-row-group codec above, W given by the
+ * operands of q4nx_repack (N = that function's M).  In fp32 per group:
+ * y += s * sum(q x) + m * sum(x), the arithmetic of _qmm_q4k_bf16
+ * (programming_examples/fused_decode/kernels/q4_k.h:39-45: c += (q*b)*scale; c += min*sum(b)).
+ * `residual` bf16 [M, N] may be NULL.  Any M >= 1 (16 rows per launch of the streaming kernel;
+ * the reference runs the prefill of these models as dense bf16 GEMMs on dequantised weights,
+ * so there is no large-M kernel for this codec).  K % 128 == 0, N % 32 == 0.
+ * Workspace: w4a16_gemm_workspace_bytes(M, K, N), initialised with w4a16_workspace_init.
+ */
+int w4a16_q4nx_gemm_bf16(const uint16_t *x, const int32_t *qweight, const uint16_t *scales, const uint16_t *mins,
+                         const uint16_t *residual, uint16_t *y, int M, int K, int N,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic),
  * "gemm_stream_max_m" (largest M given to the streaming kernel, 0 = default 96, otherwise >= 16) and

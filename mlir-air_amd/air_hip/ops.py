@@ -240,6 +240,58 @@ def decode_attention(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, out=None
     return out
 
 
+def q4nx_dequant(blocks, M, K, mode=0, out=None):
+    """Dense W[M, K] bf16 from Q4NX / Q4_0 blocks (uint8 [M/32 * K/256, 5120] on the GPU);
+    mode 0 w = s q + m, 1 w = s (q - m), 2 signed q with w = s q."""
+    lib = _lib.load_library()
+    _need_cuda(blocks)
+    if blocks.numel() * blocks.element_size() != (M // 32) * (K // 256) * 5120:
+        raise ValueError(f"blocks hold {blocks.numel() * blocks.element_size()} bytes, [M, K] = {[M, K]} needs {(M // 32) * (K // 256) * 5120}")
+    if out is None:
+        out = torch.empty((M, K), dtype=torch.bfloat16, device=blocks.device)
+    _lib.check(lib.q4nx_dequant_bf16(_ptr(blocks), _ptr(out), M, K, mode, _stream()))
+    return out
+
+
+def q4nx_repack(blocks, M, K, mode=0):
+    """Blocks -> (qweight int32 [K, M/8], scales bf16 [K/32, M], mins bf16 [K/32, M]), the
+    operands of q4nx_gemm; done once per tensor at load time."""
+    lib = _lib.load_library()
+    _need_cuda(blocks)
+    if blocks.numel() * blocks.element_size() != (M // 32) * (K // 256) * 5120:
+        raise ValueError(f"blocks hold {blocks.numel() * blocks.element_size()} bytes, [M, K] = {[M, K]} needs {(M // 32) * (K // 256) * 5120}")
+    qweight = torch.empty((K, M // 8), dtype=torch.int32, device=blocks.device)
+    scales = torch.empty((K // 32, M), dtype=torch.bfloat16, device=blocks.device)
+    mins = torch.empty((K // 32, M), dtype=torch.bfloat16, device=blocks.device)
+    _lib.check(lib.q4nx_repack(_ptr(blocks), _ptr(qweight), _ptr(scales), _ptr(mins), M, K, mode, _stream()))
+    return qweight, scales, mins
+
+
+def q4nx_gemm(x, qweight, scales, mins, residual=None, out=None):
+    """y = bf16(x . W + residual) for the operands of q4nx_repack; x [rows, K] or a vector [K]."""
+    lib = _lib.load_library()
+    _need_cuda(x, qweight, scales, mins)
+    vec = x.dim() == 1
+    x2 = x.unsqueeze(0) if vec else x
+    M, K = x2.shape
+    if qweight.shape[0] != K:
+        raise ValueError(f"x has K={K} but qweight has {qweight.shape[0]} rows")
+    N = qweight.shape[1] * 8
+    if scales.shape != (K // 32, N) or mins.shape != (K // 32, N):
+        raise ValueError(f"scales / mins must be [{K // 32}, {N}], got {tuple(scales.shape)} / {tuple(mins.shape)}")
+    if residual is not None:
+        _need_cuda(residual)
+        if residual.numel() != M * N:
+            raise ValueError("residual must have the shape of the result")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    ws = workspace(lib.w4a16_gemm_workspace_bytes(M, K, N), x.device)
+    _lib.check(lib.w4a16_q4nx_gemm_bf16(_ptr(_bits(x2)), _ptr(qweight), _ptr(_bits(scales)), _ptr(_bits(mins)),
+                                        _ptr(_bits(residual)) if residual is not None else None, _ptr(out),
+                                        M, K, N, _ptr(ws), ws.numel(), _stream()))
+    return out.squeeze(0) if vec else out
+
+
 def tune(key, value):
     lib = _lib.load_library()
     _lib.check(lib.w4a16_tune(key.encode(), int(value)))

@@ -317,6 +317,45 @@ int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_ro
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+int q4nx_dequant_bf16(const void *blocks, uint16_t *out_bf16, int M, int K, int mode, void *stream) {
+    if (!blocks || !out_bf16) return W4A16_ERR_NULL;
+    if (M <= 0 || K <= 0 || M % 32 != 0 || K % 256 != 0 || mode < 0 || mode > 2) return W4A16_ERR_SHAPE;
+    if (misaligned(blocks) || misaligned(out_bf16)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_q4nx_dequant(blocks, out_bf16, M, K, mode, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t *mins, int M, int K, int mode,
+                void *stream) {
+    if (!blocks || !qweight || !scales || !mins) return W4A16_ERR_NULL;
+    if (M <= 0 || K <= 0 || M % 32 != 0 || K % 256 != 0 || mode < 0 || mode > 2) return W4A16_ERR_SHAPE;
+    if (misaligned(blocks) || misaligned(qweight) || misaligned(scales) || misaligned(mins)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_q4nx_repack(blocks, qweight, scales, mins, M, K, mode, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_q4nx_gemm_bf16(const uint16_t *x, const int32_t *qweight, const uint16_t *scales, const uint16_t *mins,
+                         const uint16_t *residual, uint16_t *y, int M, int K, int N, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+    if (!x || !y || !qweight || !scales || !mins) return W4A16_ERR_NULL;
+    if (M <= 0 || K <= 0 || N <= 0 || K % 128 != 0 || N % 32 != 0) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(y) || misaligned(qweight) || misaligned(scales) || misaligned(mins) ||
+        misaligned(residual))
+        return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_gemm_workspace_bytes(M, K, N)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = hipSuccess;
+    for (int m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
+        const int rows = M - m0 < 16 ? M - m0 : 16;
+        StreamExtras extras;
+        extras.mins = mins;
+        extras.residual = residual ? residual + (size_t)m0 * N : nullptr;
+        e = launch_stream(x + (size_t)m0 * K, qweight, nullptr, scales, nullptr, nullptr, nullptr, y + (size_t)m0 * N,
+                          rows, K, N, workspace, static_cast<hipStream_t>(stream), extras);
+    }
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_tune(const char *key, int value) {
     if (!key || value < 0) return W4A16_ERR_TUNE;
     if (!strcmp(key, "gemv_lw")) {

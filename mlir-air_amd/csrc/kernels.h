@@ -45,6 +45,9 @@ struct StreamExtras {
     const float *sumsq_in = nullptr;
     int sumsq_n = 0;
     float *sumsq_out = nullptr;
+    // Affine codec with 32-row groups (w = q * s + m): per-group minimum [K / 32, N] bf16.  `scales` is then
+    // [K / 32, N] too and `qzeros` is not read.  Single matrix, no norm_w.
+    const uint16_t *mins = nullptr;
 };
 
 // y[M, N] = bf16(x[M, K] . W), M <= 16.  With `up_*` given (SwiGLU epilogue, M == 1) the
@@ -58,6 +61,11 @@ hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const 
                                const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream);
 
 hipError_t launch_fill_workspace(void *ptr, size_t bytes, hipStream_t stream);
+
+// Q4NX / Q4_0 block codec (q4nx.hip).  mode: 0 w = s q + m, 1 w = s (q - m), 2 signed q, w = s q.
+hipError_t launch_q4nx_dequant(const void *blocks, uint16_t *out, int M, int K, int mode, hipStream_t stream);
+hipError_t launch_q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t *mins, int M, int K,
+                              int mode, hipStream_t stream);
 
 // Decode attention (attention.hip).  The scratch buffer holds per-chunk softmax partials and
 // needs no initialisation.

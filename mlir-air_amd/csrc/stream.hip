@@ -50,6 +50,7 @@ struct StreamParams {
     const uint32_t *qw[2];
     const uint32_t *qz[2];
     const uint16_t *sc[2];
+    const uint16_t *mn;   // affine codec: per-group minimum [K / 32, N] bf16 (qz unused), else null
     uint16_t *y;
     uint32_t *header;   // workspace header: word 0 = poll timeouts seen
     float *partial;     // [nmat * ksplit][ntiles][M * tile columns]
@@ -127,7 +128,10 @@ struct Words<1> { typedef uint32_t type __attribute__((ext_vector_type(1))); };
 // RMS    x is RMS-normalised on the fly: every wave computes 1/sqrt(mean(x^2) + eps) of its
 //        rows itself (x is K bf16 values, L2-resident) while its weight loads are in
 //        flight, and feeds bf16((x * rstd) * norm_w) to the matrix cores.  M <= 4.
-template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS>
+// AFF    affine codec with groups of 32 rows (one K-step): w = q * s + m with unsigned q, s and m
+//        bf16 [K / 32, N].  Every K-step is flushed on its own:
+//        y += s * sum (128 + q) x  +  (m - 128 s) * sum x.
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS, bool AFF>
 __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParams p) {
     constexpr int SLOTS = WAVES;   // one LDS slot per wave: a single write round, no read-modify-write
     typedef typename Words<LW>::type wvec;
@@ -161,6 +165,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     const char *qw_s = reinterpret_cast<const char *>(p.qw[mat]);
     const char *qz_s = reinterpret_cast<const char *>(p.qz[mat]);
     const char *sc_s = reinterpret_cast<const char *>(p.sc[mat]);
+    const char *mn_s = reinterpret_cast<const char *>(p.mn);
     const uint32_t qw_lane = (uint32_t)(((size_t)chunk_c * LW + (size_t)(8 * lg) * p.nb) * sizeof(uint32_t));
     const uint32_t qz_lane = (uint32_t)((size_t)chunk_c * LW * sizeof(uint32_t));
     const uint32_t sc_lane = (uint32_t)((size_t)chunk_c * LC * sizeof(uint16_t));
@@ -243,11 +248,25 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             for (int i = 0; i < 8; ++i)
                 w[s][i] = __builtin_nontemporal_load(reinterpret_cast<const wvec *>(qw_s + (krow + i) * row_bytes + qw_lane));
         }
-        const wvec zw = *reinterpret_cast<const wvec *>(qz_s + (size_t)g * row_bytes + qz_lane);
+        wvec zw;
         u32x4 sv[LW];
+        u32x4 gs[AFF ? KSTEPS : 1][LW], gm[AFF ? KSTEPS : 1][LW];   // affine codec: scales and minima of each K-step
+        if constexpr (AFF) {
 #pragma unroll
-        for (int c = 0; c < LW; ++c)
-            sv[c] = *reinterpret_cast<const u32x4 *>(sc_s + ((size_t)g * p.N + 8 * c) * sizeof(uint16_t) + sc_lane);
+            for (int s = 0; s < KSTEPS; ++s) {
+#pragma unroll
+                for (int c = 0; c < LW; ++c) {
+                    const size_t off = ((size_t)(kstep0 + s) * p.N + 8 * c) * sizeof(uint16_t) + sc_lane;
+                    gs[s][c] = *reinterpret_cast<const u32x4 *>(sc_s + off);
+                    gm[s][c] = *reinterpret_cast<const u32x4 *>(mn_s + off);
+                }
+            }
+        } else {
+            zw = *reinterpret_cast<const wvec *>(qz_s + (size_t)g * row_bytes + qz_lane);
+#pragma unroll
+            for (int c = 0; c < LW; ++c)
+                sv[c] = *reinterpret_cast<const u32x4 *>(sc_s + ((size_t)g * p.N + 8 * c) * sizeof(uint16_t) + sc_lane);
+        }
         // Keep every load of the unit above this point: left alone, the scheduler sinks half of
         // them below the first MFMAs to save registers, and a wave then waits for memory twice
         // (GEMV 10.55 -> 10.25 us).  It costs ~27 registers, i.e. the third wave per SIMD, which the
@@ -276,25 +295,17 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s)
             if (!a_valid) av[s] = u32x4{0u, 0u, 0u, 0u};
-        floatx4 xs = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < KSTEPS; ++s)
-            xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av[s]), ones, xs, 0, 0, 0);
-
-        // WB packed words (8 * WB MFMA tiles) at a time: K-steps outer so that work starts as
-        // soon as a K-step's loads have landed, then the group flush of those words.
-        // acc[cc * 8 + pos]: word cb + cc, nibble position pos (= 2 * byte + nibble-in-byte).
-#pragma unroll
-        for (int cb = 0; cb < LW; cb += WB) {
-            floatx4 acc[8 * WB];
-#pragma unroll
-            for (int t = 0; t < 8 * WB; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+        if constexpr (AFF) {
+            // One group per K-step: the MFMA tiles of a K-step start from zero and are folded into
+            // yacc right away.  Column mapping as in the group flush below.
+            const floatx4 zero4 = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int s = 0; s < KSTEPS; ++s) {
                 const bf16x8 a = __builtin_bit_cast(bf16x8, av[s]);
+                const floatx4 xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ones, zero4, 0, 0, 0);
 #pragma unroll
-                for (int cc = 0; cc < WB; ++cc) {
-                    const int c = cb + cc;
+                for (int c = 0; c < LW; ++c) {
+                    floatx4 acc[8];
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
                         const uint32_t sel = 0x0C000C00u | ((4u + b) << 16) | (uint32_t)b;
@@ -305,28 +316,76 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
                             lo[v] = (pr & nib_mask) | magic;
                             hi[v] = ((pr >> 4) & nib_mask) | magic;
                         }
-                        const int t = cc * 8 + 2 * b;
-                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, lo), acc[t], 0, 0, 0);
-                        acc[t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, hi), acc[t + 1], 0, 0, 0);
+                        acc[2 * b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, lo), zero4, 0, 0, 0);
+                        acc[2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, hi), zero4, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t sw = gs[s][c][q], mw = gm[s][c][q];
+                        const float s_lo = __builtin_bit_cast(float, sw << 16), s_hi = __builtin_bit_cast(float, sw & 0xFFFF0000u);
+                        const float m_lo = __builtin_bit_cast(float, mw << 16), m_hi = __builtin_bit_cast(float, mw & 0xFFFF0000u);
+                        const float c_lo = fmaf(-128.f, s_lo, m_lo), c_hi = fmaf(-128.f, s_hi, m_hi);
+#pragma unroll
+                        for (int i = 0; i < MI; ++i) {
+                            yacc[c * 8 + 2 * q][i] = fmaf(s_lo, acc[q][i], fmaf(c_lo, xs[i], yacc[c * 8 + 2 * q][i]));
+                            yacc[c * 8 + 2 * q + 1][i] = fmaf(s_hi, acc[q + 4][i], fmaf(c_hi, xs[i], yacc[c * 8 + 2 * q + 1][i]));
+                        }
                     }
                 }
             }
-            // Group flush.  Nibble positions (q, q + 4) of a word are natural columns (2q, 2q + 1),
-            // i.e. the two halves of scale word q; (zw >> 4q) & 0x000F000F | 0x43004300 is the bf16
-            // pair (128 + z) of the same two columns.  yacc[c * 8 + j] is natural column 8c + j.
-#pragma unroll
-            for (int cc = 0; cc < WB; ++cc) {
-                const int c = cb + cc;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const uint32_t zp = ((zw[c] >> (4 * q)) & nib_mask) | magic;
-                    const uint32_t sw = sv[c][q];
-                    const float z_lo = __builtin_bit_cast(float, zp << 16), z_hi = __builtin_bit_cast(float, zp & 0xFFFF0000u);
-                    const float s_lo = __builtin_bit_cast(float, sw << 16), s_hi = __builtin_bit_cast(float, sw & 0xFFFF0000u);
-#pragma unroll
-                    for (int i = 0; i < MI; ++i) {
-                        yacc[c * 8 + 2 * q][i] = fmaf(s_lo, fmaf(-z_lo, xs[i], acc[cc * 8 + q][i]), yacc[c * 8 + 2 * q][i]);
-                        yacc[c * 8 + 2 * q + 1][i] = fmaf(s_hi, fmaf(-z_hi, xs[i], acc[cc * 8 + q + 4][i]), yacc[c * 8 + 2 * q + 1][i]);
+        } else {
+            floatx4 xs = floatx4{0.f, 0.f, 0.f, 0.f};
+    #pragma unroll
+            for (int s = 0; s < KSTEPS; ++s)
+                xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av[s]), ones, xs, 0, 0, 0);
+
+            // WB packed words (8 * WB MFMA tiles) at a time: K-steps outer so that work starts as
+            // soon as a K-step's loads have landed, then the group flush of those words.
+            // acc[cc * 8 + pos]: word cb + cc, nibble position pos (= 2 * byte + nibble-in-byte).
+    #pragma unroll
+            for (int cb = 0; cb < LW; cb += WB) {
+                floatx4 acc[8 * WB];
+    #pragma unroll
+                for (int t = 0; t < 8 * WB; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    #pragma unroll
+                for (int s = 0; s < KSTEPS; ++s) {
+                    const bf16x8 a = __builtin_bit_cast(bf16x8, av[s]);
+    #pragma unroll
+                    for (int cc = 0; cc < WB; ++cc) {
+                        const int c = cb + cc;
+    #pragma unroll
+                        for (int b = 0; b < 4; ++b) {
+                            const uint32_t sel = 0x0C000C00u | ((4u + b) << 16) | (uint32_t)b;
+                            u32x4 lo, hi;
+    #pragma unroll
+                            for (int v = 0; v < 4; ++v) {
+                                const uint32_t pr = __builtin_amdgcn_perm(w[s][2 * v + 1][c], w[s][2 * v][c], sel);
+                                lo[v] = (pr & nib_mask) | magic;
+                                hi[v] = ((pr >> 4) & nib_mask) | magic;
+                            }
+                            const int t = cc * 8 + 2 * b;
+                            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, lo), acc[t], 0, 0, 0);
+                            acc[t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, hi), acc[t + 1], 0, 0, 0);
+                        }
+                    }
+                }
+                // Group flush.  Nibble positions (q, q + 4) of a word are natural columns (2q, 2q + 1),
+                // i.e. the two halves of scale word q; (zw >> 4q) & 0x000F000F | 0x43004300 is the bf16
+                // pair (128 + z) of the same two columns.  yacc[c * 8 + j] is natural column 8c + j.
+    #pragma unroll
+                for (int cc = 0; cc < WB; ++cc) {
+                    const int c = cb + cc;
+    #pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t zp = ((zw[c] >> (4 * q)) & nib_mask) | magic;
+                        const uint32_t sw = sv[c][q];
+                        const float z_lo = __builtin_bit_cast(float, zp << 16), z_hi = __builtin_bit_cast(float, zp & 0xFFFF0000u);
+                        const float s_lo = __builtin_bit_cast(float, sw << 16), s_hi = __builtin_bit_cast(float, sw & 0xFFFF0000u);
+    #pragma unroll
+                        for (int i = 0; i < MI; ++i) {
+                            yacc[c * 8 + 2 * q][i] = fmaf(s_lo, fmaf(-z_lo, xs[i], acc[cc * 8 + q][i]), yacc[c * 8 + 2 * q][i]);
+                            yacc[c * 8 + 2 * q + 1][i] = fmaf(s_hi, fmaf(-z_hi, xs[i], acc[cc * 8 + q + 4][i]), yacc[c * 8 + 2 * q + 1][i]);
+                        }
                     }
                 }
             }
@@ -516,20 +575,27 @@ StreamPlan plan_stream(int M, int K, int N) {
     return pl;
 }
 
-template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false>
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false, bool AFF = false>
 static hipError_t launch_one(const StreamParams &p, dim3 grid, hipStream_t stream) {
     const size_t lds = (size_t)WAVES * p.M * 8 * LW * 17 * sizeof(float);   // <= 136 KB at M = 16, LW = 2, 8 waves
     if (lds > 64 * 1024) {   // more than 64 KB of dynamic LDS needs the attribute (per device, so set it every time)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS>), grid, dim3(WAVES * 64), lds, stream, p);
+    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF>), grid, dim3(WAVES * 64), lds, stream, p);
     return hipGetLastError();
 }
 
 template <int LW, int WB, int KSTEPS, int WAVES>
 static hipError_t launch_mi(int mi, const StreamParams &p, dim3 grid, hipStream_t stream) {
+    if (p.mn) {   // affine codec: single matrix, no RMSNorm prologue (checked by the caller)
+        switch (mi) {
+            case 1: return launch_one<LW, WB, KSTEPS, WAVES, 1, 1, false, true>(p, grid, stream);
+            case 2: return launch_one<LW, WB, KSTEPS, WAVES, 2, 1, false, true>(p, grid, stream);
+            default: return launch_one<LW, WB, KSTEPS, WAVES, 4, 1, false, true>(p, grid, stream);
+        }
+    }
     if (p.norm_w)   // M <= 4 checked by the caller
         return p.nmat == 2 ? launch_one<LW, WB, KSTEPS, WAVES, 1, 2, true>(p, grid, stream)
                            : launch_one<LW, WB, KSTEPS, WAVES, 1, 1, true>(p, grid, stream);
@@ -565,6 +631,7 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.qw[1] = reinterpret_cast<const uint32_t *>(up_qweight ? up_qweight : qweight);
     p.qz[1] = reinterpret_cast<const uint32_t *>(up_qzeros ? up_qzeros : qzeros);
     p.sc[1] = up_scales ? up_scales : scales;
+    p.mn = extras.mins;
     p.y = y;
     p.header = reinterpret_cast<uint32_t *>(workspace);
     p.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + kHeaderBytes);
