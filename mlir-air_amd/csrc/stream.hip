@@ -137,9 +137,10 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     typedef typename Words<LW>::type wvec;
     constexpr int TC = 128 * LW;            // tile columns
     constexpr int LC = 8 * LW;              // columns per lane
-    constexpr int ROWF = LC * 17;           // LDS floats per output row: [j (LC)][ln (16) + 1 pad]
+    constexpr int ROWF = LC * 16;           // LDS floats per output row: [ln (16)][LC], 16-byte chunks XOR-swizzled
+    constexpr int NCH = LC / 4;             // 16-byte chunks per lane
     constexpr int QPR = TC / 4;             // 4-column quads per output row
-    extern __shared__ float red[];
+    extern __shared__ __attribute__((aligned(16))) float red[];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses built from it stay on the SALU
@@ -409,16 +410,21 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             if (j < nprod) va[j] = slot_load(tile_partial + (size_t)threadIdx.x * 4 + j * slice_stride);
     }
 
-    // ---- cross-wave combine in LDS: red[slot][m][j * 17 + ln], j = natural column in the lane's chunk ----
+    // ---- cross-wave combine in LDS: red[slot][m][ln][LC], moved as 16-byte chunks (4 columns).  Chunk jj
+    // of lane ln sits at position jj ^ key(ln), key = (ln * LC / 32) % NCH, so that 8 neighbouring
+    // lanes cover all 32 banks both when a lane writes its chunks and when 8 threads read 8 neighbouring quads.
     const int slot_stride = p.M * ROWF;
     {
-        float *dst = red + wave * slot_stride;
+        float *dst = red + wave * slot_stride + ln * LC;
+        const int key = (ln * LC / 32) % NCH;
 #pragma unroll
-        for (int j = 0; j < LC; ++j) {
+        for (int jj = 0; jj < NCH; ++jj) {
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 const int m = lg + 4 * i;
-                if (m < p.M) dst[m * ROWF + j * 17 + ln] = yacc[j][i];
+                if (m < p.M)
+                    *reinterpret_cast<floatx4 *>(dst + m * ROWF + 4 * (jj ^ key)) =
+                        floatx4{yacc[4 * jj][i], yacc[4 * jj + 1][i], yacc[4 * jj + 2][i], yacc[4 * jj + 3][i]};
             }
         }
     }
@@ -429,11 +435,11 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         const int m = e / QPR;
         const int col = (e % QPR) * 4;
         floatx4 own = floatx4{0.f, 0.f, 0.f, 0.f};
+        {
+            const int qi = e % QPR, qln = qi / NCH, qjj = qi % NCH;
+            const float *src = red + m * ROWF + qln * LC + 4 * (qjj ^ ((qln * LC / 32) % NCH));
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float *src = red + m * ROWF + ((col + q) % LC) * 17 + ((col + q) / LC);
-#pragma unroll
-            for (int s = 0; s < SLOTS; ++s) own[q] += src[s * slot_stride];
+            for (int s = 0; s < SLOTS; ++s) own += *reinterpret_cast<const floatx4 *>(src + s * slot_stride);
         }
         float *slot0 = tile_partial + (size_t)e * 4;
         if (!reducer) {
@@ -577,7 +583,7 @@ StreamPlan plan_stream(int M, int K, int N) {
 
 template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false, bool AFF = false>
 static hipError_t launch_one(const StreamParams &p, dim3 grid, hipStream_t stream) {
-    const size_t lds = (size_t)WAVES * p.M * 8 * LW * 17 * sizeof(float);   // <= 136 KB at M = 16, LW = 2, 8 waves
+    const size_t lds = (size_t)WAVES * p.M * 8 * LW * 16 * sizeof(float);   // 128 KB at M = 16, LW = 2, 8 waves
     if (lds > 64 * 1024) {   // more than 64 KB of dynamic LDS needs the attribute (per device, so set it every time)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
