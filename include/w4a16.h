@@ -263,6 +263,27 @@ int w4a16_q4nx_gemm_bf16(const uint16_t *x, const int32_t *qweight, const uint16
                          void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The decode-layer entry points for the affine codec: w4a16_rms_gemv_bf16 and w4a16_o_gemv_ffn_bf16
+ * with every weight triple given as (qweight, scales, mins) from q4nx_repack.  Same arithmetic,
+ * stages, workspace sizes and optional outputs as their AWQ counterparts above; they cover the
+ * proj / O / FFN phases of the fused decode dispatch
+ * (programming_examples/fused_decode/fused_decode.py: proj_qmm, rms_residual, glu kernels) around
+ * w4a16_decode_attention_bf16.
+ */
+int w4a16_q4nx_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps,
+                             const int32_t *qweight, const uint16_t *scales, const uint16_t *mins,
+                             uint16_t *y, int K, int N,
+                             void *workspace, size_t workspace_bytes, void *stream);
+int w4a16_q4nx_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual,
+                               const uint16_t *ffn_norm_weight, float eps,
+                               const int32_t *o_qweight, const uint16_t *o_scales, const uint16_t *o_mins,
+                               const int32_t *gate_qweight, const uint16_t *gate_scales, const uint16_t *gate_mins,
+                               const int32_t *up_qweight, const uint16_t *up_scales, const uint16_t *up_mins,
+                               const int32_t *down_qweight, const uint16_t *down_scales, const uint16_t *down_mins,
+                               uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int E, int H,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic),
  * "gemm_stream_max_m" (largest M given to the streaming kernel, 0 = default 96, otherwise >= 16) and

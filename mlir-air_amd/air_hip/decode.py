@@ -40,6 +40,34 @@ class DecodeLayer:
     w_gate: tuple
     w_up: tuple
     w_down: tuple
+    codec: str = "awq"   # "awq": triples are (qweight, qzeros, scales); "q4nx": (qweight, scales, mins) from q4nx_repack
+
+
+def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda") -> DecodeLayer:
+    """A Q4NX / Q4_0 layer -> DecodeLayer.  `blocks` maps q, k, v, o, gate, up, down to the tensor's
+    blocks (uint8 [n_blocks, 5120], numpy or torch) in (row-block, col-block) order as a model.q4nx
+    bundle stores them; Q, K, V are fused by concatenating their blocks (whole row-blocks of the output
+    axis), and every matrix is repacked on the GPU once.  Norm weights are bf16 bit patterns or tensors."""
+    E, H = config.emb_dim, config.hidden_dim
+    nq, nkv = config.n_heads * config.head_dim, config.kv_dim
+
+    def dev_blocks(b):
+        t = b if isinstance(b, torch.Tensor) else torch.from_numpy(np.ascontiguousarray(np.asarray(b).view(np.uint8)))
+        return t.to(device).reshape(-1, 5120)
+
+    def dev_vec(a):
+        if isinstance(a, torch.Tensor):
+            return a.to(device)
+        return torch.from_numpy(np.ascontiguousarray(np.asarray(a).view(np.int16))).to(device).view(torch.bfloat16)
+
+    def repack(t, M, K):
+        return ops.q4nx_repack(t.contiguous(), M, K, mode)
+
+    qkv = torch.cat([dev_blocks(blocks[n]) for n in ("q", "k", "v")], dim=0)
+    return DecodeLayer(attn_norm=dev_vec(attn_norm), ffn_norm=dev_vec(ffn_norm),
+                       wqkv=repack(qkv, nq + 2 * nkv, E), wo=repack(dev_blocks(blocks["o"]), E, nq),
+                       w_gate=repack(dev_blocks(blocks["gate"]), H, E), w_up=repack(dev_blocks(blocks["up"]), H, E),
+                       w_down=repack(dev_blocks(blocks["down"]), E, H), codec="q4nx")
 
 
 def prepare_layer(layer: wmod.LayerWeights, device="cuda") -> DecodeLayer:
@@ -66,9 +94,10 @@ def new_kv_cache(config, max_seq, device="cuda"):
 def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer, current_pos, rope_lut):
     """One transformer block for one decode token; x bf16 [emb] -> bf16 [emb].  The caches are
     updated in place at current_pos."""
-    qkv = ops.w4a16_rms_gemv(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps)
+    q4nx = layer.codec == "q4nx"
+    qkv = (ops.q4nx_rms_gemv if q4nx else ops.w4a16_rms_gemv)(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps)
     attn_out = ops.decode_attention(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads)
-    return ops.o_gemv_ffn(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
+    return (ops.q4nx_o_gemv_ffn if q4nx else ops.o_gemv_ffn)(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
 
 
 def decode_token(token_id, layers, embed_table, final_norm, lm_head, config, kv_cache, current_pos, rope_lut):

@@ -292,6 +292,50 @@ def q4nx_gemm(x, qweight, scales, mins, residual=None, out=None):
     return out.squeeze(0) if vec else out
 
 
+def _qptrs(w):
+    """(qweight, scales, mins) of the affine codec as C-ABI pointers."""
+    return [_ptr(w[0]), _ptr(_bits(w[1])), _ptr(_bits(w[2]))]
+
+
+def q4nx_rms_gemv(x, norm_weight, qweight, scales, mins, eps=1e-5):
+    """y[N] = bf16(rms_norm(x, norm_weight) . W) for the operands of q4nx_repack."""
+    lib = _lib.load_library()
+    _need_cuda(x, norm_weight, qweight, scales, mins)
+    K = x.numel()
+    if qweight.shape[0] != K or norm_weight.numel() != K:
+        raise ValueError(f"x has K={K}, qweight {qweight.shape[0]} rows, norm weight {norm_weight.numel()}")
+    N = qweight.shape[1] * 8
+    out = torch.empty((N,), dtype=torch.bfloat16, device=x.device)
+    ws = workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
+    _lib.check(lib.w4a16_q4nx_rms_gemv_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
+                                            *_qptrs((qweight, scales, mins)), _ptr(out), K, N,
+                                            _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def q4nx_o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, return_intermediates=False):
+    """o_gemv_ffn for the affine codec: wo/gate/up/down are (qweight, scales, mins) from q4nx_repack."""
+    lib = _lib.load_library()
+    _need_cuda(attn_out, x_residual, ffn_norm_weight, *wo, *gate, *up, *down)
+    E = attn_out.numel()
+    H = gate[0].shape[1] * 8
+    if (wo[0].shape[0] != E or wo[0].shape[1] * 8 != E or gate[0].shape[0] != E or up[0].shape != gate[0].shape
+            or down[0].shape[0] != H or down[0].shape[1] * 8 != E or x_residual.numel() != E
+            or ffn_norm_weight.numel() != E):
+        raise ValueError("q4nx_o_gemv_ffn: wo must be [E, E/8], gate/up [E, H/8], down [H, E/8], vectors [E]")
+    dev = attn_out.device
+    y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
+    res1 = torch.empty((E,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
+    h = torch.empty((H,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
+    ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev)
+    _lib.check(lib.w4a16_q4nx_o_gemv_ffn_bf16(
+        _ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
+        *_qptrs(wo), *_qptrs(gate), *_qptrs(up), *_qptrs(down), _ptr(y),
+        _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
+        E, H, _ptr(ws), ws.numel(), _stream()))
+    return (y, res1, h) if return_intermediates else y
+
+
 def tune(key, value):
     lib = _lib.load_library()
     _lib.check(lib.w4a16_tune(key.encode(), int(value)))

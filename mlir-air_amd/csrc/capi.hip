@@ -34,6 +34,106 @@ size_t stream_partial_bytes(int M, int N, int nmat) {
     return round256((size_t)nmat * kMaxKSplit * (size_t)(M < 16 ? M : 16) * ((size_t)N + 512) * sizeof(float));
 }
 
+// One quantised matrix in either codec: AWQ (qweight, qzeros, scales [K / 128, N]) or the affine
+// 32-row-group codec of q4nx_repack (qweight, mins, scales [K / 32, N]).
+struct QuantW {
+    const int32_t *qw;
+    const void *aux;   // qzeros int32 or mins bf16
+    const uint16_t *sc;
+};
+
+int check_affine(const QuantW &w, int K, int N) {
+    if (!w.qw || !w.aux || !w.sc) return W4A16_ERR_NULL;
+    if (K <= 0 || N <= 0 || K % kGroup != 0 || N % 32 != 0) return W4A16_ERR_SHAPE;
+    if (misaligned(w.qw) || misaligned(w.aux) || misaligned(w.sc)) return W4A16_ERR_ALIGN;
+    return W4A16_OK;
+}
+
+int check_w(bool affine, const QuantW &w, int K, int N, int group) {
+    return affine ? check_affine(w, K, N) : check_quant(w.qw, w.aux, w.sc, K, N, group, 32);
+}
+
+hipError_t stream_w(bool affine, const uint16_t *x, const QuantW &a, const QuantW *up, uint16_t *y, int M, int K, int N,
+                    void *workspace, hipStream_t st, StreamExtras ex) {
+    if (affine) {
+        ex.mins = static_cast<const uint16_t *>(a.aux);
+        ex.up_mins = up ? static_cast<const uint16_t *>(up->aux) : nullptr;
+        return launch_stream(x, a.qw, nullptr, a.sc, up ? up->qw : nullptr, nullptr, up ? up->sc : nullptr, y, M, K, N,
+                             workspace, st, ex);
+    }
+    return launch_stream(x, a.qw, static_cast<const int32_t *>(a.aux), a.sc, up ? up->qw : nullptr,
+                         up ? static_cast<const int32_t *>(up->aux) : nullptr, up ? up->sc : nullptr, y, M, K, N,
+                         workspace, st, ex);
+}
+
+int rms_gemv_impl(bool affine, const uint16_t *x, const uint16_t *norm_weight, float eps, const QuantW &w, uint16_t *y,
+                  int K, int N, int group, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!x || !y || !norm_weight) return W4A16_ERR_NULL;
+    int rc = check_w(affine, w, K, N, group);
+    if (rc) return rc;
+    if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(y) || misaligned(norm_weight)) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_gemm_workspace_bytes(1, K, N)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    StreamExtras ex;
+    ex.norm_w = norm_weight;
+    ex.eps = eps;
+    hipError_t e = stream_w(affine, x, w, nullptr, y, 1, K, N, workspace, static_cast<hipStream_t>(stream), ex);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                    float eps, const QuantW &wo, const QuantW &wg, const QuantW &wu, const QuantW &wd, uint16_t *y,
+                    uint16_t *res1_out, uint16_t *h_out, int E, int H, int group, void *workspace,
+                    size_t workspace_bytes, void *stream) {
+    if (!attn_out || !x_residual || !ffn_norm_weight || !y) return W4A16_ERR_NULL;
+    int rc = check_w(affine, wo, E, E, group);
+    if (rc) return rc;
+    rc = check_w(affine, wg, E, H, group);
+    if (rc) return rc;
+    rc = check_w(affine, wu, E, H, group);
+    if (rc) return rc;
+    rc = check_w(affine, wd, H, E, group);
+    if (rc) return rc;
+    if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(attn_out) || misaligned(x_residual) || misaligned(ffn_norm_weight) || misaligned(y) ||
+        (res1_out && misaligned(res1_out)) || (h_out && misaligned(h_out)))
+        return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_block_workspace_bytes(E, H)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    char *tail = static_cast<char *>(workspace) + w4a16_block_workspace_bytes(E, H) - 256;
+    float *res1_sumsq = reinterpret_cast<float *>(tail);
+    uint16_t *res1 = res1_out ? res1_out : reinterpret_cast<uint16_t *>(tail - round256((size_t)E * sizeof(uint16_t)));
+    uint16_t *h = h_out ? h_out
+                        : reinterpret_cast<uint16_t *>(tail - round256((size_t)E * sizeof(uint16_t)) -
+                                                       round256((size_t)H * sizeof(uint16_t)));
+    // stage 1: res1 = bf16(attn_out . Wo + x_residual); its reducers also leave sum(res1^2) per column
+    // tile, so that stage 2 does not have to read res1 again for the norm
+    const int res1_tiles = plan_stream(1, E, E, affine).ntiles;
+    const bool chain_norm = res1_tiles <= 64;
+    StreamExtras add;
+    add.residual = x_residual;
+    if (chain_norm) add.sumsq_out = res1_sumsq;
+    hipError_t e = stream_w(affine, attn_out, wo, nullptr, res1, 1, E, E, workspace, st, add);
+    if (e != hipSuccess) return hip_fail(e);
+    // stage 2: h = swiglu(rms_norm(res1) . Wgate, rms_norm(res1) . Wup)
+    StreamExtras rms;
+    rms.norm_w = ffn_norm_weight;
+    rms.eps = eps;
+    if (chain_norm) {
+        rms.sumsq_in = res1_sumsq;
+        rms.sumsq_n = res1_tiles;
+    }
+    e = stream_w(affine, res1, wg, &wu, h, 1, E, H, workspace, st, rms);
+    if (e != hipSuccess) return hip_fail(e);
+    // stage 3: y = bf16(h . Wdown + res1)
+    add.sumsq_out = nullptr;
+    add.residual = res1;
+    e = stream_w(affine, h, wd, nullptr, y, 1, H, E, workspace, st, add);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 }  // namespace
 
 extern "C" {
@@ -191,19 +291,8 @@ int w4a16_gemv_add_bf16(const uint16_t *x, const int32_t *qweight, const int32_t
 int w4a16_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const int32_t *qweight,
                         const int32_t *qzeros, const uint16_t *scales, uint16_t *y, int K, int N, int group,
                         void *workspace, size_t workspace_bytes, void *stream) {
-    if (!x || !y || !norm_weight) return W4A16_ERR_NULL;
-    int rc = check_quant(qweight, qzeros, scales, K, N, group, 32);
-    if (rc) return rc;
-    if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
-    if (misaligned(x) || misaligned(y) || misaligned(norm_weight)) return W4A16_ERR_ALIGN;
-    if (!workspace || workspace_bytes < w4a16_gemm_workspace_bytes(1, K, N)) return W4A16_ERR_WORKSPACE;
-    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
-    StreamExtras ex;
-    ex.norm_w = norm_weight;
-    ex.eps = eps;
-    hipError_t e = launch_stream(x, qweight, qzeros, scales, nullptr, nullptr, nullptr, y, 1, K, N, workspace,
-                                 static_cast<hipStream_t>(stream), ex);
-    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+    return rms_gemv_impl(false, x, norm_weight, eps, QuantW{qweight, qzeros, scales}, y, K, N, group, workspace,
+                         workspace_bytes, stream);
 }
 
 int w4a16_rms_gemv_swiglu_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps,
@@ -243,55 +332,10 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, 
                           const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
                           uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int E, int H, int group, void *workspace,
                           size_t workspace_bytes, void *stream) {
-    if (!attn_out || !x_residual || !ffn_norm_weight || !y) return W4A16_ERR_NULL;
-    int rc = check_quant(o_qweight, o_qzeros, o_scales, E, E, group, 32);
-    if (rc) return rc;
-    rc = check_quant(gate_qweight, gate_qzeros, gate_scales, E, H, group, 32);
-    if (rc) return rc;
-    rc = check_quant(up_qweight, up_qzeros, up_scales, E, H, group, 32);
-    if (rc) return rc;
-    rc = check_quant(down_qweight, down_qzeros, down_scales, H, E, group, 32);
-    if (rc) return rc;
-    if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
-    if (misaligned(attn_out) || misaligned(x_residual) || misaligned(ffn_norm_weight) || misaligned(y) ||
-        (res1_out && misaligned(res1_out)) || (h_out && misaligned(h_out)))
-        return W4A16_ERR_ALIGN;
-    if (!workspace || workspace_bytes < w4a16_block_workspace_bytes(E, H)) return W4A16_ERR_WORKSPACE;
-    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    char *tail = static_cast<char *>(workspace) + w4a16_block_workspace_bytes(E, H) - 256;
-    float *res1_sumsq = reinterpret_cast<float *>(tail);
-    uint16_t *res1 = res1_out ? res1_out : reinterpret_cast<uint16_t *>(tail - round256((size_t)E * sizeof(uint16_t)));
-    uint16_t *h = h_out ? h_out
-                        : reinterpret_cast<uint16_t *>(tail - round256((size_t)E * sizeof(uint16_t)) -
-                                                       round256((size_t)H * sizeof(uint16_t)));
-    // stage 1: res1 = bf16(attn_out . Wo + x_residual); its reducers also leave sum(res1^2) per column
-    // tile, so that stage 2 does not have to read res1 again for the norm
-    const int res1_tiles = plan_stream(1, E, E).ntiles;
-    const bool chain_norm = res1_tiles <= 64;
-    StreamExtras add;
-    add.residual = x_residual;
-    if (chain_norm) add.sumsq_out = res1_sumsq;
-    hipError_t e = launch_stream(attn_out, o_qweight, o_qzeros, o_scales, nullptr, nullptr, nullptr, res1, 1, E, E,
-                                 workspace, st, add);
-    if (e != hipSuccess) return hip_fail(e);
-    // stage 2: h = swiglu(rms_norm(res1) . Wgate, rms_norm(res1) . Wup)
-    StreamExtras rms;
-    rms.norm_w = ffn_norm_weight;
-    rms.eps = eps;
-    if (chain_norm) {
-        rms.sumsq_in = res1_sumsq;
-        rms.sumsq_n = res1_tiles;
-    }
-    add.sumsq_out = nullptr;
-    e = launch_stream(res1, gate_qweight, gate_qzeros, gate_scales, up_qweight, up_qzeros, up_scales, h, 1, E, H,
-                      workspace, st, rms);
-    if (e != hipSuccess) return hip_fail(e);
-    // stage 3: y = bf16(h . Wdown + res1)
-    add.residual = res1;
-    e = launch_stream(h, down_qweight, down_qzeros, down_scales, nullptr, nullptr, nullptr, y, 1, H, E, workspace, st,
-                      add);
-    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+    return o_gemv_ffn_impl(false, attn_out, x_residual, ffn_norm_weight, eps, QuantW{o_qweight, o_qzeros, o_scales},
+                           QuantW{gate_qweight, gate_qzeros, gate_scales}, QuantW{up_qweight, up_qzeros, up_scales},
+                           QuantW{down_qweight, down_qzeros, down_scales}, y, res1_out, h_out, E, H, group, workspace,
+                           workspace_bytes, stream);
 }
 
 size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim) {
@@ -354,6 +398,26 @@ int w4a16_q4nx_gemm_bf16(const uint16_t *x, const int32_t *qweight, const uint16
                           rows, K, N, workspace, static_cast<hipStream_t>(stream), extras);
     }
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_q4nx_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const int32_t *qweight,
+                             const uint16_t *scales, const uint16_t *mins, uint16_t *y, int K, int N, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+    return rms_gemv_impl(true, x, norm_weight, eps, QuantW{qweight, mins, scales}, y, K, N, 32, workspace,
+                         workspace_bytes, stream);
+}
+
+int w4a16_q4nx_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                               float eps, const int32_t *o_qweight, const uint16_t *o_scales, const uint16_t *o_mins,
+                               const int32_t *gate_qweight, const uint16_t *gate_scales, const uint16_t *gate_mins,
+                               const int32_t *up_qweight, const uint16_t *up_scales, const uint16_t *up_mins,
+                               const int32_t *down_qweight, const uint16_t *down_scales, const uint16_t *down_mins,
+                               uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int E, int H, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+    return o_gemv_ffn_impl(true, attn_out, x_residual, ffn_norm_weight, eps, QuantW{o_qweight, o_mins, o_scales},
+                           QuantW{gate_qweight, gate_mins, gate_scales}, QuantW{up_qweight, up_mins, up_scales},
+                           QuantW{down_qweight, down_mins, down_scales}, y, res1_out, h_out, E, H, 32, workspace,
+                           workspace_bytes, stream);
 }
 
 int w4a16_tune(const char *key, int value) {

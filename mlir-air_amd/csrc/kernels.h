@@ -28,7 +28,7 @@ extern StreamTune g_stream_tune;
 struct StreamPlan {
     int lw, ksteps, waves, units, ksplit, ntiles, mi;
 };
-StreamPlan plan_stream(int M, int K, int N);
+StreamPlan plan_stream(int M, int K, int N, bool fixed_shape = false);   // fixed_shape: 256-column tiles, 8 waves, whatever the tune keys say
 
 hipError_t launch_dequant(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, uint16_t *out,
                           int K, int N, hipStream_t stream);
@@ -46,8 +46,9 @@ struct StreamExtras {
     int sumsq_n = 0;
     float *sumsq_out = nullptr;
     // Affine codec with 32-row groups (w = q * s + m): per-group minimum [K / 32, N] bf16.  `scales` is then
-    // [K / 32, N] too and `qzeros` is not read.  Single matrix, no norm_w.
+    // [K / 32, N] too and `qzeros` is not read.  `up_mins` belongs to the second matrix of a SwiGLU launch.
     const uint16_t *mins = nullptr;
+    const uint16_t *up_mins = nullptr;
 };
 
 // y[M, N] = bf16(x[M, K] . W), M <= 16.  With `up_*` given (SwiGLU epilogue, M == 1) the

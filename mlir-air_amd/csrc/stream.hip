@@ -50,7 +50,7 @@ struct StreamParams {
     const uint32_t *qw[2];
     const uint32_t *qz[2];
     const uint16_t *sc[2];
-    const uint16_t *mn;   // affine codec: per-group minimum [K / 32, N] bf16 (qz unused), else null
+    const uint16_t *mn[2];   // affine codec: per-group minimum [K / 32, N] bf16 of each matrix (qz unused), else null
     uint16_t *y;
     uint32_t *header;   // workspace header: word 0 = poll timeouts seen
     float *partial;     // [nmat * ksplit][ntiles][M * tile columns]
@@ -166,7 +166,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     const char *qw_s = reinterpret_cast<const char *>(p.qw[mat]);
     const char *qz_s = reinterpret_cast<const char *>(p.qz[mat]);
     const char *sc_s = reinterpret_cast<const char *>(p.sc[mat]);
-    const char *mn_s = reinterpret_cast<const char *>(p.mn);
+    const char *mn_s = reinterpret_cast<const char *>(p.mn[mat]);
     const uint32_t qw_lane = (uint32_t)(((size_t)chunk_c * LW + (size_t)(8 * lg) * p.nb) * sizeof(uint32_t));
     const uint32_t qz_lane = (uint32_t)((size_t)chunk_c * LW * sizeof(uint32_t));
     const uint32_t sc_lane = (uint32_t)((size_t)chunk_c * LC * sizeof(uint16_t));
@@ -547,7 +547,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 // by 9 %, so the split is only capped at 16 (two polling rounds of the reducer) for M <= 4.
 // For M > 4 the fp32 partials are M times larger and the cap is 4 (M = 16: split 4 16.3 us,
 // split 8 32.6 us, split 2 19.4 us), more units per wave instead.
-StreamPlan plan_stream(int M, int K, int N) {
+StreamPlan plan_stream(int M, int K, int N, bool fixed_shape) {
     StreamPlan pl;
     pl.mi = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     const int nksteps = K / 32;
@@ -555,9 +555,9 @@ StreamPlan plan_stream(int M, int K, int N) {
     pl.ksteps = 4;
     pl.waves = 8;
     pl.units = 1;
-    if (g_stream_tune.lw) pl.lw = g_stream_tune.lw == 1 ? 1 : 2;
+    if (g_stream_tune.lw && !fixed_shape) pl.lw = g_stream_tune.lw == 1 ? 1 : 2;
     if (g_stream_tune.ksteps) pl.ksteps = g_stream_tune.ksteps == 2 ? 2 : 4;
-    if (g_stream_tune.waves) pl.waves = g_stream_tune.waves == 4 ? 4 : 8;
+    if (g_stream_tune.waves && !fixed_shape) pl.waves = g_stream_tune.waves == 4 ? 4 : 8;
     pl.ntiles = (N + 128 * pl.lw - 1) / (128 * pl.lw);
     // Few tiles and a short K (e.g. a 4096 x 4096 projection: 16 tiles, 64 workgroups): halve the
     // unit so that twice as many workgroups share the stream (9.1 us instead of 10.1 us there).
@@ -595,11 +595,19 @@ static hipError_t launch_one(const StreamParams &p, dim3 grid, hipStream_t strea
 
 template <int LW, int WB, int KSTEPS, int WAVES>
 static hipError_t launch_mi(int mi, const StreamParams &p, dim3 grid, hipStream_t stream) {
-    if (p.mn) {   // affine codec: single matrix, no RMSNorm prologue (checked by the caller)
-        switch (mi) {
-            case 1: return launch_one<LW, WB, KSTEPS, WAVES, 1, 1, false, true>(p, grid, stream);
-            case 2: return launch_one<LW, WB, KSTEPS, WAVES, 2, 1, false, true>(p, grid, stream);
-            default: return launch_one<LW, WB, KSTEPS, WAVES, 4, 1, false, true>(p, grid, stream);
+    if (p.mn[0]) {   // affine codec: only the default launch shape is instantiated
+        if constexpr (LW == 2 && WAVES == 8) {
+            if (p.norm_w)   // M <= 4 checked by the caller
+                return p.nmat == 2 ? launch_one<LW, WB, KSTEPS, WAVES, 1, 2, true, true>(p, grid, stream)
+                                   : launch_one<LW, WB, KSTEPS, WAVES, 1, 1, true, true>(p, grid, stream);
+            if (p.nmat == 2) return launch_one<LW, WB, KSTEPS, WAVES, 1, 2, false, true>(p, grid, stream);
+            switch (mi) {
+                case 1: return launch_one<LW, WB, KSTEPS, WAVES, 1, 1, false, true>(p, grid, stream);
+                case 2: return launch_one<LW, WB, KSTEPS, WAVES, 2, 1, false, true>(p, grid, stream);
+                default: return launch_one<LW, WB, KSTEPS, WAVES, 4, 1, false, true>(p, grid, stream);
+            }
+        } else {
+            return hipErrorInvalidValue;
         }
     }
     if (p.norm_w)   // M <= 4 checked by the caller
@@ -627,7 +635,7 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
                          const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
                          uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream,
                          const StreamExtras &extras) {
-    const StreamPlan pl = plan_stream(M, K, N);
+    const StreamPlan pl = plan_stream(M, K, N, extras.mins != nullptr);
     StreamParams p;
     p.x = x;
     p.qw[0] = reinterpret_cast<const uint32_t *>(qweight);
@@ -637,7 +645,8 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.qw[1] = reinterpret_cast<const uint32_t *>(up_qweight ? up_qweight : qweight);
     p.qz[1] = reinterpret_cast<const uint32_t *>(up_qzeros ? up_qzeros : qzeros);
     p.sc[1] = up_scales ? up_scales : scales;
-    p.mn = extras.mins;
+    p.mn[0] = extras.mins;
+    p.mn[1] = extras.up_mins ? extras.up_mins : extras.mins;
     p.y = y;
     p.header = reinterpret_cast<uint32_t *>(workspace);
     p.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + kHeaderBytes);

@@ -20,6 +20,9 @@ Follows (FD = programming_examples/fused_decode, LLM = programming_examples/llms
   dequant_q4_0           LLM/qwen25_3b_q4/qwen25_3b_q4_weights.py:86-95
   gemv_reference         FD/kernels/q4_k.h:39-45 restated exactly: per group
                          c += (sum q b) * scale + min * sum b, in float64
+  rms_gemv_reference, block_staged_reference
+                         the RMSNorm + GEMV and O + FFN block stagings of oracle/reference.py
+                         (rms_norm_bf16, o_gemv_ffn_staged_reference) with gemv_reference as the GEMV
 
 bf16 tensors are uint16 bit patterns.  Pins (tests/test_oracle_q4nx.py): a block written byte
 by byte from the layout comment of proj_qmm_pack.py:4-9, loop packer == vectorised packer,
@@ -183,3 +186,26 @@ def gemv_reference(q, scale_bits, min_bits, x_bits, mode=ADDITIVE):
     dot = np.einsum("mgk,rgk->rmg", qg, xg)                   # sum q x per group
     xsum = xg.sum(2)                                          # [rows, ng]
     return (dot * s[None] + m[None] * xsum[:, None, :]).sum(2)
+
+
+def rms_gemv_reference(w, x_bits, norm_w_bits, eps=1e-5):
+    """bf16 bits [M]: the GEMV on bf16((x * rstd) * norm_w).  w = (q, scale bits, min bits) of W[M, K]."""
+    from . import reference as ref
+    normed = f32_to_bf16_bits(ref.rms_norm_bf16(x_bits, norm_w_bits, eps))
+    return f32_to_bf16_bits(gemv_reference(*w, normed)[0].astype(np.float32))
+
+
+def block_staged_reference(wo, wg, wu, wd, attn_out_bits, x_residual_bits, ffn_norm_w_bits, eps=1e-5):
+    """The O + FFN decode block in the staging of the int4 path (oracle/reference.py
+    o_gemv_ffn_staged_reference), on affine-codec weights: res1 = bf16(attn . Wo + x),
+    h = bf16(silu(bf16(n . Wg)) * bf16(n . Wu)) with n = bf16 RMSNorm of res1, y = bf16(h . Wd + res1).
+    Returns (res1 bits, h bits, y bits)."""
+    from . import reference as ref
+    res1 = f32_to_bf16_bits((gemv_reference(*wo, attn_out_bits)[0]
+                             + bf16_bits_to_f32(x_residual_bits).astype(np.float64)).astype(np.float32))
+    normed = f32_to_bf16_bits(ref.rms_norm_bf16(res1, ffn_norm_w_bits, eps))
+    gate = bf16_bits_to_f32(f32_to_bf16_bits(gemv_reference(*wg, normed)[0].astype(np.float32)))
+    up = bf16_bits_to_f32(f32_to_bf16_bits(gemv_reference(*wu, normed)[0].astype(np.float32)))
+    h = f32_to_bf16_bits(ref.silu_tanh_f32(gate) * up)
+    y = f32_to_bf16_bits((gemv_reference(*wd, h)[0] + bf16_bits_to_f32(res1).astype(np.float64)).astype(np.float32))
+    return res1, h, y

@@ -174,3 +174,118 @@ def test_argument_errors(ops):
     assert lib.q4nx_dequant_bf16(blocks.data_ptr(), blocks.data_ptr(), 48, 256, 0, None) == _lib.ERR_SHAPE
     assert lib.w4a16_q4nx_gemm_bf16(blocks.data_ptr(), blocks.data_ptr(), blocks.data_ptr(), blocks.data_ptr(), None,
                                     blocks.data_ptr(), 1, 128, 32, None, 0, None) == _lib.ERR_WORKSPACE
+
+
+# ---- decode-layer entry points on the affine codec ----
+
+def _norm_w(K, seed):
+    rng = np.random.default_rng(seed)
+    return f32_to_bf16_bits((rng.standard_normal(K) * 0.1 + 1.0).astype(np.float32))
+
+
+def _vec(K, seed):
+    return f32_to_bf16_bits(np.random.default_rng(seed).standard_normal(K).astype(np.float32))
+
+
+def _weights(ops, M, K, seed):
+    """(host (q, s, m), device (qweight, scales, mins)) of one W[M, K]."""
+    w = make(M, K, seed)
+    return w, ops.q4nx_repack(dev(oq.pack_matrix(*w)), M, K, oq.ADDITIVE)
+
+
+@pytest.mark.parametrize("M,K", [(32, 256), (1056, 512), (6144, 4096), (2048, 8192)])
+def test_rms_gemv(ops, M, K):
+    print(f"q4nx rms_gemv M={M} K={K}", flush=True)
+    w, wd = _weights(ops, M, K, seed=M + K)
+    x, nw = _vec(K, 70), _norm_w(K, 71)
+    y = ops.q4nx_rms_gemv(dev(x), dev(nw), *wd)
+    torch.cuda.synchronize()
+    # the kernel's normalised vector can differ from the oracle's by one bf16 ulp in single elements
+    want = oq.rms_gemv_reference(w, x, nw)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(y)), bf16_bits_to_f32(want), rtol=0.1, atol=0.05, min_correlation=0.999)
+    normed = f32_to_bf16_bits(oref.rms_norm_bf16(x, nw))
+    y2 = ops.q4nx_gemm(dev(normed), *wd)     # same GEMV without the prologue, fed the oracle's vector
+    torch.cuda.synchronize()
+    a, b = bf16_bits_to_f32(bits(y)).astype(np.float64), bf16_bits_to_f32(bits(y2)).astype(np.float64)
+    from helpers import bf16_ulp
+    assert np.all(np.abs(a - b) <= 2 * bf16_ulp(b) + 2e-2), np.abs(a - b).max()
+
+
+@pytest.mark.parametrize("E,H", [(256, 512), (2048, 8192), (4096, 14336)])
+def test_o_gemv_ffn_block(ops, E, H):
+    print(f"q4nx o_gemv_ffn E={E} H={H}", flush=True)
+    wo, wo_d = _weights(ops, E, E, seed=E)
+    wg, wg_d = _weights(ops, H, E, seed=E + 1)
+    wu, wu_d = _weights(ops, H, E, seed=E + 2)
+    wd, wd_d = _weights(ops, E, H, seed=E + 3)
+    attn, xres, nw = _vec(E, 80), _vec(E, 81), _norm_w(E, 82)
+    y, res1, h = ops.q4nx_o_gemv_ffn(dev(attn), dev(xres), dev(nw), wo_d, wg_d, wu_d, wd_d, return_intermediates=True)
+    torch.cuda.synchronize()
+    # stage by stage against the float64 oracle, each stage fed the kernel's own previous output
+    want1 = oq.gemv_reference(*wo, attn)[0] + bf16_bits_to_f32(xres)
+    assert_bf16_close(bits(res1), want1, ulps=1.0, atol=2e-3, what="res1")
+    want3 = oq.gemv_reference(*wd, bits(h))[0] + bf16_bits_to_f32(bits(res1))
+    assert_bf16_close(bits(y), want3, ulps=1.0, atol=2e-3, what="block y")
+    normed = f32_to_bf16_bits(oref.rms_norm_bf16(bits(res1), nw))
+    gate = bf16_bits_to_f32(f32_to_bf16_bits(oq.gemv_reference(*wg, normed)[0].astype(np.float32)))
+    up = bf16_bits_to_f32(f32_to_bf16_bits(oq.gemv_reference(*wu, normed)[0].astype(np.float32)))
+    h_want = bf16_bits_to_f32(f32_to_bf16_bits(oref.silu_tanh_f32(gate) * up))
+    assert oref.check_outputs(bf16_bits_to_f32(bits(h)), h_want, rtol=0.15, atol=0.5, min_correlation=0.99)
+    # end to end against the staged oracle under the reference's gates
+    r1, hh, yy = oq.block_staged_reference(wo, wg, wu, wd, attn, xres, nw)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(res1)), bf16_bits_to_f32(r1), rtol=0.1, atol=0.05, min_correlation=0.999)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(h)), bf16_bits_to_f32(hh), rtol=0.15, atol=0.5, min_correlation=0.99)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(y)), bf16_bits_to_f32(yy), rtol=0.2, atol=2.0, min_correlation=0.99)
+    # repeat calls are deterministic and leave the workspace clean
+    y2 = ops.q4nx_o_gemv_ffn(dev(attn), dev(xres), dev(nw), wo_d, wg_d, wu_d, wd_d)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y2), bits(y))
+
+
+def test_decode_block_q4nx_matches_the_oracle_chain(ops):
+    """run_decode_block on a Q4NX layer (fused Q|K|V by block concatenation, RoPE + cache append +
+    attention, O + FFN) against the oracle's pieces chained on the host."""
+    from air_hip import decode, weights
+    from helpers import bf16_ulp
+    from oracle import decode as odec
+
+    cfg = weights.LlamaConfig(n_layers=1, emb_dim=512, n_heads=8, head_dim=64, n_kv_heads=2, hidden_dim=1024, vocab_size=32)
+    E, H, nq, nkv = cfg.emb_dim, cfg.hidden_dim, cfg.n_heads * cfg.head_dim, cfg.kv_dim
+    max_seq = 96
+
+    def qw(M, K, seed):   # small weights: w in about [-0.04, 0.04] so that activations stay O(1)
+        rng = np.random.default_rng(seed)
+        W = (rng.standard_normal((M, K)) * 0.02).astype(np.float32)
+        q, sc, mn = oq.requant_q4k(W)
+        return q, f32_to_bf16_bits(sc), f32_to_bf16_bits(mn)
+
+    w = {"q": qw(nq, E, 1), "k": qw(nkv, E, 2), "v": qw(nkv, E, 3), "o": qw(E, nq, 4),
+         "gate": qw(H, E, 5), "up": qw(H, E, 6), "down": qw(E, H, 7)}
+    attn_norm, ffn_norm = _norm_w(E, 8), _norm_w(E, 9)
+    layer = decode.prepare_layer_q4nx({k: oq.pack_matrix(*v) for k, v in w.items()}, attn_norm, ffn_norm, cfg)
+    assert layer.codec == "q4nx" and layer.wqkv[0].shape == (E, (nq + 2 * nkv) // 8)
+    lut_bits = odec.generate_rope_lut(cfg.head_dim, cfg.rope_base, max_seq)
+    lut = decode.generate_rope_lut(cfg, max_seq)
+    (kc, vc), = decode.new_kv_cache(cfg, max_seq)
+    kc_ref = np.zeros((cfg.n_kv_heads, max_seq, cfg.head_dim), np.uint16)
+    vc_ref = np.zeros_like(kc_ref)
+    for pos in range(5):
+        print(f"q4nx decode block pos={pos}", flush=True)
+        x = _vec(E, 500 + pos)
+        y = decode.run_decode_block(dev(x), layer, cfg, kc, vc, pos, lut)
+        torch.cuda.synchronize()
+        q = oq.rms_gemv_reference(w["q"], x, attn_norm)
+        k = oq.rms_gemv_reference(w["k"], x, attn_norm)
+        v = oq.rms_gemv_reference(w["v"], x, attn_norm)
+        q_r = odec.rope_halfsplit(q.reshape(cfg.n_heads, cfg.head_dim), lut_bits[pos]).reshape(-1)
+        kc_ref[:, pos] = odec.rope_halfsplit(k.reshape(cfg.n_kv_heads, cfg.head_dim), lut_bits[pos])
+        vc_ref[:, pos] = v.reshape(cfg.n_kv_heads, cfg.head_dim)
+        attn = odec.decode_attention_cpu(q_r, kc_ref, vc_ref, pos, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim)
+        _, _, want = oq.block_staged_reference(w["o"], w["gate"], w["up"], w["down"], attn, x, ffn_norm)
+        got_f, want_f = bf16_bits_to_f32(bits(y)), bf16_bits_to_f32(want)
+        assert oref.check_outputs(got_f, want_f, rtol=0.2, atol=2.0, min_correlation=0.99)
+        assert np.max(np.abs(got_f - want_f)) <= 8 * 2.0**-8 * np.max(np.abs(want_f)), np.max(np.abs(got_f - want_f))
+        kd = np.abs(bf16_bits_to_f32(bits(kc)[:, pos]) - bf16_bits_to_f32(kc_ref[:, pos]))
+        assert np.all(kd <= 2 * bf16_ulp(bf16_bits_to_f32(kc_ref[:, pos])) + 2e-2), kd.max()
+        kc[:, pos] = dev(kc_ref[:, pos])
+        vc[:, pos] = dev(vc_ref[:, pos])
