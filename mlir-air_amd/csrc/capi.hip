@@ -29,6 +29,19 @@ int check_quant(const void *qweight, const void *qzeros, const void *scales, int
 
 size_t round256(size_t v) { return (v + 255) & ~size_t(255); }
 
+// Compute units of the current device (cached per device id; 0 if the query fails).
+int current_cus() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (!cached[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 size_t stream_partial_bytes(int M, int N, int nmat) {
     // tiles are at most 512 columns wide; a ragged last tile is stored in full
     return round256((size_t)nmat * kMaxKSplit * (size_t)(M < 16 ? M : 16) * ((size_t)N + 512) * sizeof(float));
@@ -262,6 +275,16 @@ int w4a16_ffn_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const 
     if (!workspace || workspace_bytes < w4a16_ffn_workspace_bytes(K, H)) return W4A16_ERR_WORKSPACE;
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // One persistent kernel when the shape fits it (every workgroup resident at once), else two launches.
+    FfnFusedPlan fpl;
+    if (!g_stream_tune.no_ffn_fused && plan_ffn_fused(K, H, current_cus(), &fpl) &&
+        kHeaderBytes + ffn_fused_scratch_bytes(K, H, fpl) <= w4a16_ffn_workspace_bytes(K, H)) {
+        const int32_t *const qw[3] = {gate_qweight, up_qweight, down_qweight};
+        const int32_t *const qz[3] = {gate_qzeros, up_qzeros, down_qzeros};
+        const uint16_t *const sc[3] = {gate_scales, up_scales, down_scales};
+        hipError_t ef = launch_ffn_fused(fpl, x, qw, qz, sc, nullptr, y, h_out, K, H, workspace, st);
+        return ef == hipSuccess ? W4A16_OK : hip_fail(ef);
+    }
     uint16_t *h = h_out;
     if (!h) h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + w4a16_ffn_workspace_bytes(K, H) -
                                              round256((size_t)H * sizeof(uint16_t)));
@@ -435,6 +458,8 @@ int w4a16_tune(const char *key, int value) {
         g_stream_tune.skip_publish = value ? 1 : 0;
     } else if (!strcmp(key, "gemv_spin_limit")) {
         g_stream_tune.spin_limit = value;
+    } else if (!strcmp(key, "ffn_fused")) {
+        g_stream_tune.no_ffn_fused = value ? 0 : 1;
     } else if (!strcmp(key, "gemm_stream_max_m")) {
         g_stream_tune.stream_max_m = value;
     } else if (!strcmp(key, "gemv_ksplit")) {

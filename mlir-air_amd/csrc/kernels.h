@@ -22,6 +22,7 @@ struct StreamTune {
     int stream_max_m = 0;   // largest M that w4a16_gemm_bf16 gives to the streaming kernel (0 = kStreamMaxM; at least 16)
     int skip_publish = 0; // tests only: producers do not publish, so reducers run into their poll bound
     int spin_limit = 0;   // reducer poll bound (0 = default); tiny values force the timeout path in tests
+    int no_ffn_fused = 0; // 1: w4a16_ffn_swiglu_bf16 always runs its two streaming launches
 };
 extern StreamTune g_stream_tune;
 
@@ -62,6 +63,17 @@ hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const 
                                const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream);
 
 hipError_t launch_fill_workspace(void *ptr, size_t bytes, hipStream_t stream);
+
+// Decode FFN as one persistent kernel (ffn_fused.hip).  plan_ffn_fused returns false for shapes
+// the kernel does not take (the caller then runs the two streaming launches).
+struct FfnFusedPlan {
+    int G, tilesA, splitA, upsA, tilesB, splitB, upsB;
+};
+bool plan_ffn_fused(int E, int H, int cus, FfnFusedPlan *pl);
+size_t ffn_fused_scratch_bytes(int E, int H, const FfnFusedPlan &pl);   // bytes after the workspace header
+hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int32_t *const qw[3], const int32_t *const qz[3],
+                            const uint16_t *const sc[3], const uint16_t *residual, uint16_t *y, uint16_t *h_out, int E, int H,
+                            void *workspace, hipStream_t stream);
 
 // Q4NX / Q4_0 block codec (q4nx.hip).  mode: 0 w = s q + m, 1 w = s (q - m), 2 signed q, w = s q.
 hipError_t launch_q4nx_dequant(const void *blocks, uint16_t *out, int M, int K, int mode, hipStream_t stream);

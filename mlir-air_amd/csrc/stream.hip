@@ -40,6 +40,7 @@
 // and reports a timeout through the workspace header instead of hanging.
 #include "common.h"
 #include "kernels.h"
+#include "slots.h"
 
 namespace w4a16 {
 
@@ -72,34 +73,7 @@ struct StreamParams {
     int skip_publish;   // fault injection for tests: producers keep their partials to themselves
 };
 
-constexpr uint32_t kEmpty = 0xFFFFFFFFu;
-#ifndef POLL_SLEEP
-#define POLL_SLEEP 1   // s_sleep units of 64 cycles between issuing the two polling rounds (0..2 measure the same, 8 and 16 slower)
-#endif
-
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-// 16-byte slot access as two 8-byte atomics.
-#ifndef SLOT_ST_SCOPE
-#define SLOT_ST_SCOPE __HIP_MEMORY_SCOPE_AGENT
-#endif
-#ifndef SLOT_LD_SCOPE
-#define SLOT_LD_SCOPE __HIP_MEMORY_SCOPE_AGENT
-#endif
-__device__ __forceinline__ void slot_store(float *p, u32x4 v) {
-    uint64_t *q = reinterpret_cast<uint64_t *>(p);
-    __hip_atomic_store(q, (uint64_t)v[0] | ((uint64_t)v[1] << 32), __ATOMIC_RELAXED, SLOT_ST_SCOPE);
-    __hip_atomic_store(q + 1, (uint64_t)v[2] | ((uint64_t)v[3] << 32), __ATOMIC_RELAXED, SLOT_ST_SCOPE);
-}
-__device__ __forceinline__ u32x4 slot_load(const float *p) {
-    const uint64_t *q = reinterpret_cast<const uint64_t *>(p);
-    const uint64_t a = __hip_atomic_load(q, __ATOMIC_RELAXED, SLOT_LD_SCOPE);
-    const uint64_t b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, SLOT_LD_SCOPE);
-    return u32x4{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
-}
-__device__ __forceinline__ bool slot_full(u32x4 v) {
-    return v[0] != kEmpty && v[1] != kEmpty && v[2] != kEmpty && v[3] != kEmpty;
-}
 
 // a0 += sum of squares of the low bf16 halves of v, a1 += of the high halves
 __device__ __forceinline__ void sumsq8(const u32x4 v, float &a0, float &a1) {
@@ -111,8 +85,6 @@ __device__ __forceinline__ void sumsq8(const u32x4 v, float &a0, float &a1) {
         a1 = fmaf(hi, hi, a1);
     }
 }
-
-__device__ __forceinline__ float silu_tanh(float g) { return g * 0.5f * (tanhf(g * 0.5f) + 1.0f); }
 
 template <int LW>
 struct Words;
