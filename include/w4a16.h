@@ -288,9 +288,8 @@ int w4a16_q4nx_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_resid
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic),
  * "gemm_stream_max_m" (largest M given to the streaming kernel, 0 = default 96, otherwise >= 16) and
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the
- * timeout test: split-K producers do not publish), "ffn_fused" (0 = default: w4a16_ffn_swiglu_bf16
- * runs two launches; 1 = one persistent kernel where the shape allows - experimental, it is faster
- * but about one call in a thousand returns wrong values, see csrc/ffn_fused.hip).  Process-wide.
+ * timeout test: split-K producers do not publish), "ffn_fused" (1 = default: w4a16_ffn_swiglu_bf16
+ * runs as one persistent kernel when the shape allows, 0 = always two launches).  Process-wide.
  */
 int w4a16_tune(const char *key, int value);
 

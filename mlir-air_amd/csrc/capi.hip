@@ -275,9 +275,9 @@ int w4a16_ffn_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const 
     if (!workspace || workspace_bytes < w4a16_ffn_workspace_bytes(K, H)) return W4A16_ERR_WORKSPACE;
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // One persistent kernel when asked for (tune key "ffn_fused") and the shape fits it, else two launches.
+    // One persistent kernel when the shape fits it (every workgroup resident at once), else two launches.
     FfnFusedPlan fpl;
-    if (g_stream_tune.ffn_fused && plan_ffn_fused(K, H, current_cus(), &fpl) &&
+    if (!g_stream_tune.no_ffn_fused && plan_ffn_fused(K, H, current_cus(), &fpl) &&
         kHeaderBytes + ffn_fused_scratch_bytes(K, H, fpl) <= w4a16_ffn_workspace_bytes(K, H)) {
         const int32_t *const qw[3] = {gate_qweight, up_qweight, down_qweight};
         const int32_t *const qz[3] = {gate_qzeros, up_qzeros, down_qzeros};
@@ -459,7 +459,7 @@ int w4a16_tune(const char *key, int value) {
     } else if (!strcmp(key, "gemv_spin_limit")) {
         g_stream_tune.spin_limit = value;
     } else if (!strcmp(key, "ffn_fused")) {
-        g_stream_tune.ffn_fused = value ? 1 : 0;
+        g_stream_tune.no_ffn_fused = value ? 0 : 1;
     } else if (!strcmp(key, "gemm_stream_max_m")) {
         g_stream_tune.stream_max_m = value;
     } else if (!strcmp(key, "gemv_ksplit")) {

@@ -25,13 +25,6 @@
 // clean again when the kernel ends.  Waits are bounded (spin_limit) and report through the
 // workspace header instead of hanging.
 //
-// STATE: switched off by default (tune key "ffn_fused").  Bit-identical to the two-launch path in
-// most calls and 14 % faster (K = 4096, H = 14336: 27.6 us against 32.1 us), but about one call in
-// a thousand returns wrong values in h: the low halves of the packed words (even columns) of 8 or
-// 16 neighbouring quads of one tile.  Variants of the kernel that put global loads in flight at
-// other points fail more often (up to every second call); the streaming kernel, with the same slot
-// protocol, is clean over 18000 launches.  The cause has not been found.
-//
 // Progress: producers never wait before they publish; gate/up reducers wait only for producers;
 // down units wait only for gate/up reducers; down reducers wait only for down producers.  All G
 // workgroups must be able to become resident (G <= number of CUs, checked by the host), so two
@@ -164,17 +157,28 @@ __device__ __forceinline__ u32x4 keep_sentinel_unique(floatx4 v) {
 
 // Adds the `n` slots base + j * stride (j < split into sum0, the rest into sum1) once they are all
 // filled, then empties them.  Two polling rounds in flight.  Returns false after spin_limit rounds.
+// Every round issues the same eight slot loads whatever n is (slots past the end re-read the last
+// one and are masked out of the test and the sum), so that the number of loads in flight at each
+// wait is fixed; with loads skipped by branches, stale registers were sporadically accepted as
+// filled slots (about one call in a thousand).
 __device__ __forceinline__ bool gather(float *base, size_t stride, int n, int split, floatx4 &sum0, floatx4 &sum1,
                                        int spin_limit) {
     bool all_ok = true;
     for (int s0 = 0; s0 < n; s0 += 8) {
         u32x4 va[8], vb[8];
-#define FFN_ISSUE(dst) _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < n) dst[j] = slot_load(base + (s0 + j) * stride)
-#define FFN_FULL(src, ok) ok = true; _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < n) ok = ok && slot_full(src[j])
-#define FFN_TAKE(src)                                                        \
-    _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < n) {          \
-        if (s0 + j >= split) sum1 += __builtin_bit_cast(floatx4, src[j]);    \
-        else sum0 += __builtin_bit_cast(floatx4, src[j]);                    \
+        const float *addr[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) addr[j] = base + (size_t)(s0 + j < n ? s0 + j : n - 1) * stride;
+#define FFN_ISSUE(dst) _Pragma("unroll") for (int j = 0; j < 8; ++j) dst[j] = slot_load(addr[j])
+#define FFN_FULL(src, ok) ok = true; _Pragma("unroll") for (int j = 0; j < 8; ++j) ok = ok && slot_full(src[j])
+#define FFN_TAKE(src)                                                                         \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                           \
+        const floatx4 v = __builtin_bit_cast(floatx4, src[j]);                                \
+        const bool live = s0 + j < n, second = s0 + j >= split;                               \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                       \
+            sum0[q] += live && !second ? v[q] : 0.f;                                          \
+            sum1[q] += live && second ? v[q] : 0.f;                                           \
+        }                                                                                     \
     }
         FFN_ISSUE(va);
         int spins = 0;
@@ -201,7 +205,7 @@ __device__ __forceinline__ bool gather(float *base, size_t stride, int n, int sp
         all_ok = all_ok && ok;
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            if (s0 + j < n) slot_store(base + (s0 + j) * stride, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
+            if (s0 + j < n) slot_store(base + (size_t)(s0 + j) * stride, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
     }
     return all_ok;
 }

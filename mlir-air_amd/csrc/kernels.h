@@ -22,7 +22,7 @@ struct StreamTune {
     int stream_max_m = 0;   // largest M that w4a16_gemm_bf16 gives to the streaming kernel (0 = kStreamMaxM; at least 16)
     int skip_publish = 0; // tests only: producers do not publish, so reducers run into their poll bound
     int spin_limit = 0;   // reducer poll bound (0 = default); tiny values force the timeout path in tests
-    int ffn_fused = 0;    // 1: w4a16_ffn_swiglu_bf16 runs the single persistent kernel where the shape fits (off: see ffn_fused.hip)
+    int no_ffn_fused = 0; // 1: w4a16_ffn_swiglu_bf16 always runs its two streaming launches
 };
 extern StreamTune g_stream_tune;
 

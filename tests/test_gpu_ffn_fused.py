@@ -2,9 +2,10 @@
 
 Both run the same arithmetic in the same order (per-wave units, LDS combine, partials added in
 slice order), so h and y must agree bit for bit; the two-launch path itself is checked against the
-oracle in test_gpu_parity.py.  Repeated calls catch races in the cross-workgroup protocol (a lost
-LDS read showed up in about one call in two while the kernel was being written), the workspace
-must be left clean, and the kernel must replay from a HIP graph.
+oracle in test_gpu_parity.py.  Repeated calls catch races in the cross-workgroup protocol (while the
+kernel was being written, a reducer sporadically accepted stale registers as filled slots: from
+one call in two down to one in a thousand, depending on the variant), the workspace must be left
+clean, and the kernel must replay from a HIP graph.
 """
 import numpy as np
 import pytest
@@ -12,9 +13,7 @@ import torch
 
 from helpers import make_awq, make_x
 
-pytestmark = [pytest.mark.gpu,
-              pytest.mark.skip(reason="the single-kernel FFN is switched off by default: about one call in a thousand "
-                                      "still returns wrong values (a 20000-call run found 30 bad calls); cause not found yet")]
+pytestmark = pytest.mark.gpu
 
 
 def dev(a):
@@ -32,7 +31,7 @@ def bits(t):
 def ops():
     from air_hip import ops
     yield ops
-    ops.tune("ffn_fused", 0)
+    ops.tune("ffn_fused", 1)
 
 
 def _weights(K, H, seed):
@@ -68,7 +67,7 @@ def test_fused_repeated_calls_stay_bit_exact_and_leave_the_workspace_clean(ops):
     (y0, h0), _ = _both(ops, x, g, u, d)
     y0t, h0t = dev(y0), dev(h0)
     bad = torch.zeros((), dtype=torch.int64, device="cuda")
-    for _ in range(200):
+    for _ in range(5000):
         y, h = ops.ffn_swiglu(x, g, u, d, return_h=True)
         bad += (y.view(torch.int16) != y0t.view(torch.int16)).sum() + (h.view(torch.int16) != h0t.view(torch.int16)).sum()
     y = ops.ffn_swiglu(x, g, u, d)          # h kept inside the kernel
