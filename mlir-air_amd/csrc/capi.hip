@@ -130,6 +130,20 @@ int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_res
     if (chain_norm) add.sumsq_out = res1_sumsq;
     hipError_t e = stream_w(affine, attn_out, wo, nullptr, res1, 1, E, E, workspace, st, add);
     if (e != hipSuccess) return hip_fail(e);
+    // stages 2 and 3 as one persistent kernel when the shape fits it (AWQ codec): h = swiglu(rms_norm(res1) . Wgate,
+    // rms_norm(res1) . Wup), y = bf16(h . Wdown + res1)
+    FfnFusedPlan fpl;
+    if (!affine && chain_norm && !g_stream_tune.no_ffn_fused && plan_ffn_fused(E, H, current_cus(), &fpl) &&
+        kHeaderBytes + ffn_fused_scratch_bytes(E, H, fpl) + 256 + round256((size_t)E * sizeof(uint16_t)) +
+                round256((size_t)H * sizeof(uint16_t)) <= w4a16_block_workspace_bytes(E, H)) {
+        const int32_t *const qw[3] = {wg.qw, wu.qw, wd.qw};
+        const int32_t *const qz[3] = {static_cast<const int32_t *>(wg.aux), static_cast<const int32_t *>(wu.aux),
+                                      static_cast<const int32_t *>(wd.aux)};
+        const uint16_t *const sc[3] = {wg.sc, wu.sc, wd.sc};
+        const FfnFusedNorm norm = {ffn_norm_weight, res1_sumsq, res1_tiles, eps};
+        e = launch_ffn_fused(fpl, res1, qw, qz, sc, res1, y, h_out, E, H, workspace, st, &norm);
+        return e == hipSuccess ? W4A16_OK : hip_fail(e);
+    }
     // stage 2: h = swiglu(rms_norm(res1) . Wgate, rms_norm(res1) . Wup)
     StreamExtras rms;
     rms.norm_w = ffn_norm_weight;

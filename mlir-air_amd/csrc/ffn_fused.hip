@@ -43,6 +43,10 @@ struct FfnParams {
     const uint32_t *qz[3];
     const uint16_t *sc[3];
     const uint16_t *residual;   // [E] added to y, or null
+    const uint16_t *norm_w;     // RMS kernels: [E] bf16, x is replaced by bf16((x * rstd) * norm_w)
+    const float *sumsq_in;      // RMS kernels: partial sums of x^2 left by the kernel that produced x (<= 64)
+    int sumsq_n;
+    float eps;
     uint16_t *y;                // [E]
     uint16_t *h_out;            // [H] or null
     uint32_t *header;
@@ -210,6 +214,10 @@ __device__ __forceinline__ bool gather(float *base, size_t stride, int n, int sp
     return all_ok;
 }
 
+// RMS: x is RMS-normalised on the fly, as in the streaming kernel's prologue for M = 1 (the sum of
+// squares comes from the launch that produced x; the norm weights are requested ahead of the packed
+// weights because one wave's loads return in order).
+template <bool RMS>
 __global__ void __launch_bounds__(512, 2) ffn_fused_kernel(const FfnParams p) {
     // gate slots [8][256], up slots [8][256], down slots [8][256]
     extern __shared__ __attribute__((aligned(16))) float red[];
@@ -232,7 +240,15 @@ __global__ void __launch_bounds__(512, 2) ffn_fused_kernel(const FfnParams p) {
     // ---- gate and up units: everything requested up front ----
     UnitRegs r0, r1;
     u32x4 av[4];
+    u32x4 nw[RMS ? 4 : 1];
+    float piece = 0.f;
     if (hasA) {
+        if constexpr (RMS) {
+            piece = lane < p.sumsq_n ? p.sumsq_in[lane] : 0.f;
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                nw[s] = *reinterpret_cast<const u32x4 *>(p.norm_w + (size_t)unitA * 128 + s * 32 + 8 * lg);
+        }
 #pragma unroll
         for (int s = 0; s < 4; ++s)
             av[s] = *reinterpret_cast<const u32x4 *>(p.x + (size_t)unitA * 128 + s * 32 + 8 * lg);
@@ -244,6 +260,23 @@ __global__ void __launch_bounds__(512, 2) ffn_fused_kernel(const FfnParams p) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) yg[j] = yu[j] = yd[j] = 0.f;
     if (hasA) {
+        if constexpr (RMS) {
+            float a = piece;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off);
+            const float rstd = 1.0f / sqrtf(a / (float)p.E + p.eps);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float x_lo = __builtin_bit_cast(float, av[s][j] << 16);
+                    const float x_hi = __builtin_bit_cast(float, av[s][j] & 0xFFFF0000u);
+                    const float w_lo = __builtin_bit_cast(float, nw[s][j] << 16);
+                    const float w_hi = __builtin_bit_cast(float, nw[s][j] & 0xFFFF0000u);
+                    av[s][j] = pack_bf16x2((x_lo * rstd) * w_lo, (x_hi * rstd) * w_hi);
+                }
+            }
+        }
 #pragma unroll
         for (int s = 0; s < 4; ++s)
             if (!a_valid) av[s] = u32x4{0u, 0u, 0u, 0u};
@@ -397,7 +430,7 @@ size_t ffn_fused_scratch_bytes(int E, int H, const FfnFusedPlan &pl) {
 
 hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int32_t *const qw[3], const int32_t *const qz[3],
                             const uint16_t *const sc[3], const uint16_t *residual, uint16_t *y, uint16_t *h_out, int E, int H,
-                            void *workspace, hipStream_t stream) {
+                            void *workspace, hipStream_t stream, const FfnFusedNorm *norm) {
     FfnParams p;
     p.x = x;
     for (int i = 0; i < 3; ++i) {
@@ -406,6 +439,10 @@ hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int
         p.sc[i] = sc[i];
     }
     p.residual = residual;
+    p.norm_w = norm ? norm->norm_w : nullptr;
+    p.sumsq_in = norm ? norm->sumsq_in : nullptr;
+    p.sumsq_n = norm ? norm->sumsq_n : 0;
+    p.eps = norm ? norm->eps : 0.f;
     p.y = y;
     p.h_out = h_out;
     p.header = reinterpret_cast<uint32_t *>(workspace);
@@ -424,7 +461,10 @@ hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int
     p.splitB = pl.splitB;
     p.upsB = pl.upsB;
     p.spin_limit = g_stream_tune.spin_limit > 0 ? g_stream_tune.spin_limit : (1 << 18);
-    hipLaunchKernelGGL(ffn_fused_kernel, dim3(pl.G), dim3(512), 3 * 8 * 256 * sizeof(float), stream, p);
+    if (norm)
+        hipLaunchKernelGGL(ffn_fused_kernel<true>, dim3(pl.G), dim3(512), 3 * 8 * 256 * sizeof(float), stream, p);
+    else
+        hipLaunchKernelGGL(ffn_fused_kernel<false>, dim3(pl.G), dim3(512), 3 * 8 * 256 * sizeof(float), stream, p);
     return hipGetLastError();
 }
 

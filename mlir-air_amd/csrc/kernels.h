@@ -71,9 +71,17 @@ struct FfnFusedPlan {
 };
 bool plan_ffn_fused(int E, int H, int cus, FfnFusedPlan *pl);
 size_t ffn_fused_scratch_bytes(int E, int H, const FfnFusedPlan &pl);   // bytes after the workspace header
+// RMSNorm prologue of the fused kernel: x is the output of a launch that left sum(x^2) in `sumsq_in`
+// (`sumsq_n` <= 64 pieces, StreamExtras::sumsq_out).
+struct FfnFusedNorm {
+    const uint16_t *norm_w;
+    const float *sumsq_in;
+    int sumsq_n;
+    float eps;
+};
 hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int32_t *const qw[3], const int32_t *const qz[3],
                             const uint16_t *const sc[3], const uint16_t *residual, uint16_t *y, uint16_t *h_out, int E, int H,
-                            void *workspace, hipStream_t stream);
+                            void *workspace, hipStream_t stream, const FfnFusedNorm *norm = nullptr);
 
 // Q4NX / Q4_0 block codec (q4nx.hip).  mode: 0 w = s q + m, 1 w = s (q - m), 2 signed q, w = s q.
 hipError_t launch_q4nx_dequant(const void *blocks, uint16_t *out, int M, int K, int mode, hipStream_t stream);
