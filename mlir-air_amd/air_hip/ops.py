@@ -38,10 +38,12 @@ def _bits(t):
     raise TypeError(f"expected a bf16 tensor (or its int16 bits), got {t.dtype}")
 
 
-def workspace(nbytes, device):
-    """Cleared workspace per (device, stream), grown on demand."""
+def workspace(nbytes, device, use="gemm"):
+    """Cleared workspace per (device, stream, use), grown on demand.  `use` names the entry point and
+    shape: the FFN and block entry points keep plain intermediates (h, res1) behind their slot area,
+    so a buffer is only shared between calls that lay it out the same way."""
     lib = _lib.load_library()
-    key = (device.index, _stream())
+    key = (device.index, _stream(), use)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
@@ -106,7 +108,7 @@ def w4a16_swiglu(x, gate, up, group=GROUP):
     if gate[0].shape[0] != K or up[0].shape != gate[0].shape:
         raise ValueError("w4a16_swiglu: gate and up must both be [K, H/8]")
     h = torch.empty((H,), dtype=torch.bfloat16, device=x.device)
-    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device)
+    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device, ("ffn", K, H))
     _lib.check(lib.w4a16_gemv_swiglu_bf16(
         _ptr(_bits(x)), _ptr(gate[0]), _ptr(gate[1]), _ptr(_bits(gate[2])),
         _ptr(up[0]), _ptr(up[1]), _ptr(_bits(up[2])), _ptr(h), K, H, group, _ptr(ws), ws.numel(), _stream()))
@@ -123,7 +125,7 @@ def ffn_swiglu(x, gate, up, down, group=GROUP, return_h=False):
         raise ValueError("ffn_swiglu: gate/up must be [K, H/8] and down [H, K/8]")
     y = torch.empty((K,), dtype=torch.bfloat16, device=x.device)
     h = torch.empty((H,), dtype=torch.bfloat16, device=x.device) if return_h else None
-    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device)
+    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device, ("ffn", K, H))
     _lib.check(lib.w4a16_ffn_swiglu_bf16(
         _ptr(_bits(x)),
         _ptr(gate[0]), _ptr(gate[1]), _ptr(_bits(gate[2])),
@@ -180,7 +182,7 @@ def w4a16_rms_swiglu(x, norm_weight, gate, up, eps=1e-5, group=GROUP):
     if gate[0].shape[0] != K or up[0].shape != gate[0].shape or norm_weight.numel() != K:
         raise ValueError("w4a16_rms_swiglu: gate and up must both be [K, H/8], norm_weight [K]")
     h = torch.empty((H,), dtype=torch.bfloat16, device=x.device)
-    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device)
+    ws = workspace(lib.w4a16_ffn_workspace_bytes(K, H), x.device, ("ffn", K, H))
     _lib.check(lib.w4a16_rms_gemv_swiglu_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
                                               *_wptrs(gate), *_wptrs(up), _ptr(h), K, H, group,
                                               _ptr(ws), ws.numel(), _stream()))
@@ -205,7 +207,7 @@ def o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e
     y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
     res1 = torch.empty((E,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
     h = torch.empty((H,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
-    ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev)
+    ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev, ("block", E, H))
     _lib.check(lib.w4a16_o_gemv_ffn_bf16(
         _ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
         *_wptrs(wo), *_wptrs(gate), *_wptrs(up), *_wptrs(down), _ptr(y),
@@ -327,7 +329,7 @@ def q4nx_o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, e
     y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
     res1 = torch.empty((E,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
     h = torch.empty((H,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
-    ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev)
+    ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev, ("block", E, H))
     _lib.check(lib.w4a16_q4nx_o_gemv_ffn_bf16(
         _ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
         *_qptrs(wo), *_qptrs(gate), *_qptrs(up), *_qptrs(down), _ptr(y),
