@@ -67,7 +67,13 @@ int awq_dequant_bf16(const int32_t *qweight, const int32_t *qzeros, const uint16
  * `*_workspace_bytes` bytes of device memory once, prepares it once with
  * w4a16_workspace_init, and may then reuse it for any number of calls that do not
  * overlap in time (each call leaves it prepared again).  Calls that run concurrently
- * (different streams) need separate workspaces.
+ * (different streams) need separate workspaces.  The FFN and block entry points keep plain
+ * intermediates (h, res1) behind the prepared area, at an offset that depends on their shapes: share
+ * a workspace only between calls of one entry point with the same shapes, or prepare it again
+ * before a call of another kind.  w4a16_ffn_swiglu_bf16 and w4a16_o_gemv_ffn_bf16 run a persistent
+ * kernel whose workgroups wait for one another; two such calls running at the same time on one
+ * GPU can starve each other into the timeout path (w4a16_workspace_check), so keep them on one stream
+ * or switch the kernel off with w4a16_tune("ffn_fused", 0).
  */
 size_t w4a16_gemm_workspace_bytes(int M, int K, int N);
 size_t w4a16_ffn_workspace_bytes(int K, int H);
