@@ -47,7 +47,7 @@ LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 204
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
 # scaled by the same counter's reading for a 256 MiB device copy: x2.000 and x1.000); the
 # summaries under profiles/ hold the commands and the raw readings.
-MEASURED_TRAFFIC_BYTES = {"gemv": 24.53e6, "prefill": 342.2e6}
+MEASURED_TRAFFIC_BYTES = {"gemv": 24.53e6, "prefill": 342.2e6, "ffn": 97.07e6}
 
 
 def weight_bytes(K, N):
@@ -391,7 +391,7 @@ def main():
         roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": value / HBM_PEAK_GBS, "traffic": None}
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
-    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel"}.get(name, "stream_kernel")
+    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel", "ffn": "ffn_fused_kernel"}.get(name, "stream_kernel")
     roof["algorithmic_per_launch"] = main_res["flops"] if name == "prefill" else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]
 
