@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -41,6 +41,8 @@ CONFIGS = {
     # projection shape of Llama-3.1-8B (programming_examples/llms/llama31_8b_q4nx)
     "q4nx_gemv": dict(M=1, K=4096, N=14336, cfg=None, desc="decode GEMV Q4NX M=1 K=4096 N=14336 g32"),
     "q4nx_gemm16": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM Q4NX M=16 K=4096 N=14336 g32"),
+    # the tail of a decode step of Llama-3.2-1B: final RMSNorm + bf16 lm_head GEMV + argmax
+    "lm_head": dict(M=1, K=2048, N=128256, cfg=None, desc="decode tail RMSNorm + bf16 lm_head GEMV + argmax E=2048 V=128256"),
 }
 LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 2048
 
@@ -63,6 +65,8 @@ def algorithmic_bytes(name):
     M, K, N = c["M"], c["K"], c["N"]
     if name.startswith("q4nx"):
         return q4nx_weight_bytes(K, N) + M * K * 2 + M * N * 2
+    if name == "lm_head":   # weights, x and norm weight in, logits out
+        return K * N * 2 + 2 * K * 2 + N * 2
     if name == "dequant":
         return weight_bytes(K, N) + K * N * 2
     if name == "ffn":
@@ -117,7 +121,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     stream = torch.cuda.Stream()
 
     q4nx = name.startswith("q4nx")
-    per_copy = q4nx_weight_bytes(K, N) if q4nx else weight_bytes(K, N) * (3 if name in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if name in ("block", "layer") else 0)
+    lm_head = name == "lm_head"
+    per_copy = K * N * 2 if lm_head else q4nx_weight_bytes(K, N) if q4nx else weight_bytes(K, N) * (3 if name in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if name in ("block", "layer") else 0)
     nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
     if name == "layer":
         per_copy += weight_bytes(K, nqkv)
@@ -136,6 +141,10 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             copies.append(c4 + ((make_weights(torch, K, nqkv, 104 + 5 * i),) if name == "layer" else ()))
         elif q4nx:
             copies.append(make_q4nx_weights(torch, K, N, 100 + i))
+        elif lm_head:
+            gw = torch.Generator(device="cuda")
+            gw.manual_seed(100 + i)
+            copies.append(((torch.randn((N, K), device="cuda", generator=gw) * 0.05).to(torch.bfloat16),))
         else:
             copies.append(make_weights(torch, K, N, 100 + i))
     gx = torch.Generator(device="cuda")
@@ -147,7 +156,11 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         outs = [torch.empty((K,), dtype=torch.bfloat16, device=dev)]
     else:
         outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev)]
-    if name in ("block", "layer"):
+    if lm_head:
+        outs = [torch.empty((N,), dtype=torch.bfloat16, device=dev)]
+        best = torch.empty((1,), dtype=torch.int32, device=dev)
+        lm_ws = torch.empty(int(lib.lm_head_workspace_bytes(N)), dtype=torch.uint8, device=dev)
+    if name in ("block", "layer", "lm_head"):
         x_residual = torch.randn((K,), device="cuda", generator=gx).to(torch.bfloat16)
         norm_w = (torch.randn((K,), device="cuda", generator=gx) * 0.1 + 1.0).to(torch.bfloat16)
     if name == "layer":
@@ -195,6 +208,9 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                 a_in = attn_out
             rc = lib.w4a16_o_gemv_ffn_bf16(a_in.data_ptr(), x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, *ptrs,
                                            outs[0].data_ptr(), None, None, K, N, 128, ws.data_ptr(), ws.numel(), st)
+        elif lm_head:
+            rc = lib.lm_head_gemv_bf16(x.data_ptr(), norm_w.data_ptr(), 1e-5, w[0].data_ptr(), outs[0].data_ptr(),
+                                       best.data_ptr(), N, K, lm_ws.data_ptr(), lm_ws.numel(), st)
         elif q4nx:
             rc = lib.w4a16_q4nx_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), None,
                                           outs[0].data_ptr(), M, K, N, ws.data_ptr(), ws.numel(), st)
@@ -256,7 +272,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                  "avg": sum(per_launch) / len(per_launch), "max": per_launch[-1]},
     }
 
-    if with_cpu_baseline and name not in ("block", "layer") and not q4nx:
+    if with_cpu_baseline and name not in ("block", "layer", "lm_head") and not q4nx:
         res["cpu_baseline"] = cpu_baseline(name, torch, copies[0], x, outs, launch, stream)
     return res
 
@@ -391,7 +407,7 @@ def main():
         roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": value / HBM_PEAK_GBS, "traffic": None}
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
-    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel", "ffn": "ffn_fused_kernel"}.get(name, "stream_kernel")
+    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel", "ffn": "ffn_fused_kernel", "lm_head": "lm_head_kernel"}.get(name, "stream_kernel")
     roof["algorithmic_per_launch"] = main_res["flops"] if name == "prefill" else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]
 
@@ -406,8 +422,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int4 weights, bf16 activations, fp32 accumulate",
-        "data": "synthetic (uniform uint4 q/z, scales |N(0,1)|*0.02+1e-3, x ~ N(0,1)), random weights",
+        "dtype": "bf16 weights and activations, fp32 accumulate" if name == "lm_head" else "int4 weights, bf16 activations, fp32 accumulate",
+        "data": "synthetic (W ~ N(0,1)*0.05 as bf16, x ~ N(0,1))" if name == "lm_head" else "synthetic (uniform uint4 q/z, scales |N(0,1)|*0.02+1e-3, x ~ N(0,1)), random weights",
         "config": {"workload": CONFIGS[name]["desc"], "group": 32 if name.startswith("q4nx") else 128,
                    "weight_copies_rotated": main_res["ncopies"], "timing": "HIP graph of K launches, events on the launch stream"},
         "roofline": roof,

@@ -220,6 +220,23 @@ int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_ro
                                 void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Tail of a decode step: final RMSNorm, bf16 lm_head GEMV and argmax in one call
+ * (run_npu_decode_step, programming_examples/llms/llama32_1b_int4/llama32_1b_int4_inference.py:459-486:
+ * host rms_norm, the `lm_head_gemv` kernel over 8 vocabulary partitions, np.argmax).
+ *   normed = bf16((x / sqrt(mean(x^2) + eps)) * norm_weight)     fp32 arithmetic (rms_norm,
+ *            programming_examples/llms/llama32_1b/llama32_1b_cpu_helpers.py:25-39); norm_weight NULL: normed = x
+ *   logits[v] = bf16(sum_e lm_head[v, e] * normed[e])             lm_head bf16 [V, E] row-major, fp32 accumulation
+ *   *argmax_out = lowest v with the largest logit                 (may be NULL; a NaN logit counts as the largest if positive)
+ * x bf16 [E], logits bf16 [V] (every V >= 1; the reference pads the vocabulary to 8 x 16384 rows
+ * instead).  E % 8 == 0, E <= 8192.  The workspace is plain scratch
+ * (no initialisation), lm_head_workspace_bytes(V).
+ */
+size_t lm_head_workspace_bytes(int V);
+int lm_head_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const uint16_t *lm_head,
+                      uint16_t *logits, int32_t *argmax_out, int V, int E,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Q4NX / Q4_0 block codec (the 4-bit formats of the fused decode examples).  W[M, K] (M output
  * features, K input features) is stored as (M / 32) x (K / 256) blocks of 5120 bytes, row-block
  * major, each holding bf16 scales[8][32], bf16 mins[8][32] (one per row and 32-column group) and

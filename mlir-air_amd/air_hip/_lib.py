@@ -31,6 +31,8 @@ SYMBOLS = {
     "w4a16_o_gemv_ffn_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 15 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_attention_workspace_bytes": (_sz, [_ci, _ci]),
     "w4a16_decode_attention_bf16": (_ci, [_vp] * 5 + [_ci] * 5 + [_vp, _sz, _vp]),
+    "lm_head_workspace_bytes": (_sz, [_ci]),
+    "lm_head_gemv_bf16": (_ci, [_vp, _vp, _cf, _vp, _vp, _vp, _ci, _ci, _vp, _sz, _vp]),
     "q4nx_dequant_bf16": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp]),
     "q4nx_repack": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_q4nx_gemm_bf16": (_ci, [_vp] * 6 + [_ci, _ci, _ci, _vp, _sz, _vp]),

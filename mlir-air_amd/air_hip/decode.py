@@ -100,14 +100,14 @@ def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer
     return (ops.q4nx_o_gemv_ffn if q4nx else ops.o_gemv_ffn)(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
 
 
-def decode_token(token_id, layers, embed_table, final_norm, lm_head, config, kv_cache, current_pos, rope_lut):
-    """Full model step: embedding row -> blocks -> final RMSNorm -> logits (fp32 [vocab]).
-    The embedding lookup, the final norm and the bf16 lm_head product are plain torch calls;
-    the reference runs the same three pieces outside its int4 kernels
-    (llama32_1b_int4_inference.py: lm_head_gemv is a bf16 GEMV)."""
+def decode_token(token_id, layers, embed_table, final_norm, lm_head, config, kv_cache, current_pos, rope_lut,
+                 return_argmax=False):
+    """Full model step: embedding row -> blocks -> final RMSNorm + bf16 lm_head GEMV (+ argmax) in one
+    kernel call (run_npu_decode_step, llama32_1b_int4_inference.py:429-486).  Returns the logits as
+    fp32 [vocab], like the reference, and with return_argmax also the greedy token as a device
+    int32 tensor [1] (no host synchronisation here)."""
     x = embed_table[token_id].contiguous()
     for layer, (kc, vc) in zip(layers, kv_cache):
         x = run_decode_block(x, layer, config, kc, vc, current_pos, rope_lut)
-    xf = x.float()
-    normed = ((xf * torch.rsqrt((xf * xf).mean() + config.rms_eps)) * final_norm.float()).to(torch.bfloat16)
-    return (lm_head @ normed).float()
+    logits, best = ops.lm_head(x, lm_head, norm_weight=final_norm, eps=config.rms_eps)
+    return (logits.float(), best) if return_argmax else logits.float()

@@ -242,6 +242,29 @@ def decode_attention(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, out=None
     return out
 
 
+def lm_head(x, lm_head_weight, norm_weight=None, eps=1e-5, return_argmax=True):
+    """Tail of a decode step: logits bf16 [V] = lm_head_weight [V, E] . rms_norm(x) (x itself when
+    norm_weight is None), and the index of the largest logit as a device int32 tensor [1]."""
+    lib = _lib.load_library()
+    _need_cuda(x, lm_head_weight)
+    V, E = lm_head_weight.shape
+    if x.numel() != E:
+        raise ValueError(f"x has {x.numel()} elements but lm_head has E={E}")
+    if not lm_head_weight.is_contiguous():
+        raise ValueError("lm_head must be contiguous [V, E]")
+    logits = torch.empty((V,), dtype=torch.bfloat16, device=x.device)
+    best = torch.empty((1,), dtype=torch.int32, device=x.device) if return_argmax else None
+    key = (x.device.index, _stream(), "lm_head", V)
+    ws = _attn_ws.get(key)
+    if ws is None:
+        ws = torch.empty(int(lib.lm_head_workspace_bytes(V)), dtype=torch.uint8, device=x.device)
+        _attn_ws[key] = ws
+    _lib.check(lib.lm_head_gemv_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)) if norm_weight is not None else None,
+                                     float(eps), _ptr(_bits(lm_head_weight)), _ptr(logits),
+                                     _ptr(best) if return_argmax else None, V, E, _ptr(ws), ws.numel(), _stream()))
+    return (logits, best) if return_argmax else logits
+
+
 def q4nx_dequant(blocks, M, K, mode=0, out=None):
     """Dense W[M, K] bf16 from Q4NX / Q4_0 blocks (uint8 [M/32 * K/256, 5120] on the GPU);
     mode 0 w = s q + m, 1 w = s (q - m), 2 signed q with w = s q."""

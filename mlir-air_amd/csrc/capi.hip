@@ -398,6 +398,24 @@ int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_ro
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+size_t lm_head_workspace_bytes(int V) { return V > 0 ? lm_head_scratch_bytes(V) : 0; }
+
+int lm_head_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const uint16_t *lm_head,
+                      uint16_t *logits, int32_t *argmax_out, int V, int E, void *workspace, size_t workspace_bytes,
+                      void *stream) {
+    if (!x || !lm_head || !logits) return W4A16_ERR_NULL;
+    if (!lm_head_supported(V, E)) return W4A16_ERR_SHAPE;
+    if (norm_weight && !(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(lm_head) || misaligned(logits) || (norm_weight && misaligned(norm_weight)))
+        return W4A16_ERR_ALIGN;
+    if (argmax_out && (reinterpret_cast<uintptr_t>(argmax_out) & 3)) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < lm_head_workspace_bytes(V)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_lm_head(x, norm_weight, eps, lm_head, logits, argmax_out, V, E, workspace,
+                                  static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int q4nx_dequant_bf16(const void *blocks, uint16_t *out_bf16, int M, int K, int mode, void *stream) {
     if (!blocks || !out_bf16) return W4A16_ERR_NULL;
     if (M <= 0 || K <= 0 || M % 32 != 0 || K % 256 != 0 || mode < 0 || mode > 2) return W4A16_ERR_SHAPE;

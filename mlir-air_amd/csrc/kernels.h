@@ -88,6 +88,13 @@ hipError_t launch_q4nx_dequant(const void *blocks, uint16_t *out, int M, int K, 
 hipError_t launch_q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t *mins, int M, int K,
                               int mode, hipStream_t stream);
 
+// Final RMSNorm + bf16 lm_head GEMV + argmax (lm_head.hip).  The scratch buffer holds one 8-byte
+// argmax key per 16 rows and needs no initialisation.
+bool lm_head_supported(int V, int E);
+size_t lm_head_scratch_bytes(int V);
+hipError_t launch_lm_head(const uint16_t *x, const uint16_t *norm_w, float eps, const uint16_t *w, uint16_t *logits,
+                          int32_t *argmax_out, int V, int E, void *workspace, hipStream_t stream);
+
 // Decode attention (attention.hip).  The scratch buffer holds per-chunk softmax partials and
 // needs no initialisation.
 constexpr int kMaxAttnSplit = 32;

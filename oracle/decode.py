@@ -16,9 +16,17 @@ Follows (LLM = programming_examples/llms):
   decode_block_reference run_decode_block (llama32_1b_int4_decode.py:176-313): the call above,
                          KV-cache append, attention, then the O + FFN block
 
+  lm_head_reference      the tail of run_npu_decode_step
+                         (LLM/llama32_1b_int4/llama32_1b_int4_inference.py:459-486): host rms_norm
+                         in float32 (LLM/llama32_1b/llama32_1b_cpu_helpers.py:25-39,
+                         (x / sqrt(mean(x^2) + eps)) * w), one rounding to bf16, the bf16
+                         lm_head GEMV with bf16 logits, np.argmax over the logits as float32
+
 bf16 tensors are uint16 bit patterns.  Pins (tests/test_oracle_decode.py): RoPE against a complex
 rotation and its norm/inverse identities; the LUT against closed forms (pos 0, index 0); attention
-against torch's scaled_dot_product_attention and the closed forms seq_len = 1 and equal keys.
+against torch's scaled_dot_product_attention and the closed forms seq_len = 1 and equal keys; the
+lm_head tail against torch's rms_norm and matmul in float64, one-hot rows (logits = the normalised
+vector), a constant vector (closed-form norm) and tied rows (first index wins).
 """
 
 import numpy as np
@@ -95,3 +103,21 @@ def decode_block_reference(x_bits, layer_l1, k_cache_bits, v_cache_bits, current
     _, _, y = ref.o_gemv_ffn_staged_reference(layer_l1["wo"], layer_l1["w_gate"], layer_l1["w_up"], layer_l1["w_down"],
                                               attn, x_bits, layer_l1["ffn_norm"], eps)
     return y
+
+
+def final_rms_norm(x_bits, w_bits, eps=1e-5):
+    """bf16 bits of (x / sqrt(mean(x^2) + eps)) * w, every step in float32 as in the host helper."""
+    x = bf16_bits_to_f32(np.asarray(x_bits)).astype(np.float32)
+    w = bf16_bits_to_f32(np.asarray(w_bits)).astype(np.float32)
+    rms = np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + np.float32(eps))
+    return f32_to_bf16_bits(((x / rms) * w).astype(np.float32))
+
+
+def lm_head_reference(x_bits, final_norm_bits, lm_head_bits, eps=1e-5):
+    """(logits bf16 bits [V], argmax).  final_norm_bits None: x is used as it is.  The product is
+    accumulated in float64 and rounded once (through float32) to bf16."""
+    normed = np.asarray(x_bits) if final_norm_bits is None else final_rms_norm(x_bits, final_norm_bits, eps)
+    w = bf16_bits_to_f32(np.asarray(lm_head_bits)).astype(np.float64)
+    acc = w @ bf16_bits_to_f32(normed).astype(np.float64)
+    logits = f32_to_bf16_bits(acc.astype(np.float32))
+    return logits, int(np.argmax(bf16_bits_to_f32(logits).astype(np.float32)))

@@ -175,6 +175,13 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     bad = list(args)
     bad[16] = fws - 1
     assert lib.w4a16_ffn_swiglu_bf16(*bad) == _lib.ERR_WORKSPACE
+    lws = lib.lm_head_workspace_bytes(100)
+    assert lws >= 8 * 7 and lib.lm_head_workspace_bytes(0) == 0
+    assert lib.lm_head_gemv_bf16(P, None, 0.0, P, None, None, 100, 512, P, lws, None) == _lib.ERR_NULL
+    assert lib.lm_head_gemv_bf16(P, None, 0.0, P, P, None, 100, 8200, P, lws, None) == _lib.ERR_SHAPE   # E above 8192
+    assert lib.lm_head_gemv_bf16(P, P, -1.0, P, P, None, 100, 512, P, lws, None) == _lib.ERR_SHAPE
+    assert lib.lm_head_gemv_bf16(P, None, 0.0, P, P, P + 2, 100, 512, P, lws, None) == _lib.ERR_ALIGN
+    assert lib.lm_head_gemv_bf16(P, None, 0.0, P, P, None, 100, 512, P, lws - 1, None) == _lib.ERR_WORKSPACE
     assert lib.w4a16_workspace_init(None, 1024, None) == _lib.ERR_NULL
     assert lib.w4a16_workspace_init(P, 16, None) == _lib.ERR_WORKSPACE
     assert lib.w4a16_tune(b"no_such_key", 1) == _lib.ERR_TUNE and lib.w4a16_tune(b"gemv_waves", 0) == 0

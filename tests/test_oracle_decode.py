@@ -60,3 +60,47 @@ def test_attention_against_library_and_closed_forms():
     me = bf16_bits_to_f32(dec.decode_attention_cpu(q, ke, v, pos, n_heads, n_kv, hd)).reshape(n_heads, hd)
     mean = bf16_bits_to_f32(v[:, :pos + 1]).astype(np.float64).mean(axis=1)
     assert np.max(np.abs(me - mean[np.arange(n_heads) // 4])) <= 2.0**-8 * np.abs(mean).max() + 1e-4
+
+
+def test_lm_head_tail_against_library_and_closed_forms():
+    V, E = 96, 512
+    rng = np.random.default_rng(70)
+    x = f32_to_bf16_bits((rng.standard_normal(E) * 3.0).astype(np.float32))
+    nw = f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32))
+    W = f32_to_bf16_bits((rng.standard_normal((V, E)) * 0.05).astype(np.float32))
+    logits, best = dec.lm_head_reference(x, nw, W, eps=1e-5)
+    # library routines in float64, one rounding per stage
+    xt, wt = torch.from_numpy(bf16_bits_to_f32(x)).double(), torch.from_numpy(bf16_bits_to_f32(nw)).double()
+    n_lib = bf16_bits_to_f32(f32_to_bf16_bits(torch.nn.functional.rms_norm(xt, (E,), wt, eps=1e-5).float().numpy()))
+    n_got = bf16_bits_to_f32(dec.final_rms_norm(x, nw))
+    assert np.mean(n_got != n_lib) <= 0.01 and np.max(np.abs(n_got - n_lib) / np.abs(n_lib)) <= 2.0**-7
+    l_lib = torch.from_numpy(bf16_bits_to_f32(W)).double() @ torch.from_numpy(n_got).double()
+    assert np.array_equal(logits, f32_to_bf16_bits(l_lib.float().numpy()))
+    assert best == int(torch.argmax(l_lib.float().bfloat16().float()))
+    # one-hot rows pick elements of the normalised vector: row v = unit vector e_(5 v mod E)
+    idx = (5 * np.arange(V)) % E
+    onehot = np.zeros((V, E), np.uint16)
+    onehot[np.arange(V), idx] = 0x3F80
+    l1, b1 = dec.lm_head_reference(x, nw, onehot)
+    assert np.array_equal(l1, dec.final_rms_norm(x, nw)[idx])
+    assert b1 == int(np.argmax(n_got[idx]))
+    # a transposed operand or a dropped norm would fail here: without the norm the logits are x itself
+    l2, _ = dec.lm_head_reference(x, None, onehot)
+    assert np.array_equal(l2, x[idx]) and not np.array_equal(l1, l2)
+    # constant x = c with unit weight: normed = c / sqrt(c^2 + eps); a sum instead of a mean gives 1 / sqrt(E)
+    c = np.float32(0.0078125)
+    n = bf16_bits_to_f32(dec.final_rms_norm(f32_to_bf16_bits(np.full(E, c, np.float32)), np.full(E, 0x3F80, np.uint16)))
+    closed = float(c) / np.sqrt(float(c) ** 2 + 1e-5)
+    assert np.max(np.abs(n - closed)) <= 2.0**-8 * closed * 1.001
+    # tied rows: the first of the equal maxima wins, also when the tie is between +0 and -0
+    Wt = W.copy()
+    Wt[40] = Wt[7]
+    Wt[80] = Wt[7]
+    lt, _ = dec.lm_head_reference(x, nw, Wt)
+    assert lt[40] == lt[7] == lt[80]
+    big = f32_to_bf16_bits(bf16_bits_to_f32(dec.final_rms_norm(x, nw)) * np.float32(0.25))   # row = 0.25 * normed: the largest possible logit direction
+    Wt[7] = Wt[40] = Wt[80] = big
+    assert dec.lm_head_reference(x, nw, Wt)[1] == 7
+    zeros = np.zeros((4, E), np.uint16)
+    zeros[0, 0] = 0x8000          # -0 * x: logits -0 or +0, all equal as floats
+    assert dec.lm_head_reference(x, nw, zeros)[1] == 0
