@@ -19,8 +19,20 @@ namespace w4a16 {
 
 namespace {
 
-constexpr int kRowsPerWave = 16;
-constexpr int kWaves = 4;
+#ifndef LM_RPW
+#define LM_RPW 16
+#endif
+#ifndef LM_WAVES
+#define LM_WAVES 4
+#endif
+#ifndef LM_RG
+#define LM_RG 4
+#endif
+#ifndef LM_NT
+#define LM_NT 1
+#endif
+constexpr int kRowsPerWave = LM_RPW;
+constexpr int kWaves = LM_WAVES;
 
 struct LmHeadParams {
     const uint16_t *x;
@@ -113,7 +125,7 @@ __global__ void __launch_bounds__(kWaves * 64) lm_head_kernel(const LmHeadParams
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
                 wv[i][c] = u32x4{0u, 0u, 0u, 0u};
-                if (in_row[c]) wv[i][c] = __builtin_nontemporal_load(src + 64 * c);
+                if (in_row[c]) wv[i][c] = LM_NT ? __builtin_nontemporal_load(src + 64 * c) : src[64 * c];
             }
         }
 #pragma unroll
@@ -144,9 +156,16 @@ __global__ void __launch_bounds__(kWaves * 64) lm_head_kernel(const LmHeadParams
 __global__ void __launch_bounds__(1024) lm_head_argmax_kernel(const unsigned long long *keys, int n, int32_t *out) {
     __shared__ unsigned long long part[16];
     unsigned long long best = 0;
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        const unsigned long long k = keys[i];
-        best = k > best ? k : best;
+    // eight independent loads per thread and round trip (one round for up to 131072 rows)
+    for (int base = 0; base < n; base += 8 * 1024) {
+        unsigned long long k[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = base + j * 1024 + (int)threadIdx.x;
+            k[j] = i < n ? keys[i] : 0ull;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) best = k[j] > best ? k[j] : best;
     }
     best = wave_max(best);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = best;
@@ -200,7 +219,7 @@ hipError_t launch_lm_head(const uint16_t *x, const uint16_t *norm_w, float eps, 
         case 1: launch_one<1, 4>(p, grid, stream); break;
         case 2: launch_one<2, 4>(p, grid, stream); break;
         case 3: launch_one<3, 4>(p, grid, stream); break;
-        case 4: launch_one<4, 4>(p, grid, stream); break;
+        case 4: launch_one<4, LM_RG>(p, grid, stream); break;
         case 6: launch_one<6, 2>(p, grid, stream); break;
         case 8: launch_one<8, 2>(p, grid, stream); break;
         case 10: launch_one<10, 1>(p, grid, stream); break;
