@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -277,6 +277,70 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     return res
 
 
+DECODE_1B_POS0 = 1024
+
+
+def run_decode_model(steps, warmup):
+    """Greedy decode of a random-weight model in the Llama-3.2-1B shape (16 layers, E=2048, H=8192,
+    32/8 heads of 64, vocabulary 128256, tied lm_head), `steps` consecutive tokens from position
+    DECODE_1B_POS0 captured as one HIP graph: per token 16 x (RMSNorm + QKV GEMV, attention,
+    O + FFN block) and the tail (final norm, lm_head GEMV, argmax), the token id staying on the device."""
+    import torch
+
+    from air_hip import decode, weights as wmod
+
+    cfg = wmod.LlamaConfig()
+    E, H, hd = cfg.emb_dim, cfg.hidden_dim, cfg.head_dim
+    nqkv = (cfg.n_heads + 2 * cfg.n_kv_heads) * hd
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+
+    def lin(K, N, seed):
+        qw, qz, sc = make_weights(torch, K, N, seed)
+        return qw, qz, (sc.float() * 0.05).to(torch.bfloat16)   # keeps the residual stream O(1) over 16 layers
+
+    def norm_w():
+        return (torch.randn((E,), device="cuda", generator=g) * 0.1 + 1.0).to(torch.bfloat16)
+
+    layers = [decode.DecodeLayer(attn_norm=norm_w(), ffn_norm=norm_w(), wqkv=lin(E, nqkv, 10 * i), wo=lin(E, E, 10 * i + 1),
+                                 w_gate=lin(E, H, 10 * i + 2), w_up=lin(E, H, 10 * i + 3), w_down=lin(H, E, 10 * i + 4))
+              for i in range(cfg.n_layers)]
+    embed = torch.randn((cfg.vocab_size, E), device="cuda", generator=g).to(torch.bfloat16)
+    final_norm = norm_w()
+    max_seq = 2048
+    assert DECODE_1B_POS0 + max(steps, warmup) <= max_seq
+    lut = decode.generate_rope_lut(cfg, max_seq)
+    cache = [(torch.randn((cfg.n_kv_heads, max_seq, hd), device="cuda", generator=g).to(torch.bfloat16),
+              torch.randn((cfg.n_kv_heads, max_seq, hd), device="cuda", generator=g).to(torch.bfloat16))
+             for _ in range(cfg.n_layers)]
+    first = torch.tensor([1], dtype=torch.int32, device=dev)
+    with torch.cuda.stream(stream):
+        decode.decode_greedy(first, warmup, layers, embed, final_norm, embed, cfg, cache, DECODE_1B_POS0, lut)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            tokens = decode.decode_greedy(first, steps, layers, embed, final_norm, embed, cfg, cache, DECODE_1B_POS0, lut)
+        graph.replay()
+        stream.synchronize()
+        ref_tokens = tokens.clone()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+    sec = e0.elapsed_time(e1) * 1e-3
+    layer_w = weight_bytes(E, nqkv) + weight_bytes(E, E) + 2 * weight_bytes(E, H) + weight_bytes(H, E)
+    kv = 2 * cfg.n_kv_heads * (DECODE_1B_POS0 + steps // 2 + 1) * hd * 2
+    per_token = cfg.n_layers * (layer_w + kv + 2 * E * 2) + 2 * cfg.vocab_size * E + 2 * cfg.vocab_size + 3 * E * 2
+    return {"us_per_token": sec / steps * 1e6, "tokens_per_s": steps / sec, "bytes_per_token": per_token,
+            "replays_agree": bool(torch.equal(ref_tokens, tokens))}
+
+
 def cpu_baseline(name, torch, w, x, outs, launch, stream):
     """The reference's NumPy path (restated in oracle/baseline.py) timed on this host's cores,
     on the same inputs as GPU launch 0; also used to sanity-check the GPU result."""
@@ -373,7 +437,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS))
+    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configs")
     ap.add_argument("--copy-probe", action="store_true",
@@ -393,6 +457,22 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if a.workload == "decode_1b":
+        steps = min(a.steps, 64)
+        r = run_decode_model(steps, min(a.warmup, 8))
+        gbs = r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9
+        print(json.dumps({
+            "metric": "int4 decode tokens/s, Llama-3.2-1B shape, batch 1", "value": r["tokens_per_s"], "unit": "tokens/s",
+            "n_gpus": 1, "steps": steps, "warmup": min(a.warmup, 8), "ms_per_step": r["us_per_token"] * 1e-3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "int4 weights (bf16 lm_head), bf16 activations, fp32 accumulate",
+            "data": "synthetic (random weights of the architecture, random KV cache up to the start position)",
+            "config": {"workload": f"greedy decode, 16 layers E=2048 H=8192 32/8 heads hd=64 V=128256 g128, positions {DECODE_1B_POS0}..{DECODE_1B_POS0 + steps - 1}",
+                       "timing": "one HIP graph of all token steps, events on the launch stream"},
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                         "traffic": None, "algorithmic_per_launch": r["bytes_per_token"], "avg_launch_us": r["us_per_token"]},
+            "replays_agree": r["replays_agree"]}))
+        return
     main_res = run_workload(a.workload, a.steps, a.warmup, not a.no_cpu_baseline)
     name = a.workload
     sec = main_res["cold_us"] * 1e-6
@@ -448,6 +528,10 @@ def main():
             else:
                 extra[other] = {"us": r["cold_us"], "GB/s": r["bytes"] / s / 1e9,
                                 "frac_hbm_peak": r["bytes"] / s / 1e9 / HBM_PEAK_GBS, "hot_us": r["hot_us"]}
+        r = run_decode_model(32, 4)
+        extra["decode_1b"] = {"us_per_token": r["us_per_token"], "tokens/s": r["tokens_per_s"],
+                              "GB/s": r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9,
+                              "frac_hbm_peak": r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9 / HBM_PEAK_GBS}
         out["other_workloads"] = extra
     print(json.dumps(out))
 

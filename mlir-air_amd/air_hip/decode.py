@@ -111,3 +111,20 @@ def decode_token(token_id, layers, embed_table, final_norm, lm_head, config, kv_
         x = run_decode_block(x, layer, config, kc, vc, current_pos, rope_lut)
     logits, best = ops.lm_head(x, lm_head, norm_weight=final_norm, eps=config.rms_eps)
     return (logits.float(), best) if return_argmax else logits.float()
+
+
+def decode_greedy(token, n_tokens, layers, embed_table, final_norm, lm_head, config, kv_cache, start_pos, rope_lut):
+    """Greedy decode loop of `generate` (llama32_1b_int4_inference.py:494-560) with nothing returning
+    to the host between tokens: `token` is a device int32 tensor [1] (the token at position
+    start_pos), each step's argmax feeds the next embedding lookup on the device.  Returns the
+    n_tokens generated ids as a device int32 tensor; the caller looks for an end-of-sequence id
+    afterwards (the reference stops at it, so later entries are to be dropped)."""
+    out = torch.empty((n_tokens,), dtype=torch.int32, device=embed_table.device)
+    tok = token.to(torch.int32).reshape(1)
+    for i in range(n_tokens):
+        x = embed_table.index_select(0, tok).reshape(-1)
+        for layer, (kc, vc) in zip(layers, kv_cache):
+            x = run_decode_block(x, layer, config, kc, vc, start_pos + i, rope_lut)
+        _, tok = ops.lm_head(x, lm_head, norm_weight=final_norm, eps=config.rms_eps)
+        out[i:i + 1] = tok
+    return out

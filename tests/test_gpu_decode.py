@@ -133,3 +133,36 @@ def test_decode_token_runs_a_two_layer_model(ops):
         assert logits.shape == (cfg.vocab_size,) and torch.isfinite(logits).all()
         tok = int(torch.argmax(logits))
     assert float(cache[1][0][:, :4].float().abs().sum()) > 0 and float(cache[1][0][:, 4:].float().abs().sum()) == 0
+
+
+def test_decode_greedy_matches_token_by_token_decoding(ops):
+    """The device-side greedy loop produces the tokens that decode_token + a host argmax produce."""
+    from air_hip import decode, weights
+
+    cfg = weights.LlamaConfig(n_layers=2, emb_dim=256, n_heads=4, head_dim=64, n_kv_heads=2, hidden_dim=512, vocab_size=200)
+    layers = []
+    for i in range(cfg.n_layers):
+        t, an, fn = _layer(cfg.emb_dim, cfg.hidden_dim, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, seed=700 + 10 * i)
+        t = {k: (v[0], v[1], f32_to_bf16_bits(bf16_bits_to_f32(v[2]) * 0.05)) for k, v in t.items()}
+        layers.append(decode.prepare_layer(weights.LayerWeights(attn_norm=an, ffn_norm=fn, **t)))
+    g = torch.Generator(device="cuda").manual_seed(2)
+    embed = torch.randn((cfg.vocab_size, cfg.emb_dim), device="cuda", generator=g).to(torch.bfloat16)
+    final_norm = (torch.randn(cfg.emb_dim, device="cuda", generator=g) * 0.1 + 1.0).to(torch.bfloat16)
+    lut = decode.generate_rope_lut(cfg, 32)
+    n = 6
+    print("greedy loop, token by token", flush=True)
+    cache = decode.new_kv_cache(cfg, 32)
+    tok, want = 5, []
+    for pos in range(n):
+        logits, best = decode.decode_token(tok, layers, embed, final_norm, embed, cfg, cache, pos, lut, return_argmax=True)
+        tok = int(torch.argmax(logits))
+        assert tok == int(best.item())
+        want.append(tok)
+    print("greedy loop, on the device", flush=True)
+    cache2 = decode.new_kv_cache(cfg, 32)
+    first = torch.tensor([5], dtype=torch.int32, device="cuda")
+    got = decode.decode_greedy(first, n, layers, embed, final_norm, embed, cfg, cache2, 0, lut)
+    torch.cuda.synchronize()
+    assert got.tolist() == want
+    for (k1, v1), (k2, v2) in zip(cache, cache2):
+        assert torch.equal(k1, k2) and torch.equal(v1, v2)
