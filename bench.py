@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|prefill_block]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -278,6 +278,56 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
 
 
 DECODE_1B_POS0 = 1024
+PREFILL_BLOCK = dict(M=2048, E=2048, H=8192)   # the reference example's dimensions (o_ffn_int4_multi.py:291-293)
+
+
+def run_prefill_block(steps, warmup):
+    """Prefill O projection + residual + RMSNorm + SwiGLU FFN + residual for 2048 tokens at the
+    Llama-3.2-1B widths (w4a16_prefill_o_ffn_bf16), `steps` calls in one HIP graph."""
+    import torch
+
+    from air_hip import _lib
+
+    lib = _lib.load_library()
+    M, E, H = PREFILL_BLOCK["M"], PREFILL_BLOCK["E"], PREFILL_BLOCK["H"]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    ws = [make_weights(torch, K, N, 300 + i) for i, (K, N) in enumerate(((E, E), (E, H), (E, H), (H, E)))]
+    ws = [(qw, qz, (sc.float() * 0.1).to(torch.bfloat16)) for qw, qz, sc in ws]
+    attn = torch.randn((M, E), device="cuda", generator=g).to(torch.bfloat16)
+    xres = torch.randn((M, E), device="cuda", generator=g).to(torch.bfloat16)
+    nw = (torch.randn((E,), device="cuda", generator=g) * 0.1 + 1.0).to(torch.bfloat16)
+    y = torch.empty((M, E), dtype=torch.bfloat16, device=dev)
+    scratch = torch.empty(int(lib.w4a16_prefill_block_workspace_bytes(M, E, H)), dtype=torch.uint8, device=dev)
+    ptrs = [t.data_ptr() for w in ws for t in w]
+
+    def launch(st):
+        _lib.check(lib.w4a16_prefill_o_ffn_bf16(attn.data_ptr(), xres.data_ptr(), nw.data_ptr(), 1e-5, *ptrs, y.data_ptr(),
+                                                None, None, M, E, H, 128, scratch.data_ptr(), scratch.numel(), st))
+
+    with torch.cuda.stream(stream):
+        for _ in range(warmup):
+            launch(stream.cuda_stream)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for _ in range(steps):
+                launch(stream.cuda_stream)
+        graph.replay()
+        stream.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+    sec = e0.elapsed_time(e1) * 1e-3 / steps
+    flops = 2 * M * (E * E + 3 * E * H)
+    return {"us": sec * 1e6, "flops": flops, "TFLOP/s": flops / sec / 1e12, "finite": bool(torch.isfinite(y.float()).all())}
 
 
 def run_decode_model(steps, warmup):
@@ -437,7 +487,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b"])
+    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b", "prefill_block"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configs")
     ap.add_argument("--copy-probe", action="store_true",
@@ -457,6 +507,21 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if a.workload == "prefill_block":
+        steps = min(a.steps, 20)
+        r = run_prefill_block(steps, min(a.warmup, 3))
+        print(json.dumps({
+            "metric": "W4A16 prefill O + FFN block TFLOP/s", "value": r["TFLOP/s"], "unit": "TFLOP/s", "n_gpus": 1,
+            "steps": steps, "warmup": min(a.warmup, 3), "ms_per_step": r["us"] * 1e-3, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights, bf16 activations, fp32 accumulate",
+            "data": "synthetic (uniform uint4 q/z, scales (|N(0,1)|*0.02+1e-3)*0.1, activations ~ N(0,1))",
+            "config": {"workload": "prefill O-proj + residual + RMSNorm + SwiGLU FFN + residual, M=2048 E=2048 H=8192 g128",
+                       "timing": "HIP graph of K calls (5 to 7 launches each), events on the launch stream"},
+            "roofline": {"bound": "mfma", "achieved": r["TFLOP/s"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_per_launch": r["flops"],
+                         "avg_launch_us": r["us"]},
+            "finite": r["finite"]}))
+        return
     if a.workload == "decode_1b":
         steps = min(a.steps, 64)
         r = run_decode_model(steps, min(a.warmup, 8))
@@ -528,6 +593,8 @@ def main():
             else:
                 extra[other] = {"us": r["cold_us"], "GB/s": r["bytes"] / s / 1e9,
                                 "frac_hbm_peak": r["bytes"] / s / 1e9 / HBM_PEAK_GBS, "hot_us": r["hot_us"]}
+        r = run_prefill_block(10, 2)
+        extra["prefill_block"] = {"us": r["us"], "TFLOP/s": r["TFLOP/s"], "frac_mfma_peak": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS}
         r = run_decode_model(32, 4)
         extra["decode_1b"] = {"us_per_token": r["us_per_token"], "tokens/s": r["tokens_per_s"],
                               "GB/s": r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9,

@@ -220,6 +220,35 @@ int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_ro
                                 void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Prefill counterpart of w4a16_o_gemv_ffn_bf16 for M tokens at once: the reference's 8-launch ELF `o_ffn_int4`
+ * (programming_examples/llms/llama32_1b_int4/multi_launch_builder/o_ffn_int4_multi.py:4-17; CPU
+ * reference :644-665) as four GEMM launches with fused epilogues and one RMSNorm launch:
+ *   res1    = bf16(bf16(attn_out . Wo) + x_residual)
+ *   normed2 = bf16((res1 / sqrt(mean(res1^2) + eps)) * ffn_norm_weight)      per row, fp32
+ *   h       = bf16(silu(bf16(normed2 . Wgate)) * bf16(normed2 . Wup))        silu(g) = g / (1 + exp(-g)), fp32
+ *   y       = bf16(bf16(h . Wdown) + res1)
+ * attn_out, x_residual, y bf16 [M, E]; optional outputs res1_out [M, E] and h_out [M, H] (NULL: kept
+ * in the workspace).  Any M >= 1 (the tiled kernel is used whatever M is), E % 128 == 0,
+ * E <= 8192, H % 128 == 0.  The workspace is plain scratch (no initialisation),
+ * w4a16_prefill_block_workspace_bytes(M, E, H): 4 M E + 4 M H bytes for res1, normed2, gate and h, plus
+ * the fp32 split-K slices (up to 16 M max(E, H) bytes) of the projections that have too few 256 x 256 tiles to
+ * fill the GPU.
+ * rms_norm_rows_bf16 is the block's RMSNorm stage on its own (the `weighted_rms_norm` launch of both
+ * prefill ELFs): out[m, :] = bf16((x[m, :] / sqrt(mean(x[m, :]^2) + eps)) * norm_weight), K % 8 == 0, K <= 8192.
+ */
+size_t w4a16_prefill_block_workspace_bytes(int M, int E, int H);
+int rms_norm_rows_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, uint16_t *out, int M, int K,
+                       void *stream);
+int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual,
+                             const uint16_t *ffn_norm_weight, float eps,
+                             const int32_t *o_qweight, const int32_t *o_qzeros, const uint16_t *o_scales,
+                             const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                             const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                             const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
+                             uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E, int H, int group,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Tail of a decode step: final RMSNorm, bf16 lm_head GEMV and argmax in one call
  * (run_npu_decode_step, programming_examples/llms/llama32_1b_int4/llama32_1b_int4_inference.py:459-486:
  * host rms_norm, the `lm_head_gemv` kernel over 8 vocabulary partitions, np.argmax).

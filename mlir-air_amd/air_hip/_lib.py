@@ -31,6 +31,9 @@ SYMBOLS = {
     "w4a16_o_gemv_ffn_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 15 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_attention_workspace_bytes": (_sz, [_ci, _ci]),
     "w4a16_decode_attention_bf16": (_ci, [_vp] * 5 + [_ci] * 5 + [_vp, _sz, _vp]),
+    "w4a16_prefill_block_workspace_bytes": (_sz, [_ci, _ci, _ci]),
+    "rms_norm_rows_bf16": (_ci, [_vp, _vp, _cf, _vp, _ci, _ci, _vp]),
+    "w4a16_prefill_o_ffn_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 15 + [_ci, _ci, _ci, _ci, _vp, _sz, _vp]),
     "lm_head_workspace_bytes": (_sz, [_ci]),
     "lm_head_gemv_bf16": (_ci, [_vp, _vp, _cf, _vp, _vp, _vp, _ci, _ci, _vp, _sz, _vp]),
     "q4nx_dequant_bf16": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp]),

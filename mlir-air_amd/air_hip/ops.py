@@ -242,6 +242,40 @@ def decode_attention(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, out=None
     return out
 
 
+def rms_norm_rows(x, norm_weight, eps=1e-5):
+    """out[m, :] = bf16((x[m, :] / sqrt(mean(x[m, :]^2) + eps)) * norm_weight) for x bf16 [M, K]."""
+    lib = _lib.load_library()
+    _need_cuda(x, norm_weight)
+    M, K = x.shape
+    out = torch.empty_like(x)
+    _lib.check(lib.rms_norm_rows_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps), _ptr(out), M, K, _stream()))
+    return out
+
+
+def prefill_o_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, group=GROUP,
+                  return_intermediates=False):
+    """Prefill O projection + residual + RMSNorm + SwiGLU FFN + residual for M tokens: bf16 [M, E] -> [M, E].
+    Every weight is an AWQ triple (qweight, qzeros, scales).  With return_intermediates also res1 [M, E]
+    and h [M, H]."""
+    lib = _lib.load_library()
+    _need_cuda(attn_out, x_residual, ffn_norm_weight)
+    M, E = attn_out.shape
+    H = gate[0].shape[1] * 8
+    y = torch.empty((M, E), dtype=torch.bfloat16, device=attn_out.device)
+    res1 = torch.empty((M, E), dtype=torch.bfloat16, device=attn_out.device) if return_intermediates else None
+    h = torch.empty((M, H), dtype=torch.bfloat16, device=attn_out.device) if return_intermediates else None
+    key = (attn_out.device.index, _stream(), "prefill_block", M, E, H)
+    ws = _attn_ws.get(key)
+    if ws is None:
+        ws = torch.empty(int(lib.w4a16_prefill_block_workspace_bytes(M, E, H)), dtype=torch.uint8, device=attn_out.device)
+        _attn_ws[key] = ws
+    _lib.check(lib.w4a16_prefill_o_ffn_bf16(_ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)),
+                                            float(eps), *_wptrs(wo), *_wptrs(gate), *_wptrs(up), *_wptrs(down), _ptr(y),
+                                            _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
+                                            M, E, H, group, _ptr(ws), ws.numel(), _stream()))
+    return (y, res1, h) if return_intermediates else y
+
+
 def lm_head(x, lm_head_weight, norm_weight=None, eps=1e-5, return_argmax=True):
     """Tail of a decode step: logits bf16 [V] = lm_head_weight [V, E] . rms_norm(x) (x itself when
     norm_weight is None), and the index of the largest logit as a device int32 tensor [1]."""

@@ -375,6 +375,50 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, 
                            workspace_bytes, stream);
 }
 
+size_t w4a16_prefill_block_workspace_bytes(int M, int E, int H) {
+    return prefill_block_supported(M, E, H) ? prefill_block_scratch_bytes(M, E, H) : 0;
+}
+
+int rms_norm_rows_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, uint16_t *out, int M, int K,
+                       void *stream) {
+    if (!x || !norm_weight || !out) return W4A16_ERR_NULL;
+    if (!prefill_block_supported(M, K, 8) || !(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(norm_weight) || misaligned(out)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_rmsnorm_rows(x, norm_weight, out, M, K, eps, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                             float eps, const int32_t *o_qweight, const int32_t *o_qzeros, const uint16_t *o_scales,
+                             const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                             const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                             const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
+                             uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E, int H, int group,
+                             void *workspace, size_t workspace_bytes, void *stream) {
+    if (!attn_out || !x_residual || !ffn_norm_weight || !y) return W4A16_ERR_NULL;
+    int rc = check_quant(o_qweight, o_qzeros, o_scales, E, E, group, 32);
+    if (rc) return rc;
+    rc = check_quant(gate_qweight, gate_qzeros, gate_scales, E, H, group, 32);
+    if (rc) return rc;
+    rc = check_quant(up_qweight, up_qzeros, up_scales, E, H, group, 32);
+    if (rc) return rc;
+    rc = check_quant(down_qweight, down_qzeros, down_scales, H, E, group, 32);
+    if (rc) return rc;
+    if (!prefill_block_supported(M, E, H) || !(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(attn_out) || misaligned(x_residual) || misaligned(ffn_norm_weight) || misaligned(y) ||
+        (res1_out && misaligned(res1_out)) || (h_out && misaligned(h_out)))
+        return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_prefill_block_workspace_bytes(M, E, H)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_prefill_o_ffn(attn_out, x_residual, ffn_norm_weight, eps,
+                                        PrefillLinear{o_qweight, o_qzeros, o_scales},
+                                        PrefillLinear{gate_qweight, gate_qzeros, gate_scales},
+                                        PrefillLinear{up_qweight, up_qzeros, up_scales},
+                                        PrefillLinear{down_qweight, down_qzeros, down_scales}, y, res1_out, h_out, M, E,
+                                        H, workspace, current_cus(), static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim) {
     if (n_heads <= 0 || head_dim <= 0) return 0;
     return round256(attention_workspace_bytes(n_heads, head_dim));

@@ -48,8 +48,12 @@ struct GemmParams {
     const uint32_t *qz;
     const uint16_t *sc;
     uint16_t *y;
+    const uint16_t *aux;   // [M, N] bf16 operand of the epilogue (residual or gate), or nullptr
+    int epi;               // kEpi*
     int M, K, N;
     int tiles_m, tiles_n;
+    float *partial;        // split-K: fp32 [gridDim.y][M][N] partial products instead of y (nullptr: no split)
+    int kt_per_split;      // K steps of 64 per blockIdx.y (even)
 };
 
 __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
@@ -165,7 +169,8 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
         b_sw[j] = (n >> 3) & 7;
     }
 
-    const int KT = p.K / BK;                        // even: K % 128 == 0
+    // K steps [kt_begin, kt_end) of this workgroup: all of them, or slice blockIdx.y of a split-K launch (even bounds)
+    const int kt_begin = blockIdx.y * p.kt_per_split, kt_end = kt_begin + p.kt_per_split;
     uint16_t *stage0 = lds, *stage1 = lds + kStageElems;
 
     // Pipeline (stage = kt % 2, one barrier per K step).  While the MFMAs of tile kt run:
@@ -177,13 +182,13 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
     // A step is one basic block (the flags are compile-time), and sched_group_barrier pins the
     // interleaving: one wave per SIMD issues in order, so VALU / LDS / global instructions only
     // overlap with the matrix pipe when they sit between MFMAs in program order.
-    dma_a(stage0, 0);
-    load_b(0, rb[0]);
-    fetch_group(0);
+    dma_a(stage0, kt_begin * BK);
+    load_b(kt_begin * BK, rb[0]);
+    fetch_group(kt_begin * BK);
     convert_group();
 #pragma unroll
     for (int part = 0; part < 4; ++part) store_b(stage0, rb[0], part);
-    load_b(BK, rb[1]);
+    load_b((kt_begin + 1) * BK, rb[1]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the x tile copy writes LDS behind the compiler's back
     __syncthreads();
 
@@ -246,33 +251,105 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
     };
     using T = std::true_type;
     using F = std::false_type;
-    int kt = 0;
-    for (; kt + 3 < KT; kt += 2) {
+    int kt = kt_begin;
+    for (; kt + 3 < kt_end; kt += 2) {
         step(kt, stage0, stage1, rb[1], rb[0], T{}, T{}, F{});
         step(kt + 1, stage1, stage0, rb[0], rb[1], T{}, T{}, T{});
     }
-    // KT is even: two steps remain
+    // the step count is even: two steps remain
     step(kt, stage0, stage1, rb[1], rb[0], T{}, F{}, F{});
     step(kt + 1, stage1, stage0, rb[0], rb[1], F{}, F{}, T{});
 
     // D layout of the 32x32 MFMA: register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
+    // One copy of the store loop per epilogue, chosen by a uniform branch.
+    auto store_tile = [&](auto EPI) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int col = n0 + wn * 128 + j * 32 + fr;
+            for (int j = 0; j < 4; ++j) {
+                const int col = n0 + wn * 128 + j * 32 + fr;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * fk + (r & 3);
-                if (row < p.M && col < p.N) p.y[(size_t)row * p.N + col] = float_to_bf16_bits(acc[i][j][r]);
+                for (int r = 0; r < 16; ++r) {
+                    const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * fk + (r & 3);
+                    if (row < p.M && col < p.N) {
+                        const size_t at = (size_t)row * p.N + col;
+                        uint16_t out = float_to_bf16_bits(acc[i][j][r]);
+                        if constexpr (decltype(EPI)::value == kEpiAddRounded) {
+                            // y = bf16(bf16(x . W) + R): the product is a bf16 tensor before the add
+                            out = float_to_bf16_bits(bf16_bits_to_float(out) + bf16_bits_to_float(p.aux[at]));
+                        } else if constexpr (decltype(EPI)::value == kEpiSiluGateMul) {
+                            // y = bf16(silu(G) * bf16(x . W)), silu(g) = g / (1 + exp(-g)) in fp32
+                            const float g = bf16_bits_to_float(p.aux[at]);
+                            out = float_to_bf16_bits(g / (1.0f + expf(-g)) * bf16_bits_to_float(out));
+                        }
+                        p.y[at] = out;
+                    }
+                }
             }
-        }
+    };
+    if (p.partial) {
+        float *dst = p.partial + (size_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = n0 + wn * 128 + j * 32 + fr;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * fk + (r & 3);
+                    if (row < p.M && col < p.N) dst[(size_t)row * p.N + col] = acc[i][j][r];
+                }
+            }
+    } else if (p.epi == kEpiAddRounded)
+        store_tile(std::integral_constant<int, kEpiAddRounded>{});
+    else if (p.epi == kEpiSiluGateMul)
+        store_tile(std::integral_constant<int, kEpiSiluGateMul>{});
+    else
+        store_tile(std::integral_constant<int, kEpiNone>{});
 }
 
 }  // namespace
 
+// y = epilogue(sum over slices of the split-K partial products), four elements per thread.
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restrict__ partial, int ksplit, size_t mn,
+                                                            uint16_t *__restrict__ y, const uint16_t *__restrict__ aux, int epi) {
+    const size_t at = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (at >= mn) return;                            // M * N is a multiple of 4 (N % 32 == 0)
+    floatx4 sum = *reinterpret_cast<const floatx4 *>(partial + at);
+    for (int s = 1; s < ksplit; ++s) sum += *reinterpret_cast<const floatx4 *>(partial + (size_t)s * mn + at);
+    uint16_t out[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        out[e] = float_to_bf16_bits(sum[e]);
+        if (epi == kEpiAddRounded) {
+            out[e] = float_to_bf16_bits(bf16_bits_to_float(out[e]) + bf16_bits_to_float(aux[at + e]));
+        } else if (epi == kEpiSiluGateMul) {
+            const float g = bf16_bits_to_float(aux[at + e]);
+            out[e] = float_to_bf16_bits(g / (1.0f + expf(-g)) * bf16_bits_to_float(out[e]));
+        }
+    }
+    *reinterpret_cast<uint2 *>(y + at) = uint2{(uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16)};
+}
+
+// Slices along K for a launch whose tiles would leave most of the chip idle: as many as fit the CUs,
+// at most 4, each an even number of K steps and at least 8 of them.
+int gemm_prefill_ksplit(int M, int K, int N, int cus) {
+    const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    const int KT = K / BK;
+    int split = 1;
+    for (int s = 2; s <= 4; s *= 2)
+        if (tiles * s <= cus && KT % (2 * s) == 0 && KT / s >= 8) split = s;
+    return split;
+}
+
+size_t gemm_prefill_splitk_bytes(int M, int K, int N, int cus) {
+    const int s = gemm_prefill_ksplit(M, K, N, cus);
+    return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+}
+
 hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
-                               const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream) {
+                               const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream,
+                               int epi, const uint16_t *aux, float *splitk_scratch, int cus) {
     // 144 KiB of dynamic LDS needs the attribute; it is per device, so it is set on every launch
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
@@ -283,14 +360,24 @@ hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const 
     p.qz = reinterpret_cast<const uint32_t *>(qzeros);
     p.sc = scales;
     p.y = y;
+    p.aux = aux;
+    p.epi = aux ? epi : kEpiNone;
     p.M = M;
     p.K = K;
     p.N = N;
     p.tiles_m = (M + BM - 1) / BM;
     p.tiles_n = (N + BN - 1) / BN;
+    const int ksplit = splitk_scratch ? gemm_prefill_ksplit(M, K, N, cus) : 1;
+    p.partial = ksplit > 1 ? splitk_scratch : nullptr;
+    p.kt_per_split = K / BK / ksplit;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    hipLaunchKernelGGL(gemm_kernel, dim3(grid), dim3(kThreads), kLdsBytes, stream, p);
+    hipLaunchKernelGGL(gemm_kernel, dim3(grid, ksplit), dim3(kThreads), kLdsBytes, stream, p);
+    e = hipGetLastError();
+    if (e != hipSuccess || ksplit == 1) return e;
+    const size_t mn = (size_t)M * N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, stream, splitk_scratch,
+                       ksplit, mn, y, p.aux, p.epi);
     return hipGetLastError();
 }
 

@@ -59,10 +59,34 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
                          uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream,
                          const StreamExtras &extras = StreamExtras());
 
+// Prefill GEMM (M > 16) with an optional epilogue on a second bf16 [M, N] operand `aux`:
+//   kEpiAddRounded   y = bf16(bf16(x . W) + aux)            (residual add of a bf16 product)
+//   kEpiSiluGateMul  y = bf16(silu(aux) * bf16(x . W))      (SwiGLU with aux = the gate projection)
+enum : int { kEpiNone = 0, kEpiAddRounded = 1, kEpiSiluGateMul = 2 };
+// With `splitk_scratch` (plain scratch of gemm_prefill_splitk_bytes) a launch with few tiles is cut into 2 or 4
+// slices along K whose fp32 partial products a second kernel sums before the epilogue.
 hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
-                               const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream);
+                               const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream,
+                               int epi = kEpiNone, const uint16_t *aux = nullptr, float *splitk_scratch = nullptr,
+                               int cus = 0);
+int gemm_prefill_ksplit(int M, int K, int N, int cus);
+size_t gemm_prefill_splitk_bytes(int M, int K, int N, int cus);
 
 hipError_t launch_fill_workspace(void *ptr, size_t bytes, hipStream_t stream);
+
+// Prefill O projection + FFN block (prefill_block.hip): five launches, intermediates in the workspace
+// (plain scratch, no initialisation).
+struct PrefillLinear {
+    const int32_t *qw, *qz;
+    const uint16_t *sc;
+};
+bool prefill_block_supported(int M, int E, int H);
+size_t prefill_block_scratch_bytes(int M, int E, int H);   // sized for split-K on a 256-CU device
+hipError_t launch_rmsnorm_rows(const uint16_t *x, const uint16_t *w, uint16_t *out, int M, int K, float eps, hipStream_t stream);
+hipError_t launch_prefill_o_ffn(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_w, float eps,
+                                const PrefillLinear &wo, const PrefillLinear &wg, const PrefillLinear &wu,
+                                const PrefillLinear &wd, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
+                                int H, void *workspace, int cus, hipStream_t stream);
 
 // Decode FFN as one persistent kernel (ffn_fused.hip).  plan_ffn_fused returns false for shapes
 // the kernel does not take (the caller then runs the two streaming launches).

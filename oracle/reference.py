@@ -25,6 +25,11 @@ Follows (PE = programming_examples, INT4 = PE/llms/llama32_1b_int4):
                              (o_gemv_ffn_int4_multi.py:4-37) chained with the
                              per-stage references above, i.e. with the bf16
                              rounding points the stages have on the device
+  o_ffn_int4_prefill_reference  the CPU reference of the 8-launch prefill ELF
+                             (INT4/multi_launch_builder/o_ffn_int4_multi.py:644-665): four
+                             matmul_cpu_reference products with bf16 outputs, residual adds
+                             and the row-wise RMSNorm in float32 (r1 / rms * w), SwiGLU
+                             with silu(g) = g / (1 + exp(-g)) in float32
   check_outputs              python/air/backend/xrt_runner.py:394-523
 
 Arrays named A_q/A_s/A_z use the examples' kernel-side layout
@@ -203,6 +208,29 @@ def o_gemv_ffn_staged_reference(wo_l1, gate_l1, up_l1, down_l1, attn_out_bits, x
     h = swiglu_rms_cpu_reference(a_q, a_s, a_z, res1, ffn_norm_w_bits, eps)
     y = matvec_add_cpu_reference(down_l1[0], down_l1[1], down_l1[2], h, res1)
     return res1, h, y
+
+
+def rms_norm_rows_bf16(x_bits, w_bits, eps=1e-5):
+    """bf16 bits of r / sqrt(mean(r^2, axis=-1) + eps) * w, row-wise, every step in float32."""
+    r = bf16_bits_to_f32(np.asarray(x_bits)).astype(np.float32)
+    rms = np.sqrt(np.mean(r**2, axis=-1, keepdims=True) + np.float32(eps))
+    return f32_to_bf16_bits((r / rms * bf16_bits_to_f32(np.asarray(w_bits)).astype(np.float32)).astype(np.float32))
+
+
+def o_ffn_int4_prefill_reference(wo_l1, gate_l1, up_l1, down_l1, attn_out_bits, x_residual_bits, ffn_norm_w_bits,
+                                 eps=1e-5, **matmul_kw):
+    """(output, res1, swiglu) as bf16 bits [M, E], [M, E], [M, H]; every weight is (A_q, A_s, A_z).
+    matmul_kw goes to matmul_cpu_reference (round_weights / accumulate)."""
+    proj = matmul_cpu_reference(*wo_l1, attn_out_bits, **matmul_kw)
+    res1 = f32_to_bf16_bits(bf16_bits_to_f32(proj).astype(np.float32) + bf16_bits_to_f32(x_residual_bits).astype(np.float32))
+    normed2 = rms_norm_rows_bf16(res1, ffn_norm_w_bits, eps)
+    gate = matmul_cpu_reference(*gate_l1, normed2, **matmul_kw)
+    up = matmul_cpu_reference(*up_l1, normed2, **matmul_kw)
+    g = bf16_bits_to_f32(gate).astype(np.float32)
+    swiglu = f32_to_bf16_bits((g / (np.float32(1.0) + np.exp(-g)) * bf16_bits_to_f32(up).astype(np.float32)).astype(np.float32))
+    down = matmul_cpu_reference(*down_l1, swiglu, **matmul_kw)
+    out = f32_to_bf16_bits(bf16_bits_to_f32(down).astype(np.float32) + bf16_bits_to_f32(res1).astype(np.float32))
+    return out, res1, swiglu
 
 
 def check_outputs(actual, expected, rtol=1e-3, atol=1e-8, max_mismatch_percentage=0, min_correlation=None):

@@ -1,0 +1,149 @@
+"""GPU parity of the prefill O projection + FFN block (four GEMMs with fused epilogues + one
+row-wise RMSNorm) against the oracle, stage by stage.
+
+Every stage is checked on the kernel's own input to that stage, so that a one-ulp flip upstream
+does not have to be propagated through a GEMM: res1 and y are bf16(bf16(P) + R) with P a float64
+product (tolerance: one ulp of the sum, one ulp of P, 2e-3 absolute), the RMSNorm rows may flip
+one ulp where fp32 sums differ in their last bit, and h = silu(bf16(G)) * bf16(U) moves by up to
+~3 ulp when G and U flip (silu' <= 1.1).  The whole block also passes the reference's own gate.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_ulp, dense_f64, make_awq, make_x
+from oracle import awq as oawq, reference as oref
+from oracle.bf16 import bf16_bits_to_f32, f32_to_bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(a).cuda()
+
+
+def bits(t):
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from air_hip import ops
+    return ops
+
+
+def _weights(E, H, seed, scale=1.0):
+    out = []
+    for i, (K, N) in enumerate(((E, E), (E, H), (E, H), (H, E))):
+        qw, qz, s = make_awq(K, N, seed=seed + i)
+        out.append((qw, qz, f32_to_bf16_bits(bf16_bits_to_f32(s) * np.float32(scale))))
+    return out
+
+
+def _norm_w(E, seed):
+    rng = np.random.default_rng(seed)
+    return f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32))
+
+
+def _close_sum(got_bits, prod64, add32, what):
+    """got = bf16(bf16(prod) + add) up to one ulp of each rounding."""
+    want = prod64 + add32
+    err = np.abs(bf16_bits_to_f32(got_bits).astype(np.float64) - want)
+    tol = bf16_ulp(want) + bf16_ulp(prod64) + 2e-3
+    assert np.all(err <= tol), f"{what}: worst {np.max(err - tol):.4g} over tolerance at {np.unravel_index(np.argmax(err - tol), err.shape)}"
+
+
+@pytest.mark.parametrize("M,E,H", [(40, 256, 512), (300, 512, 1152), (17, 128, 128), (260, 1024, 2048)])
+def test_prefill_block_stage_by_stage(ops, M, E, H):
+    print(f"prefill block M={M} E={E} H={H}", flush=True)
+    wo, wg, wu, wd = _weights(E, H, seed=M + E, scale=0.25)
+    attn, xres, nw = make_x((M, E), seed=M), make_x((M, E), seed=M + 1), _norm_w(E, M + 2)
+    y, res1, h = ops.prefill_o_ffn(dev(attn), dev(xres), dev(nw), tuple(map(dev, wo)), tuple(map(dev, wg)),
+                                   tuple(map(dev, wu)), tuple(map(dev, wd)), return_intermediates=True)
+    y2 = ops.prefill_o_ffn(dev(attn), dev(xres), dev(nw), tuple(map(dev, wo)), tuple(map(dev, wg)),
+                           tuple(map(dev, wu)), tuple(map(dev, wd)))
+    torch.cuda.synchronize()
+    y_b, res1_b, h_b = bits(y), bits(res1), bits(h)
+    assert np.array_equal(bits(y2), y_b), "intermediates kept in the workspace give another result"
+    f = lambda b: bf16_bits_to_f32(b).astype(np.float64)
+    # 1. O projection + residual
+    _close_sum(res1_b, f(attn) @ dense_f64(*wo, rounded=True), f(xres), "res1")
+    # 2. row-wise RMSNorm of the kernel's res1
+    n_gpu = bits(ops.rms_norm_rows(res1, dev(nw)))
+    n_ref = oref.rms_norm_rows_bf16(res1_b, nw)
+    nd = np.abs(f(n_gpu) - f(n_ref))
+    assert np.all(nd <= bf16_ulp(f(n_ref))) and np.mean(n_gpu != n_ref) < 0.01, (nd.max(), np.mean(n_gpu != n_ref))
+    # 3. gate / up + SwiGLU on the kernel's normalised rows
+    G, U = f(n_gpu) @ dense_f64(*wg, rounded=True), f(n_gpu) @ dense_f64(*wu, rounded=True)
+    gb, ub = f(f32_to_bf16_bits(G.astype(np.float32))), f(f32_to_bf16_bits(U.astype(np.float32)))
+    h_want = gb / (1.0 + np.exp(-gb)) * ub
+    h_tol = 4 * bf16_ulp(h_want) + 1.2 * bf16_ulp(gb) * np.abs(ub) + bf16_ulp(ub) * np.abs(gb) + 1e-3
+    assert np.all(np.abs(f(h_b) - h_want) <= h_tol), np.max(np.abs(f(h_b) - h_want) - h_tol)
+    # 4. down projection + residual on the kernel's h and res1
+    _close_sum(y_b, f(h_b) @ dense_f64(*wd, rounded=True), f(res1_b), "y")
+    # the whole block against the restated CPU reference, under the reference's gate and a tighter one
+    l1 = [oawq.repack_hf_awq_linear(*w, 128) for w in (wo, wg, wu, wd)]
+    want, _, _ = oref.o_ffn_int4_prefill_reference(*l1, attn, xres, nw)
+    got_f, want_f = bf16_bits_to_f32(y_b), bf16_bits_to_f32(want)
+    assert oref.check_outputs(got_f, want_f, rtol=0.5, atol=10.0, max_mismatch_percentage=0.5, min_correlation=0.99)
+    assert np.max(np.abs(got_f - want_f)) <= 8 * 2.0**-8 * np.max(np.abs(want_f)), np.max(np.abs(got_f - want_f))
+
+
+def test_prefill_block_zero_projections_are_exact(ops):
+    """q == z makes a projection exactly zero: res1 is the residual and y is res1, bit for bit."""
+    M, E, H = 200, 256, 512
+    wo, wg, wu, wd = _weights(E, H, seed=90)
+    zero = lambda w: (w[1].repeat(128, axis=0), w[1], w[2])      # every q row equals its group's z row
+    attn, xres, nw = make_x((M, E), seed=91), make_x((M, E), seed=92), _norm_w(E, 93)
+    print("prefill block, zero O and down projections", flush=True)
+    y, res1, h = ops.prefill_o_ffn(dev(attn), dev(xres), dev(nw), tuple(map(dev, zero(wo))), tuple(map(dev, wg)),
+                                   tuple(map(dev, wu)), tuple(map(dev, zero(wd))), return_intermediates=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(res1), xres) and np.array_equal(bits(y), xres)
+    # a zero gate projection gives h = 0 whatever up is
+    _, _, h0 = ops.prefill_o_ffn(dev(attn), dev(xres), dev(nw), tuple(map(dev, wo)), tuple(map(dev, zero(wg))),
+                                 tuple(map(dev, wu)), tuple(map(dev, wd)), return_intermediates=True)
+    assert np.all((bits(h0) & 0x7FFF) == 0)
+
+
+def test_prefill_block_llama32_1b_size(ops):
+    """The reference example's dimensions (seq 2048, emb 2048, hidden 8192) against a float64 chain on the GPU."""
+    M, E, H = 2048, 2048, 8192
+    print("prefill block M=2048 E=2048 H=8192", flush=True)
+    wo, wg, wu, wd = _weights(E, H, seed=7, scale=0.1)
+    attn, xres, nw = make_x((M, E), seed=8), make_x((M, E), seed=9), _norm_w(E, 10)
+    y, res1, h = ops.prefill_o_ffn(dev(attn), dev(xres), dev(nw), tuple(map(dev, wo)), tuple(map(dev, wg)),
+                                   tuple(map(dev, wu)), tuple(map(dev, wd)), return_intermediates=True)
+    torch.cuda.synchronize()
+    d64 = lambda w: torch.from_numpy(dense_f64(*w, rounded=True)).cuda()
+    rnd = lambda t: t.to(torch.bfloat16).double()
+    res1_t = rnd(rnd(dev(attn).double() @ d64(wo)) + dev(xres).double())
+    err = (res1.double() - res1_t).abs()
+    assert float(err.max()) <= 2.0**-7 * float(res1_t.abs().max()) and float((err > 0).double().mean()) < 0.02
+    # the later stages on the kernel's own intermediates
+    n_t = rnd(torch.nn.functional.rms_norm(res1.double(), (E,), dev(nw).double(), eps=1e-5))
+    g_t, u_t = rnd(n_t @ d64(wg)), rnd(n_t @ d64(wu))
+    h_t = rnd(torch.nn.functional.silu(g_t) * u_t)
+    herr = (h.double() - h_t).abs()
+    assert float(herr.max()) <= 8 * 2.0**-8 * float(h_t.abs().max()) and float((herr > 0).double().mean()) < 0.1
+    y_t = rnd(rnd(h.double() @ d64(wd)) + res1.double())
+    yerr = (y.double() - y_t).abs()
+    assert float(yerr.max()) <= 2.0**-7 * float(y_t.abs().max()) and float((yerr > 0).double().mean()) < 0.02
+
+
+def test_prefill_block_rejects_bad_arguments(ops):
+    from air_hip import _lib
+    lib = _lib.load_library()
+    P = torch.zeros(1 << 16, dtype=torch.int32, device="cuda").data_ptr()
+    ws = lib.w4a16_prefill_block_workspace_bytes(32, 128, 128)
+    args = [P, P, P, 1e-5] + [P] * 12 + [P, None, None, 32, 128, 128, 128, P, ws, None]
+    bad = list(args); bad[24] = ws - 1
+    assert lib.w4a16_prefill_o_ffn_bf16(*bad) == _lib.ERR_WORKSPACE
+    bad = list(args); bad[20] = 100
+    assert lib.w4a16_prefill_o_ffn_bf16(*bad) == _lib.ERR_SHAPE
+    bad = list(args); bad[0] = None
+    assert lib.w4a16_prefill_o_ffn_bf16(*bad) == _lib.ERR_NULL
+    assert lib.rms_norm_rows_bf16(P, P, 1e-5, P, 4, 8200, None) == _lib.ERR_SHAPE

@@ -213,3 +213,52 @@ def test_check_outputs_semantics():
     assert not ref.check_outputs(a, e, rtol=0.1, atol=0.05, max_mismatch_percentage=0.49)  # int(4.9)=4
     # constant actual -> NaN correlation -> fail
     assert not ref.check_outputs(np.ones(10), np.ones(10), rtol=1, atol=1, min_correlation=0.5)
+
+
+def test_prefill_block_reference_against_library_and_closed_forms():
+    M, E, H, gs = 24, 256, 512, 128
+    _, oq, os_, oz, _ = _l1(E, E, gs, 60)
+    _, gq, gs_, gz, _ = _l1(H, E, gs, 61)
+    _, uq, us_, uz, _ = _l1(H, E, gs, 62)
+    _, dq, ds, dz, _ = _l1(E, H, gs, 63)
+    rng = np.random.default_rng(64)
+    attn = f32_to_bf16_bits(rng.standard_normal((M, E)).astype(np.float32))
+    xres = f32_to_bf16_bits(rng.standard_normal((M, E)).astype(np.float32))
+    w = f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32))
+    wo, wg, wu, wd = (oq, os_, oz), (gq, gs_, gz), (uq, us_, uz), (dq, ds, dz)
+    out, res1, h = ref.o_ffn_int4_prefill_reference(wo, wg, wu, wd, attn, xres, w)
+
+    # the same chain with library routines in float64 and one rounding per stage
+    def dense(l1, k):
+        return torch.from_numpy(ref._dequant_l1_f64(*l1, k).T.copy())          # [K, N] float64
+
+    def rnd(t):
+        return torch.from_numpy(bf16_bits_to_f32(f32_to_bf16_bits(t.float().numpy()))).double()
+
+    a, r = torch.from_numpy(bf16_bits_to_f32(attn)).double(), torch.from_numpy(bf16_bits_to_f32(xres)).double()
+    res1_t = rnd(rnd(a @ dense(wo, E)) + r)
+    n_t = rnd(torch.nn.functional.rms_norm(res1_t, (E,), torch.from_numpy(bf16_bits_to_f32(w)).double(), eps=1e-5))
+    g_t, u_t = rnd(n_t @ dense(wg, E)), rnd(n_t @ dense(wu, E))
+    h_t = rnd(torch.nn.functional.silu(g_t) * u_t)
+    out_t = rnd(rnd(h_t @ dense(wd, H)) + res1_t)
+    for got, want, name in ((res1, res1_t, "res1"), (h, h_t, "h"), (out, out_t, "out")):
+        g = bf16_bits_to_f32(got).astype(np.float64)
+        wv = want.numpy()
+        # float32 BLAS sums and one-ulp flips upstream: a few bf16 ulps of the tensor's scale, almost everywhere equal
+        assert np.max(np.abs(g - wv)) <= 4 * 2.0**-8 * np.max(np.abs(wv)), name
+        assert np.mean(g != wv) < 0.1, name
+    # Wo = 0 (z = q): res1 = x_residual exactly; Wdown = 0: out = res1
+    zo = (np.zeros_like(oq), os_, np.zeros_like(oz))
+    zd = (np.zeros_like(dq), ds, np.zeros_like(dz))
+    out0, res10, _ = ref.o_ffn_int4_prefill_reference(zo, wg, wu, zd, attn, xres, w)
+    assert np.array_equal(res10, xres) and np.array_equal(out0, xres)
+    # rows are independent: a row subset gives the same rows
+    out_s, res1_s, h_s = ref.o_ffn_int4_prefill_reference(wo, wg, wu, wd, attn[5:9], xres[5:9], w)
+    assert np.array_equal(out_s, out[5:9]) and np.array_equal(h_s, h[5:9])
+    # the row-wise norm against its closed form for constant rows (a sum instead of a mean would give 1 / sqrt(E))
+    c = np.float32(0.0078125)
+    n = bf16_bits_to_f32(ref.rms_norm_rows_bf16(f32_to_bf16_bits(np.full((3, E), c, np.float32)), np.full(E, 0x3F80, np.uint16)))
+    assert np.max(np.abs(n - float(c) / np.sqrt(float(c) ** 2 + 1e-5))) <= 2.0**-8
+    # gate = 0 gives h = 0 whatever up is (silu(0) = 0); the tanh form used by the decode kernels agrees with this one
+    gvals = np.linspace(-8, 8, 101).astype(np.float32)
+    assert np.allclose(gvals / (1 + np.exp(-gvals)), ref.silu_tanh_f32(gvals), rtol=1e-5, atol=1e-6)
