@@ -260,32 +260,52 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
     step(kt, stage0, stage1, rb[1], rb[0], T{}, F{}, F{});
     step(kt + 1, stage1, stage0, rb[0], rb[1], F{}, F{}, T{});
 
-    // D layout of the 32x32 MFMA: register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
-    // One copy of the store loop per epilogue, chosen by a uniform branch.
+    // D layout of the 32x32 MFMA: register r of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32:
+    // a lane holds a column, so stores straight from the registers are 2-byte stores in 64-byte runs
+    // (256 store instructions per thread, ~8 us per tile).  Instead the bf16 tile is transposed through
+    // LDS, which the K loop no longer needs (its last step ended with a barrier): rows padded to 528 B
+    // (the two row groups of a wave instruction, 4 rows apart, land 16 banks apart), then read back as
+    // 16-byte chunks so that a wave stores two whole 512-byte rows per instruction and the epilogue
+    // operand is loaded the same way.
+    constexpr int LDC = BN + 8;
+    static_assert((size_t)BM * LDC * sizeof(uint16_t) <= kLdsBytes, "the output tile must fit the K loop's LDS");
     auto store_tile = [&](auto EPI) {
+        uint16_t *ct = lds;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int col = n0 + wn * 128 + j * 32 + fr;
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * fk + (r & 3);
-                    if (row < p.M && col < p.N) {
-                        const size_t at = (size_t)row * p.N + col;
-                        uint16_t out = float_to_bf16_bits(acc[i][j][r]);
-                        if constexpr (decltype(EPI)::value == kEpiAddRounded) {
-                            // y = bf16(bf16(x . W) + R): the product is a bf16 tensor before the add
-                            out = float_to_bf16_bits(bf16_bits_to_float(out) + bf16_bits_to_float(p.aux[at]));
-                        } else if constexpr (decltype(EPI)::value == kEpiSiluGateMul) {
-                            // y = bf16(silu(G) * bf16(x . W)), silu(g) = g / (1 + exp(-g)) in fp32
-                            const float g = bf16_bits_to_float(p.aux[at]);
-                            out = float_to_bf16_bits(g / (1.0f + expf(-g)) * bf16_bits_to_float(out));
-                        }
-                        p.y[at] = out;
+                for (int r = 0; r < 16; ++r)
+                    ct[(wm * 128 + i * 32 + 8 * (r >> 2) + 4 * fk + (r & 3)) * LDC + wn * 128 + j * 32 + fr] =
+                        float_to_bf16_bits(acc[i][j][r]);
+        __syncthreads();
+#pragma unroll 4
+        for (int k = 0; k < BM * BN / 8 / kThreads; ++k) {
+            const int chunk = tid + kThreads * k;
+            const int row = chunk >> 5, c = chunk & 31;           // 32 chunks of 8 columns per row
+            const int grow = m0 + row, gcol = n0 + 8 * c;
+            if (grow >= p.M || gcol >= p.N) continue;             // N % 8 == 0: a chunk is inside or outside
+            u32x4 v = *reinterpret_cast<const u32x4 *>(&ct[row * LDC + 8 * c]);
+            const size_t at = (size_t)grow * p.N + gcol;
+            if constexpr (decltype(EPI)::value != kEpiNone) {
+                const u32x4 a = *reinterpret_cast<const u32x4 *>(p.aux + at);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t vw = v[e], aw = a[e];
+                    const float v0 = bf16_bits_to_float(vw & 0xFFFFu), v1 = bf16_bits_to_float(vw >> 16);
+                    const float a0 = bf16_bits_to_float(aw & 0xFFFFu), a1 = bf16_bits_to_float(aw >> 16);
+                    if constexpr (decltype(EPI)::value == kEpiAddRounded) {
+                        // y = bf16(bf16(x . W) + R): the product is a bf16 tensor before the add
+                        v[e] = pack_bf16x2(v0 + a0, v1 + a1);
+                    } else {
+                        // y = bf16(silu(G) * bf16(x . W)), silu(g) = g / (1 + exp(-g)) in fp32
+                        v[e] = pack_bf16x2(a0 / (1.0f + expf(-a0)) * v0, a1 / (1.0f + expf(-a1)) * v1);
                     }
                 }
             }
+            *reinterpret_cast<u32x4 *>(p.y + at) = v;
+        }
     };
     if (p.partial) {
         float *dst = p.partial + (size_t)blockIdx.y * p.M * p.N;
