@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|prefill_block]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -330,16 +330,24 @@ def run_prefill_block(steps, warmup):
     return {"us": sec * 1e6, "flops": flops, "TFLOP/s": flops / sec / 1e12, "finite": bool(torch.isfinite(y.float()).all())}
 
 
-def run_decode_model(steps, warmup):
+DECODE_MODELS = {
+    # Llama-3.2-1B (programming_examples/llms/llama32_1b/llama32_1b_weights.py:35-47) and Llama-3.1-8B
+    "decode_1b": dict(n_layers=16, emb_dim=2048, n_heads=32, head_dim=64, n_kv_heads=8, hidden_dim=8192, vocab_size=128256),
+    "decode_8b": dict(n_layers=32, emb_dim=4096, n_heads=32, head_dim=128, n_kv_heads=8, hidden_dim=14336, vocab_size=128256),
+}
+
+
+def run_decode_model(steps, warmup, model="decode_1b"):
     """Greedy decode of a random-weight model in the Llama-3.2-1B shape (16 layers, E=2048, H=8192,
-    32/8 heads of 64, vocabulary 128256, tied lm_head), `steps` consecutive tokens from position
-    DECODE_1B_POS0 captured as one HIP graph: per token 16 x (RMSNorm + QKV GEMV, attention,
-    O + FFN block) and the tail (final norm, lm_head GEMV, argmax), the token id staying on the device."""
+    32/8 heads of 64, vocabulary 128256, tied lm_head) or the Llama-3.1-8B shape, `steps` consecutive
+    tokens from position DECODE_1B_POS0 captured as one HIP graph: per token n_layers x (RMSNorm + QKV
+    GEMV, attention, O + FFN block) and the tail (final norm, lm_head GEMV, argmax), the token id
+    staying on the device."""
     import torch
 
     from air_hip import decode, weights as wmod
 
-    cfg = wmod.LlamaConfig()
+    cfg = wmod.LlamaConfig(**DECODE_MODELS[model])
     E, H, hd = cfg.emb_dim, cfg.hidden_dim, cfg.head_dim
     nqkv = (cfg.n_heads + 2 * cfg.n_kv_heads) * hd
     dev = torch.device("cuda:0")
@@ -487,7 +495,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b", "prefill_block"])
+    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b", "decode_8b", "prefill_block"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configs")
     ap.add_argument("--copy-probe", action="store_true",
@@ -522,17 +530,18 @@ def main():
                          "avg_launch_us": r["us"]},
             "finite": r["finite"]}))
         return
-    if a.workload == "decode_1b":
+    if a.workload in DECODE_MODELS:
         steps = min(a.steps, 64)
-        r = run_decode_model(steps, min(a.warmup, 8))
+        r = run_decode_model(steps, min(a.warmup, 8), a.workload)
+        m = DECODE_MODELS[a.workload]
         gbs = r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9
         print(json.dumps({
-            "metric": "int4 decode tokens/s, Llama-3.2-1B shape, batch 1", "value": r["tokens_per_s"], "unit": "tokens/s",
+            "metric": "int4 decode tokens/s, Llama-3.%s shape, batch 1" % ("2-1B" if a.workload == "decode_1b" else "1-8B"), "value": r["tokens_per_s"], "unit": "tokens/s",
             "n_gpus": 1, "steps": steps, "warmup": min(a.warmup, 8), "ms_per_step": r["us_per_token"] * 1e-3,
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "int4 weights (bf16 lm_head), bf16 activations, fp32 accumulate",
             "data": "synthetic (random weights of the architecture, random KV cache up to the start position)",
-            "config": {"workload": f"greedy decode, 16 layers E=2048 H=8192 32/8 heads hd=64 V=128256 g128, positions {DECODE_1B_POS0}..{DECODE_1B_POS0 + steps - 1}",
+            "config": {"workload": f"greedy decode, {m['n_layers']} layers E={m['emb_dim']} H={m['hidden_dim']} {m['n_heads']}/{m['n_kv_heads']} heads hd={m['head_dim']} V={m['vocab_size']} g128, positions {DECODE_1B_POS0}..{DECODE_1B_POS0 + steps - 1}",
                        "timing": "one HIP graph of all token steps, events on the launch stream"},
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                          "traffic": None, "algorithmic_per_launch": r["bytes_per_token"], "avg_launch_us": r["us_per_token"]},
@@ -595,10 +604,11 @@ def main():
                                 "frac_hbm_peak": r["bytes"] / s / 1e9 / HBM_PEAK_GBS, "hot_us": r["hot_us"]}
         r = run_prefill_block(10, 2)
         extra["prefill_block"] = {"us": r["us"], "TFLOP/s": r["TFLOP/s"], "frac_mfma_peak": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS}
-        r = run_decode_model(32, 4)
-        extra["decode_1b"] = {"us_per_token": r["us_per_token"], "tokens/s": r["tokens_per_s"],
-                              "GB/s": r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9,
-                              "frac_hbm_peak": r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9 / HBM_PEAK_GBS}
+        for model in DECODE_MODELS:
+            r = run_decode_model(32 if model == "decode_1b" else 16, 4, model)
+            extra[model] = {"us_per_token": r["us_per_token"], "tokens/s": r["tokens_per_s"],
+                            "GB/s": r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9,
+                            "frac_hbm_peak": r["bytes_per_token"] / (r["us_per_token"] * 1e-6) / 1e9 / HBM_PEAK_GBS}
         out["other_workloads"] = extra
     print(json.dumps(out))
 
