@@ -249,6 +249,25 @@ int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residua
                              void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Prefill counterpart of w4a16_rms_gemv_bf16 + the RoPE of w4a16_decode_attention_bf16 for M tokens at
+ * positions pos0 .. pos0 + M - 1: the reference's 6-launch ELF `rms_gemms_rope_int4`
+ * (programming_examples/llms/llama32_1b_int4/multi_launch_builder/rms_gemms_rope_int4_multi.py:4-17; CPU reference
+ * :414-436 and :543-561) as one RMSNorm launch and one GEMM over the Q|K|V weights concatenated along N:
+ *   normed   = bf16((x / sqrt(mean(x^2) + eps)) * attn_norm_weight)          per row, fp32
+ *   q, k, v  = bf16(normed . Wq), bf16(normed . Wk), bf16(normed . Wv)
+ *   q, k     = half-split RoPE per head with row pos0 + m of the table      (_rope_ref; fp32, one rounding)
+ * x bf16 [M, E]; qkv_out bf16 [M, (n_heads + 2 n_kv_heads) * head_dim] = Q | K | V per row; rope_lut bf16
+ * [rope_lut_rows, head_dim], cos then sin (generate_rope_lut), pos0 + M <= rope_lut_rows.  head_dim 64 or 128,
+ * E % 128 == 0, E <= 8192.  The workspace is plain scratch, w4a16_prefill_qkv_workspace_bytes(M, E) = 2 M E bytes.
+ */
+size_t w4a16_prefill_qkv_workspace_bytes(int M, int E);
+int w4a16_prefill_rms_qkv_rope_bf16(const uint16_t *x, const uint16_t *attn_norm_weight, float eps,
+                                    const int32_t *qkv_qweight, const int32_t *qkv_qzeros, const uint16_t *qkv_scales,
+                                    const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out,
+                                    int M, int E, int n_heads, int n_kv_heads, int head_dim, int group,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Tail of a decode step: final RMSNorm, bf16 lm_head GEMV and argmax in one call
  * (run_npu_decode_step, programming_examples/llms/llama32_1b_int4/llama32_1b_int4_inference.py:459-486:
  * host rms_norm, the `lm_head_gemv` kernel over 8 vocabulary partitions, np.argmax).

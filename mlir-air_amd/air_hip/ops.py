@@ -252,6 +252,26 @@ def rms_norm_rows(x, norm_weight, eps=1e-5):
     return out
 
 
+def prefill_rms_qkv_rope(x, attn_norm_weight, wqkv, rope_lut, pos0, n_heads, n_kv_heads, head_dim, eps=1e-5, group=GROUP):
+    """RMSNorm + fused Q|K|V projection + RoPE on the Q and K heads for M tokens at positions pos0..:
+    x bf16 [M, E] -> bf16 [M, (n_heads + 2 n_kv_heads) * head_dim].  wqkv is the AWQ triple of the
+    concatenated weights, rope_lut bf16 [positions, head_dim]."""
+    lib = _lib.load_library()
+    _need_cuda(x, attn_norm_weight, rope_lut)
+    M, E = x.shape
+    N = (n_heads + 2 * n_kv_heads) * head_dim
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    key = (x.device.index, _stream(), "prefill_qkv", M, E)
+    ws = _attn_ws.get(key)
+    if ws is None:
+        ws = torch.empty(int(lib.w4a16_prefill_qkv_workspace_bytes(M, E)), dtype=torch.uint8, device=x.device)
+        _attn_ws[key] = ws
+    _lib.check(lib.w4a16_prefill_rms_qkv_rope_bf16(_ptr(_bits(x)), _ptr(_bits(attn_norm_weight)), float(eps), *_wptrs(wqkv),
+                                                   _ptr(_bits(rope_lut)), rope_lut.shape[0], int(pos0), _ptr(out), M, E,
+                                                   n_heads, n_kv_heads, head_dim, group, _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
 def prefill_o_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, group=GROUP,
                   return_intermediates=False):
     """Prefill O projection + residual + RMSNorm + SwiGLU FFN + residual for M tokens: bf16 [M, E] -> [M, E].

@@ -388,6 +388,32 @@ int rms_norm_rows_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+size_t w4a16_prefill_qkv_workspace_bytes(int M, int E) {
+    return prefill_block_supported(M, E, 8) ? round256((size_t)M * E * sizeof(uint16_t)) : 0;
+}
+
+int w4a16_prefill_rms_qkv_rope_bf16(const uint16_t *x, const uint16_t *attn_norm_weight, float eps,
+                                    const int32_t *qkv_qweight, const int32_t *qkv_qzeros, const uint16_t *qkv_scales,
+                                    const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out, int M, int E,
+                                    int n_heads, int n_kv_heads, int head_dim, int group, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
+    if (!x || !attn_norm_weight || !rope_lut || !qkv_out) return W4A16_ERR_NULL;
+    if (head_dim != 64 && head_dim != 128) return W4A16_ERR_SHAPE;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads > 1024 || n_kv_heads > 1024) return W4A16_ERR_SHAPE;
+    const int N = (n_heads + 2 * n_kv_heads) * head_dim;
+    int rc = check_quant(qkv_qweight, qkv_qzeros, qkv_scales, E, N, group, 32);
+    if (rc) return rc;
+    if (!prefill_block_supported(M, E, 8) || !(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (pos0 < 0 || rope_lut_rows <= 0 || pos0 > rope_lut_rows - M) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(attn_norm_weight) || misaligned(rope_lut) || misaligned(qkv_out)) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_prefill_qkv_workspace_bytes(M, E)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_prefill_rms_qkv_rope(x, attn_norm_weight, eps, PrefillLinear{qkv_qweight, qkv_qzeros, qkv_scales},
+                                               rope_lut, pos0, qkv_out, M, E, n_heads, n_kv_heads, head_dim,
+                                               static_cast<uint16_t *>(workspace), static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
                              float eps, const int32_t *o_qweight, const int32_t *o_qzeros, const uint16_t *o_scales,
                              const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,

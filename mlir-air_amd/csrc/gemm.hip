@@ -52,6 +52,7 @@ struct GemmParams {
     int epi;               // kEpi*
     int M, K, N;
     int tiles_m, tiles_n;
+    int rope_cols, rope_hd, rope_pos0;   // kEpiRope: columns [0, rope_cols) are heads of rope_hd to rotate, row m is position rope_pos0 + m
     float *partial;        // split-K: fp32 [gridDim.y][M][N] partial products instead of y (nullptr: no split)
     int kt_per_split;      // K steps of 64 per blockIdx.y (even)
 };
@@ -288,7 +289,30 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
             if (grow >= p.M || gcol >= p.N) continue;             // N % 8 == 0: a chunk is inside or outside
             u32x4 v = *reinterpret_cast<const u32x4 *>(&ct[row * LDC + 8 * c]);
             const size_t at = (size_t)grow * p.N + gcol;
-            if constexpr (decltype(EPI)::value != kEpiNone) {
+            if constexpr (decltype(EPI)::value == kEpiRope) {
+                // Half-split rotation of the bf16 product: out[i] = x[i] cos[i] - x[i + h] sin[i],
+                // out[i + h] = x[i + h] cos[i] + x[i] sin[i]; the partner chunk is in the same tile
+                // (a tile is a whole number of heads).  Products of two bf16 values are exact in fp32,
+                // so each element is rounded once, fused multiply-add or not.
+                if (gcol < p.rope_cols) {
+                    const int hd = p.rope_hd, half = hd >> 1;
+                    const int i = gcol & (hd - 1);
+                    const bool low = i < half;
+                    const u32x4 w = *reinterpret_cast<const u32x4 *>(&ct[row * LDC + 8 * c + (low ? half : -half)]);
+                    const uint16_t *lut = p.aux + (size_t)(p.rope_pos0 + grow) * hd + (low ? i : i - half);
+                    const u32x4 cs = *reinterpret_cast<const u32x4 *>(lut), sn = *reinterpret_cast<const u32x4 *>(lut + half);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t vw = v[e], ww = w[e], cw = cs[e], sw = sn[e];
+                        const float x0 = bf16_bits_to_float(vw & 0xFFFFu), x1 = bf16_bits_to_float(vw >> 16);
+                        const float y0 = bf16_bits_to_float(ww & 0xFFFFu), y1 = bf16_bits_to_float(ww >> 16);
+                        const float c0 = bf16_bits_to_float(cw & 0xFFFFu), c1 = bf16_bits_to_float(cw >> 16);
+                        const float s0 = bf16_bits_to_float(sw & 0xFFFFu), s1 = bf16_bits_to_float(sw >> 16);
+                        v[e] = low ? pack_bf16x2(x0 * c0 - y0 * s0, x1 * c1 - y1 * s1)
+                                   : pack_bf16x2(x0 * c0 + y0 * s0, x1 * c1 + y1 * s1);
+                    }
+                }
+            } else if constexpr (decltype(EPI)::value != kEpiNone) {
                 const u32x4 a = *reinterpret_cast<const u32x4 *>(p.aux + at);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -324,6 +348,8 @@ __global__ void __launch_bounds__(kThreads, 1) gemm_kernel(const GemmParams p) {
         store_tile(std::integral_constant<int, kEpiAddRounded>{});
     else if (p.epi == kEpiSiluGateMul)
         store_tile(std::integral_constant<int, kEpiSiluGateMul>{});
+    else if (p.epi == kEpiRope)
+        store_tile(std::integral_constant<int, kEpiRope>{});
     else
         store_tile(std::integral_constant<int, kEpiNone>{});
 }
@@ -369,7 +395,7 @@ size_t gemm_prefill_splitk_bytes(int M, int K, int N, int cus) {
 
 hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
                                const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream,
-                               int epi, const uint16_t *aux, float *splitk_scratch, int cus) {
+                               int epi, const uint16_t *aux, float *splitk_scratch, int cus, const GemmRope *rope) {
     // 144 KiB of dynamic LDS needs the attribute; it is per device, so it is set on every launch
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
@@ -382,12 +408,17 @@ hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const 
     p.y = y;
     p.aux = aux;
     p.epi = aux ? epi : kEpiNone;
+    p.rope_cols = rope ? rope->cols : 0;
+    p.rope_hd = rope ? rope->head_dim : 64;
+    p.rope_pos0 = rope ? rope->pos0 : 0;
+    if (p.epi == kEpiRope && !rope) return hipErrorInvalidValue;
     p.M = M;
     p.K = K;
     p.N = N;
     p.tiles_m = (M + BM - 1) / BM;
     p.tiles_n = (N + BN - 1) / BN;
-    const int ksplit = splitk_scratch ? gemm_prefill_ksplit(M, K, N, cus) : 1;
+    // the reduction kernel of the split has no rotation epilogue
+    const int ksplit = splitk_scratch && p.epi != kEpiRope ? gemm_prefill_ksplit(M, K, N, cus) : 1;
     p.partial = ksplit > 1 ? splitk_scratch : nullptr;
     p.kt_per_split = K / BK / ksplit;
     const int total = p.tiles_m * p.tiles_n;

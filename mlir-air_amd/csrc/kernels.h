@@ -62,13 +62,18 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
 // Prefill GEMM (M > 16) with an optional epilogue on a second bf16 [M, N] operand `aux`:
 //   kEpiAddRounded   y = bf16(bf16(x . W) + aux)            (residual add of a bf16 product)
 //   kEpiSiluGateMul  y = bf16(silu(aux) * bf16(x . W))      (SwiGLU with aux = the gate projection)
-enum : int { kEpiNone = 0, kEpiAddRounded = 1, kEpiSiluGateMul = 2 };
+//   kEpiRope         half-split RoPE of the bf16 product on columns [0, rope.cols) (whole heads of rope.head_dim,
+//                    64 or 128), aux = the LUT [positions, head_dim] (cos then sin), row m at position rope.pos0 + m
+enum : int { kEpiNone = 0, kEpiAddRounded = 1, kEpiSiluGateMul = 2, kEpiRope = 3 };
+struct GemmRope {
+    int cols, head_dim, pos0;
+};
 // With `splitk_scratch` (plain scratch of gemm_prefill_splitk_bytes) a launch with few tiles is cut into 2 or 4
 // slices along K whose fp32 partial products a second kernel sums before the epilogue.
 hipError_t launch_gemm_prefill(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
                                const uint16_t *scales, uint16_t *y, int M, int K, int N, hipStream_t stream,
                                int epi = kEpiNone, const uint16_t *aux = nullptr, float *splitk_scratch = nullptr,
-                               int cus = 0);
+                               int cus = 0, const GemmRope *rope = nullptr);
 int gemm_prefill_ksplit(int M, int K, int N, int cus);
 size_t gemm_prefill_splitk_bytes(int M, int K, int N, int cus);
 
@@ -83,6 +88,10 @@ struct PrefillLinear {
 bool prefill_block_supported(int M, int E, int H);
 size_t prefill_block_scratch_bytes(int M, int E, int H);   // sized for split-K on a 256-CU device
 hipError_t launch_rmsnorm_rows(const uint16_t *x, const uint16_t *w, uint16_t *out, int M, int K, float eps, hipStream_t stream);
+// RMSNorm rows + fused Q|K|V GEMM + RoPE on the Q and K heads (prefill_block.hip); `normed` [M, E] is scratch.
+hipError_t launch_prefill_rms_qkv_rope(const uint16_t *x, const uint16_t *norm_w, float eps, const PrefillLinear &wqkv,
+                                       const uint16_t *rope_lut, int pos0, uint16_t *qkv_out, int M, int E, int n_heads,
+                                       int n_kv, int head_dim, uint16_t *normed, hipStream_t stream);
 hipError_t launch_prefill_o_ffn(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_w, float eps,
                                 const PrefillLinear &wo, const PrefillLinear &wg, const PrefillLinear &wu,
                                 const PrefillLinear &wd, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,

@@ -94,6 +94,20 @@ hipError_t launch_rmsnorm_rows(const uint16_t *x, const uint16_t *w, uint16_t *o
     return hipGetLastError();
 }
 
+// The reference's 6-launch prefill ELF rms_gemms_rope_int4
+// (programming_examples/llms/llama32_1b_int4/multi_launch_builder/rms_gemms_rope_int4_multi.py:4-17, CPU reference
+// :414-436, 543-561) as two launches: row-wise RMSNorm, then one GEMM over the Q|K|V weights concatenated along
+// N whose epilogue rotates the Q and K heads (row m at position pos0 + m).
+hipError_t launch_prefill_rms_qkv_rope(const uint16_t *x, const uint16_t *norm_w, float eps, const PrefillLinear &wqkv,
+                                       const uint16_t *rope_lut, int pos0, uint16_t *qkv_out, int M, int E, int n_heads,
+                                       int n_kv, int head_dim, uint16_t *normed, hipStream_t stream) {
+    hipError_t e = launch_rmsnorm_rows(x, norm_w, normed, M, E, eps, stream);
+    if (e != hipSuccess) return e;
+    const GemmRope rope = {(n_heads + n_kv) * head_dim, head_dim, pos0};
+    return launch_gemm_prefill(normed, wqkv.qw, wqkv.qz, wqkv.sc, qkv_out, M, E, (n_heads + 2 * n_kv) * head_dim, stream,
+                               kEpiRope, rope_lut, nullptr, 0, &rope);
+}
+
 hipError_t launch_prefill_o_ffn(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_w, float eps,
                                 const PrefillLinear &wo, const PrefillLinear &wg, const PrefillLinear &wu,
                                 const PrefillLinear &wd, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,

@@ -16,6 +16,11 @@ Follows (LLM = programming_examples/llms):
   decode_block_reference run_decode_block (llama32_1b_int4_decode.py:176-313): the call above,
                          KV-cache append, attention, then the O + FFN block
 
+  rope_rows, prefill_rms_qkv_rope_reference
+                         the CPU reference of the 6-launch prefill ELF rms_gemms_rope_int4
+                         (LLM/llama32_1b_int4/multi_launch_builder/rms_gemms_rope_int4_multi.py:414-436,
+                         543-561): row-wise RMSNorm to bf16, three matmul_int4_packed products to bf16,
+                         half-split RoPE of every Q and K head with the LUT row of the token's position
   lm_head_reference      the tail of run_npu_decode_step
                          (LLM/llama32_1b_int4/llama32_1b_int4_inference.py:459-486): host rms_norm
                          in float32 (LLM/llama32_1b/llama32_1b_cpu_helpers.py:25-39,
@@ -25,6 +30,8 @@ Follows (LLM = programming_examples/llms):
 bf16 tensors are uint16 bit patterns.  Pins (tests/test_oracle_decode.py): RoPE against a complex
 rotation and its norm/inverse identities; the LUT against closed forms (pos 0, index 0); attention
 against torch's scaled_dot_product_attention and the closed forms seq_len = 1 and equal keys; the
+per-row RoPE against the complex rotation by the position's angles and, for equal LUT rows, against
+rope_halfsplit; the prefill QKV reference against its stages and the decode-step reference row by row; the
 lm_head tail against torch's rms_norm and matmul in float64, one-hot rows (logits = the normalised
 vector), a constant vector (closed-form norm) and tied rows (first index wins).
 """
@@ -121,3 +128,30 @@ def lm_head_reference(x_bits, final_norm_bits, lm_head_bits, eps=1e-5):
     acc = w @ bf16_bits_to_f32(normed).astype(np.float64)
     logits = f32_to_bf16_bits(acc.astype(np.float32))
     return logits, int(np.argmax(bf16_bits_to_f32(logits).astype(np.float32)))
+
+
+def rope_rows(x_bits, lut_bits):
+    """x bf16 bits [rows, dim] rotated with its own LUT row each (lut bf16 bits [rows, dim], cos then sin)."""
+    x = bf16_bits_to_f32(np.asarray(x_bits)).astype(np.float32)
+    lut = bf16_bits_to_f32(np.asarray(lut_bits)).astype(np.float32)
+    half = x.shape[1] // 2
+    cos, sin = lut[:, :half], lut[:, half:]
+    x1, x2 = x[:, :half], x[:, half:]
+    out = np.empty_like(x)
+    out[:, :half] = x1 * cos - x2 * sin
+    out[:, half:] = x2 * cos + x1 * sin
+    return f32_to_bf16_bits(out)
+
+
+def prefill_rms_qkv_rope_reference(x_bits, norm_w_bits, wq_l1, wk_l1, wv_l1, lut_bits, pos0, n_heads, n_kv_heads,
+                                   head_dim, eps=1e-5, **matmul_kw):
+    """bf16 bits [M, (n_heads + 2 n_kv_heads) * head_dim] = roped Q | roped K | V for tokens at positions pos0.."""
+    M = np.asarray(x_bits).shape[0]
+    normed = ref.rms_norm_rows_bf16(x_bits, norm_w_bits, eps)
+    q = ref.matmul_cpu_reference(*wq_l1, normed, **matmul_kw)
+    k = ref.matmul_cpu_reference(*wk_l1, normed, **matmul_kw)
+    v = ref.matmul_cpu_reference(*wv_l1, normed, **matmul_kw)
+    rows = np.asarray(lut_bits)[pos0:pos0 + M]
+    q = rope_rows(q.reshape(M * n_heads, head_dim), np.repeat(rows, n_heads, axis=0)).reshape(M, -1)
+    k = rope_rows(k.reshape(M * n_kv_heads, head_dim), np.repeat(rows, n_kv_heads, axis=0)).reshape(M, -1)
+    return np.concatenate([q, k, v], axis=1)

@@ -35,6 +35,15 @@ def ops():
     return ops
 
 
+@pytest.fixture
+def tiled_gemm(ops):
+    """w4a16_gemm runs the tiled prefill kernel for every M > 16, so that its output can be compared bit for bit
+    with the product inside the fused prefill calls (the streaming kernel sums in another order)."""
+    ops.tune("gemm_stream_max_m", 16)
+    yield
+    ops.tune("gemm_stream_max_m", 0)
+
+
 def _weights(E, H, seed, scale=1.0):
     out = []
     for i, (K, N) in enumerate(((E, E), (E, H), (E, H), (H, E))):
@@ -147,3 +156,89 @@ def test_prefill_block_rejects_bad_arguments(ops):
     bad = list(args); bad[0] = None
     assert lib.w4a16_prefill_o_ffn_bf16(*bad) == _lib.ERR_NULL
     assert lib.rms_norm_rows_bf16(P, P, 1e-5, P, 4, 8200, None) == _lib.ERR_SHAPE
+
+
+def _qkv_weights(E, nh, nkv, hd, seed, scale=0.25):
+    parts = []
+    for i, N in enumerate((nh * hd, nkv * hd, nkv * hd)):
+        qw, qz, s = make_awq(E, N, seed=seed + i)
+        parts.append((qw, qz, f32_to_bf16_bits(bf16_bits_to_f32(s) * np.float32(scale))))
+    fused = tuple(np.concatenate([p[j] for p in parts], axis=1) for j in range(3))
+    return parts, fused
+
+
+@pytest.mark.parametrize("M,E,nh,nkv,hd,pos0", [(40, 256, 4, 2, 64, 0), (300, 512, 8, 8, 64, 7), (130, 256, 2, 1, 128, 100),
+                                                 (17, 128, 3, 1, 64, 1)])
+def test_prefill_rms_qkv_rope(ops, tiled_gemm, M, E, nh, nkv, hd, pos0):
+    from oracle import decode as odec
+    print(f"prefill qkv rope M={M} E={E} heads {nh}/{nkv} hd={hd} pos0={pos0}", flush=True)
+    parts, fused = _qkv_weights(E, nh, nkv, hd, seed=M + E)
+    x, nw = make_x((M, E), seed=M + 3), _norm_w(E, M + 4)
+    lut = odec.generate_rope_lut(hd, 500000.0, pos0 + M + 5)
+    dw = tuple(map(dev, fused))
+    out = ops.prefill_rms_qkv_rope(dev(x), dev(nw), dw, dev(lut), pos0, nh, nkv, hd)
+    normed = ops.rms_norm_rows(dev(x), dev(nw))
+    plain = ops.w4a16_gemm(normed, *dw)
+    torch.cuda.synchronize()
+    got = bits(out)
+    f = lambda b: bf16_bits_to_f32(b).astype(np.float64)
+    nq, nk = nh * hd, nkv * hd
+    # V columns are the plain product, bit for bit the GEMM entry point's
+    assert np.array_equal(got[:, nq + nk:], bits(plain)[:, nq + nk:])
+    # Q and K: the rotation of the kernel's own bf16 product is reproduced exactly by the oracle's rotation
+    rows = lut[pos0:pos0 + M]
+    for lo, n in ((0, nh), (nq, nkv)):
+        prod = bits(plain)[:, lo:lo + n * hd].reshape(M * n, hd)
+        want = odec.rope_rows(prod, np.repeat(rows, n, axis=0)).reshape(M, n * hd)
+        assert np.array_equal(got[:, lo:lo + n * hd], want)
+    # and the whole call against the restated CPU reference (float32 BLAS products, one-ulp flips upstream)
+    l1 = [oawq.repack_hf_awq_linear(*w, 128) for w in parts]
+    ref_out = odec.prefill_rms_qkv_rope_reference(x, nw, *l1, lut, pos0, nh, nkv, hd)
+    err = np.abs(f(got) - f(ref_out))
+    assert np.max(err) <= 4 * 2.0**-8 * np.max(np.abs(f(ref_out))), err.max()
+    # with the weights rounded to bf16 first, as the kernel's tiles hold them, most outputs agree bit for bit
+    ref_r = odec.prefill_rms_qkv_rope_reference(x, nw, *l1, lut, pos0, nh, nkv, hd, round_weights=True)
+    assert np.mean(got != ref_r) < 0.1, np.mean(got != ref_r)
+
+
+def test_prefill_rms_qkv_rope_position_zero_is_the_identity(ops, tiled_gemm):
+    """Every row at position 0 (a one-row table, cos = 1, sin = 0) leaves Q and K unrotated: the fused call equals
+    RMSNorm + plain GEMM bit for bit; and shifting pos0 equals shifting the table."""
+    from oracle import decode as odec
+    E, nh, nkv, hd = 256, 4, 2, 64
+    _, fused = _qkv_weights(E, nh, nkv, hd, seed=5)
+    dw = tuple(map(dev, fused))
+    nw = _norm_w(E, 6)
+    lut = odec.generate_rope_lut(hd, 500000.0, 64)
+    x = make_x((40, E), seed=7)
+    print("prefill qkv rope, position 0 and shifted tables", flush=True)
+    plain = ops.w4a16_gemm(ops.rms_norm_rows(dev(x), dev(nw)), *dw)
+    for m in (0, 17, 39):
+        one = ops.prefill_rms_qkv_rope(dev(x[m:m + 1]), dev(nw), dw, dev(lut[:1]), 0, nh, nkv, hd)
+        assert torch.equal(one.view(torch.int16), plain[m:m + 1].view(torch.int16))
+    a = ops.prefill_rms_qkv_rope(dev(x), dev(nw), dw, dev(lut), 9, nh, nkv, hd)
+    b = ops.prefill_rms_qkv_rope(dev(x), dev(nw), dw, dev(lut[9:]), 0, nh, nkv, hd)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_prefill_rms_qkv_rope_llama32_1b_size(ops, tiled_gemm):
+    from oracle import decode as odec
+    M, E, nh, nkv, hd = 2048, 2048, 32, 8, 64
+    print("prefill qkv rope M=2048 E=2048 32/8 heads", flush=True)
+    _, fused = _qkv_weights(E, nh, nkv, hd, seed=15, scale=0.1)
+    dw = tuple(map(dev, fused))
+    x, nw = make_x((M, E), seed=16), _norm_w(E, 17)
+    lut = odec.generate_rope_lut(hd, 500000.0, M)
+    out = ops.prefill_rms_qkv_rope(dev(x), dev(nw), dw, dev(lut), 0, nh, nkv, hd)
+    plain = ops.w4a16_gemm(ops.rms_norm_rows(dev(x), dev(nw)), *dw)
+    torch.cuda.synchronize()
+    got, prod = bits(out), bits(plain)
+    nq = nh * hd
+    want_q = odec.rope_rows(prod[:, :nq].reshape(M * nh, hd), np.repeat(lut, nh, axis=0)).reshape(M, nq)
+    assert np.array_equal(got[:, :nq], want_q)
+    assert np.array_equal(got[:, nq + nkv * hd:], prod[:, nq + nkv * hd:])
+    # rotations preserve the norm of every (i, i + 32) pair up to the bf16 roundings
+    g = bf16_bits_to_f32(got[:, :nq]).reshape(M, nh, 2, hd // 2).astype(np.float64)
+    p = bf16_bits_to_f32(prod[:, :nq]).reshape(M, nh, 2, hd // 2).astype(np.float64)
+    n_g, n_p = np.sqrt((g**2).sum(axis=2)), np.sqrt((p**2).sum(axis=2))
+    assert np.max(np.abs(n_g - n_p)) <= 2.0**-6 * np.max(n_p)

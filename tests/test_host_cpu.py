@@ -175,6 +175,25 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     bad = list(args)
     bad[16] = fws - 1
     assert lib.w4a16_ffn_swiglu_bf16(*bad) == _lib.ERR_WORKSPACE
+    qws = lib.w4a16_prefill_qkv_workspace_bytes(64, 256)
+    assert qws >= 64 * 256 * 2 and lib.w4a16_prefill_qkv_workspace_bytes(64, 8200) == 0
+    qargs = [P, P, 1e-5, P, P, P, P, 128, 0, P, 64, 256, 4, 2, 64, 128, P, qws, None]
+    bad = list(qargs); bad[14] = 96
+    assert lib.w4a16_prefill_rms_qkv_rope_bf16(*bad) == _lib.ERR_SHAPE        # head_dim 64 or 128
+    bad = list(qargs); bad[8] = 65
+    assert lib.w4a16_prefill_rms_qkv_rope_bf16(*bad) == _lib.ERR_SHAPE        # pos0 + M beyond the table
+    bad = list(qargs); bad[17] = qws - 1
+    assert lib.w4a16_prefill_rms_qkv_rope_bf16(*bad) == _lib.ERR_WORKSPACE
+    bad = list(qargs); bad[6] = None
+    assert lib.w4a16_prefill_rms_qkv_rope_bf16(*bad) == _lib.ERR_NULL
+    pws = lib.w4a16_prefill_block_workspace_bytes(64, 256, 512)
+    assert pws >= 4 * 64 * (256 + 512)
+    pargs = [P, P, P, 1e-5] + [P] * 12 + [P, None, None, 64, 256, 512, 128, P, pws, None]
+    bad = list(pargs); bad[21] = 500
+    assert lib.w4a16_prefill_o_ffn_bf16(*bad) == _lib.ERR_SHAPE
+    bad = list(pargs); bad[24] = pws - 1
+    assert lib.w4a16_prefill_o_ffn_bf16(*bad) == _lib.ERR_WORKSPACE
+    assert lib.rms_norm_rows_bf16(P, P, 1e-5, P, 4, 100, None) == _lib.ERR_SHAPE    # K % 8
     lws = lib.lm_head_workspace_bytes(100)
     assert lws >= 8 * 7 and lib.lm_head_workspace_bytes(0) == 0
     assert lib.lm_head_gemv_bf16(P, None, 0.0, P, None, None, 100, 512, P, lws, None) == _lib.ERR_NULL

@@ -104,3 +104,46 @@ def test_lm_head_tail_against_library_and_closed_forms():
     zeros = np.zeros((4, E), np.uint16)
     zeros[0, 0] = 0x8000          # -0 * x: logits -0 or +0, all equal as floats
     assert dec.lm_head_reference(x, nw, zeros)[1] == 0
+
+
+def _l1(M, K, gs, seed):
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 16, size=(M, K), dtype=np.uint8)
+    a_q = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)
+    a_s = f32_to_bf16_bits(rng.uniform(0.005, 0.02, size=(K // gs, M)).astype(np.float32))
+    a_z = rng.integers(0, 16, size=(K // gs, M), dtype=np.uint8)
+    return a_q, a_s, a_z
+
+
+def test_prefill_qkv_rope_reference_against_its_stages_and_the_decode_step():
+    from oracle import reference as ref
+
+    M, E, nh, nkv, hd, pos0 = 6, 256, 4, 2, 64, 3
+    rng = np.random.default_rng(80)
+    x = f32_to_bf16_bits(rng.standard_normal((M, E)).astype(np.float32))
+    nw = f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32))
+    wq, wk, wv = _l1(nh * hd, E, 128, 81), _l1(nkv * hd, E, 128, 82), _l1(nkv * hd, E, 128, 83)
+    lut = dec.generate_rope_lut(hd, 500000.0, 16)
+    out = dec.prefill_rms_qkv_rope_reference(x, nw, wq, wk, wv, lut, pos0, nh, nkv, hd)
+    assert out.shape == (M, (nh + 2 * nkv) * hd)
+    # per-row rotation: the complex rotation by that row's angles; equal LUT rows reduce to rope_halfsplit
+    xr = f32_to_bf16_bits(rng.standard_normal((5, hd)).astype(np.float32))
+    rows = lut[[1, 4, 4, 9, 0]]
+    got = bf16_bits_to_f32(dec.rope_rows(xr, rows))
+    xf, l = bf16_bits_to_f32(xr).astype(np.float64), bf16_bits_to_f32(rows).astype(np.float64)
+    z = (xf[:, :32] + 1j * xf[:, 32:]) * (l[:, :32] + 1j * l[:, 32:])
+    assert np.max(np.abs(got - np.concatenate([z.real, z.imag], axis=1))) <= 2.0**-8 * np.max(np.abs(xf)) * 1.5
+    assert np.array_equal(dec.rope_rows(xr, np.repeat(lut[7:8], 5, axis=0)), dec.rope_halfsplit(xr, lut[7]))
+    assert np.array_equal(dec.rope_rows(xr, rows)[4], xr[4])                      # position 0 is the identity
+    # stages: V is the plain product of the normalised rows; Q of row m is rope(product) with LUT row pos0 + m
+    normed = ref.rms_norm_rows_bf16(x, nw)
+    assert np.array_equal(out[:, (nh + nkv) * hd:], ref.matmul_cpu_reference(*wv, normed))
+    qm = ref.matmul_cpu_reference(*wq, normed)
+    for m in (0, M - 1):
+        assert np.array_equal(out[m, :nh * hd].reshape(nh, hd), dec.rope_halfsplit(qm[m].reshape(nh, hd), lut[pos0 + m]))
+    # a single row is what the decode-step reference computes for that token (GEMV = one-row GEMM up to
+    # the float32 BLAS summation order and the norm's x * rstd against x / rms: a few one-ulp flips)
+    m = 2
+    one = dec.rms_qkv_rope_reference(x[m], nw, wq, wk, wv, lut[pos0 + m], nh, nkv, hd)
+    a, b = bf16_bits_to_f32(np.concatenate([np.ravel(t) for t in one])), bf16_bits_to_f32(out[m])
+    assert a.shape == b.shape and np.max(np.abs(a - b)) <= 2.0**-6 * np.max(np.abs(b)) and np.mean(a != b) < 0.2
