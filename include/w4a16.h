@@ -268,6 +268,18 @@ int w4a16_prefill_rms_qkv_rope_bf16(const uint16_t *x, const uint16_t *attn_norm
                                     void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Causal grouped-query attention over the M tokens of a prefill: the `flash_attn` step between the two prefill ELFs
+ * (programming_examples/llms/llama32_1b_int4/llama32_1b_int4_prefill.py:302-326; CPU form attention_reference,
+ * programming_examples/llms/llama32_1b/llama32_1b_cpu_helpers.py:50-88: softmax(Q K^T / sqrt(head_dim) + causal
+ * mask) V per head, query head h reading KV head h / (n_heads / n_kv_heads)).
+ * qkv bf16 [M, (n_heads + 2 n_kv_heads) * head_dim] is the output of w4a16_prefill_rms_qkv_rope_bf16 (roped Q | roped
+ * K | V per row); attn_out bf16 [M, n_heads * head_dim].  Token m attends to tokens 0..m of the same call (no earlier
+ * cache).  fp32 softmax with the probabilities rounded to bf16 for the P.V product.  head_dim 64 or 128.
+ */
+int w4a16_prefill_attention_bf16(const uint16_t *qkv, uint16_t *attn_out, int M, int n_heads, int n_kv_heads,
+                                 int head_dim, void *stream);
+
+/*
  * Tail of a decode step: final RMSNorm, bf16 lm_head GEMV and argmax in one call
  * (run_npu_decode_step, programming_examples/llms/llama32_1b_int4/llama32_1b_int4_inference.py:459-486:
  * host rms_norm, the `lm_head_gemv` kernel over 8 vocabulary partitions, np.argmax).

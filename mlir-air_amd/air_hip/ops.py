@@ -272,6 +272,19 @@ def prefill_rms_qkv_rope(x, attn_norm_weight, wqkv, rope_lut, pos0, n_heads, n_k
     return out
 
 
+def prefill_attention(qkv, n_heads, n_kv_heads, head_dim):
+    """Causal GQA attention over the M rows of qkv bf16 [M, (n_heads + 2 n_kv_heads) * head_dim] (roped Q | roped K | V):
+    returns bf16 [M, n_heads * head_dim]."""
+    lib = _lib.load_library()
+    _need_cuda(qkv)
+    M = qkv.shape[0]
+    if qkv.shape[1] != (n_heads + 2 * n_kv_heads) * head_dim:
+        raise ValueError("qkv must be [M, (n_heads + 2 n_kv_heads) * head_dim]")
+    out = torch.empty((M, n_heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    _lib.check(lib.w4a16_prefill_attention_bf16(_ptr(_bits(qkv)), _ptr(out), M, n_heads, n_kv_heads, head_dim, _stream()))
+    return out
+
+
 def prefill_o_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, group=GROUP,
                   return_intermediates=False):
     """Prefill O projection + residual + RMSNorm + SwiGLU FFN + residual for M tokens: bf16 [M, E] -> [M, E].

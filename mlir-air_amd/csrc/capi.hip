@@ -414,6 +414,16 @@ int w4a16_prefill_rms_qkv_rope_bf16(const uint16_t *x, const uint16_t *attn_norm
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+int w4a16_prefill_attention_bf16(const uint16_t *qkv, uint16_t *attn_out, int M, int n_heads, int n_kv_heads, int head_dim,
+                                 void *stream) {
+    if (!qkv || !attn_out) return W4A16_ERR_NULL;
+    if (head_dim != 64 && head_dim != 128) return W4A16_ERR_SHAPE;
+    if (M <= 0 || n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || n_heads > 65535) return W4A16_ERR_SHAPE;
+    if (misaligned(qkv) || misaligned(attn_out)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_prefill_attention(qkv, attn_out, M, n_heads, n_kv_heads, head_dim, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
                              float eps, const int32_t *o_qweight, const int32_t *o_qzeros, const uint16_t *o_scales,
                              const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,

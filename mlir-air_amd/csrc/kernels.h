@@ -88,6 +88,9 @@ struct PrefillLinear {
 bool prefill_block_supported(int M, int E, int H);
 size_t prefill_block_scratch_bytes(int M, int E, int H);   // sized for split-K on a 256-CU device
 hipError_t launch_rmsnorm_rows(const uint16_t *x, const uint16_t *w, uint16_t *out, int M, int K, float eps, hipStream_t stream);
+// Causal GQA attention over the M rows of a prefill (prefill_attention.hip); qkv is [M, (n_heads + 2 n_kv) * head_dim].
+hipError_t launch_prefill_attention(const uint16_t *qkv, uint16_t *attn_out, int M, int n_heads, int n_kv, int head_dim,
+                                    hipStream_t stream);
 // RMSNorm rows + fused Q|K|V GEMM + RoPE on the Q and K heads (prefill_block.hip); `normed` [M, E] is scratch.
 hipError_t launch_prefill_rms_qkv_rope(const uint16_t *x, const uint16_t *norm_w, float eps, const PrefillLinear &wqkv,
                                        const uint16_t *rope_lut, int pos0, uint16_t *qkv_out, int M, int E, int n_heads,

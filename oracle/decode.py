@@ -21,6 +21,8 @@ Follows (LLM = programming_examples/llms):
                          (LLM/llama32_1b_int4/multi_launch_builder/rms_gemms_rope_int4_multi.py:414-436,
                          543-561): row-wise RMSNorm to bf16, three matmul_int4_packed products to bf16,
                          half-split RoPE of every Q and K head with the LUT row of the token's position
+  prefill_attention_reference  attention_reference (LLM/llama32_1b/llama32_1b_cpu_helpers.py:50-88): causal GQA
+                         attention over the tokens of a prefill, float32 softmax per head
   lm_head_reference      the tail of run_npu_decode_step
                          (LLM/llama32_1b_int4/llama32_1b_int4_inference.py:459-486): host rms_norm
                          in float32 (LLM/llama32_1b/llama32_1b_cpu_helpers.py:25-39,
@@ -155,3 +157,23 @@ def prefill_rms_qkv_rope_reference(x_bits, norm_w_bits, wq_l1, wk_l1, wv_l1, lut
     q = rope_rows(q.reshape(M * n_heads, head_dim), np.repeat(rows, n_heads, axis=0)).reshape(M, -1)
     k = rope_rows(k.reshape(M * n_kv_heads, head_dim), np.repeat(rows, n_kv_heads, axis=0)).reshape(M, -1)
     return np.concatenate([q, k, v], axis=1)
+
+
+def prefill_attention_reference(q_bits, k_bits, v_bits, n_heads, n_kv_heads):
+    """q [M, n_heads * hd], k, v [M, n_kv_heads * hd] bf16 bits -> float32 [M, n_heads * hd]."""
+    q, k, v = (bf16_bits_to_f32(np.asarray(t)).astype(np.float32) for t in (q_bits, k_bits, v_bits))
+    M = q.shape[0]
+    hd = q.shape[1] // n_heads
+    group = n_heads // n_kv_heads
+    q = q.reshape(M, n_heads, hd).transpose(1, 0, 2)
+    k = k.reshape(M, n_kv_heads, hd).transpose(1, 0, 2)
+    v = v.reshape(M, n_kv_heads, hd).transpose(1, 0, 2)
+    scale = np.float32(1.0 / np.sqrt(hd))
+    mask = np.triu(np.full((M, M), -np.inf, dtype=np.float32), k=1)
+    out = np.empty((n_heads, M, hd), dtype=np.float32)
+    for h in range(n_heads):
+        scores = q[h] @ k[h // group].T * scale + mask
+        probs = np.exp(scores - scores.max(axis=-1, keepdims=True))
+        probs = probs / probs.sum(axis=-1, keepdims=True)
+        out[h] = probs @ v[h // group]
+    return out.transpose(1, 0, 2).reshape(M, n_heads * hd)

@@ -242,3 +242,62 @@ def test_prefill_rms_qkv_rope_llama32_1b_size(ops, tiled_gemm):
     p = bf16_bits_to_f32(prod[:, :nq]).reshape(M, nh, 2, hd // 2).astype(np.float64)
     n_g, n_p = np.sqrt((g**2).sum(axis=2)), np.sqrt((p**2).sum(axis=2))
     assert np.max(np.abs(n_g - n_p)) <= 2.0**-6 * np.max(n_p)
+
+
+@pytest.mark.parametrize("M,nh,nkv,hd", [(40, 4, 2, 64), (64, 2, 2, 64), (65, 4, 1, 128), (300, 8, 2, 64), (1, 2, 1, 64),
+                                         (200, 8, 1, 128), (33, 3, 3, 64)])
+def test_prefill_attention(ops, M, nh, nkv, hd):
+    from oracle import decode as odec
+    print(f"prefill attention M={M} heads {nh}/{nkv} hd={hd}", flush=True)
+    rng = np.random.default_rng(M + nh + hd)
+    qkv = f32_to_bf16_bits(rng.standard_normal((M, (nh + 2 * nkv) * hd)).astype(np.float32))
+    out = ops.prefill_attention(dev(qkv), nh, nkv, hd)
+    torch.cuda.synchronize()
+    nq, nk = nh * hd, nkv * hd
+    want = odec.prefill_attention_reference(qkv[:, :nq], qkv[:, nq:nq + nk], qkv[:, nq + nk:], nh, nkv)
+    got = bf16_bits_to_f32(bits(out)).astype(np.float64)
+    # probabilities are rounded to bf16 before the P.V product: each of up to M terms carries 2^-9 relative error
+    # (errors of random sign), plus the output rounding
+    tol = bf16_ulp(want) + 2.0**-8 * np.max(np.abs(bf16_bits_to_f32(qkv[:, nq + nk:]))) + 1e-3
+    assert np.all(np.abs(got - want) <= tol), np.max(np.abs(got - want) - tol)
+    # the first token attends to itself only: its output is its V row, bit for bit (P = 1)
+    v0 = qkv[0, nq + nk:].reshape(nkv, hd).repeat(nh // nkv, axis=0).reshape(-1)
+    assert np.array_equal(bits(out)[0], v0)
+
+
+def test_prefill_attention_matches_the_decode_kernel_row_by_row(ops):
+    """Row m of the prefill attention against the single-query decode kernel at position m over the same keys
+    (that kernel applies RoPE itself, so it is fed unrotated rows and a position-0 table row)."""
+    from oracle import decode as odec
+    M, nh, nkv, hd = 150, 8, 2, 64
+    rng = np.random.default_rng(3)
+    qkv = f32_to_bf16_bits(rng.standard_normal((M, (nh + 2 * nkv) * hd)).astype(np.float32))
+    print("prefill attention vs decode attention", flush=True)
+    out = ops.prefill_attention(dev(qkv), nh, nkv, hd)
+    ident = dev(odec.generate_rope_lut(hd, 500000.0, 1)[0])          # cos = 1, sin = 0
+    nq, nk = nh * hd, nkv * hd
+    kc = torch.zeros((nkv, M, hd), dtype=torch.bfloat16, device="cuda")
+    vc = torch.zeros((nkv, M, hd), dtype=torch.bfloat16, device="cuda")
+    d = dev(qkv)
+    for m in range(M):
+        one = ops.decode_attention(d[m].contiguous(), ident, kc, vc, m, nh)
+        if m in (0, 63, 64, 149):
+            err = (one.float() - out[m].float()).abs().max().item()
+            assert err <= 2.0**-6 * out[m].float().abs().max().item(), (m, err)
+    # the decode kernel filled the caches with exactly the K and V columns
+    assert torch.equal(kc.transpose(0, 1).reshape(M, nk), d[:, nq:nq + nk]) and torch.equal(vc.transpose(0, 1).reshape(M, nk), d[:, nq + nk:])
+
+
+def test_prefill_attention_llama32_1b_size(ops):
+    M, nh, nkv, hd = 2048, 32, 8, 64
+    print("prefill attention M=2048 32/8 heads", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(4)
+    qkv = torch.randn((M, (nh + 2 * nkv) * hd), device="cuda", generator=g).to(torch.bfloat16)
+    out = ops.prefill_attention(qkv, nh, nkv, hd)
+    nq, nk = nh * hd, nkv * hd
+    t = lambda x, n: x.double().reshape(M, n, hd).transpose(0, 1)
+    want = torch.nn.functional.scaled_dot_product_attention(t(qkv[:, :nq], nh), t(qkv[:, nq:nq + nk], nkv).repeat_interleave(nh // nkv, dim=0),
+                                                            t(qkv[:, nq + nk:], nkv).repeat_interleave(nh // nkv, dim=0), is_causal=True)
+    want = want.transpose(0, 1).reshape(M, nq)
+    err = (out.double() - want).abs()
+    assert float(err.max()) <= 2.0**-7 * float(qkv[:, nq + nk:].float().abs().max()), float(err.max())

@@ -147,3 +147,27 @@ def test_prefill_qkv_rope_reference_against_its_stages_and_the_decode_step():
     one = dec.rms_qkv_rope_reference(x[m], nw, wq, wk, wv, lut[pos0 + m], nh, nkv, hd)
     a, b = bf16_bits_to_f32(np.concatenate([np.ravel(t) for t in one])), bf16_bits_to_f32(out[m])
     assert a.shape == b.shape and np.max(np.abs(a - b)) <= 2.0**-6 * np.max(np.abs(b)) and np.mean(a != b) < 0.2
+
+
+def test_prefill_attention_reference_against_library_and_the_decode_reference():
+    M, nh, nkv, hd = 23, 4, 2, 64
+    rng = np.random.default_rng(90)
+    q = f32_to_bf16_bits(rng.standard_normal((M, nh * hd)).astype(np.float32))
+    k = f32_to_bf16_bits(rng.standard_normal((M, nkv * hd)).astype(np.float32))
+    v = f32_to_bf16_bits(rng.standard_normal((M, nkv * hd)).astype(np.float32))
+    got = dec.prefill_attention_reference(q, k, v, nh, nkv)
+    t = lambda b, n: torch.from_numpy(bf16_bits_to_f32(b)).double().reshape(M, n, hd).transpose(0, 1)
+    want = torch.nn.functional.scaled_dot_product_attention(t(q, nh), t(k, nkv).repeat_interleave(nh // nkv, dim=0),
+                                                            t(v, nkv).repeat_interleave(nh // nkv, dim=0), is_causal=True)
+    want = want.transpose(0, 1).reshape(M, nh * hd).numpy()
+    assert np.max(np.abs(got - want)) <= 1e-5
+    # the first token only sees itself: its output is its own V row, for every query head of the group
+    assert np.allclose(got[0].reshape(nh, hd), bf16_bits_to_f32(v[0]).reshape(nkv, hd).repeat(nh // nkv, axis=0), atol=1e-6)
+    # row m is what the single-query decode attention gives for position m over the cache of rows 0..m
+    m = 11
+    kc = k.reshape(M, nkv, hd).transpose(1, 0, 2).copy()
+    vc = v.reshape(M, nkv, hd).transpose(1, 0, 2).copy()
+    one = bf16_bits_to_f32(dec.decode_attention_cpu(q[m], kc, vc, m, nh, nkv, hd))
+    assert np.max(np.abs(one - got[m])) <= 2.0**-8 * np.max(np.abs(got[m])) + 1e-6
+    # a non-causal softmax would let row 0 see everything
+    assert not np.allclose(got[0], got[M - 1])
