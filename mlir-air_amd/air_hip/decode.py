@@ -128,3 +128,33 @@ def decode_greedy(token, n_tokens, layers, embed_table, final_norm, lm_head, con
         _, tok = ops.lm_head(x, lm_head, norm_weight=final_norm, eps=config.rms_eps)
         out[i:i + 1] = tok
     return out
+
+
+def run_prefill_layer(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer, rope_lut):
+    """One transformer block over the M prompt tokens at positions 0..M-1 (_run_layer_int4,
+    programming_examples/llms/llama32_1b_int4/llama32_1b_int4_prefill.py:241-390): RMSNorm + fused Q|K|V GEMM +
+    RoPE, causal attention, O projection + FFN block; x bf16 [M, emb] -> bf16 [M, emb].  The roped K and V
+    rows are written to the caches [n_kv_heads, max_seq, head_dim] at positions 0..M-1, where the decode
+    steps that follow expect them."""
+    if layer.codec != "awq":
+        raise ValueError("the prefill kernels take AWQ layers (the reference prefills its Q4NX models in bf16)")
+    M = x.shape[0]
+    nh, nkv, hd = config.n_heads, config.n_kv_heads, config.head_dim
+    qkv = ops.prefill_rms_qkv_rope(x, layer.attn_norm, layer.wqkv, rope_lut, 0, nh, nkv, hd, eps=config.rms_eps)
+    nq, nk = nh * hd, nkv * hd
+    k_cache_layer[:, :M].copy_(qkv[:, nq:nq + nk].reshape(M, nkv, hd).transpose(0, 1))
+    v_cache_layer[:, :M].copy_(qkv[:, nq + nk:].reshape(M, nkv, hd).transpose(0, 1))
+    attn_out = ops.prefill_attention(qkv, nh, nkv, hd)
+    return ops.prefill_o_ffn(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
+
+
+def prefill(token_ids, layers, embed_table, final_norm, lm_head, config, kv_cache, rope_lut):
+    """Prompt pass (run_npu_prefill, llama32_1b_int4_inference.py:335-427): all prompt tokens through every
+    layer at once, KV caches filled for positions 0..M-1, then the decode tail on the last row only.
+    token_ids: device integer tensor [M].  Returns (logits fp32 [vocab] of the last position, greedy next
+    token as a device int32 tensor [1])."""
+    x = embed_table.index_select(0, token_ids.to(torch.int32)).contiguous()
+    for layer, (kc, vc) in zip(layers, kv_cache):
+        x = run_prefill_layer(x, layer, config, kc, vc, rope_lut)
+    logits, best = ops.lm_head(x[-1].contiguous(), lm_head, norm_weight=final_norm, eps=config.rms_eps)
+    return logits.float(), best

@@ -166,3 +166,41 @@ def test_decode_greedy_matches_token_by_token_decoding(ops):
     assert got.tolist() == want
     for (k1, v1), (k2, v2) in zip(cache, cache2):
         assert torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
+def test_prefill_then_decode_agrees_with_token_by_token_decoding(ops):
+    """The prompt pass (tiled GEMMs, causal attention) and the decode path (streaming GEMVs, single-query
+    attention) are two implementations of the same model: after the same 20 tokens their KV caches and
+    last-position logits agree to bf16 noise, and decoding continues from either."""
+    from air_hip import decode, weights
+
+    cfg = weights.LlamaConfig(n_layers=2, emb_dim=256, n_heads=4, head_dim=64, n_kv_heads=2, hidden_dim=512, vocab_size=300)
+    layers = []
+    for i in range(cfg.n_layers):
+        t, an, fn = _layer(cfg.emb_dim, cfg.hidden_dim, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, seed=900 + 10 * i)
+        t = {k: (v[0], v[1], f32_to_bf16_bits(bf16_bits_to_f32(v[2]) * 0.05)) for k, v in t.items()}
+        layers.append(decode.prepare_layer(weights.LayerWeights(attn_norm=an, ffn_norm=fn, **t)))
+    g = torch.Generator(device="cuda").manual_seed(3)
+    embed = torch.randn((cfg.vocab_size, cfg.emb_dim), device="cuda", generator=g).to(torch.bfloat16)
+    final_norm = (torch.randn(cfg.emb_dim, device="cuda", generator=g) * 0.1 + 1.0).to(torch.bfloat16)
+    lut = decode.generate_rope_lut(cfg, 64)
+    prompt = torch.randint(0, cfg.vocab_size, (20,), device="cuda", generator=g, dtype=torch.int64)
+    print("prefill of 20 tokens", flush=True)
+    cache_p = decode.new_kv_cache(cfg, 64)
+    logits_p, best_p = decode.prefill(prompt, layers, embed, final_norm, embed, cfg, cache_p, lut)
+    print("the same 20 tokens one by one", flush=True)
+    cache_d = decode.new_kv_cache(cfg, 64)
+    for pos, tok in enumerate(prompt.tolist()):
+        logits_d = decode.decode_token(tok, layers, embed, final_norm, embed, cfg, cache_d, pos, lut)
+    torch.cuda.synchronize()
+    assert int(best_p.item()) == int(torch.argmax(logits_p))
+    scale = float(logits_d.abs().max())
+    assert float((logits_p - logits_d).abs().max()) <= 0.05 * scale, float((logits_p - logits_d).abs().max()) / scale
+    for (kp, vp), (kd, vd) in zip(cache_p, cache_d):
+        for a, b in ((kp, kd), (vp, vd)):
+            assert float((a[:, :20].float() - b[:, :20].float()).abs().max()) <= 0.05 * float(b.float().abs().max())
+            assert float(a[:, 20:].float().abs().sum()) == 0
+    # decoding goes on from the prefilled caches
+    nxt = decode.decode_token(int(best_p.item()), layers, embed, final_norm, embed, cfg, cache_p, 20, lut)
+    ref = decode.decode_token(int(best_p.item()), layers, embed, final_norm, embed, cfg, cache_d, 20, lut)
+    assert float((nxt - ref).abs().max()) <= 0.05 * float(ref.abs().max())
