@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_1b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -399,6 +399,58 @@ def run_decode_model(steps, warmup, model="decode_1b"):
             "replays_agree": bool(torch.equal(ref_tokens, tokens))}
 
 
+def run_prefill_model(model="decode_1b", M=2048, reps=3):
+    """Prompt pass of M tokens through a random-weight model (air_hip.decode.prefill: per layer RMSNorm + QKV GEMM
+    + RoPE, causal attention, O + FFN block; then the decode tail on the last row), captured as one HIP graph."""
+    import torch
+
+    from air_hip import decode, weights as wmod
+
+    cfg = wmod.LlamaConfig(**DECODE_MODELS[model])
+    E, H, hd = cfg.emb_dim, cfg.hidden_dim, cfg.head_dim
+    nqkv = (cfg.n_heads + 2 * cfg.n_kv_heads) * hd
+    torch.cuda.set_device(0)
+    stream = torch.cuda.Stream()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(6)
+
+    def lin(K, N, seed):
+        qw, qz, sc = make_weights(torch, K, N, seed)
+        return qw, qz, (sc.float() * 0.05).to(torch.bfloat16)
+
+    def norm_w():
+        return (torch.randn((E,), device="cuda", generator=g) * 0.1 + 1.0).to(torch.bfloat16)
+
+    layers = [decode.DecodeLayer(attn_norm=norm_w(), ffn_norm=norm_w(), wqkv=lin(E, nqkv, 10 * i), wo=lin(E, E, 10 * i + 1),
+                                 w_gate=lin(E, H, 10 * i + 2), w_up=lin(E, H, 10 * i + 3), w_down=lin(H, E, 10 * i + 4))
+              for i in range(cfg.n_layers)]
+    embed = torch.randn((cfg.vocab_size, E), device="cuda", generator=g).to(torch.bfloat16)
+    final_norm = norm_w()
+    lut = decode.generate_rope_lut(cfg, M)
+    cache = decode.new_kv_cache(cfg, M)
+    prompt = torch.randint(0, cfg.vocab_size, (M,), device="cuda", generator=g, dtype=torch.int64)
+    with torch.cuda.stream(stream):
+        decode.prefill(prompt, layers, embed, final_norm, embed, cfg, cache, lut)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            logits, best = decode.prefill(prompt, layers, embed, final_norm, embed, cfg, cache, lut)
+        graph.replay()
+        stream.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(reps):
+            graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+    sec = e0.elapsed_time(e1) * 1e-3 / reps
+    flops = cfg.n_layers * (2 * M * (E * nqkv + E * E + 3 * E * H) + 2 * M * M * hd * cfg.n_heads) + 2 * E * cfg.vocab_size
+    return {"ms": sec * 1e3, "tokens_per_s": M / sec, "flops": flops, "TFLOP/s": flops / sec / 1e12,
+            "finite": bool(torch.isfinite(logits).all())}
+
+
 def cpu_baseline(name, torch, w, x, outs, launch, stream):
     """The reference's NumPy path (restated in oracle/baseline.py) timed on this host's cores,
     on the same inputs as GPU launch 0; also used to sanity-check the GPU result."""
@@ -495,7 +547,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b", "decode_8b", "prefill_block"])
+    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b", "decode_8b", "prefill_block", "prefill_1b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configs")
     ap.add_argument("--copy-probe", action="store_true",
@@ -515,6 +567,20 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if a.workload == "prefill_1b":
+        r = run_prefill_model("decode_1b", 2048, max(1, min(a.steps, 5)))
+        print(json.dumps({
+            "metric": "int4 prefill tokens/s, Llama-3.2-1B shape, 2048-token prompt", "value": r["tokens_per_s"], "unit": "tokens/s",
+            "n_gpus": 1, "steps": max(1, min(a.steps, 5)), "warmup": 1, "ms_per_step": r["ms"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights (bf16 lm_head), bf16 activations, fp32 accumulate",
+            "data": "synthetic (random weights of the architecture, random prompt)",
+            "config": {"workload": "prompt pass, 16 layers E=2048 H=8192 32/8 heads hd=64 V=128256 g128, 2048 tokens, causal attention, KV caches filled",
+                       "timing": "one HIP graph of the whole pass, events on the launch stream"},
+            "roofline": {"bound": "mfma", "achieved": r["TFLOP/s"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_per_launch": r["flops"],
+                         "avg_launch_us": r["ms"] * 1e3},
+            "finite": r["finite"]}))
+        return
     if a.workload == "prefill_block":
         steps = min(a.steps, 20)
         r = run_prefill_block(steps, min(a.warmup, 3))
@@ -604,6 +670,9 @@ def main():
                                 "frac_hbm_peak": r["bytes"] / s / 1e9 / HBM_PEAK_GBS, "hot_us": r["hot_us"]}
         r = run_prefill_block(10, 2)
         extra["prefill_block"] = {"us": r["us"], "TFLOP/s": r["TFLOP/s"], "frac_mfma_peak": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS}
+        r = run_prefill_model("decode_1b", 2048, 2)
+        extra["prefill_1b"] = {"ms": r["ms"], "tokens/s": r["tokens_per_s"], "TFLOP/s": r["TFLOP/s"],
+                               "frac_mfma_peak": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS}
         for model in DECODE_MODELS:
             r = run_decode_model(32 if model == "decode_1b" else 16, 4, model)
             extra[model] = {"us_per_token": r["us_per_token"], "tokens/s": r["tokens_per_s"],

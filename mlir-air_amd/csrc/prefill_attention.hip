@@ -58,24 +58,40 @@ __global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillAttnPara
     float m = kMasked, l = 0.f;
 
     const int kend = qb + 64 < p.M ? qb + 64 : p.M;           // causal: no query of the workgroup sees a later key
-    for (int kb = 0; kb < kend; kb += 32) {
-        __syncthreads();                                       // the previous block's tiles have been read
-        for (int c = tid; c < 32 * HD / 8; c += 256) {
-            const int key = c / (HD / 8), e8 = c % (HD / 8);
+    // K and V rows of the next block travel global -> registers while the current block is multiplied, then
+    // registers -> LDS between the two barriers.  A thread moves chunk c = tid (+ 256) of 8 elements: key c % 32, elements 8 (c / 32)..
+    constexpr int NCH = 32 * HD / 8 / 256;
+    u32x4 kreg[NCH], vreg[NCH];
+    auto fetch = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + 256 * i;
+            const int key = c & 31, e8 = c >> 5;
             const int gk = kb + key < p.M ? kb + key : p.M - 1;
             const uint16_t *row = p.qkv + (size_t)gk * p.ld;
-            *reinterpret_cast<u32x4 *>(&kt[key * KP + 8 * e8]) = *reinterpret_cast<const u32x4 *>(row + k_off + 8 * e8);
-            const u32x4 vv = *reinterpret_cast<const u32x4 *>(row + v_off + 8 * e8);
+            kreg[i] = *reinterpret_cast<const u32x4 *>(row + k_off + 8 * e8);
+            vreg[i] = *reinterpret_cast<const u32x4 *>(row + v_off + 8 * e8);
+        }
+    };
+    fetch(0);
+    for (int kb = 0; kb < kend; kb += 32) {
+        __syncthreads();                                       // the previous block's tiles have been read
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + 256 * i;
+            const int key = c & 31, e8 = c >> 5;                // lanes = keys: the 2-byte V^T stores of a half-wave fill 64 contiguous bytes of one row
+            *reinterpret_cast<u32x4 *>(&kt[key * KP + 8 * e8]) = kreg[i];
             // key -> k slot of the second product: half b = key / 16, r = key % 16: slot 8 (r / 4) + r % 4 + 4 b
             const int slot = 8 * ((key & 15) >> 2) + (key & 3) + 4 * (key >> 4);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t word = vv[e];
+                const uint32_t word = vreg[i][e];
                 vt[(8 * e8 + 2 * e) * VP + slot] = (uint16_t)(word & 0xFFFFu);
                 vt[(8 * e8 + 2 * e + 1) * VP + slot] = (uint16_t)(word >> 16);
             }
         }
         __syncthreads();
+        if (kb + 32 < kend) fetch(kb + 32);
         if (kb > q0 + 15) continue;                            // every key of the block is after this wave's queries
 
         floatx4 s[2];
@@ -102,13 +118,15 @@ __global__ void __launch_bounds__(256) prefill_attn_kernel(const PrefillAttnPara
         bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
         bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
         const float m_new = fmaxf(m, bm);                      // finite from the first block on: key 0 is visible to every query
-        const float alpha = exp2f(m - m_new);
+        // v_exp_f32 directly: arguments are <= 0, results that would be denormal may flush to zero, and a masked
+        // score (-1e30 minus a finite maximum) gives exactly 0
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
         float psum = 0.f;
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float e = s[b][r] == kMasked ? 0.f : exp2f(s[b][r] - m_new);
+                const float e = __builtin_amdgcn_exp2f(s[b][r] - m_new);
                 s[b][r] = e;
                 psum += e;
             }
