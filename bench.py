@@ -553,12 +553,19 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one device copy of 256 MiB (a dispatch of known traffic that calibrates "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="set a library tuning key (w4a16_tune) before the run, e.g. --tune colgemv=1; repeatable")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures the single-GPU W4A16 kernels; --gpus must be 1 "
               "(this build has no multi-GPU path and every box has one GPU)", file=sys.stderr)
         sys.exit(2)
 
+    if a.tune:
+        from air_hip import ops
+        for kv in a.tune:
+            key, _, val = kv.partition("=")
+            ops.tune(key, int(val))
     if a.copy_probe:
         import torch
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)

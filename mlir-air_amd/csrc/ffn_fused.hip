@@ -65,9 +65,20 @@ struct UnitRegs {
     u32x4 sv[2];
 };
 
-// All loads of one unit: rows [128 * unit, +128) of a [K, N/8] matrix, the lane's two words of tile `tile`.
-__device__ __forceinline__ void load_unit(UnitRegs &u, const uint32_t *qw, const uint32_t *qz, const uint16_t *sc, int N,
-                                          int tile, int unit, int lg, int ln) {
+// The loads of one unit: rows [128 * unit, +128) of a [K, N/8] matrix, the lane's two words of tile `tile`.
+// Zero points and scales are requested first (a wave's loads return in order, and they are small), the
+// weights K-step by K-step with the order pinned, so that compute_unit can start on K-step 0 while the
+// later ones are still in flight (left alone, the load clustering mixes the K-steps).
+__device__ __forceinline__ void load_unit_meta(UnitRegs &u, const uint32_t *qz, const uint16_t *sc, int N, int tile, int unit,
+                                               int ln) {
+    const int nb = N >> 3;
+    const size_t word = (size_t)(tile * 16 + ln) * 2;
+    u.zw = *reinterpret_cast<const u32x2f *>(qz + (size_t)unit * nb + word);
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+        u.sv[c] = *reinterpret_cast<const u32x4 *>(sc + (size_t)unit * N + (size_t)(tile * 16 + ln) * 16 + 8 * c);
+}
+__device__ __forceinline__ void load_unit_weights(UnitRegs &u, const uint32_t *qw, int N, int tile, int unit, int lg, int ln) {
     const int nb = N >> 3;
     const size_t word = (size_t)(tile * 16 + ln) * 2;
 #pragma unroll
@@ -77,11 +88,13 @@ __device__ __forceinline__ void load_unit(UnitRegs &u, const uint32_t *qw, const
             const size_t row = (size_t)unit * 128 + s * 32 + 8 * lg + i;
             u.w[s][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x2f *>(qw + row * nb + word));
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
-    u.zw = *reinterpret_cast<const u32x2f *>(qz + (size_t)unit * nb + word);
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-        u.sv[c] = *reinterpret_cast<const u32x4 *>(sc + (size_t)unit * N + (size_t)(tile * 16 + ln) * 16 + 8 * c);
+}
+__device__ __forceinline__ void load_unit(UnitRegs &u, const uint32_t *qw, const uint32_t *qz, const uint16_t *sc, int N,
+                                          int tile, int unit, int lg, int ln) {
+    load_unit_meta(u, qz, sc, N, tile, unit, ln);
+    load_unit_weights(u, qw, N, tile, unit, lg, ln);
 }
 
 // yacc[j] += row 0 of x . W for the lane's 16 columns (natural order), as in the streaming kernel:
@@ -117,6 +130,7 @@ __device__ __forceinline__ void compute_unit(const UnitRegs &u, const u32x4 (&av
                 acc[t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, hi), acc[t + 1], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);   // K-step s + 1 stays below: its operands are built when its loads have landed
     }
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
@@ -252,8 +266,11 @@ __global__ void __launch_bounds__(512, 2) ffn_fused_kernel(const FfnParams p) {
 #pragma unroll
         for (int s = 0; s < 4; ++s)
             av[s] = *reinterpret_cast<const u32x4 *>(p.x + (size_t)unitA * 128 + s * 32 + 8 * lg);
-        load_unit(r0, p.qw[0], p.qz[0], p.sc[0], p.H, tileA, unitA, lg, ln);
-        load_unit(r1, p.qw[1], p.qz[1], p.sc[1], p.H, tileA, unitA, lg, ln);
+        load_unit_meta(r0, p.qz[0], p.sc[0], p.H, tileA, unitA, ln);
+        load_unit_meta(r1, p.qz[1], p.sc[1], p.H, tileA, unitA, ln);
+        __builtin_amdgcn_sched_barrier(0);
+        load_unit_weights(r0, p.qw[0], p.H, tileA, unitA, lg, ln);
+        load_unit_weights(r1, p.qw[1], p.H, tileA, unitA, lg, ln);
     }
     __builtin_amdgcn_sched_barrier(0);
     float yg[16], yu[16], yd[16];

@@ -213,13 +213,18 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
             for (int s = 0; s < KSTEPS; ++s)
                 nw[s] = *reinterpret_cast<const u32x4 *>(p.norm_w + (size_t)(kstep0 + s) * 32 + 8 * lg);
         }
+        // x first (a wave's loads return in order and the x sum needs every K-step's x), then the weights
+        // K-step by K-step, so that K-step s can be consumed while the later ones are still in flight.
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+            av[s] = *reinterpret_cast<const u32x4 *>(x_s + (size_t)(kstep0 + s) * 32 * sizeof(uint16_t) + x_lane);
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
             const size_t krow = (size_t)(kstep0 + s) * 32;          // scalar
-            av[s] = *reinterpret_cast<const u32x4 *>(x_s + krow * sizeof(uint16_t) + x_lane);
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 w[s][i] = __builtin_nontemporal_load(reinterpret_cast<const wvec *>(qw_s + (krow + i) * row_bytes + qw_lane));
+            if constexpr (NMAT == 1 || RMS) __builtin_amdgcn_sched_barrier(0);   // the load clustering would mix the K-steps
         }
         wvec zw;
         u32x4 sv[LW];
@@ -341,6 +346,10 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
                             acc[t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, hi), acc[t + 1], 0, 0, 0);
                         }
                     }
+                    // Nothing of K-step s + 1 moves above this point: left alone, the scheduler interleaves the
+                    // operand construction of later K-steps with the first MFMAs and the wave then waits for
+                    // three quarters of its loads before it starts.
+                    if constexpr (NMAT == 1 || RMS) __builtin_amdgcn_sched_barrier(0);
                 }
                 // Group flush.  Nibble positions (q, q + 4) of a word are natural columns (2q, 2q + 1),
                 // i.e. the two halves of scale word q; (zw >> 4q) & 0x000F000F | 0x43004300 is the bf16
