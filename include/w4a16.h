@@ -214,6 +214,20 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual,
  * The workspace is plain scratch (no initialisation), w4a16_attention_workspace_bytes().
  */
 size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim);
+
+/*
+ * Half-split RoPE on its own, for callers that keep the reference's launch structure (launches L5 and L6
+ * of rms_qkv_int4_rope, programming_examples/llms/llama32_1b_int4/multi_launch_builder/rms_qkv_int4_rope_multi.py:4-30):
+ *   out[r, i]        = bf16(x[r, i] * cos[r, i] - x[r, i + dim/2] * sin[r, i])
+ *   out[r, i + dim/2] = bf16(x[r, i + dim/2] * cos[r, i] + x[r, i] * sin[r, i])          i < dim/2, fp32
+ * with lut[r, :] = [cos_0 .. cos_{dim/2-1}, sin_0 .. sin_{dim/2-1}] (one LUT row per row of x, the tiled
+ * lut_q / lut_k buffers of that ABI).  Replaces the device kernel
+ * rope(bfloat16 *input, bfloat16 *lut, bfloat16 *output, int32_t dims)
+ * (programming_examples/rope_halfsplit/rope_halfsplit.cc:86-89); CPU form _cpu_rope
+ * (programming_examples/llms/llama32_1b_int4/llama32_1b_int4_prefill.py:508-524).  x, lut, out bf16 [rows, dim],
+ * dim % 16 == 0, out may not alias x.
+ */
+int rope_halfsplit_bf16(const uint16_t *x, const uint16_t *lut, uint16_t *out, int rows, int dim, void *stream);
 int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_row,
                                 uint16_t *k_cache, uint16_t *v_cache, uint16_t *attn_out,
                                 int pos, int max_seq, int n_heads, int n_kv_heads, int head_dim,

@@ -1,0 +1,429 @@
+"""KernelCache and Profiler: the call boundary of the reference's LLM decode path on the GPU.
+
+The reference's decode loop never talks to a backend directly; every device call is
+`cache.load_and_run(name, backend_kwargs, *arrays, output_indices=..., static_input_indices=...,
+intermediate_indices=..., bo_key=...)` (programming_examples/llms/shared/infra/cache.py:494-737)
+on three multi-launch ELFs compiled once by `compile_and_cache` (:447-492):
+
+  rms_qkv_int4_rope   13 args  (llama32_1b_int4/multi_launch_builder/rms_qkv_int4_rope_multi.py:4-30)
+  o_gemv_ffn_int4     15 args  (llama32_1b_int4/multi_launch_builder/o_gemv_ffn_int4_multi.py:14-32)
+  lm_head_gemv        1 + 2 P  (shared/builders/lm_head_gemv_multi.py:39-46; call site
+                               llama32_1b_int4/llama32_1b_int4_inference.py:459-486)
+
+This module keeps that interface - names, argument slots, which slots are static / intermediate /
+read back, one result per argument with empty arrays for slots that are not read back - so that
+`run_decode_block` (llama32_1b_int4/llama32_1b_int4_decode.py:176-313) and `run_npu_decode_step` can
+be pointed at it unchanged.  The packed weight slots take the reference's decode buffers (uint8
+[tiles, tile_bytes], `matvec_int4_packed.pack_inputs`); on the first call of a `bo_key` they are
+unpacked to the AutoAWQ layout the HIP kernels read and stay in HBM, the counterpart of the
+reference's write-once buffer objects.  "Compiling" validates a module description against the
+kernels' shape rules; there is nothing to build at run time.
+
+bf16 arrays are `air_hip.bf16.BF16Array` (uint16 bit patterns) or ml_dtypes bfloat16 arrays; results
+come back in the dtype of the argument they replace, flat, like the reference's buffer views.
+"""
+
+import dataclasses
+import json
+import time
+from pathlib import Path
+
+import numpy as np
+
+from . import awq, bf16
+from .backend.abc import AirBackendError
+
+KERNELS = ("rms_qkv_int4_rope", "o_gemv_ffn_int4", "lm_head_gemv")
+
+
+@dataclasses.dataclass(frozen=True)
+class DecodeModule:
+    """Description of one decode ELF (what the reference's build_*_module returns as MLIR)."""
+
+    kernel: str
+    emb_dim: int = 2048
+    kv_dim: int = 512
+    n_heads: int = 32
+    n_kv_heads: int = 8
+    head_dim: int = 64
+    hidden_dim: int = 8192
+    gs: int = 128
+    m_tile: int = 8
+    k_chunk: int = 2048
+    n_cores: int = 8
+    n_partitions: int = 8
+    n_part: int = 16384
+    eps: float = 1e-5
+
+    def __str__(self):
+        return f"hip.decode_module @{self.kernel} {dataclasses.asdict(self)}"
+
+
+def build_rms_qkv_int4_rope_module(emb_dim=2048, kv_dim=512, n_heads=32, n_kv_heads=8, head_dim=64, gs=128, m_tile=8,
+                                   k_chunk=2048, n_cores=8, **ignored):
+    """Same arguments and shape rules as build_rms_qkv_int4_rope_module
+    (rms_qkv_int4_rope_multi.py:361-382): Q heads fill the embedding, one K chunk."""
+    assert n_heads * head_dim == emb_dim
+    assert n_kv_heads * head_dim == kv_dim
+    assert k_chunk == emb_dim, "K_CHUNK must equal emb_dim for single-chunk GEMV"
+    return DecodeModule("rms_qkv_int4_rope", emb_dim=emb_dim, kv_dim=kv_dim, n_heads=n_heads, n_kv_heads=n_kv_heads,
+                        head_dim=head_dim, gs=gs, m_tile=m_tile, k_chunk=k_chunk, n_cores=n_cores)
+
+
+def build_o_gemv_ffn_int4_module(emb_dim=2048, hidden_dim=8192, gs=128, m_tile=8, k_chunk=2048, n_cores=8):
+    """Same arguments and shape rules as build_o_gemv_ffn_int4_module (o_gemv_ffn_int4_multi.py:110-123)."""
+    assert emb_dim % k_chunk == 0 and hidden_dim % k_chunk == 0
+    assert emb_dim == k_chunk, f"Stage 2 int4 swiglu_rms requires emb_dim ({emb_dim}) == k_chunk ({k_chunk})"
+    return DecodeModule("o_gemv_ffn_int4", emb_dim=emb_dim, hidden_dim=hidden_dim, gs=gs, m_tile=m_tile,
+                        k_chunk=k_chunk, n_cores=n_cores)
+
+
+def build_lm_head_gemv_module(emb_dim=2048, n_partitions=8, n_part=16384, **ignored):
+    """Same leading arguments as build_lm_head_gemv_module (shared/builders/lm_head_gemv_multi.py:39-46)."""
+    return DecodeModule("lm_head_gemv", emb_dim=emb_dim, n_partitions=n_partitions, n_part=n_part)
+
+
+class Profiler:
+    """Per-kernel and per-layer wall times with the reference's recording interface
+    (shared/infra/cache.py:70-306).  Disabled by default; every method is then a no-op."""
+
+    def __init__(self, enabled=False):
+        self.enabled = enabled
+        self.compile_times = {}
+        self.kernel_times = {}
+        self.cpu_times = {}
+        self.layer_times = []
+        self.kernel_breakdowns = {}
+
+    def record_compile(self, name, duration):
+        if self.enabled:
+            self.compile_times[name] = duration
+
+    def record_kernel(self, name, duration):
+        if self.enabled:
+            self.kernel_times.setdefault(name, []).append(duration)
+
+    def record_cpu(self, name, duration):
+        if self.enabled:
+            self.cpu_times.setdefault(name, []).append(duration)
+
+    def record_breakdown(self, name, write_ms, kernel_ms, read_ms, n_written, bytes_written, n_readback):
+        if self.enabled:
+            self.kernel_breakdowns.setdefault(name, []).append(
+                dict(write_ms=write_ms, kernel_ms=kernel_ms, read_ms=read_ms, n_written=n_written,
+                     bytes_written=bytes_written, n_readback=n_readback))
+
+    def start_layer(self):
+        return time.perf_counter() if self.enabled else None
+
+    def end_layer(self, layer_idx, t0):
+        if self.enabled and t0 is not None:
+            self.layer_times.append((layer_idx, time.perf_counter() - t0))
+
+    def time_cpu(self, name):
+        """`with profiler.time_cpu("decode_attention_cpu"): ...` records the block as a host operation."""
+        prof = self
+
+        class _Timer:
+            def __enter__(self):
+                self.t0 = time.perf_counter() if prof.enabled else None
+                return self
+
+            def __exit__(self, *exc):
+                if self.t0 is not None:
+                    prof.record_cpu(name, time.perf_counter() - self.t0)
+                return False
+
+        return _Timer()
+
+    def per_token_walls_ms(self, n_layers):
+        if not self.enabled or not self.layer_times or len(self.layer_times) % n_layers:
+            return []
+        walls = [t for _, t in self.layer_times]
+        return [sum(walls[i:i + n_layers]) * 1000.0 for i in range(0, len(walls), n_layers)]
+
+    def report(self):
+        if not self.enabled:
+            return
+        print("Kernel calls (host write + launch + read back):")
+        for name, ts in sorted(self.kernel_times.items()):
+            print(f"  {name:24s} n={len(ts):5d} avg={1e3 * sum(ts) / len(ts):8.3f} ms total={sum(ts):7.3f} s")
+            bd = self.kernel_breakdowns.get(name)
+            if bd:
+                avg = lambda k: sum(b[k] for b in bd) / len(bd)
+                print(f"  {'':24s} write {avg('write_ms'):.3f} ms, kernel {avg('kernel_ms'):.3f} ms, read {avg('read_ms'):.3f} ms")
+        if self.cpu_times:
+            print("Host operations:")
+            for name, ts in sorted(self.cpu_times.items()):
+                print(f"  {name:24s} n={len(ts):5d} avg={1e3 * sum(ts) / len(ts):8.3f} ms")
+
+
+def _check_shared_alias(shared_alias, static_input_indices, n_args):
+    """The reference validates the alias map before it touches the device (cache.py:576-603)."""
+    static = set(static_input_indices or [])
+    clash = sorted(set(shared_alias) & static)
+    if clash:
+        raise ValueError(f"shared_alias must not target static_input_indices {clash}: "
+                         f"static BOs are per-bo_key, aliases are process-wide")
+    oob = sorted(i for i in shared_alias if not 0 <= i < n_args)
+    if oob:
+        raise ValueError(f"shared_alias indices {oob} out of range for {n_args} args")
+    unnamed = sorted(i for i, n in shared_alias.items() if not isinstance(n, str) or not n)
+    if unnamed:
+        raise ValueError(f"shared_alias pool names must be non-empty strings; bad at arg indices {unnamed}")
+
+
+class KernelCache:
+    """Registers decode modules once and runs them with device-resident static arguments."""
+
+    MANIFEST_FILE = "manifest.json"
+
+    def __init__(self, cache_dir=None, verbose=False, profiler=None):
+        self.cache_dir = Path(cache_dir) if cache_dir is not None else None
+        if self.cache_dir is not None:
+            self.cache_dir.mkdir(parents=True, exist_ok=True)
+        self.verbose = verbose
+        self.profiler = profiler or Profiler()
+        self.artifacts = {}      # name -> DecodeModule
+        self._cached_bos = {}    # bo_key -> {arg index or derived name: device tensors}
+        self._shared_bos = {}    # (alias, bytes) -> device tensor handed from a producer to a consumer
+
+    def _log(self, msg):
+        if self.verbose:
+            print(f"  [KernelCache] {msg}")
+
+    # -- registration ----------------------------------------------------------------
+    def compile_and_cache(self, name, mlir_module, backend_kwargs=None, output_binary_name="air"):
+        t0 = time.time()
+        if not isinstance(mlir_module, DecodeModule):
+            raise AirBackendError(f"compile_and_cache expects a DecodeModule, got {type(mlir_module).__name__}")
+        m = mlir_module
+        if m.kernel not in KERNELS:
+            raise AirBackendError(f"unknown decode kernel '{m.kernel}' (known: {', '.join(KERNELS)})")
+        if m.gs != awq.GROUP:
+            raise AirBackendError(f"group size {m.gs} is not supported (only {awq.GROUP})")
+        if m.emb_dim <= 0 or m.emb_dim % awq.GROUP:
+            raise AirBackendError(f"emb_dim = {m.emb_dim} must be a positive multiple of {awq.GROUP}")
+        if m.kernel == "o_gemv_ffn_int4" and (m.hidden_dim <= 0 or m.hidden_dim % awq.GROUP):
+            raise AirBackendError(f"hidden_dim = {m.hidden_dim} must be a positive multiple of {awq.GROUP}")
+        if m.kernel == "rms_qkv_int4_rope" and (m.head_dim % 16 or (m.emb_dim + 2 * m.kv_dim) % 32):
+            raise AirBackendError("head_dim must be a multiple of 16 and emb_dim + 2 kv_dim a multiple of 32")
+        self.artifacts[name] = m
+        self.profiler.record_compile(name, time.time() - t0)
+        self._log(f"registered {name}: {m}")
+
+    def _save_manifest(self):
+        if self.cache_dir is None:
+            return
+        data = {name: dataclasses.asdict(m) for name, m in self.artifacts.items()}
+        (self.cache_dir / self.MANIFEST_FILE).write_text(json.dumps(data, indent=1))
+
+    def load_manifest(self):
+        """True if a manifest written by _save_manifest was found and loaded (the reference's --run-only path)."""
+        if self.cache_dir is None or not (self.cache_dir / self.MANIFEST_FILE).exists():
+            return False
+        data = json.loads((self.cache_dir / self.MANIFEST_FILE).read_text())
+        self.artifacts = {name: DecodeModule(**fields) for name, fields in data.items()}
+        return True
+
+    # -- execution -------------------------------------------------------------------
+    def load_and_run(self, name, backend_kwargs, *inputs, output_indices=None, static_input_indices=None,
+                     intermediate_indices=None, bo_key=None, shared_nonstatic=False, shared_alias=None):
+        if name not in self.artifacts:
+            raise RuntimeError(f"Kernel '{name}' not found in cache. Available: {list(self.artifacts.keys())}")
+        if shared_alias:
+            _check_shared_alias(shared_alias, static_input_indices, len(inputs))
+        mod = self.artifacts[name]
+        n_expected = {"rms_qkv_int4_rope": 13, "o_gemv_ffn_int4": 15, "lm_head_gemv": 1 + 2 * mod.n_partitions}[mod.kernel]
+        if len(inputs) != n_expected:
+            raise AirBackendError(f"{name} takes {n_expected} arguments, got {len(inputs)}")
+
+        import torch
+
+        from . import _lib
+
+        try:
+            _lib.load_library()
+        except _lib.LibraryNotBuiltError as e:
+            raise AirBackendError(str(e))
+        if not torch.cuda.is_available():
+            raise AirBackendError("no GPU visible: the HIP backend has no CPU fallback")
+
+        key = bo_key if bo_key is not None else name
+        first_call = key not in self._cached_bos
+        slots = self._cached_bos.setdefault(key, {})
+        static = set(static_input_indices or [])
+        intermediate = set(intermediate_indices or [])
+        alias = shared_alias or {}
+        readback = {len(inputs) - 1} if output_indices is None else set(output_indices)
+        stats = {"n": 0, "bytes": 0}
+
+        def resident(i):
+            """Slot i keeps what an earlier call wrote: static and intermediate slots after the first call."""
+            return not first_call and (i in static or i in intermediate)
+
+        def vec(i, shape):
+            """bf16 argument i on the device; an aliased intermediate slot takes the producer's tensor."""
+            a = inputs[i]
+            nbytes = int(np.asarray(a).size) * 2
+            if i in alias and i in intermediate and (alias[i], nbytes) in self._shared_bos:
+                return self._shared_bos[(alias[i], nbytes)].reshape(shape)
+            if resident(i) and i in slots:
+                return slots[i]
+            t = torch.from_numpy(bf16.bits_of(a).view(np.int16).reshape(shape)).cuda().view(torch.bfloat16)
+            stats["n"] += 1
+            stats["bytes"] += nbytes
+            if i in static:
+                slots[i] = t
+            return t
+
+        def linear(i, M, K):
+            """Packed decode buffer i -> kernel-side arrays (A_q [M, K/2], A_s, A_z [K/gs, M])."""
+            stats["n"] += 1
+            stats["bytes"] += int(np.asarray(inputs[i]).size)
+            return awq.unpack_bo_tiles(np.asarray(inputs[i]).view(np.uint8), M, K, mod.gs, mod.m_tile,
+                                       min(mod.k_chunk, K), mod.n_cores, M)
+
+        def to_awq_dev(l1):
+            qw, qz, sc = awq.awq_from_l1(*l1)
+            dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+            return dev(qw), dev(qz), dev(bf16.bits_of(sc).view(np.int16)).view(torch.bfloat16)
+
+        def weights(tag, indices, build):
+            """Device weights derived from packed slots `indices`; kept while all of them are resident."""
+            if tag in slots and all(resident(i) for i in indices):
+                return slots[tag]
+            w = build()
+            if all(i in static for i in indices):
+                slots[tag] = w
+            return w
+
+        t0 = time.time()
+        t_write = time.perf_counter()
+        try:
+            if mod.kernel == "rms_qkv_int4_rope":
+                run, outputs = self._stage_rms_qkv(mod, vec, linear, to_awq_dev, weights)
+            elif mod.kernel == "o_gemv_ffn_int4":
+                run, outputs = self._stage_o_gemv_ffn(mod, vec, linear, to_awq_dev, weights)
+            else:
+                run, outputs = self._stage_lm_head(mod, vec, slots, static, resident, inputs, stats)
+            torch.cuda.synchronize()
+            t_write_ms = (time.perf_counter() - t_write) * 1e3
+            t_kernel = time.perf_counter()
+            produced = run(readback)
+            torch.cuda.synchronize()
+            t_kernel_ms = (time.perf_counter() - t_kernel) * 1e3
+        except _lib.W4A16Error as e:
+            raise AirBackendError(str(e))
+        unknown = sorted(readback - set(outputs))
+        if unknown:
+            raise AirBackendError(f"{name}: argument slots {unknown} are not outputs of this kernel (outputs: {sorted(outputs)})")
+
+        t_read = time.perf_counter()
+        results = []
+        for i, a in enumerate(inputs):
+            a = np.asarray(a) if not isinstance(a, np.ndarray) else a
+            if i not in readback:
+                results.append(np.empty(0, dtype=a.dtype))
+                continue
+            t = produced[i].contiguous()
+            if i in alias:
+                self._shared_bos[(alias[i], t.numel() * 2)] = t
+            host = t.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1)
+            results.append(host.view(bf16.BF16Array) if isinstance(a, bf16.BF16Array) or a.dtype.itemsize != 2
+                           else host.view(a.dtype))
+        t_read_ms = (time.perf_counter() - t_read) * 1e3
+        self.profiler.record_kernel(name, time.time() - t0)
+        self.profiler.record_breakdown(name, t_write_ms, t_kernel_ms, t_read_ms, stats["n"], stats["bytes"], len(readback))
+        return tuple(results)
+
+    # Each _stage_* uploads what the call needs and returns (run, output slots); run(readback) launches the
+    # kernels and returns {slot: device tensor} for the slots asked for.
+    @staticmethod
+    def _stage_rms_qkv(mod, vec, linear, to_awq_dev, weights):
+        from . import ops
+
+        E, KV, nh, nkv, hd = mod.emb_dim, mod.kv_dim, mod.n_heads, mod.n_kv_heads, mod.head_dim
+        x = vec(0, (E,))
+        norm_w = vec(1, (E,))
+
+        def fused():   # Q | K | V along the output axis: one GEMV instead of three
+            parts = [linear(3, E, E), linear(5, KV, E), linear(7, KV, E)]
+            a_q = np.concatenate([p[0] for p in parts], axis=0)
+            a_s = np.concatenate([bf16.bits_of(p[1]) for p in parts], axis=1)
+            a_z = np.concatenate([p[2] for p in parts], axis=1)
+            return to_awq_dev((a_q, bf16.from_bits(a_s), a_z))
+
+        wqkv = weights("wqkv", (3, 5, 7), fused)
+        lut_q = vec(9, (nh, hd))
+        lut_k = vec(10, (nkv, hd))
+
+        def run(readback):
+            qkv = ops.w4a16_rms_gemv(x, norm_w, *wqkv, eps=mod.eps)
+            q, k, v = qkv[:E], qkv[E:E + KV], qkv[E + KV:]
+            out = {4: q, 6: k, 8: v}
+            if 11 in readback:
+                out[11] = ops.rope_halfsplit(q.reshape(nh, hd), lut_q)
+            if 12 in readback:
+                out[12] = ops.rope_halfsplit(k.reshape(nkv, hd), lut_k)
+            if 2 in readback:
+                out[2] = ops.rms_norm_rows(x.reshape(1, E), norm_w, eps=mod.eps)
+            return out
+
+        return run, (2, 4, 6, 8, 11, 12)
+
+    @staticmethod
+    def _stage_o_gemv_ffn(mod, vec, linear, to_awq_dev, weights):
+        import torch
+
+        from . import ops
+
+        E, H = mod.emb_dim, mod.hidden_dim
+        attn_out = vec(1, (E,))
+        x_residual = vec(3, (E,))
+        rms_buf = vec(6, (2, E))   # row 0: res1 (written by stage 1), row 1: ffn_norm_w
+        wo = weights("wo", (0,), lambda: to_awq_dev(linear(0, E, E)))
+
+        def gate_up():             # rows 2i = gate[i], 2i + 1 = up[i] (llama32_1b_int4_weights.py:173-207)
+            gate, up = awq.deinterleave_rows(*linear(7, 2 * H, E))
+            return to_awq_dev(gate), to_awq_dev(up)
+
+        wg, wu = weights("wgateup", (7,), gate_up)
+        wd = weights("wdown", (12,), lambda: to_awq_dev(linear(12, E, H)))
+
+        def run(readback):
+            y, res1, h = ops.o_gemv_ffn(attn_out, x_residual, rms_buf[1].contiguous(), wo, wg, wu, wd, eps=mod.eps,
+                                        return_intermediates=True)
+            out = {14: y, 11: h}
+            if 6 in readback:
+                out[6] = torch.stack([res1, rms_buf[1]])
+            return out
+
+        return run, (6, 11, 14)
+
+    @staticmethod
+    def _stage_lm_head(mod, vec, slots, static, resident, inputs, stats):
+        import torch
+
+        from . import ops
+
+        E = mod.emb_dim
+        x = vec(0, (E,))
+        parts = []
+        for p in range(mod.n_partitions):
+            i = 1 + 2 * p
+            if resident(i) and i in slots:
+                parts.append(slots[i])
+                continue
+            w = torch.from_numpy(bf16.bits_of(inputs[i]).view(np.int16).reshape(mod.n_part, E)).cuda().view(torch.bfloat16)
+            stats["n"] += 1
+            stats["bytes"] += w.numel() * 2
+            if i in static:
+                slots[i] = w
+            parts.append(w)
+
+        def run(readback):
+            return {2 + 2 * p: ops.lm_head(x, parts[p], norm_weight=None, return_argmax=False)
+                    for p in range(mod.n_partitions) if 2 + 2 * p in readback}
+
+        return run, tuple(2 + 2 * p for p in range(mod.n_partitions))

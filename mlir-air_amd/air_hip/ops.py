@@ -242,6 +242,18 @@ def decode_attention(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, out=None
     return out
 
 
+def rope_halfsplit(x, lut):
+    """Half-split RoPE of x bf16 [rows, dim] with one LUT row (cos then sin) per row: lut bf16 [rows, dim]."""
+    lib = _lib.load_library()
+    _need_cuda(x, lut)
+    if x.dim() != 2 or lut.shape != x.shape:
+        raise ValueError("rope_halfsplit: x and lut must both be [rows, dim]")
+    rows, dim = x.shape
+    out = torch.empty_like(x)
+    _lib.check(lib.rope_halfsplit_bf16(_ptr(_bits(x)), _ptr(_bits(lut)), _ptr(out), rows, dim, _stream()))
+    return out
+
+
 def rms_norm_rows(x, norm_weight, eps=1e-5):
     """out[m, :] = bf16((x[m, :] / sqrt(mean(x[m, :]^2) + eps)) * norm_weight) for x bf16 [M, K]."""
     lib = _lib.load_library()

@@ -292,4 +292,40 @@ hipError_t launch_decode_attention(const uint16_t *qkv, const uint16_t *lut_row,
     return hipGetLastError();
 }
 
+// Half-split RoPE of `rows` independent rows of `dim` elements, each with its own LUT row
+// (cos then sin).  One thread rotates 8 consecutive elements of one row; dim % 16 == 0.
+__global__ void __launch_bounds__(256) rope_rows_kernel(const uint16_t *x, const uint16_t *lut, uint16_t *out, int rows,
+                                                        int dim) {
+    const int per_row = dim >> 3;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= rows * per_row) return;
+    const int row = t / per_row, e0 = 8 * (t % per_row);
+    const int half = dim >> 1;
+    const bool low = e0 < half;
+    const int i0 = low ? e0 : e0 - half;
+    const uint16_t *src = x + (size_t)row * dim;
+    const uint16_t *l = lut + (size_t)row * dim;
+    float a[8], b[8], c[8], s[8];
+    unpack8(*reinterpret_cast<const u32x4 *>(src + e0), a);
+    unpack8(*reinterpret_cast<const u32x4 *>(src + (low ? e0 + half : e0 - half)), b);
+    unpack8(*reinterpret_cast<const u32x4 *>(l + i0), c);
+    unpack8(*reinterpret_cast<const u32x4 *>(l + half + i0), s);
+    u32x4 o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        // products of two bf16 values are exact in fp32: one rounding to fp32, one to bf16, as in NumPy
+        const float r0 = low ? a[2 * j] * c[2 * j] - b[2 * j] * s[2 * j] : a[2 * j] * c[2 * j] + b[2 * j] * s[2 * j];
+        const float r1 = low ? a[2 * j + 1] * c[2 * j + 1] - b[2 * j + 1] * s[2 * j + 1]
+                             : a[2 * j + 1] * c[2 * j + 1] + b[2 * j + 1] * s[2 * j + 1];
+        o[j] = pack_bf16x2(r0, r1);
+    }
+    *reinterpret_cast<u32x4 *>(out + (size_t)row * dim + e0) = o;
+}
+
+hipError_t launch_rope_rows(const uint16_t *x, const uint16_t *lut, uint16_t *out, int rows, int dim, hipStream_t stream) {
+    const int threads = rows * (dim >> 3);
+    hipLaunchKernelGGL(rope_rows_kernel, dim3((threads + 255) / 256), dim3(256), 0, stream, x, lut, out, rows, dim);
+    return hipGetLastError();
+}
+
 }  // namespace w4a16

@@ -478,6 +478,14 @@ int w4a16_decode_attention_bf16(const uint16_t *qkv, const uint16_t *rope_lut_ro
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+int rope_halfsplit_bf16(const uint16_t *x, const uint16_t *lut, uint16_t *out, int rows, int dim, void *stream) {
+    if (!x || !lut || !out) return W4A16_ERR_NULL;
+    if (rows <= 0 || dim <= 0 || dim % 16 != 0 || (long long)rows * dim > (1ll << 30)) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(lut) || misaligned(out)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_rope_rows(x, lut, out, rows, dim, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 size_t lm_head_workspace_bytes(int V) { return V > 0 ? lm_head_scratch_bytes(V) : 0; }
 
 int lm_head_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const uint16_t *lm_head,

@@ -140,4 +140,7 @@ hipError_t launch_decode_attention(const uint16_t *qkv, const uint16_t *lut_row,
                                    uint16_t *out, int pos, int max_seq, int n_heads, int n_kv, int head_dim,
                                    void *workspace, hipStream_t stream);
 
+// Half-split RoPE of rows x dim bf16 with one LUT row (cos then sin) per row (attention.hip).
+hipError_t launch_rope_rows(const uint16_t *x, const uint16_t *lut, uint16_t *out, int rows, int dim, hipStream_t stream);
+
 }  // namespace w4a16

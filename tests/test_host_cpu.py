@@ -201,8 +201,67 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.lm_head_gemv_bf16(P, P, -1.0, P, P, None, 100, 512, P, lws, None) == _lib.ERR_SHAPE
     assert lib.lm_head_gemv_bf16(P, None, 0.0, P, P, P + 2, 100, 512, P, lws, None) == _lib.ERR_ALIGN
     assert lib.lm_head_gemv_bf16(P, None, 0.0, P, P, None, 100, 512, P, lws - 1, None) == _lib.ERR_WORKSPACE
+    assert lib.rope_halfsplit_bf16(P, P, None, 8, 64, None) == _lib.ERR_NULL
+    assert lib.rope_halfsplit_bf16(P, P, P, 8, 24, None) == _lib.ERR_SHAPE        # dim % 16
+    assert lib.rope_halfsplit_bf16(P, P, P, 0, 64, None) == _lib.ERR_SHAPE
+    assert lib.rope_halfsplit_bf16(P, P + 8, P, 8, 64, None) == _lib.ERR_ALIGN
     assert lib.w4a16_workspace_init(None, 1024, None) == _lib.ERR_NULL
     assert lib.w4a16_workspace_init(P, 16, None) == _lib.ERR_WORKSPACE
     assert lib.w4a16_tune(b"no_such_key", 1) == _lib.ERR_TUNE and lib.w4a16_tune(b"gemv_waves", 0) == 0
     with pytest.raises(_lib.W4A16Error):
         _lib.check(_lib.ERR_ALIGN)
+
+
+def test_kernel_cache_host_contract(tmp_path):
+    """What KernelCache decides before it touches the device: module shape rules, registration, the manifest,
+    unknown kernels, the shared_alias checks (the reference makes these before any XRT call,
+    shared/infra/cache.py:569-603) and the profiler's bookkeeping."""
+    from air_hip import cache as kc
+
+    with pytest.raises(AssertionError):
+        kc.build_rms_qkv_int4_rope_module(emb_dim=2048, kv_dim=512, n_heads=16, n_kv_heads=8, head_dim=64)
+    with pytest.raises(AssertionError):
+        kc.build_rms_qkv_int4_rope_module(emb_dim=1024, kv_dim=256, n_heads=16, n_kv_heads=4, head_dim=64)   # k_chunk != emb
+    with pytest.raises(AssertionError):
+        kc.build_o_gemv_ffn_int4_module(emb_dim=2048, hidden_dim=3072)
+    with pytest.raises(AssertionError):
+        kc.build_o_gemv_ffn_int4_module(emb_dim=4096, hidden_dim=8192)
+    c = kc.KernelCache(cache_dir=tmp_path, profiler=kc.Profiler(enabled=True))
+    with pytest.raises(AirBackendError):
+        c.compile_and_cache("x", "not a module", {})
+    with pytest.raises(AirBackendError):
+        c.compile_and_cache("x", kc.DecodeModule("o_gemv_ffn_int4", emb_dim=2048, hidden_dim=8192, gs=64), {})
+    c.compile_and_cache("rms_qkv_int4_rope", kc.build_rms_qkv_int4_rope_module(), {"verbose": False})
+    c.compile_and_cache("o_gemv_ffn_int4", kc.build_o_gemv_ffn_int4_module(), {})
+    c.compile_and_cache("lm_head_gemv", kc.build_lm_head_gemv_module(2048), {})
+    assert set(c.profiler.compile_times) == {"rms_qkv_int4_rope", "o_gemv_ffn_int4", "lm_head_gemv"}
+    c._save_manifest()
+    c2 = kc.KernelCache(cache_dir=tmp_path)
+    assert c2.load_manifest() and c2.artifacts == c.artifacts
+    assert not kc.KernelCache().load_manifest()
+
+    with pytest.raises(RuntimeError, match="not found in cache"):
+        c.load_and_run("attn_gemms", {}, np.zeros(4, np.uint16))
+    z = bf16.from_f32(np.zeros(2048))
+    args = [z] * 15
+    with pytest.raises(ValueError, match="must not target static_input_indices"):
+        c.load_and_run("o_gemv_ffn_int4", {}, *args, static_input_indices={0, 6}, shared_alias={6: "res"})
+    with pytest.raises(ValueError, match="out of range"):
+        c.load_and_run("o_gemv_ffn_int4", {}, *args, shared_alias={15: "res"})
+    with pytest.raises(ValueError, match="non-empty strings"):
+        c.load_and_run("o_gemv_ffn_int4", {}, *args, shared_alias={14: ""})
+    with pytest.raises(AirBackendError, match="takes 15 arguments"):
+        c.load_and_run("o_gemv_ffn_int4", {}, *args[:14])
+
+    prof = kc.Profiler(enabled=True)
+    with prof.time_cpu("decode_attention_cpu"):
+        pass
+    for layer in range(4):
+        prof.end_layer(layer % 2, prof.start_layer())
+    prof.record_kernel("k", 0.5)
+    prof.record_breakdown("k", 1.0, 2.0, 3.0, 4, 5, 6)
+    assert len(prof.cpu_times["decode_attention_cpu"]) == 1 and len(prof.per_token_walls_ms(2)) == 2
+    assert prof.per_token_walls_ms(3) == [] and prof.kernel_breakdowns["k"][0]["bytes_written"] == 5
+    off = kc.Profiler()
+    off.record_kernel("k", 1.0)
+    assert off.start_layer() is None and off.kernel_times == {} and off.per_token_walls_ms(1) == []
