@@ -144,6 +144,21 @@ def unpack_bo_tiles(packed, M, K, GS=GROUP, M_TILE=8, K_CHUNK=2048, N_CORES=8, M
     return np.ascontiguousarray(A_q), bf16.from_bits(np.ascontiguousarray(A_s)), np.ascontiguousarray(A_z)
 
 
+def pack_gemm_tiles(W_q, W_s, W_z, K, N, GS=GROUP, N_TILE=16, K_CHUNK=128):
+    """Kernel-side arrays of a prefill weight (W_q [N, K/2] u8 output-major, W_s, W_z [K/GS, N]) -> uint8
+    [N / N_TILE, K / K_CHUNK, tile_bytes] in the layout of the reference's int4 GEMM buffers
+    (matmul_int4_packed.pack_inputs, programming_examples/matrix_multiplication/int4_awq/matmul_int4_packed.py:57-86;
+    what awq_pack_for_npu emits, llama32_1b_int4/awq_pack.py:112-146).  A tile is the decode tile with
+    N_TILE output rows, and tiles are ordered output block, then K chunk."""
+    t = pack_bo_tiles(W_q, W_s, W_z, N, K, GS, N_TILE, K_CHUNK, 1, N)
+    return t.reshape(N // N_TILE, K // K_CHUNK, -1)
+
+
+def unpack_gemm_tiles(packed, K, N, GS=GROUP, N_TILE=16, K_CHUNK=128):
+    """Inverse of pack_gemm_tiles: a buffer packed by the reference -> (W_q, W_s, W_z)."""
+    return unpack_bo_tiles(np.asarray(packed).reshape(-1), N, K, GS, N_TILE, K_CHUNK, 1, N)
+
+
 # --- single packed buffer ("BO") ------------------------------------------------------
 
 def _round256(v):

@@ -3,18 +3,25 @@
 The reference's decode loop never talks to a backend directly; every device call is
 `cache.load_and_run(name, backend_kwargs, *arrays, output_indices=..., static_input_indices=...,
 intermediate_indices=..., bo_key=...)` (programming_examples/llms/shared/infra/cache.py:494-737)
-on three multi-launch ELFs compiled once by `compile_and_cache` (:447-492):
+on multi-launch ELFs compiled once by `compile_and_cache` (:447-492).  Decode:
 
   rms_qkv_int4_rope   13 args  (llama32_1b_int4/multi_launch_builder/rms_qkv_int4_rope_multi.py:4-30)
   o_gemv_ffn_int4     15 args  (llama32_1b_int4/multi_launch_builder/o_gemv_ffn_int4_multi.py:14-32)
   lm_head_gemv        1 + 2 P  (shared/builders/lm_head_gemv_multi.py:39-46; call site
                                llama32_1b_int4/llama32_1b_int4_inference.py:459-486)
 
+and the int4 prompt pass (`_run_layer_int4`, llama32_1b_int4/llama32_1b_int4_prefill.py:241-364):
+
+  rms_gemms_rope_int4 13 args  (multi_launch_builder/rms_gemms_rope_int4_multi.py:4-17)
+  flash_attn           4 args  (q_roped, k_roped, v, out; causal grouped-query attention)
+  o_ffn_int4          15 args  (multi_launch_builder/o_ffn_int4_multi.py:4-17)
+
 This module keeps that interface - names, argument slots, which slots are static / intermediate /
 read back, one result per argument with empty arrays for slots that are not read back - so that
-`run_decode_block` (llama32_1b_int4/llama32_1b_int4_decode.py:176-313) and `run_npu_decode_step` can
-be pointed at it unchanged.  The packed weight slots take the reference's decode buffers (uint8
-[tiles, tile_bytes], `matvec_int4_packed.pack_inputs`); on the first call of a `bo_key` they are
+`run_decode_block` (llama32_1b_int4/llama32_1b_int4_decode.py:176-313), `run_npu_decode_step` and
+`_run_layer_int4` can be pointed at it unchanged.  The packed weight slots take the reference's
+buffers (decode: uint8 [tiles, tile_bytes], `matvec_int4_packed.pack_inputs`; prefill: uint8
+[N / tile_n, K / 128, tile_bytes], `awq_pack_for_npu`); on the first call of a `bo_key` they are
 unpacked to the AutoAWQ layout the HIP kernels read and stay in HBM, the counterpart of the
 reference's write-once buffer objects.  "Compiling" validates a module description against the
 kernels' shape rules; there is nothing to build at run time.
@@ -33,7 +40,7 @@ import numpy as np
 from . import awq, bf16
 from .backend.abc import AirBackendError
 
-KERNELS = ("rms_qkv_int4_rope", "o_gemv_ffn_int4", "lm_head_gemv")
+KERNELS = ("rms_qkv_int4_rope", "o_gemv_ffn_int4", "lm_head_gemv", "rms_gemms_rope_int4", "flash_attn", "o_ffn_int4")
 
 
 @dataclasses.dataclass(frozen=True)
@@ -54,6 +61,9 @@ class DecodeModule:
     n_partitions: int = 8
     n_part: int = 16384
     eps: float = 1e-5
+    seq_len: int = 1        # prefill modules: rows per call
+    tile_n: int = 16        # prefill modules: output columns per packed weight tile
+    tile_k: int = 128       # prefill modules: K chunk of a packed weight tile
 
     def __str__(self):
         return f"hip.decode_module @{self.kernel} {dataclasses.asdict(self)}"
@@ -81,6 +91,32 @@ def build_o_gemv_ffn_int4_module(emb_dim=2048, hidden_dim=8192, gs=128, m_tile=8
 def build_lm_head_gemv_module(emb_dim=2048, n_partitions=8, n_part=16384, **ignored):
     """Same leading arguments as build_lm_head_gemv_module (shared/builders/lm_head_gemv_multi.py:39-46)."""
     return DecodeModule("lm_head_gemv", emb_dim=emb_dim, n_partitions=n_partitions, n_part=n_part)
+
+
+def build_rms_gemms_rope_int4_module(seq_len=2048, emb_dim=2048, kv_dim=512, n_heads=32, n_kv_heads=8, head_dim=64,
+                                     gs=128, tile_m=16, tile_n=16, tile_k_l1=128, **ignored):
+    """Same leading arguments as build_rms_gemms_rope_int4_module (rms_gemms_rope_int4_multi.py:196-212)."""
+    assert n_heads * head_dim == emb_dim
+    assert n_kv_heads * head_dim == kv_dim
+    return DecodeModule("rms_gemms_rope_int4", emb_dim=emb_dim, kv_dim=kv_dim, n_heads=n_heads, n_kv_heads=n_kv_heads,
+                        head_dim=head_dim, gs=gs, seq_len=seq_len, tile_n=tile_n, tile_k=tile_k_l1)
+
+
+def build_o_ffn_int4_module(seq_len=2048, emb_dim=2048, hidden_dim=8192, gs=128, tile_m=16, tile_n=16, tile_k_l1=128,
+                            **ignored):
+    """Same leading arguments as build_o_ffn_int4_module (o_ffn_int4_multi.py:290-298)."""
+    return DecodeModule("o_ffn_int4", emb_dim=emb_dim, hidden_dim=hidden_dim, gs=gs, seq_len=seq_len, tile_n=tile_n,
+                        tile_k=tile_k_l1)
+
+
+def build_attn(lk=2048, lkp=64, lq=2048, lqp=256, dk=64, dv=64, num_q_tiles=4, num_cascade_stages=4, num_heads=32,
+               num_kv_heads=8, causal=True, **ignored):
+    """The flash attention module as the int4 prompt pass builds it (llama32_1b_int4_prefill.py:1219-1233): lq
+    queries and lk keys of num_heads / num_kv_heads heads of dk.  Only the causal self-attention of that call
+    site is provided: lq == lk, dk == dv, causal."""
+    assert lq == lk and dk == dv and causal, "only causal self-attention (lq == lk, dk == dv) is provided"
+    return DecodeModule("flash_attn", emb_dim=num_heads * dk, kv_dim=num_kv_heads * dk, n_heads=num_heads,
+                        n_kv_heads=num_kv_heads, head_dim=dk, seq_len=lq)
 
 
 class Profiler:
@@ -208,6 +244,14 @@ class KernelCache:
             raise AirBackendError(f"hidden_dim = {m.hidden_dim} must be a positive multiple of {awq.GROUP}")
         if m.kernel == "rms_qkv_int4_rope" and (m.head_dim % 16 or (m.emb_dim + 2 * m.kv_dim) % 32):
             raise AirBackendError("head_dim must be a multiple of 16 and emb_dim + 2 kv_dim a multiple of 32")
+        if m.kernel in ("rms_gemms_rope_int4", "flash_attn"):
+            g = m.n_heads // max(m.n_kv_heads, 1)
+            if m.head_dim not in (64, 128) or m.n_heads % m.n_kv_heads or g not in (1, 2, 4, 8):
+                raise AirBackendError("head_dim must be 64 or 128 and n_heads / n_kv_heads one of 1, 2, 4, 8")
+        if m.kernel in ("rms_gemms_rope_int4", "o_ffn_int4", "flash_attn") and m.seq_len <= 0:
+            raise AirBackendError(f"seq_len = {m.seq_len} must be positive")
+        if m.kernel == "o_ffn_int4" and (m.hidden_dim <= 0 or m.hidden_dim % awq.GROUP or m.emb_dim > 8192):
+            raise AirBackendError("hidden_dim must be a positive multiple of 128 and emb_dim at most 8192")
         self.artifacts[name] = m
         self.profiler.record_compile(name, time.time() - t0)
         self._log(f"registered {name}: {m}")
@@ -234,7 +278,8 @@ class KernelCache:
         if shared_alias:
             _check_shared_alias(shared_alias, static_input_indices, len(inputs))
         mod = self.artifacts[name]
-        n_expected = {"rms_qkv_int4_rope": 13, "o_gemv_ffn_int4": 15, "lm_head_gemv": 1 + 2 * mod.n_partitions}[mod.kernel]
+        n_expected = {"rms_qkv_int4_rope": 13, "o_gemv_ffn_int4": 15, "lm_head_gemv": 1 + 2 * mod.n_partitions,
+                      "rms_gemms_rope_int4": 13, "flash_attn": 4, "o_ffn_int4": 15}[mod.kernel]
         if len(inputs) != n_expected:
             raise AirBackendError(f"{name} takes {n_expected} arguments, got {len(inputs)}")
 
@@ -284,6 +329,12 @@ class KernelCache:
             return awq.unpack_bo_tiles(np.asarray(inputs[i]).view(np.uint8), M, K, mod.gs, mod.m_tile,
                                        min(mod.k_chunk, K), mod.n_cores, M)
 
+        def gemm_linear(i, K, N):
+            """Packed prefill buffer i -> kernel-side arrays (W_q [N, K/2], W_s, W_z [K/gs, N])."""
+            stats["n"] += 1
+            stats["bytes"] += int(np.asarray(inputs[i]).size)
+            return awq.unpack_gemm_tiles(np.asarray(inputs[i]).view(np.uint8), K, N, mod.gs, mod.tile_n, mod.tile_k)
+
         def to_awq_dev(l1):
             qw, qz, sc = awq.awq_from_l1(*l1)
             dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
@@ -305,6 +356,12 @@ class KernelCache:
                 run, outputs = self._stage_rms_qkv(mod, vec, linear, to_awq_dev, weights)
             elif mod.kernel == "o_gemv_ffn_int4":
                 run, outputs = self._stage_o_gemv_ffn(mod, vec, linear, to_awq_dev, weights)
+            elif mod.kernel == "rms_gemms_rope_int4":
+                run, outputs = self._stage_rms_gemms_rope(mod, vec, gemm_linear, to_awq_dev, weights)
+            elif mod.kernel == "flash_attn":
+                run, outputs = self._stage_flash_attn(mod, vec)
+            elif mod.kernel == "o_ffn_int4":
+                run, outputs = self._stage_o_ffn(mod, vec, gemm_linear, to_awq_dev, weights)
             else:
                 run, outputs = self._stage_lm_head(mod, vec, slots, static, resident, inputs, stats)
             torch.cuda.synchronize()
@@ -400,6 +457,71 @@ class KernelCache:
             return out
 
         return run, (6, 11, 14)
+
+    @staticmethod
+    def _stage_rms_gemms_rope(mod, vec, gemm_linear, to_awq_dev, weights):
+        import torch
+
+        from . import ops
+
+        M, E, KV, nh, nkv, hd = mod.seq_len, mod.emb_dim, mod.kv_dim, mod.n_heads, mod.n_kv_heads, mod.head_dim
+        x = vec(0, (M, E))
+        norm_w = vec(1, (E,))
+
+        def fused():
+            parts = [gemm_linear(3, E, E), gemm_linear(5, E, KV), gemm_linear(7, E, KV)]
+            a_q = np.concatenate([p[0] for p in parts], axis=0)
+            a_s = np.concatenate([bf16.bits_of(p[1]) for p in parts], axis=1)
+            a_z = np.concatenate([p[2] for p in parts], axis=1)
+            return to_awq_dev((a_q, bf16.from_bits(a_s), a_z))
+
+        wqkv = weights("wqkv", (3, 5, 7), fused)
+        # slot 9 repeats LUT row m for every Q head of token m ([M, n_heads, head_dim]); the kernel reads the table itself
+        lut = vec(9, (M, nh, hd))[:, 0].contiguous()
+
+        def run(readback):
+            qkv = ops.prefill_rms_qkv_rope(x, norm_w, wqkv, lut, 0, nh, nkv, hd, eps=mod.eps)
+            out = {11: qkv[:, :E], 12: qkv[:, E:E + KV], 8: qkv[:, E + KV:]}
+            if readback & {2, 4, 6}:   # the unrotated projections and the normalised input, for diagnosis
+                normed = ops.rms_norm_rows(x, norm_w, eps=mod.eps)
+                plain = ops.w4a16_gemm(normed, *wqkv)
+                out.update({2: normed, 4: plain[:, :E], 6: plain[:, E:E + KV]})
+            return out
+
+        return run, (2, 4, 6, 8, 11, 12)
+
+    @staticmethod
+    def _stage_flash_attn(mod, vec):
+        import torch
+
+        from . import ops
+
+        M, E, KV = mod.seq_len, mod.emb_dim, mod.kv_dim
+        q, k, v = vec(0, (M, E)), vec(1, (M, KV)), vec(2, (M, KV))
+
+        def run(readback):
+            return {3: ops.prefill_attention(torch.cat([q, k, v], dim=1).contiguous(), mod.n_heads, mod.n_kv_heads, mod.head_dim)}
+
+        return run, (3,)
+
+    @staticmethod
+    def _stage_o_ffn(mod, vec, gemm_linear, to_awq_dev, weights):
+        from . import ops
+
+        M, E, H = mod.seq_len, mod.emb_dim, mod.hidden_dim
+        attn_out = vec(0, (M, E))
+        x_residual = vec(3, (M, E))
+        norm_w = vec(5, (E,))
+        wo = weights("wo", (1,), lambda: to_awq_dev(gemm_linear(1, E, E)))
+        wg = weights("wgate", (7,), lambda: to_awq_dev(gemm_linear(7, E, H)))
+        wu = weights("wup", (9,), lambda: to_awq_dev(gemm_linear(9, E, H)))
+        wd = weights("wdown", (12,), lambda: to_awq_dev(gemm_linear(12, H, E)))
+
+        def run(readback):
+            y, res1, h = ops.prefill_o_ffn(attn_out, x_residual, norm_w, wo, wg, wu, wd, eps=mod.eps, return_intermediates=True)
+            return {14: y, 4: res1, 11: h}
+
+        return run, (4, 11, 14)
 
     @staticmethod
     def _stage_lm_head(mod, vec, slots, static, resident, inputs, stats):

@@ -199,6 +199,19 @@ def reference_decode_buffers(layer: LayerWeights, group_size=awq.GROUP, m_tile=8
     return out
 
 
+def reference_prefill_buffers(layer: LayerWeights, group_size=awq.GROUP, n_tile=16, k_chunk=128):
+    """The per-layer dict of packed GEMM buffers the reference's int4 prefill consumes (`layers_packed[i]` of
+    load_awq_weights, llama32_1b_int4/awq_pack.py:246-266: wq, wk, wv, wo, w_gate, w_up, w_down, each
+    awq_pack_for_npu of the checkpoint tensors), for interchange with it."""
+    out = {}
+    for field in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
+        qw, qz, sc = getattr(layer, field)
+        w_q, w_s, w_z = awq.l1_from_awq(qw, qz, bf16.from_bits(sc))
+        N, K = w_q.shape[0], w_q.shape[1] * 2
+        out[field] = awq.pack_gemm_tiles(w_q, w_s, w_z, K, N, group_size, n_tile, k_chunk)
+    return out
+
+
 def to_device(weights: LlamaWeights, device="cuda"):
     """Copy a loaded model into HBM as torch tensors (bf16 where the host holds bf16 bits)."""
     import torch

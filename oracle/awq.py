@@ -157,3 +157,26 @@ def pack_inputs_loop(a_q, a_s_bits, a_z, M, K, GS, M_TILE, K_CHUNK, N_CORES, M_P
                             t[q_bytes + s_bytes + g * M_TILE + r] = a_z[kc * n_gpc + g, row0 + r]
                     tiles.append(t)
     return np.stack(tiles)
+
+
+def pack_inputs_gemm_loop(w_q, w_s_bits, w_z, K, N, GS, N_TILE, K_CHUNK):
+    """Scalar restatement of the prefill GEMM weight tiling (matmul_int4_packed.py:57-86): uint8
+    [N / N_TILE, K / K_CHUNK, tile_bytes], tile (n_outer, k_outer) =
+    [Q: N_TILE rows x K_CHUNK/2 bytes][S: K_CHUNK/GS groups x N_TILE bf16][Z: K_CHUNK/GS x N_TILE u8].
+    Pure Python loops over bytes: small shapes only."""
+    n_gpc = K_CHUNK // GS
+    q_bytes, s_bytes, z_bytes = N_TILE * (K_CHUNK // 2), n_gpc * N_TILE * 2, n_gpc * N_TILE
+    out = np.zeros((N // N_TILE, K // K_CHUNK, q_bytes + s_bytes + z_bytes), dtype=np.uint8)
+    for n_outer in range(N // N_TILE):
+        for k_outer in range(K // K_CHUNK):
+            t = out[n_outer, k_outer]
+            for r in range(N_TILE):
+                for b in range(K_CHUNK // 2):
+                    t[r * (K_CHUNK // 2) + b] = w_q[n_outer * N_TILE + r, k_outer * (K_CHUNK // 2) + b]
+            for g in range(n_gpc):
+                for r in range(N_TILE):
+                    v = int(w_s_bits[k_outer * n_gpc + g, n_outer * N_TILE + r])
+                    o = q_bytes + 2 * (g * N_TILE + r)
+                    t[o], t[o + 1] = v & 0xFF, v >> 8
+                    t[q_bytes + s_bytes + g * N_TILE + r] = w_z[k_outer * n_gpc + g, n_outer * N_TILE + r]
+    return out

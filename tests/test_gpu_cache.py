@@ -189,3 +189,65 @@ def test_lm_head_partitions_through_the_kernel_cache():
     want = bf16_bits_to_f32(w).astype(np.float64) @ bf16_bits_to_f32(x).astype(np.float64)
     assert_bf16_close(logits, want, ulps=1.0, atol=2e-3, what="lm_head partitions")
     assert int(np.argmax(bf16_bits_to_f32(logits))) == odec.lm_head_reference(x, None, w)[1]
+
+
+def test_prompt_layer_through_the_kernel_cache_matches_the_oracle():
+    """The call sequence of _run_layer_int4 (llama32_1b_int4_prefill.py:241-364): rms_gemms_rope_int4, flash_attn,
+    o_ffn_int4, with the packed GEMM buffers awq_pack_for_npu makes, stage by stage against the oracle."""
+    from air_hip import bf16, cache as kc, weights
+
+    M, E, H, nh, nkv, hd = 72, 256, 512, 4, 2, 64
+    kv = nkv * hd
+    host, l1 = _model(E, H, nh, nkv, hd, seed=1200)
+    # larger Q/K/V scales than the decode tests use: attention scores with some spread
+    big = lambda w: (w[0], w[1], f32_to_bf16_bits(bf16_bits_to_f32(w[2]) * 5.0))
+    for f in ("wq", "wk", "wv"):
+        setattr(host, f, big(getattr(host, f)))
+        l1[f] = oawq.repack_hf_awq_linear(*getattr(host, f), 128)
+    packed = weights.reference_prefill_buffers(host, n_tile=16, k_chunk=128)
+    cache = kc.KernelCache()
+    cache.compile_and_cache("rms_gemms_rope_int4", kc.build_rms_gemms_rope_int4_module(M, E, kv, nh, nkv, hd, tile_n=16), {})
+    cache.compile_and_cache("flash_attn", kc.build_attn(lk=M, lkp=hd, lq=M, lqp=256, dk=hd, dv=hd, num_heads=nh,
+                                                        num_kv_heads=nkv, causal=True), {})
+    cache.compile_and_cache("o_ffn_int4", kc.build_o_ffn_int4_module(M, E, H, tile_n=16), {})
+    lut = odec.generate_rope_lut(hd, 500000.0, M)
+    x = make_x((M, E), seed=1300)
+    z = lambda *shape: bf16.from_bits(np.zeros(shape, np.uint16))
+    f = lambda b: bf16_bits_to_f32(np.asarray(b).view(np.uint16)).astype(np.float64)
+    print("kernel cache prompt layer: rms_gemms_rope_int4", flush=True)
+    r = cache.load_and_run(
+        "rms_gemms_rope_int4", {}, bf16.from_bits(x), bf16.from_bits(host.attn_norm), z(M, E), packed["wq"], z(M, E),
+        packed["wk"], z(M, kv), packed["wv"], z(M, kv), bf16.from_bits(np.repeat(lut, nh, axis=0).reshape(-1)),
+        bf16.from_bits(np.repeat(lut, nkv, axis=0).reshape(-1)), z(M, E), z(M, kv),
+        output_indices=[2, 4, 6, 8, 11, 12], static_input_indices={1, 3, 5, 7, 9, 10},
+        intermediate_indices={2, 4, 6, 8, 11, 12}, bo_key="rms_int4_L0")
+    v, q_roped, k_roped = (np.asarray(r[i]).view(np.uint16) for i in (8, 11, 12))
+    want = odec.prefill_rms_qkv_rope_reference(x, host.attn_norm, l1["wq"], l1["wk"], l1["wv"], lut, 0, nh, nkv, hd)
+    got = np.concatenate([q_roped.reshape(M, E), k_roped.reshape(M, kv), v.reshape(M, kv)], axis=1)
+    assert np.max(np.abs(f(got) - f(want))) <= 4 * 2.0**-8 * np.max(np.abs(f(want)))
+    # the diagnostic slots: normed input, and Q before the rotation (at this M the plain product comes from the
+    # streaming kernel, whose weights are not rounded to bf16 first: rotating it gives slot 11 up to one-ulp flips)
+    assert np.mean(np.asarray(r[2]).view(np.uint16).reshape(M, E) != oref.rms_norm_rows_bf16(x, host.attn_norm, 1e-5)) < 0.02
+    q_plain = np.asarray(r[4]).view(np.uint16).reshape(M * nh, hd)
+    rerot = odec.rope_rows(q_plain, np.repeat(lut, nh, axis=0)).reshape(-1)
+    assert np.max(np.abs(f(rerot) - f(q_roped))) <= 2 * 2.0**-8 * np.max(np.abs(f(q_roped)))
+
+    print("kernel cache prompt layer: flash_attn", flush=True)
+    r = cache.load_and_run("flash_attn", {}, bf16.from_bits(q_roped.reshape(M, E)), bf16.from_bits(k_roped.reshape(M, kv)),
+                           bf16.from_bits(v.reshape(M, kv)), z(M, E), output_indices=[3], bo_key="flash_attn_L0")
+    attn = np.asarray(r[3]).view(np.uint16).reshape(M, E)
+    want_attn = odec.prefill_attention_reference(q_roped.reshape(M, E), k_roped.reshape(M, kv), v.reshape(M, kv), nh, nkv)
+    tol = bf16_ulp(want_attn) + 2.0**-8 * np.max(np.abs(f(v))) + 1e-3
+    assert np.all(np.abs(f(attn) - want_attn) <= tol)
+
+    print("kernel cache prompt layer: o_ffn_int4", flush=True)
+    r = cache.load_and_run(
+        "o_ffn_int4", {}, bf16.from_bits(attn), packed["wo"], z(M, E), bf16.from_bits(x), z(M, E),
+        bf16.from_bits(host.ffn_norm), z(M, E), packed["w_gate"], z(M, H), packed["w_up"], z(M, H), z(M, H),
+        packed["w_down"], z(M, E), z(M * E), output_indices=[14], static_input_indices={1, 5, 7, 9, 12},
+        intermediate_indices={2, 4, 6, 8, 10, 11, 13, 14}, bo_key="offn_int4_L0")
+    assert r[14].shape == (M * E,) and r[4].size == 0
+    y = np.asarray(r[14]).view(np.uint16).reshape(M, E)
+    want_y, _, _ = oref.o_ffn_int4_prefill_reference(l1["wo"], l1["w_gate"], l1["w_up"], l1["w_down"], attn, x, host.ffn_norm)
+    assert oref.check_outputs(f(y), f(want_y), rtol=0.2, atol=2.0, min_correlation=0.99)
+    assert np.max(np.abs(f(y) - f(want_y))) <= 8 * 2.0**-8 * np.max(np.abs(f(want_y)))

@@ -148,3 +148,41 @@ def test_concat_and_reference_decode_buffers(tmp_path):
     g = awq.unpack_bo_tiles(bufs["_wgateup_packed"], 1024, 256, 128, 8, 256, 2)
     gate, up = awq.deinterleave_rows(*g)
     assert np.array_equal(awq.awq_from_l1(*gate)[0], layer.w_gate[0]) and np.array_equal(awq.awq_from_l1(*up)[0], layer.w_up[0])
+
+
+def test_gemm_tiles_match_the_loop_restatement_invert_and_follow_an_element_by_hand():
+    K, N, GS, N_TILE, K_CHUNK = 512, 48, 128, 16, 256
+    w_q, w_s, w_z = _l1(N, K, GS, 11)
+    got = awq.pack_gemm_tiles(w_q, bf16.from_bits(w_s), w_z, K, N, GS, N_TILE, K_CHUNK)
+    want = oawq.pack_inputs_gemm_loop(w_q, w_s, w_z, K, N, GS, N_TILE, K_CHUNK)
+    assert got.shape == want.shape == (3, 2, 16 * 128 + 2 * 16 * 2 + 2 * 16)
+    assert np.array_equal(got, want)
+    b_q, b_s, b_z = awq.unpack_gemm_tiles(got, K, N, GS, N_TILE, K_CHUNK)
+    assert np.array_equal(b_q, w_q) and np.array_equal(bf16.bits_of(b_s), w_s) and np.array_equal(b_z, w_z)
+    # one element by hand: output column 37, k = 301 (high nibble of byte 150), group 2
+    z_q, z_s, z_z = np.zeros_like(w_q), np.zeros_like(w_s), np.zeros_like(w_z)
+    z_q[37, 150], z_s[2, 37], z_z[2, 37] = 0xB0, 0x3D34, 6
+    for packed in (awq.pack_gemm_tiles(z_q, bf16.from_bits(z_s), z_z, K, N, GS, N_TILE, K_CHUNK),
+                   oawq.pack_inputs_gemm_loop(z_q, z_s, z_z, K, N, GS, N_TILE, K_CHUNK)):
+        tile = packed[2, 1]            # columns 32..47, k 256..511; row 5 of the tile, byte 22 and group 0 of the chunk
+        q_bytes, s_bytes = 16 * 128, 2 * 16 * 2
+        assert tile[5 * 128 + 22] == 0xB0 and tile[q_bytes + 2 * 5] == 0x34 and tile[q_bytes + 2 * 5 + 1] == 0x3D
+        assert tile[q_bytes + s_bytes + 5] == 6 and int(packed.astype(np.int64).sum()) == 0xB0 + 0x34 + 0x3D + 6
+
+
+def test_awq_tensors_to_gemm_tiles_is_the_reference_prefill_packing():
+    """awq_pack_for_npu (awq_pack.py:112-146): unpack the AutoAWQ words, transpose to output-major, pair
+    k-neighbours into bytes, tile.  Restated step by step with the oracle's unpacker."""
+    K, N, GS = 256, 64, 128
+    rng = np.random.default_rng(5)
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(K // GS, N), dtype=np.uint8)
+    sc = f32_to_bf16_bits(rng.uniform(0.005, 0.02, size=(K // GS, N)).astype(np.float32))
+    qw, qz = oawq.pack_awq_int32(q), oawq.pack_awq_int32(z)
+    layer = weights.LayerWeights(attn_norm=None, ffn_norm=None, **{f: (qw, qz, sc) for f in
+                                 ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")})
+    got = weights.reference_prefill_buffers(layer, n_tile=16, k_chunk=128)["w_up"]
+    w_nk = np.ascontiguousarray(oawq.unpack_awq_int32(qw).T)
+    w_q = (w_nk[:, 0::2] | (w_nk[:, 1::2] << 4)).astype(np.uint8)
+    want = oawq.pack_inputs_gemm_loop(w_q, sc, oawq.unpack_awq_int32(qz), K, N, GS, 16, 128)
+    assert np.array_equal(got, want)
