@@ -158,3 +158,41 @@ def prefill(token_ids, layers, embed_table, final_norm, lm_head, config, kv_cach
         x = run_prefill_layer(x, layer, config, kc, vc, rope_lut)
     logits, best = ops.lm_head(x[-1].contiguous(), lm_head, norm_weight=final_norm, eps=config.rms_eps)
     return logits.float(), best
+
+
+def generate(prompt_tokens, layers, embed_table, final_norm, lm_head, config, rope_lut, n_tokens=10,
+             eos_token_ids=(128001, 128009), on_token=None):
+    """Prompt pass + greedy decode (generate, programming_examples/llms/llama32_1b_int4/llama32_1b_int4_inference.py:494-575):
+    returns [first token predicted by the prompt pass] + the tokens decoded after it, at most n_tokens of them,
+    ending with the first end-of-sequence id if one is produced.  prompt_tokens: a sequence of ints.
+
+    Without `on_token` the whole decode loop runs on the device (decode_greedy) and the ids come back once; tokens
+    after an end-of-sequence id are computed and dropped.  With `on_token(token_id)` every token is brought to the
+    host as it is produced (the reference's streaming mode) and the loop stops at an end-of-sequence id."""
+    seq_len = len(prompt_tokens)
+    max_seq = seq_len + n_tokens
+    if rope_lut.shape[0] < max_seq:
+        raise ValueError(f"the RoPE table has {rope_lut.shape[0]} rows, the run needs {max_seq}")
+    kv_cache = new_kv_cache(config, max_seq, device=embed_table.device)
+    ids = torch.as_tensor(list(prompt_tokens), dtype=torch.int32, device=embed_table.device)
+    _, first = prefill(ids, layers, embed_table, final_norm, lm_head, config, kv_cache, rope_lut)
+    eos = set(int(t) for t in eos_token_ids)
+    if on_token is None:
+        rest = decode_greedy(first, n_tokens, layers, embed_table, final_norm, lm_head, config, kv_cache, seq_len, rope_lut)
+        out = [int(first.item())] + [int(t) for t in rest.cpu().tolist()]
+        for i in range(1, len(out)):
+            if out[i] in eos:
+                return out[:i + 1]
+        return out
+    tok = int(first.item())
+    out = [tok]
+    on_token(tok)
+    for i in range(n_tokens):
+        _, best = decode_token(tok, layers, embed_table, final_norm, lm_head, config, kv_cache, seq_len + i, rope_lut,
+                               return_argmax=True)
+        tok = int(best.item())
+        out.append(tok)
+        on_token(tok)
+        if tok in eos:
+            break
+    return out

@@ -204,3 +204,47 @@ def test_prefill_then_decode_agrees_with_token_by_token_decoding(ops):
     nxt = decode.decode_token(int(best_p.item()), layers, embed, final_norm, embed, cfg, cache_p, 20, lut)
     ref = decode.decode_token(int(best_p.item()), layers, embed, final_norm, embed, cfg, cache_d, 20, lut)
     assert float((nxt - ref).abs().max()) <= 0.05 * float(ref.abs().max())
+
+
+def test_generate_is_prefill_plus_greedy_decoding_and_stops_at_eos(ops):
+    """generate() against its parts: the first token is the prompt pass's argmax, the rest equals a token-by-token
+    greedy loop from the prefilled caches; the device loop and the streaming loop agree; an end-of-sequence id ends
+    the output with that id."""
+    from air_hip import decode, weights
+
+    cfg = weights.LlamaConfig(n_layers=2, emb_dim=256, n_heads=4, head_dim=64, n_kv_heads=2, hidden_dim=512, vocab_size=300)
+    layers = []
+    for i in range(cfg.n_layers):
+        t, an, fn = _layer(cfg.emb_dim, cfg.hidden_dim, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, seed=1100 + 10 * i)
+        t = {k: (v[0], v[1], f32_to_bf16_bits(bf16_bits_to_f32(v[2]) * 0.05)) for k, v in t.items()}
+        layers.append(decode.prepare_layer(weights.LayerWeights(attn_norm=an, ffn_norm=fn, **t)))
+    g = torch.Generator(device="cuda").manual_seed(5)
+    embed = torch.randn((cfg.vocab_size, cfg.emb_dim), device="cuda", generator=g).to(torch.bfloat16)
+    final_norm = (torch.randn(cfg.emb_dim, device="cuda", generator=g) * 0.1 + 1.0).to(torch.bfloat16)
+    lut = decode.generate_rope_lut(cfg, 64)
+    prompt = torch.randint(0, cfg.vocab_size, (12,), device="cuda", generator=g, dtype=torch.int64).tolist()
+    n = 9
+    print("generate: device loop", flush=True)
+    got = decode.generate(prompt, layers, embed, final_norm, embed, cfg, lut, n_tokens=n, eos_token_ids=())
+    assert len(got) == n + 1
+    print("generate: reference loop from its parts", flush=True)
+    cache = decode.new_kv_cache(cfg, len(prompt) + n)
+    _, first = decode.prefill(torch.tensor(prompt, device="cuda"), layers, embed, final_norm, embed, cfg, cache, lut)
+    want = [int(first.item())]
+    for i in range(n):
+        logits = decode.decode_token(want[-1], layers, embed, final_norm, embed, cfg, cache, len(prompt) + i, lut)
+        want.append(int(torch.argmax(logits)))
+    assert got == want
+    print("generate: streaming", flush=True)
+    seen = []
+    streamed = decode.generate(prompt, layers, embed, final_norm, embed, cfg, lut, n_tokens=n, eos_token_ids=(), on_token=seen.append)
+    assert streamed == want and seen == want
+    # an end-of-sequence id ends the output at its first occurrence among the decoded tokens, in both modes (the
+    # prompt pass's own token is not tested, as in the reference's loop)
+    for eos in (want[1], want[-1]):
+        cut = next(i for i in range(1, len(want)) if want[i] == eos)
+        for cb in (None, lambda t: None):
+            out = decode.generate(prompt, layers, embed, final_norm, embed, cfg, lut, n_tokens=n, eos_token_ids=(eos,), on_token=cb)
+            assert out == want[:cut + 1]
+    with pytest.raises(ValueError):
+        decode.generate(prompt, layers, embed, final_norm, embed, cfg, lut, n_tokens=60)
