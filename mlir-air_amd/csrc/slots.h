@@ -31,6 +31,18 @@ __device__ __forceinline__ u32x4 slot_load(const float *p) {
     const uint64_t b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, SLOT_LD_SCOPE);
     return u32x4{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
 }
+// The same slot split over two planes `plane` floats apart: thread e keeps words 0, 1 at pa and words 2, 3 at
+// pa + plane, with pa = base + 2 e.  Each of the two 8-byte accesses of a wavefront then covers 512 contiguous
+// bytes (the interleaved form writes every 32-byte sector twice, half of it each time).
+__device__ __forceinline__ void slot_store_planes(float *pa, size_t plane, u32x4 v) {
+    __hip_atomic_store(reinterpret_cast<uint64_t *>(pa), (uint64_t)v[0] | ((uint64_t)v[1] << 32), __ATOMIC_RELAXED, SLOT_ST_SCOPE);
+    __hip_atomic_store(reinterpret_cast<uint64_t *>(pa + plane), (uint64_t)v[2] | ((uint64_t)v[3] << 32), __ATOMIC_RELAXED, SLOT_ST_SCOPE);
+}
+__device__ __forceinline__ u32x4 slot_load_planes(const float *pa, size_t plane) {
+    const uint64_t a = __hip_atomic_load(reinterpret_cast<const uint64_t *>(pa), __ATOMIC_RELAXED, SLOT_LD_SCOPE);
+    const uint64_t b = __hip_atomic_load(reinterpret_cast<const uint64_t *>(pa + plane), __ATOMIC_RELAXED, SLOT_LD_SCOPE);
+    return u32x4{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
+}
 __device__ __forceinline__ bool slot_full(u32x4 v) {
     return v[0] != kEmpty && v[1] != kEmpty && v[2] != kEmpty && v[3] != kEmpty;
 }

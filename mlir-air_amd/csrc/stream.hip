@@ -54,7 +54,7 @@ struct StreamParams {
     const uint16_t *mn[2];   // affine codec: per-group minimum [K / 32, N] bf16 of each matrix (qz unused), else null
     uint16_t *y;
     uint32_t *header;   // workspace header: word 0 = poll timeouts seen
-    float *partial;     // [nmat * ksplit][ntiles][M * tile columns]
+    float *partial;     // [nmat * ksplit][ntiles][2 planes][M * tile columns / 2]: a quad's words 0, 1 and words 2, 3
     int M, K, N;
     int nb;        // N / 8 packed words per row
     int ntiles;    // ceil(N / tile columns)
@@ -380,6 +380,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     const int col0 = tile * TC;
     const size_t slice_stride = (size_t)p.ntiles * nquads * 4;                 // floats per (mat, kslice)
     float *tile_partial = p.partial + (size_t)tile * nquads * 4;
+    const size_t plane = (size_t)nquads * 2;   // a tile's slots are two planes of 8 bytes per quad
 
     // The reducer's first polling round is issued before the LDS combine, so that its latency
     // (one trip to L2 per slot) is hidden behind the combine and its barriers.
@@ -388,7 +389,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     if (prefetched) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            if (j < nprod) va[j] = slot_load(tile_partial + (size_t)threadIdx.x * 4 + j * slice_stride);
+            if (j < nprod) va[j] = slot_load_planes(tile_partial + (size_t)threadIdx.x * 2 + j * slice_stride, plane);
     }
 
     // ---- cross-wave combine in LDS: red[slot][m][ln][LC], moved as 16-byte chunks (4 columns).  Chunk jj
@@ -422,12 +423,12 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s) own += *reinterpret_cast<const floatx4 *>(src + s * slot_stride);
         }
-        float *slot0 = tile_partial + (size_t)e * 4;
+        float *slot0 = tile_partial + (size_t)e * 2;   // words 0, 1 here, words 2, 3 one plane further
         if (!reducer) {
             u32x4 bits = __builtin_bit_cast(u32x4, own);
 #pragma unroll
             for (int q = 0; q < 4; ++q) bits[q] = bits[q] == kEmpty ? 0x7FC00000u : bits[q];   // keep the sentinel unique
-            if (!p.skip_publish) slot_store(slot0 + sub * slice_stride, bits);
+            if (!p.skip_publish) slot_store_planes(slot0 + sub * slice_stride, plane, bits);
             continue;
         }
         // Reducer: fetch the producers' slots eight at a time (all loads of a round in flight
@@ -437,7 +438,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         floatx4 sum0 = floatx4{0.f, 0.f, 0.f, 0.f}, sum1 = floatx4{0.f, 0.f, 0.f, 0.f};
         for (int s0 = 0; s0 < nprod; s0 += 8) {
 #define W4A16_POLL_ISSUE(dst)                                                                 \
-    _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < nprod) dst[j] = slot_load(slot0 + (s0 + j) * slice_stride)
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < nprod) dst[j] = slot_load_planes(slot0 + (s0 + j) * slice_stride, plane)
 #define W4A16_POLL_FULL(src, ok)                                                              \
     ok = true;                                                                                \
     _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < nprod) ok = ok && slot_full(src[j])
@@ -473,7 +474,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 #undef W4A16_POLL_TAKE
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                if (s0 + j < nprod) slot_store(slot0 + (s0 + j) * slice_stride, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
+                if (s0 + j < nprod) slot_store_planes(slot0 + (s0 + j) * slice_stride, plane, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
         }
         floatx4 out;
         if (NMAT == 2) {
