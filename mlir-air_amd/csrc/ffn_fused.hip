@@ -15,8 +15,8 @@
 //
 // Cross-workgroup traffic uses the sentinel slots of slots.h, all inside the caller's workspace
 // (every word 0xFFFFFFFF between calls):
-//   partialA  [2 * (splitA - 1)][tilesA][64 quads]   gate and up partials of the producers
-//   partialB  [splitB - 1][tilesB][64 quads]
+//   partialA  [2 * (splitA - 1)][tilesA][2 planes][64 quads / 2]   gate and up partials of the producers
+//   partialB  [splitB - 1][tilesB][2 planes][64 quads / 2]
 //   hpriv     [tilesB][H / 2] words                  one private copy of h (bf16 pairs) per down tile
 // The reducer of a gate/up tile (last slice = highest workgroup ids = dispatched last) adds the
 // partials in fixed order, applies SwiGLU and writes its 256 values of h into all tilesB copies;
@@ -174,7 +174,8 @@ __device__ __forceinline__ u32x4 keep_sentinel_unique(floatx4 v) {
 }
 
 // Adds the `n` slots base + j * stride (j < split into sum0, the rest into sum1) once they are all
-// filled, then empties them.  Two polling rounds in flight.  Returns false after spin_limit rounds.
+// filled, then empties them.  A tile's 64 slots are two planes of 128 floats (slot_store_planes): base is
+// the tile's region + 2 * lane.  Two polling rounds in flight.  Returns false after spin_limit rounds.
 // Every round issues the same eight slot loads whatever n is (slots past the end re-read the last
 // one and are masked out of the test and the sum), so that the number of loads in flight at each
 // wait is fixed; with loads skipped by branches, stale registers were sporadically accepted as
@@ -187,7 +188,7 @@ __device__ __forceinline__ bool gather(float *base, size_t stride, int n, int sp
         const float *addr[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) addr[j] = base + (size_t)(s0 + j < n ? s0 + j : n - 1) * stride;
-#define FFN_ISSUE(dst) _Pragma("unroll") for (int j = 0; j < 8; ++j) dst[j] = slot_load(addr[j])
+#define FFN_ISSUE(dst) _Pragma("unroll") for (int j = 0; j < 8; ++j) dst[j] = slot_load_planes(addr[j], 128)
 #define FFN_FULL(src, ok) ok = true; _Pragma("unroll") for (int j = 0; j < 8; ++j) ok = ok && slot_full(src[j])
 #define FFN_TAKE(src)                                                                         \
     _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                           \
@@ -223,7 +224,7 @@ __device__ __forceinline__ bool gather(float *base, size_t stride, int n, int sp
         all_ok = all_ok && ok;
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            if (s0 + j < n) slot_store(base + (size_t)(s0 + j) * stride, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
+            if (s0 + j < n) slot_store_planes(base + (size_t)(s0 + j) * stride, 128, u32x4{kEmpty, kEmpty, kEmpty, kEmpty});
     }
     return all_ok;
 }
@@ -328,8 +329,8 @@ __global__ void __launch_bounds__(512, 2) ffn_fused_kernel(const FfnParams p) {
     // SwiGLU reduction runs ----
     if (!reducerA) {
         if (wave < 2) {
-            float *slot = p.partialA + (((size_t)(wave * nprodA + sliceA) * p.tilesA + tileA) * 64 + lane) * 4;
-            slot_store(slot, keep_sentinel_unique(own0));
+            float *slot = p.partialA + ((size_t)(wave * nprodA + sliceA) * p.tilesA + tileA) * 256 + lane * 2;
+            slot_store_planes(slot, 128, keep_sentinel_unique(own0));
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -338,7 +339,7 @@ __global__ void __launch_bounds__(512, 2) ffn_fused_kernel(const FfnParams p) {
     if (gather_wave) {
         floatx4 g = own0, u = own1;
         floatx4 sg = floatx4{0.f, 0.f, 0.f, 0.f}, su = floatx4{0.f, 0.f, 0.f, 0.f};
-        float *base = p.partialA + ((size_t)tileA * 64 + lane) * 4;
+        float *base = p.partialA + (size_t)tileA * 256 + lane * 2;
         if (!gather(base, (size_t)p.tilesA * 256, 2 * nprodA, nprodA, sg, su, p.spin_limit))
             __hip_atomic_store(p.header, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         g += sg;
@@ -401,11 +402,11 @@ __global__ void __launch_bounds__(512, 2) ffn_fused_kernel(const FfnParams p) {
     floatx4 own = lds_sum(redB, lane);
     const int nprodB = p.splitB - 1;
     if (!reducerB) {
-        slot_store(p.partialB + (((size_t)sliceB * p.tilesB + tileB) * 64 + lane) * 4, keep_sentinel_unique(own));
+        slot_store_planes(p.partialB + ((size_t)sliceB * p.tilesB + tileB) * 256 + lane * 2, 128, keep_sentinel_unique(own));
         return;
     }
     floatx4 sum = floatx4{0.f, 0.f, 0.f, 0.f}, unused = floatx4{0.f, 0.f, 0.f, 0.f};
-    if (!gather(p.partialB + ((size_t)tileB * 64 + lane) * 4, (size_t)p.tilesB * 256, nprodB, nprodB, sum, unused, p.spin_limit))
+    if (!gather(p.partialB + (size_t)tileB * 256 + lane * 2, (size_t)p.tilesB * 256, nprodB, nprodB, sum, unused, p.spin_limit))
         __hip_atomic_store(p.header, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     floatx4 out = sum + own;
     const int col = tileB * 256 + lane * 4;
