@@ -46,6 +46,30 @@ __device__ __forceinline__ void unpack8(const u32x4 v, float (&f)[8]) {
     }
 }
 
+// 2^x for x <= 0 as the bare v_exp_f32: the library routine's rescaling of very negative arguments only
+// changes results below 2^-126, which vanish against the running sums they are added to.
+__device__ __forceinline__ float exp2_nonpos(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Sum over a group of LPP = 8 or 16 neighbouring lanes (a group never crosses a row of 16 lanes), every lane
+// of the group receiving the sum: an xor butterfly on data-parallel-primitive moves (quad permutes for
+// distances 1 and 2, half-row and row mirrors for 4 and 8: once the quads agree, mirroring meets the
+// partner quad), i.e. full-rate VALU adds instead of LDS-routed shuffles.  Bit-identical to the butterfly
+// with shuffles: every step adds the same two partial sums.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+    return v + __builtin_bit_cast(float, moved);
+}
+template <int LPP>
+__device__ __forceinline__ float group_sum(float s) {
+    static_assert(LPP == 8 || LPP == 16, "lane groups of 8 or 16");
+    s = dpp_add<0xB1>(s);    // quad_perm [1, 0, 3, 2]
+    s = dpp_add<0x4E>(s);    // quad_perm [2, 3, 0, 1]
+    s = dpp_add<0x141>(s);   // row_half_mirror
+    if constexpr (LPP == 16) s = dpp_add<0x140>(s);   // row_mirror
+    return s;
+}
+
 // Half-split RoPE of elements [e0, e0 + 8) of one head: x at src, rounded to bf16 (returned as floats).
 template <int HD>
 __device__ __forceinline__ void rope8(const uint16_t *src, const uint16_t *lut, int e0, float (&out)[8]) {
@@ -139,11 +163,10 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const AttnParams p) {
                 float s = 0.f;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) s = fmaf(q[h][j], k[j], s);
-#pragma unroll
-                for (int off = 1; off < LPP; off <<= 1) s += __shfl_xor(s, off);
+                s = group_sum<LPP>(s);
                 const float mn = fmaxf(m[h], s);
-                const float corr = exp2f(m[h] - mn);
-                const float pr = exp2f(s - mn);
+                const float corr = exp2_nonpos(m[h] - mn);
+                const float pr = exp2_nonpos(s - mn);
                 m[h] = mn;
                 l[h] = l[h] * corr + pr;
 #pragma unroll
@@ -159,7 +182,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(const AttnParams p) {
         for (int h = 0; h < G; ++h) {
             const float m2 = __shfl_xor(m[h], off), l2 = __shfl_xor(l[h], off);
             const float mn = fmaxf(m[h], m2);
-            const float c1 = exp2f(m[h] - mn), c2 = exp2f(m2 - mn);
+            const float c1 = exp2_nonpos(m[h] - mn), c2 = exp2_nonpos(m2 - mn);
             m[h] = mn;
             l[h] = l[h] * c1 + l2 * c2;
 #pragma unroll
