@@ -123,11 +123,21 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     // consecutive numbers go to consecutive XCDs, so with gridDim.x a multiple of 8 all workgroups
     // of a tile share an XCD (tile % 8); they are dispatched in that order too, so the reducer,
     // the last K-slice of the last matrix, starts after all of its producers.
+    const int kslice = blockIdx.y;
+    const int mat = blockIdx.z;
+    // Every kernel argument the main path reads is requested here, before the first branch: left to the
+    // compiler the scalar loads are issued one use at a time behind the early exits, four dependent
+    // round trips to the constant cache before the first weight load is requested.
+    {
+        const int i0 = p.ntiles, i1 = p.M, i2 = p.K, i3 = p.N, i4 = p.nb, i5 = p.ksplit, i6 = p.units, i7 = p.slice_units,
+                  i8 = p.slice_extra, i9 = p.nmat;
+        const void *q0 = p.x, *q1 = p.qw[mat], *q2 = p.qz[mat], *q3 = p.sc[mat];
+        asm volatile("" ::"s"(i0), "s"(i1), "s"(i2), "s"(i3), "s"(i4), "s"(i5), "s"(i6), "s"(i7), "s"(i8), "s"(i9), "s"(q0),
+                     "s"(q1), "s"(q2), "s"(q3));
+    }
     const int per_tile = p.nmat * p.ksplit;
     const int tile = blockIdx.x;
     if (tile >= p.ntiles) return;
-    const int kslice = blockIdx.y;
-    const int mat = blockIdx.z;
     const int sub = mat * p.ksplit + kslice;
 
     const int nchunks = p.nb / LW;
