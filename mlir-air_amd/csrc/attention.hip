@@ -16,6 +16,8 @@
 //
 // Rounding points follow the reference's decode step: Q and K are rounded to bf16 after RoPE,
 // scores, softmax and the weighted sum are fp32, the output is rounded to bf16 once.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -68,6 +70,24 @@ __device__ __forceinline__ float group_sum(float s) {
     s = dpp_add<0x141>(s);   // row_half_mirror
     if constexpr (LPP == 16) s = dpp_add<0x140>(s);   // row_mirror
     return s;
+}
+
+// Maximum / sum over the 64 lanes of a wavefront, every lane receiving the result: the four steps inside a row of
+// 16 lanes on DPP moves as in group_sum, the two steps across rows by shuffle.
+template <bool MAX>
+__device__ __forceinline__ float wave_reduce(float v) {
+    auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+    auto dpp = [&](auto ctrl) {
+        constexpr int CTRL = decltype(ctrl)::value;
+        const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+        v = op(v, __builtin_bit_cast(float, moved));
+    };
+    dpp(std::integral_constant<int, 0xB1>());    // quad_perm [1, 0, 3, 2]
+    dpp(std::integral_constant<int, 0x4E>());    // quad_perm [2, 3, 0, 1]
+    dpp(std::integral_constant<int, 0x141>());   // row_half_mirror
+    dpp(std::integral_constant<int, 0x140>());   // row_mirror
+    v = op(v, __shfl_xor(v, 16));
+    return op(v, __shfl_xor(v, 32));
 }
 
 // Half-split RoPE of elements [e0, e0 + 8) of one head: x at src, rounded to bf16 (returned as floats).
@@ -246,13 +266,9 @@ __global__ void attn_combine_kernel(const float *part_ml, const float *part_acc,
         const bool live = e < nsplit;
         const float m = live ? part_ml[2 * ((size_t)head * nsplit + e)] : kNegBig;
         const float l = live ? part_ml[2 * ((size_t)head * nsplit + e) + 1] : 0.f;
-        float mn = m;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) mn = fmaxf(mn, __shfl_xor(mn, off));
+        const float mn = wave_reduce<true>(m);
         const float c = exp2f(m - mn);
-        float ls = l * c;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) ls += __shfl_xor(ls, off);
+        const float ls = wave_reduce<false>(l * c);
         if (e < kMaxAttnSplit) wgt[e] = live ? c : 0.f;
         if (e == 0) inv_l = 1.0f / ls;
     }
