@@ -216,6 +216,27 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual,
 size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim);
 
 /*
+ * w4a16_decode_attention_bf16 followed by w4a16_o_gemv_ffn_bf16 as one call: everything of a decode layer after
+ * the Q|K|V projection (RoPE, cache append and attention of run_decode_block, then the o_gemv_ffn_int4 ELF,
+ * programming_examples/llms/llama32_1b_int4/llama32_1b_int4_decode.py:270-313).  When the attention runs over
+ * several sequence chunks and the O projection's work units lie inside one head (head_dim % 64 == 0 and a short
+ * enough E), the O projection merges the chunk partials itself, with the merge kernel's arithmetic in the merge
+ * kernel's order, and the merge launch is dropped: y is the same bit for bit as from the two calls.  `attn_out`
+ * bf16 [E] is scratch (it holds the attention output whenever the merge launch did run).  E == n_heads * head_dim;
+ * other constraints and both workspaces as for the two calls.  w4a16_tune("attn_fuse", 0) keeps the merge launch.
+ */
+int w4a16_decode_attn_o_gemv_ffn_bf16(const uint16_t *qkv, const uint16_t *rope_lut_row, uint16_t *k_cache,
+                                      uint16_t *v_cache, uint16_t *attn_out, int pos, int max_seq, int n_heads,
+                                      int n_kv_heads, int head_dim, void *attn_workspace, size_t attn_workspace_bytes,
+                                      const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                                      const int32_t *o_qweight, const int32_t *o_qzeros, const uint16_t *o_scales,
+                                      const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                                      const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                                      const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
+                                      uint16_t *y, int E, int H, int group, void *workspace, size_t workspace_bytes,
+                                      void *stream);
+
+/*
  * Half-split RoPE on its own, for callers that keep the reference's launch structure (launches L5 and L6
  * of rms_qkv_int4_rope, programming_examples/llms/llama32_1b_int4/multi_launch_builder/rms_qkv_int4_rope_multi.py:4-30):
  *   out[r, i]        = bf16(x[r, i] * cos[r, i] - x[r, i + dim/2] * sin[r, i])

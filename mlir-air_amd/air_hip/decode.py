@@ -6,7 +6,8 @@ The reference issues two NPU calls per layer (rms_qkv_int4_rope: 6 launches; o_g
 is five kernel launches, all on the device:
 
   1. RMSNorm + fused Q|K|V int4 GEMV (one matrix, concatenated along the output axis)
-  2. RoPE(Q, K) + cache append + grouped-query attention (+ 3. the chunk combine for long contexts)
+  2. RoPE(Q, K) + cache append + grouped-query attention (+ 3. the chunk combine for long contexts, unless the O
+     projection can merge the chunks itself)
   4-6. O projection + residual, RMSNorm + gate/up + SwiGLU, down projection + residual
 """
 
@@ -96,6 +97,9 @@ def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer
     updated in place at current_pos."""
     q4nx = layer.codec == "q4nx"
     qkv = (ops.q4nx_rms_gemv if q4nx else ops.w4a16_rms_gemv)(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps)
+    if not q4nx:   # attention + block as one call: the O projection merges the attention's chunk partials where it can
+        return ops.decode_attn_o_gemv_ffn(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads,
+                                          x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
     attn_out = ops.decode_attention(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads)
     return (ops.q4nx_o_gemv_ffn if q4nx else ops.o_gemv_ffn)(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
 

@@ -242,6 +242,36 @@ def decode_attention(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, out=None
     return out
 
 
+def decode_attn_o_gemv_ffn(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, x_residual, ffn_norm_weight, wo, gate, up, down,
+                           eps=1e-5, group=GROUP):
+    """decode_attention followed by o_gemv_ffn in one call; over several sequence chunks the O projection merges the
+    attention partials itself (one launch fewer), with the same result bit for bit.  Returns y bf16 [E]."""
+    lib = _lib.load_library()
+    _need_cuda(qkv, rope_lut_row, k_cache, v_cache, x_residual, ffn_norm_weight, *wo, *gate, *up, *down)
+    n_kv, max_seq, hd = k_cache.shape
+    E = n_heads * hd
+    H = gate[0].shape[1] * 8
+    if v_cache.shape != k_cache.shape or qkv.numel() != (n_heads + 2 * n_kv) * hd or rope_lut_row.numel() != hd:
+        raise ValueError("decode_attn_o_gemv_ffn: qkv must be [(n_heads + 2 n_kv) * hd], caches [n_kv, max_seq, hd], lut row [hd]")
+    if (wo[0].shape[0] != E or wo[0].shape[1] * 8 != E or gate[0].shape[0] != E or up[0].shape != gate[0].shape
+            or down[0].shape[0] != H or down[0].shape[1] * 8 != E or x_residual.numel() != E or ffn_norm_weight.numel() != E):
+        raise ValueError("decode_attn_o_gemv_ffn: wo must be [E, E/8], gate/up [E, H/8], down [H, E/8], vectors [E]")
+    dev = qkv.device
+    y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
+    attn_out = torch.empty((E,), dtype=torch.bfloat16, device=dev)
+    key = (dev.index, _stream(), n_heads, hd)
+    aws = _attn_ws.get(key)
+    if aws is None:
+        aws = torch.empty(int(lib.w4a16_attention_workspace_bytes(n_heads, hd)), dtype=torch.uint8, device=dev)
+        _attn_ws[key] = aws
+    ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev, ("block", E, H))
+    _lib.check(lib.w4a16_decode_attn_o_gemv_ffn_bf16(
+        _ptr(_bits(qkv)), _ptr(_bits(rope_lut_row)), _ptr(_bits(k_cache)), _ptr(_bits(v_cache)), _ptr(attn_out), int(pos),
+        max_seq, n_heads, n_kv, hd, _ptr(aws), aws.numel(), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
+        *_wptrs(wo), *_wptrs(gate), *_wptrs(up), *_wptrs(down), _ptr(y), E, H, group, _ptr(ws), ws.numel(), _stream()))
+    return y
+
+
 def rope_halfsplit(x, lut):
     """Half-split RoPE of x bf16 [rows, dim] with one LUT row (cos then sin) per row: lut bf16 [rows, dim]."""
     lib = _lib.load_library()

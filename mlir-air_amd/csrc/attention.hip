@@ -16,8 +16,6 @@
 //
 // Rounding points follow the reference's decode step: Q and K are rounded to bf16 after RoPE,
 // scores, softmax and the weighted sum are fp32, the output is rounded to bf16 once.
-#include <type_traits>
-
 #include "common.h"
 #include "kernels.h"
 
@@ -25,7 +23,7 @@ namespace w4a16 {
 
 namespace {
 
-constexpr float kNegBig = -1e30f;   // "no score yet": finite, so differences of two of them are 0, not NaN
+constexpr float kNegBig = kAttnNegBig;
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct AttnParams {
@@ -70,24 +68,6 @@ __device__ __forceinline__ float group_sum(float s) {
     s = dpp_add<0x141>(s);   // row_half_mirror
     if constexpr (LPP == 16) s = dpp_add<0x140>(s);   // row_mirror
     return s;
-}
-
-// Maximum / sum over the 64 lanes of a wavefront, every lane receiving the result: the four steps inside a row of
-// 16 lanes on DPP moves as in group_sum, the two steps across rows by shuffle.
-template <bool MAX>
-__device__ __forceinline__ float wave_reduce(float v) {
-    auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
-    auto dpp = [&](auto ctrl) {
-        constexpr int CTRL = decltype(ctrl)::value;
-        const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
-        v = op(v, __builtin_bit_cast(float, moved));
-    };
-    dpp(std::integral_constant<int, 0xB1>());    // quad_perm [1, 0, 3, 2]
-    dpp(std::integral_constant<int, 0x4E>());    // quad_perm [2, 3, 0, 1]
-    dpp(std::integral_constant<int, 0x141>());   // row_half_mirror
-    dpp(std::integral_constant<int, 0x140>());   // row_mirror
-    v = op(v, __shfl_xor(v, 16));
-    return op(v, __shfl_xor(v, 32));
 }
 
 // Half-split RoPE of elements [e0, e0 + 8) of one head: x at src, rounded to bf16 (returned as floats).
@@ -305,7 +285,7 @@ size_t attention_workspace_bytes(int n_heads, int head_dim) {
 
 hipError_t launch_decode_attention(const uint16_t *qkv, const uint16_t *lut_row, uint16_t *k_cache, uint16_t *v_cache,
                                    uint16_t *out, int pos, int max_seq, int n_heads, int n_kv, int head_dim,
-                                   void *workspace, hipStream_t stream) {
+                                   void *workspace, hipStream_t stream, bool combine) {
     AttnParams p;
     p.qkv = qkv;
     p.lut = lut_row;
@@ -325,7 +305,7 @@ hipError_t launch_decode_attention(const uint16_t *qkv, const uint16_t *lut_row,
     const dim3 grid(p.nsplit, n_kv);
     hipError_t e = head_dim == 64 ? launch_g<64>(n_heads / n_kv, p, grid, stream)
                                   : launch_g<128>(n_heads / n_kv, p, grid, stream);
-    if (e != hipSuccess || p.nsplit == 1) return e;
+    if (e != hipSuccess || p.nsplit == 1 || !combine) return e;
     hipLaunchKernelGGL(attn_combine_kernel, dim3(n_heads), dim3(head_dim), 0, stream, p.part_ml, p.part_acc, out,
                        p.nsplit, head_dim);
     return hipGetLastError();

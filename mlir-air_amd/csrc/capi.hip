@@ -95,10 +95,16 @@ int rms_gemv_impl(bool affine, const uint16_t *x, const uint16_t *norm_weight, f
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+// The decode attention's chunk partials, when stage 1 of the block merges them itself (StreamExtras::attn_*).
+struct AttnPartials {
+    const float *ml, *acc;
+    int nsplit, hd;
+};
+
 int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
                     float eps, const QuantW &wo, const QuantW &wg, const QuantW &wu, const QuantW &wd, uint16_t *y,
                     uint16_t *res1_out, uint16_t *h_out, int E, int H, int group, void *workspace,
-                    size_t workspace_bytes, void *stream) {
+                    size_t workspace_bytes, void *stream, const AttnPartials *partials = nullptr, bool check_only = false) {
     if (!attn_out || !x_residual || !ffn_norm_weight || !y) return W4A16_ERR_NULL;
     int rc = check_w(affine, wo, E, E, group);
     if (rc) return rc;
@@ -114,6 +120,7 @@ int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_res
         return W4A16_ERR_ALIGN;
     if (!workspace || workspace_bytes < w4a16_block_workspace_bytes(E, H)) return W4A16_ERR_WORKSPACE;
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    if (check_only) return W4A16_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     char *tail = static_cast<char *>(workspace) + w4a16_block_workspace_bytes(E, H) - 256;
     float *res1_sumsq = reinterpret_cast<float *>(tail);
@@ -128,7 +135,14 @@ int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_res
     StreamExtras add;
     add.residual = x_residual;
     if (chain_norm) add.sumsq_out = res1_sumsq;
+    if (partials) {
+        add.attn_ml = partials->ml;
+        add.attn_acc = partials->acc;
+        add.attn_nsplit = partials->nsplit;
+        add.attn_hd = partials->hd;
+    }
     hipError_t e = stream_w(affine, attn_out, wo, nullptr, res1, 1, E, E, workspace, st, add);
+    add.attn_ml = add.attn_acc = nullptr;   // stage 3 reuses `add` for the down projection
     if (e != hipSuccess) return hip_fail(e);
     // stages 2 and 3 as one persistent kernel when the shape fits it (AWQ codec): h = swiglu(rms_norm(res1) . Wgate,
     // rms_norm(res1) . Wup), y = bf16(h . Wdown + res1)
@@ -486,6 +500,44 @@ int rope_halfsplit_bf16(const uint16_t *x, const uint16_t *lut, uint16_t *out, i
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+int w4a16_decode_attn_o_gemv_ffn_bf16(const uint16_t *qkv, const uint16_t *rope_lut_row, uint16_t *k_cache,
+                                      uint16_t *v_cache, uint16_t *attn_out, int pos, int max_seq, int n_heads,
+                                      int n_kv_heads, int head_dim, void *attn_workspace, size_t attn_workspace_bytes,
+                                      const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                                      const int32_t *o_qweight, const int32_t *o_qzeros, const uint16_t *o_scales,
+                                      const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
+                                      const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
+                                      const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
+                                      uint16_t *y, int E, int H, int group, void *workspace, size_t workspace_bytes,
+                                      void *stream) {
+    if (!qkv || !rope_lut_row || !k_cache || !v_cache || !attn_out) return W4A16_ERR_NULL;
+    if (head_dim != 64 && head_dim != 128) return W4A16_ERR_SHAPE;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || n_heads * head_dim != E) return W4A16_ERR_SHAPE;
+    const int g = n_heads / n_kv_heads;
+    if (g != 1 && g != 2 && g != 4 && g != 8) return W4A16_ERR_SHAPE;
+    if (max_seq <= 0 || pos < 0 || pos >= max_seq) return W4A16_ERR_SHAPE;
+    if (misaligned(qkv) || misaligned(rope_lut_row) || misaligned(k_cache) || misaligned(v_cache)) return W4A16_ERR_ALIGN;
+    if (!attn_workspace || attn_workspace_bytes < w4a16_attention_workspace_bytes(n_heads, head_dim)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(attn_workspace)) return W4A16_ERR_ALIGN;
+    const QuantW wo{o_qweight, o_qzeros, o_scales}, wg{gate_qweight, gate_qzeros, gate_scales},
+        wu{up_qweight, up_qzeros, up_scales}, wd{down_qweight, down_qzeros, down_scales};
+    int rc = o_gemv_ffn_impl(false, attn_out, x_residual, ffn_norm_weight, eps, wo, wg, wu, wd, y, nullptr, nullptr, E, H,
+                             group, workspace, workspace_bytes, stream, nullptr, true);
+    if (rc) return rc;
+    // With several sequence chunks and an O projection whose units lie inside one head, the projection merges the
+    // chunk partials itself and the merge launch is dropped; attn_out is then not written.
+    AttnPartials ap;
+    ap.nsplit = attention_nsplit(pos + 1);
+    ap.hd = head_dim;
+    attention_partials(attn_workspace, n_heads, &ap.ml, &ap.acc);
+    const bool fuse = !g_stream_tune.no_attn_fuse && stream_attn_fusable(E, E, head_dim, ap.nsplit);
+    hipError_t e = launch_decode_attention(qkv, rope_lut_row, k_cache, v_cache, attn_out, pos, max_seq, n_heads, n_kv_heads,
+                                           head_dim, attn_workspace, static_cast<hipStream_t>(stream), !fuse);
+    if (e != hipSuccess) return hip_fail(e);
+    return o_gemv_ffn_impl(false, attn_out, x_residual, ffn_norm_weight, eps, wo, wg, wu, wd, y, nullptr, nullptr, E, H,
+                           group, workspace, workspace_bytes, stream, fuse ? &ap : nullptr);
+}
+
 size_t lm_head_workspace_bytes(int V) { return V > 0 ? lm_head_scratch_bytes(V) : 0; }
 
 int lm_head_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const uint16_t *lm_head,
@@ -580,6 +632,8 @@ int w4a16_tune(const char *key, int value) {
         g_stream_tune.spin_limit = value;
     } else if (!strcmp(key, "ffn_fused")) {
         g_stream_tune.no_ffn_fused = value ? 0 : 1;
+    } else if (!strcmp(key, "attn_fuse")) {
+        g_stream_tune.no_attn_fuse = value ? 0 : 1;
     } else if (!strcmp(key, "gemm_stream_max_m")) {
         g_stream_tune.stream_max_m = value;
     } else if (!strcmp(key, "gemv_ksplit")) {

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace w4a16 {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -55,6 +57,28 @@ __device__ __forceinline__ void unpack8_f32(uint32_t w, float (&q)[8]) {
     q[3] = static_cast<float>((o >> 16) & 0xFFu);
     q[7] = static_cast<float>(o >> 24);
 }
+
+// Maximum / sum over the 64 lanes of a wavefront, every lane receiving the result: the four steps inside a row of
+// 16 lanes on DPP moves (quad permutes for distances 1 and 2, half-row and row mirrors for 4 and 8: once the
+// quads agree, mirroring meets the partner quad), the two steps across rows by shuffle.
+template <bool MAX>
+__device__ __forceinline__ float wave_reduce(float v) {
+    auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+    auto dpp = [&](auto ctrl) {
+        constexpr int CTRL = decltype(ctrl)::value;
+        const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+        v = op(v, __builtin_bit_cast(float, moved));
+    };
+    dpp(std::integral_constant<int, 0xB1>());    // quad_perm [1, 0, 3, 2]
+    dpp(std::integral_constant<int, 0x4E>());    // quad_perm [2, 3, 0, 1]
+    dpp(std::integral_constant<int, 0x141>());   // row_half_mirror
+    dpp(std::integral_constant<int, 0x140>());   // row_mirror
+    v = op(v, __shfl_xor(v, 16));
+    return op(v, __shfl_xor(v, 32));
+}
+
+// "No score yet" of the attention partials: finite, so differences of two of them are 0, not NaN.
+constexpr float kAttnNegBig = -1e30f;
 
 // Agent-scope (all XCDs) relaxed accesses for data exchanged between workgroups.
 __device__ __forceinline__ void store_agent(float *p, float v) {

@@ -23,6 +23,7 @@ struct StreamTune {
     int skip_publish = 0; // tests only: producers do not publish, so reducers run into their poll bound
     int spin_limit = 0;   // reducer poll bound (0 = default); tiny values force the timeout path in tests
     int no_ffn_fused = 0; // 1: w4a16_ffn_swiglu_bf16 always runs its two streaming launches
+    int no_attn_fuse = 0; // 1: w4a16_decode_attn_o_gemv_ffn_bf16 always runs the attention merge launch
 };
 extern StreamTune g_stream_tune;
 
@@ -50,7 +51,14 @@ struct StreamExtras {
     // [K / 32, N] too and `qzeros` is not read.  `up_mins` belongs to the second matrix of a SwiGLU launch.
     const uint16_t *mins = nullptr;
     const uint16_t *up_mins = nullptr;
+    // M == 1: x is not read; it is the merge of the decode attention's per-chunk partials (attention_partials below),
+    // computed by every wave for the rows of its units exactly as the attention merge kernel computes it.  Only where
+    // stream_attn_fusable says so.
+    const float *attn_ml = nullptr;    // [n_heads, nsplit, 2]
+    const float *attn_acc = nullptr;   // [n_heads, nsplit, head_dim]
+    int attn_nsplit = 0, attn_hd = 0;
 };
+bool stream_attn_fusable(int K, int N, int head_dim, int nsplit);
 
 // y[M, N] = bf16(x[M, K] . W), M <= 16.  With `up_*` given (SwiGLU epilogue, M == 1) the
 // kernel streams both weight sets and writes y = bf16(silu(bf16(x.Wg)) * bf16(x.Wu)).
@@ -138,7 +146,12 @@ int attention_nsplit(int seq_len);
 size_t attention_workspace_bytes(int n_heads, int head_dim);
 hipError_t launch_decode_attention(const uint16_t *qkv, const uint16_t *lut_row, uint16_t *k_cache, uint16_t *v_cache,
                                    uint16_t *out, int pos, int max_seq, int n_heads, int n_kv, int head_dim,
-                                   void *workspace, hipStream_t stream);
+                                   void *workspace, hipStream_t stream, bool combine = true);
+// Where launch_decode_attention(..., combine = false) leaves its partials inside the attention scratch buffer.
+inline void attention_partials(void *workspace, int n_heads, const float **ml, const float **acc) {
+    *ml = reinterpret_cast<const float *>(workspace);
+    *acc = *ml + (size_t)n_heads * kMaxAttnSplit * 2;
+}
 
 // Half-split RoPE of rows x dim bf16 with one LUT row (cos then sin) per row (attention.hip).
 hipError_t launch_rope_rows(const uint16_t *x, const uint16_t *lut, uint16_t *out, int rows, int dim, hipStream_t stream);

@@ -69,6 +69,8 @@ struct StreamParams {
     const float *sumsq_in;      // RMS, M == 1: partial sums of x^2 written by the kernel that produced x, or null
     int sumsq_n;
     float *sumsq_out;           // M == 1: sum of squares of this launch's bf16 outputs, one float per column tile, or null
+    const float *attn_ml, *attn_acc;   // ATT kernels: the decode attention's partials (StreamExtras)
+    int attn_nsplit, attn_hd;
     int spin_limit;
     int skip_publish;   // fault injection for tests: producers keep their partials to themselves
 };
@@ -103,7 +105,10 @@ struct Words<1> { typedef uint32_t type __attribute__((ext_vector_type(1))); };
 // AFF    affine codec with groups of 32 rows (one K-step): w = q * s + m with unsigned q, s and m
 //        bf16 [K / 32, N].  Every K-step is flushed on its own:
 //        y += s * sum (128 + q) x  +  (m - 128 s) * sum x.
-template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS, bool AFF>
+// ATT    M == 1: x is the merge of the decode attention's chunk partials, computed by every wave for the 64 rows of
+//        its unit (KSTEPS == 2, inside one head) with the merge kernel's arithmetic in the merge kernel's order,
+//        so the result is the same bit for bit; the partials are requested ahead of the weights.
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS, bool AFF, bool ATT = false>
 __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParams p) {
     constexpr int SLOTS = WAVES;   // one LDS slot per wave: a single write round, no read-modify-write
     typedef typename Words<LW>::type wvec;
@@ -225,9 +230,25 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         }
         // x first (a wave's loads return in order and the x sum needs every K-step's x), then the weights
         // K-step by K-step, so that K-step s can be consumed while the later ones are still in flight.
+        float attn_a[ATT ? kMaxAttnSplit : 1];
+        float attn_m = kAttnNegBig, attn_l = 0.f;
+        if constexpr (ATT) {
+            static_assert(!ATT || (KSTEPS == 2 && MI == 1 && NMAT == 1 && !RMS && !AFF), "attention merge prologue: plain M = 1 units of 64 rows");
+            const int head = (kstep0 * 32) / p.attn_hd;                 // scalar: the unit lies inside one head
+            const int e = kstep0 * 32 - head * p.attn_hd + lane;        // this lane's element of the head
+            const float *src = p.attn_acc + (size_t)head * p.attn_nsplit * p.attn_hd + e;
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s)
-            av[s] = *reinterpret_cast<const u32x4 *>(x_s + (size_t)(kstep0 + s) * 32 * sizeof(uint16_t) + x_lane);
+            for (int c = 0; c < kMaxAttnSplit; ++c) attn_a[c] = c < p.attn_nsplit ? src[(size_t)c * p.attn_hd] : 0.f;
+            if (lane < p.attn_nsplit) {                                 // lane c owns chunk c
+                const float *ml = p.attn_ml + 2 * ((size_t)head * p.attn_nsplit + lane);
+                attn_m = ml[0];
+                attn_l = ml[1];
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s)
+                av[s] = *reinterpret_cast<const u32x4 *>(x_s + (size_t)(kstep0 + s) * 32 * sizeof(uint16_t) + x_lane);
+        }
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
             const size_t krow = (size_t)(kstep0 + s) * 32;          // scalar
@@ -279,6 +300,24 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
                     av[s][j] = pack_bf16x2((x_lo * rstd) * w_lo, (x_hi * rstd) * w_hi);
                 }
             }
+        }
+        if constexpr (ATT) {
+            // out[e] = sum_c acc_c[e] 2^(m_c - M) / sum_c l_c 2^(m_c - M), as in attn_combine_kernel
+            const float mn = wave_reduce<true>(attn_m);
+            const float wgt = lane < p.attn_nsplit ? exp2f(attn_m - mn) : 0.f;
+            const float inv_l = 1.0f / wave_reduce<false>(attn_l * wgt);
+            float as = 0.f;
+#pragma unroll
+            for (int c = 0; c < kMaxAttnSplit; ++c)
+                as = fmaf(attn_a[c], __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wgt), c)), as);
+            // lane i holds row i of the unit; the MFMA operand wants 8 consecutive rows in lanes 0, 16, 32, 48: through
+            // the wave's own part of the combine buffer (LDS operations of one wave are carried out in order)
+            uint16_t *stage = reinterpret_cast<uint16_t *>(red + wave * (p.M * ROWF));
+            stage[lane] = float_to_bf16_bits(as * inv_l);
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) av[s] = *reinterpret_cast<const u32x4 *>(stage + 32 * s + 8 * lg);
+            asm volatile("" ::: "memory");
         }
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s)
@@ -573,15 +612,21 @@ StreamPlan plan_stream(int M, int K, int N, bool fixed_shape) {
     return pl;
 }
 
-template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false, bool AFF = false>
+bool stream_attn_fusable(int K, int N, int head_dim, int nsplit) {
+    if (head_dim <= 0 || head_dim % 64 != 0 || K % head_dim != 0 || nsplit < 2 || nsplit > kMaxAttnSplit) return false;
+    const StreamPlan pl = plan_stream(1, K, N);
+    return pl.lw == 2 && pl.ksteps == 2 && pl.waves == 8;   // units of 64 rows: a unit never straddles two heads
+}
+
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false, bool AFF = false, bool ATT = false>
 static hipError_t launch_one(const StreamParams &p, dim3 grid, hipStream_t stream) {
     const size_t lds = (size_t)WAVES * p.M * 8 * LW * 16 * sizeof(float);   // 128 KB at M = 16, LW = 2, 8 waves
     if (lds > 64 * 1024) {   // more than 64 KB of dynamic LDS needs the attribute (per device, so set it every time)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF, ATT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF>), grid, dim3(WAVES * 64), lds, stream, p);
+    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF, ATT>), grid, dim3(WAVES * 64), lds, stream, p);
     return hipGetLastError();
 }
 
@@ -658,9 +703,19 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.sumsq_in = extras.sumsq_in;
     p.sumsq_n = extras.sumsq_n;
     p.sumsq_out = extras.sumsq_out;
+    p.attn_ml = extras.attn_ml;
+    p.attn_acc = extras.attn_acc;
+    p.attn_nsplit = extras.attn_nsplit;
+    p.attn_hd = extras.attn_hd;
     p.skip_publish = g_stream_tune.skip_publish;
     p.spin_limit = g_stream_tune.spin_limit > 0 ? g_stream_tune.spin_limit : (1 << 18);
     const dim3 grid(((pl.ntiles + 7) / 8) * 8, pl.ksplit, p.nmat);
+    if (extras.attn_acc) {   // x comes from the attention partials: one instantiation, shapes checked by stream_attn_fusable
+        if (M != 1 || up_qweight || extras.norm_w || extras.mins || !extras.attn_ml ||
+            !stream_attn_fusable(K, N, extras.attn_hd, extras.attn_nsplit))
+            return hipErrorInvalidValue;
+        return launch_one<2, 2, 2, 8, 1, 1, false, false, true>(p, grid, stream);
+    }
     return pl.lw == 1 ? launch_ksteps<1, 1>(pl.ksteps, pl.waves, pl.mi, p, grid, stream)
                       : launch_ksteps<2, 2>(pl.ksteps, pl.waves, pl.mi, p, grid, stream);
 }

@@ -248,3 +248,38 @@ def test_generate_is_prefill_plus_greedy_decoding_and_stops_at_eos(ops):
             assert out == want[:cut + 1]
     with pytest.raises(ValueError):
         decode.generate(prompt, layers, embed, final_norm, embed, cfg, lut, n_tokens=60)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,H,max_seq,positions", [
+    (32, 8, 128, 14336, 2048, [0, 63, 64, 500, 2047]),   # Llama-3-8B layer: fused from position 64 on (2 .. 32 chunks)
+    (32, 8, 64, 8192, 2048, [100, 2047]),                # Llama-3.2-1B layer
+    (8, 2, 64, 1024, 300, [10, 299]),                    # small E
+])
+def test_attention_and_block_in_one_call_equal_the_two_calls(ops, n_heads, n_kv, hd, H, max_seq, positions):
+    """w4a16_decode_attn_o_gemv_ffn_bf16 against w4a16_decode_attention_bf16 + w4a16_o_gemv_ffn_bf16: the same output bit
+    for bit (the O projection's merge of the attention partials repeats the merge kernel's arithmetic in its order), the
+    same cache update, with the merge launch kept (tune attn_fuse = 0) and dropped."""
+    E = n_heads * hd
+    rng = np.random.default_rng(n_heads + hd + H)
+    wo, wg, wu, wd = (tuple(map(dev, make_awq(a, b, seed=50 + i))) for i, (a, b) in enumerate([(E, E), (E, H), (E, H), (H, E)]))
+    small = lambda w: (w[0], w[1], (w[2].float() * 0.05).to(torch.bfloat16))
+    wo, wg, wu, wd = map(small, (wo, wg, wu, wd))
+    norm_w = dev(f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32)))
+    lut = dev(odec.generate_rope_lut(hd, 500000.0, max_seq))
+    kc0 = f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32))
+    vc0 = f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32))
+    for pos in positions:
+        print(f"attention + block in one call: heads {n_heads}/{n_kv} hd={hd} pos={pos}", flush=True)
+        qkv = dev(make_x(((n_heads + 2 * n_kv) * hd,), seed=pos + 1))
+        x_res = dev(make_x((E,), seed=pos + 2))
+        ka, va = dev(kc0), dev(vc0)
+        attn = ops.decode_attention(qkv, lut[pos], ka, va, pos, n_heads)
+        want = ops.o_gemv_ffn(attn, x_res, norm_w, wo, wg, wu, wd)
+        for fuse in (1, 0):
+            ops.tune("attn_fuse", fuse)
+            kb, vb = dev(kc0), dev(vc0)
+            got = ops.decode_attn_o_gemv_ffn(qkv, lut[pos], kb, vb, pos, n_heads, x_res, norm_w, wo, wg, wu, wd)
+            torch.cuda.synchronize()
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (pos, fuse)
+            assert torch.equal(kb.view(torch.int16), ka.view(torch.int16)) and torch.equal(vb.view(torch.int16), va.view(torch.int16))
+        ops.tune("attn_fuse", 1)
