@@ -34,8 +34,8 @@ CONFIGS = {
     "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128"),
     # beyond the five headline configs: the O projection + RMSNorm + FFN decode block with residuals (3 launches)
     "block": dict(M=1, K=4096, N=14336, cfg=None, desc="decode block O-proj + RMSNorm + SwiGLU FFN W4A16 E=4096 H=14336 g128"),
-    # one whole decode layer: RMSNorm + fused QKV GEMV, RoPE + KV append + GQA attention over 2048 cached
-    # positions (32 heads, 8 KV heads, head_dim 128), then the block above
+    # one whole decode layer: RMSNorm + fused QKV GEMV, then RoPE + KV append + GQA attention over 2048 cached
+    # positions (32 heads, 8 KV heads, head_dim 128) and the block above as one call
     "layer": dict(M=1, K=4096, N=14336, cfg=None, desc="decode layer W4A16 E=4096 H=14336 32/8 heads hd=128 pos=2047 g128"),
     # the Q4NX codec (w = q * s + m, 32-column groups) through the same streaming kernel: the gate / up
     # projection shape of Llama-3.1-8B (programming_examples/llms/llama31_8b_q4nx)
@@ -201,11 +201,12 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                 _lib.check(lib.w4a16_rms_gemv_bf16(x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, qw[0].data_ptr(),
                                                    qw[1].data_ptr(), qw[2].data_ptr(), qkv.data_ptr(), K, nqkv, 128,
                                                    ws.data_ptr(), ws.numel(), st))
-                _lib.check(lib.w4a16_decode_attention_bf16(qkv.data_ptr(), lut_row.data_ptr(), k_cache.data_ptr(),
-                                                           v_cache.data_ptr(), attn_out.data_ptr(), LAYER_POS, LAYER_MAXSEQ,
-                                                           LAYER_HEADS, LAYER_KV, LAYER_HD, attn_ws.data_ptr(),
-                                                           attn_ws.numel(), st))
-                a_in = attn_out
+                # attention + block as one call (the O projection merges the attention's chunk partials itself)
+                _lib.check(lib.w4a16_decode_attn_o_gemv_ffn_bf16(
+                    qkv.data_ptr(), lut_row.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), attn_out.data_ptr(), LAYER_POS,
+                    LAYER_MAXSEQ, LAYER_HEADS, LAYER_KV, LAYER_HD, attn_ws.data_ptr(), attn_ws.numel(), x_residual.data_ptr(),
+                    norm_w.data_ptr(), 1e-5, *ptrs, outs[0].data_ptr(), K, N, 128, ws.data_ptr(), ws.numel(), st))
+                return
             rc = lib.w4a16_o_gemv_ffn_bf16(a_in.data_ptr(), x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, *ptrs,
                                            outs[0].data_ptr(), None, None, K, N, 128, ws.data_ptr(), ws.numel(), st)
         elif lm_head:
