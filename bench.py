@@ -171,6 +171,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         qkv = torch.empty((nqkv,), dtype=torch.bfloat16, device=dev)
         attn_out = torch.empty((K,), dtype=torch.bfloat16, device=dev)
         attn_ws = torch.empty(int(lib.w4a16_attention_workspace_bytes(LAYER_HEADS, LAYER_HD)), dtype=torch.uint8, device=dev)
+        x_sumsq = (x_residual.float() ** 2).reshape(K // 256, 256).sum(dim=1).contiguous()
+        y_sumsq = torch.empty((K // 256,), dtype=torch.float32, device=dev)
 
     if name == "ffn":
         ws_bytes = lib.w4a16_ffn_workspace_bytes(K, N)
@@ -198,14 +200,16 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             a_in = x
             if name == "layer":
                 qw = w[4]
-                _lib.check(lib.w4a16_rms_gemv_bf16(x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, qw[0].data_ptr(),
-                                                   qw[1].data_ptr(), qw[2].data_ptr(), qkv.data_ptr(), K, nqkv, 128,
-                                                   ws.data_ptr(), ws.numel(), st))
+                # the sum of squares of x per 256-column tile comes from the block before (here: computed once)
+                _lib.check(lib.w4a16_rms_gemv_sumsq_bf16(x_residual.data_ptr(), x_sumsq.data_ptr(), x_sumsq.numel(),
+                                                         norm_w.data_ptr(), 1e-5, qw[0].data_ptr(), qw[1].data_ptr(),
+                                                         qw[2].data_ptr(), qkv.data_ptr(), K, nqkv, 128, ws.data_ptr(),
+                                                         ws.numel(), st))
                 # attention + block as one call (the O projection merges the attention's chunk partials itself)
                 _lib.check(lib.w4a16_decode_attn_o_gemv_ffn_bf16(
                     qkv.data_ptr(), lut_row.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), attn_out.data_ptr(), LAYER_POS,
                     LAYER_MAXSEQ, LAYER_HEADS, LAYER_KV, LAYER_HD, attn_ws.data_ptr(), attn_ws.numel(), x_residual.data_ptr(),
-                    norm_w.data_ptr(), 1e-5, *ptrs, outs[0].data_ptr(), K, N, 128, ws.data_ptr(), ws.numel(), st))
+                    norm_w.data_ptr(), 1e-5, *ptrs, outs[0].data_ptr(), y_sumsq.data_ptr(), K, N, 128, ws.data_ptr(), ws.numel(), st))
                 return
             rc = lib.w4a16_o_gemv_ffn_bf16(a_in.data_ptr(), x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, *ptrs,
                                            outs[0].data_ptr(), None, None, K, N, 128, ws.data_ptr(), ws.numel(), st)

@@ -224,7 +224,14 @@ size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim);
  * kernel's order, and the merge launch is dropped: y is the same bit for bit as from the two calls.  `attn_out`
  * bf16 [E] is scratch (it holds the attention output whenever the merge launch did run).  E == n_heads * head_dim;
  * other constraints and both workspaces as for the two calls.  w4a16_tune("attn_fuse", 0) keeps the merge launch.
+ * y_sumsq (NULL, or E / 256 floats with E % 256 == 0, E <= 16384): receives the sum of squares of the bf16 values
+ * of y per 256-column tile, which w4a16_rms_gemv_sumsq_bf16 of the next layer takes in place of its own pass over
+ * x: there x_sumsq holds n_pieces (<= 64) partial sums of x^2, and the result is that of w4a16_rms_gemv_bf16 up to
+ * the summation order of the mean (the RMSNorm front of rms_qkv_int4_rope, rms_qkv_int4_rope_multi.py:4-30).
  */
+int w4a16_rms_gemv_sumsq_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
+                              const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, uint16_t *y, int K,
+                              int N, int group, void *workspace, size_t workspace_bytes, void *stream);
 int w4a16_decode_attn_o_gemv_ffn_bf16(const uint16_t *qkv, const uint16_t *rope_lut_row, uint16_t *k_cache,
                                       uint16_t *v_cache, uint16_t *attn_out, int pos, int max_seq, int n_heads,
                                       int n_kv_heads, int head_dim, void *attn_workspace, size_t attn_workspace_bytes,
@@ -233,8 +240,8 @@ int w4a16_decode_attn_o_gemv_ffn_bf16(const uint16_t *qkv, const uint16_t *rope_
                                       const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
                                       const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
                                       const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
-                                      uint16_t *y, int E, int H, int group, void *workspace, size_t workspace_bytes,
-                                      void *stream);
+                                      uint16_t *y, float *y_sumsq, int E, int H, int group, void *workspace,
+                                      size_t workspace_bytes, void *stream);
 
 /*
  * Half-split RoPE on its own, for callers that keep the reference's launch structure (launches L5 and L6

@@ -92,16 +92,21 @@ def new_kv_cache(config, max_seq, device="cuda"):
             for _ in range(config.n_layers)]
 
 
-def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer, current_pos, rope_lut):
+def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer, current_pos, rope_lut, x_sumsq=None,
+                     return_sumsq=False):
     """One transformer block for one decode token; x bf16 [emb] -> bf16 [emb].  The caches are
-    updated in place at current_pos."""
+    updated in place at current_pos.  x_sumsq / return_sumsq chain the sum of squares of the block's output into
+    the next block's RMSNorm (AWQ layers): with return_sumsq the result is (y, sumsq or None)."""
     q4nx = layer.codec == "q4nx"
-    qkv = (ops.q4nx_rms_gemv if q4nx else ops.w4a16_rms_gemv)(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps)
     if not q4nx:   # attention + block as one call: the O projection merges the attention's chunk partials where it can
+        qkv = ops.w4a16_rms_gemv(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps, x_sumsq=x_sumsq)
         return ops.decode_attn_o_gemv_ffn(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads,
-                                          x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
+                                          x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps,
+                                          return_sumsq=return_sumsq)
+    qkv = ops.q4nx_rms_gemv(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps)
     attn_out = ops.decode_attention(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads)
-    return (ops.q4nx_o_gemv_ffn if q4nx else ops.o_gemv_ffn)(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
+    y = ops.q4nx_o_gemv_ffn(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
+    return (y, None) if return_sumsq else y
 
 
 def decode_token(token_id, layers, embed_table, final_norm, lm_head, config, kv_cache, current_pos, rope_lut,
@@ -111,8 +116,9 @@ def decode_token(token_id, layers, embed_table, final_norm, lm_head, config, kv_
     fp32 [vocab], like the reference, and with return_argmax also the greedy token as a device
     int32 tensor [1] (no host synchronisation here)."""
     x = embed_table[token_id].contiguous()
+    sumsq = None   # every block leaves the sum of squares of its output for the next block's norm
     for layer, (kc, vc) in zip(layers, kv_cache):
-        x = run_decode_block(x, layer, config, kc, vc, current_pos, rope_lut)
+        x, sumsq = run_decode_block(x, layer, config, kc, vc, current_pos, rope_lut, x_sumsq=sumsq, return_sumsq=True)
     logits, best = ops.lm_head(x, lm_head, norm_weight=final_norm, eps=config.rms_eps)
     return (logits.float(), best) if return_argmax else logits.float()
 
@@ -127,8 +133,9 @@ def decode_greedy(token, n_tokens, layers, embed_table, final_norm, lm_head, con
     tok = token.to(torch.int32).reshape(1)
     for i in range(n_tokens):
         x = embed_table.index_select(0, tok).reshape(-1)
+        sumsq = None
         for layer, (kc, vc) in zip(layers, kv_cache):
-            x = run_decode_block(x, layer, config, kc, vc, start_pos + i, rope_lut)
+            x, sumsq = run_decode_block(x, layer, config, kc, vc, start_pos + i, rope_lut, x_sumsq=sumsq, return_sumsq=True)
         _, tok = ops.lm_head(x, lm_head, norm_weight=final_norm, eps=config.rms_eps)
         out[i:i + 1] = tok
     return out

@@ -157,8 +157,10 @@ def w4a16_gemv_add(x, qweight, qzeros, scales, residual, group=GROUP, out=None):
     return out
 
 
-def w4a16_rms_gemv(x, norm_weight, qweight, qzeros, scales, eps=1e-5, group=GROUP):
-    """y[N] = bf16(rms_norm(x, norm_weight) . W), the normalised vector rounded to bf16 first."""
+def w4a16_rms_gemv(x, norm_weight, qweight, qzeros, scales, eps=1e-5, group=GROUP, x_sumsq=None):
+    """y[N] = bf16(rms_norm(x, norm_weight) . W), the normalised vector rounded to bf16 first.  x_sumsq: float32
+    partial sums of x^2 (at most 64) left by the call that produced x (decode_attn_o_gemv_ffn), used for the mean
+    instead of a pass over x."""
     lib = _lib.load_library()
     _need_cuda(x, norm_weight, qweight, qzeros, scales)
     K = x.numel()
@@ -167,6 +169,13 @@ def w4a16_rms_gemv(x, norm_weight, qweight, qzeros, scales, eps=1e-5, group=GROU
     N = qweight.shape[1] * 8
     out = torch.empty((N,), dtype=torch.bfloat16, device=x.device)
     ws = workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
+    if x_sumsq is not None:
+        if x_sumsq.dtype != torch.float32 or not x_sumsq.is_cuda or not x_sumsq.is_contiguous():
+            raise ValueError("x_sumsq must be a contiguous float32 GPU tensor")
+        _lib.check(lib.w4a16_rms_gemv_sumsq_bf16(_ptr(_bits(x)), _ptr(x_sumsq), x_sumsq.numel(), _ptr(_bits(norm_weight)),
+                                                 float(eps), *_wptrs((qweight, qzeros, scales)), _ptr(out), K, N, group,
+                                                 _ptr(ws), ws.numel(), _stream()))
+        return out
     _lib.check(lib.w4a16_rms_gemv_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
                                        *_wptrs((qweight, qzeros, scales)), _ptr(out), K, N, group,
                                        _ptr(ws), ws.numel(), _stream()))
@@ -243,9 +252,11 @@ def decode_attention(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, out=None
 
 
 def decode_attn_o_gemv_ffn(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, x_residual, ffn_norm_weight, wo, gate, up, down,
-                           eps=1e-5, group=GROUP):
+                           eps=1e-5, group=GROUP, return_sumsq=False):
     """decode_attention followed by o_gemv_ffn in one call; over several sequence chunks the O projection merges the
-    attention partials itself (one launch fewer), with the same result bit for bit.  Returns y bf16 [E]."""
+    attention partials itself (one launch fewer), with the same result bit for bit.  Returns y bf16 [E], with
+    return_sumsq also float32 [E / 256]: the sum of squares of y per 256-column tile for the next layer's
+    w4a16_rms_gemv (None where E is not a multiple of 256)."""
     lib = _lib.load_library()
     _need_cuda(qkv, rope_lut_row, k_cache, v_cache, x_residual, ffn_norm_weight, *wo, *gate, *up, *down)
     n_kv, max_seq, hd = k_cache.shape
@@ -265,11 +276,13 @@ def decode_attn_o_gemv_ffn(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, x_
         aws = torch.empty(int(lib.w4a16_attention_workspace_bytes(n_heads, hd)), dtype=torch.uint8, device=dev)
         _attn_ws[key] = aws
     ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev, ("block", E, H))
+    sumsq = torch.empty((E // 256,), dtype=torch.float32, device=dev) if return_sumsq and E % 256 == 0 and E <= 16384 else None
     _lib.check(lib.w4a16_decode_attn_o_gemv_ffn_bf16(
         _ptr(_bits(qkv)), _ptr(_bits(rope_lut_row)), _ptr(_bits(k_cache)), _ptr(_bits(v_cache)), _ptr(attn_out), int(pos),
         max_seq, n_heads, n_kv, hd, _ptr(aws), aws.numel(), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
-        *_wptrs(wo), *_wptrs(gate), *_wptrs(up), *_wptrs(down), _ptr(y), E, H, group, _ptr(ws), ws.numel(), _stream()))
-    return y
+        *_wptrs(wo), *_wptrs(gate), *_wptrs(up), *_wptrs(down), _ptr(y), _ptr(sumsq) if sumsq is not None else None, E, H, group,
+        _ptr(ws), ws.numel(), _stream()))
+    return (y, sumsq) if return_sumsq else y
 
 
 def rope_halfsplit(x, lut):

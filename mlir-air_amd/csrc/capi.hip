@@ -80,7 +80,8 @@ hipError_t stream_w(bool affine, const uint16_t *x, const QuantW &a, const Quant
 }
 
 int rms_gemv_impl(bool affine, const uint16_t *x, const uint16_t *norm_weight, float eps, const QuantW &w, uint16_t *y,
-                  int K, int N, int group, void *workspace, size_t workspace_bytes, void *stream) {
+                  int K, int N, int group, void *workspace, size_t workspace_bytes, void *stream,
+                  const float *x_sumsq = nullptr, int n_pieces = 0) {
     if (!x || !y || !norm_weight) return W4A16_ERR_NULL;
     int rc = check_w(affine, w, K, N, group);
     if (rc) return rc;
@@ -91,6 +92,8 @@ int rms_gemv_impl(bool affine, const uint16_t *x, const uint16_t *norm_weight, f
     StreamExtras ex;
     ex.norm_w = norm_weight;
     ex.eps = eps;
+    ex.sumsq_in = x_sumsq;
+    ex.sumsq_n = x_sumsq ? n_pieces : 0;
     hipError_t e = stream_w(affine, x, w, nullptr, y, 1, K, N, workspace, static_cast<hipStream_t>(stream), ex);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
@@ -104,7 +107,8 @@ struct AttnPartials {
 int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
                     float eps, const QuantW &wo, const QuantW &wg, const QuantW &wu, const QuantW &wd, uint16_t *y,
                     uint16_t *res1_out, uint16_t *h_out, int E, int H, int group, void *workspace,
-                    size_t workspace_bytes, void *stream, const AttnPartials *partials = nullptr, bool check_only = false) {
+                    size_t workspace_bytes, void *stream, const AttnPartials *partials = nullptr, bool check_only = false,
+                    float *y_sumsq = nullptr) {
     if (!attn_out || !x_residual || !ffn_norm_weight || !y) return W4A16_ERR_NULL;
     int rc = check_w(affine, wo, E, E, group);
     if (rc) return rc;
@@ -155,7 +159,7 @@ int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_res
                                       static_cast<const int32_t *>(wd.aux)};
         const uint16_t *const sc[3] = {wg.sc, wu.sc, wd.sc};
         const FfnFusedNorm norm = {ffn_norm_weight, res1_sumsq, res1_tiles, eps};
-        e = launch_ffn_fused(fpl, res1, qw, qz, sc, res1, y, h_out, E, H, workspace, st, &norm);
+        e = launch_ffn_fused(fpl, res1, qw, qz, sc, res1, y, h_out, E, H, workspace, st, &norm, y_sumsq);
         return e == hipSuccess ? W4A16_OK : hip_fail(e);
     }
     // stage 2: h = swiglu(rms_norm(res1) . Wgate, rms_norm(res1) . Wup)
@@ -169,7 +173,7 @@ int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_res
     e = stream_w(affine, res1, wg, &wu, h, 1, E, H, workspace, st, rms);
     if (e != hipSuccess) return hip_fail(e);
     // stage 3: y = bf16(h . Wdown + res1)
-    add.sumsq_out = nullptr;
+    add.sumsq_out = y_sumsq;
     add.residual = res1;
     e = stream_w(affine, h, wd, nullptr, y, 1, H, E, workspace, st, add);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
@@ -346,6 +350,16 @@ int w4a16_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float ep
                          workspace_bytes, stream);
 }
 
+int w4a16_rms_gemv_sumsq_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
+                              const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, uint16_t *y, int K,
+                              int N, int group, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!x_sumsq) return W4A16_ERR_NULL;
+    if (n_pieces < 1 || n_pieces > 64) return W4A16_ERR_SHAPE;
+    if (misaligned(x_sumsq)) return W4A16_ERR_ALIGN;
+    return rms_gemv_impl(false, x, norm_weight, eps, QuantW{qweight, qzeros, scales}, y, K, N, group, workspace,
+                         workspace_bytes, stream, x_sumsq, n_pieces);
+}
+
 int w4a16_rms_gemv_swiglu_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps,
                                const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
                                const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
@@ -508,9 +522,11 @@ int w4a16_decode_attn_o_gemv_ffn_bf16(const uint16_t *qkv, const uint16_t *rope_
                                       const int32_t *gate_qweight, const int32_t *gate_qzeros, const uint16_t *gate_scales,
                                       const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
                                       const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
-                                      uint16_t *y, int E, int H, int group, void *workspace, size_t workspace_bytes,
-                                      void *stream) {
+                                      uint16_t *y, float *y_sumsq, int E, int H, int group, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
     if (!qkv || !rope_lut_row || !k_cache || !v_cache || !attn_out) return W4A16_ERR_NULL;
+    if (y_sumsq && (E % 256 != 0 || E / 256 > 64)) return W4A16_ERR_SHAPE;
+    if (y_sumsq && misaligned(y_sumsq)) return W4A16_ERR_ALIGN;
     if (head_dim != 64 && head_dim != 128) return W4A16_ERR_SHAPE;
     if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || n_heads * head_dim != E) return W4A16_ERR_SHAPE;
     const int g = n_heads / n_kv_heads;
@@ -535,7 +551,7 @@ int w4a16_decode_attn_o_gemv_ffn_bf16(const uint16_t *qkv, const uint16_t *rope_
                                            head_dim, attn_workspace, static_cast<hipStream_t>(stream), !fuse);
     if (e != hipSuccess) return hip_fail(e);
     return o_gemv_ffn_impl(false, attn_out, x_residual, ffn_norm_weight, eps, wo, wg, wu, wd, y, nullptr, nullptr, E, H,
-                           group, workspace, workspace_bytes, stream, fuse ? &ap : nullptr);
+                           group, workspace, workspace_bytes, stream, fuse ? &ap : nullptr, false, y_sumsq);
 }
 
 size_t lm_head_workspace_bytes(int V) { return V > 0 ? lm_head_scratch_bytes(V) : 0; }

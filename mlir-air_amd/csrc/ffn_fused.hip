@@ -49,6 +49,7 @@ struct FfnParams {
     float eps;
     uint16_t *y;                // [E]
     uint16_t *h_out;            // [H] or null
+    float *sumsq_out;           // [E / 256] or null: sum of squares of the bf16 y values of each 256-column tile
     uint32_t *header;
     float *partialA;
     float *partialB;
@@ -417,7 +418,16 @@ __global__ void __launch_bounds__(512, 2) ffn_fused_kernel(const FfnParams p) {
         out[2] += __builtin_bit_cast(float, r.y << 16);
         out[3] += __builtin_bit_cast(float, r.y & 0xFFFF0000u);
     }
-    *reinterpret_cast<uint2 *>(p.y + col) = uint2{pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3])};
+    const uint2 o = uint2{pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3])};
+    *reinterpret_cast<uint2 *>(p.y + col) = o;
+    if (p.sumsq_out) {   // same expression and order as the streaming kernel's epilogue, so either path feeds the next norm alike
+        const float r0 = __builtin_bit_cast(float, o.x << 16), r1 = __builtin_bit_cast(float, o.x & 0xFFFF0000u);
+        const float r2 = __builtin_bit_cast(float, o.y << 16), r3 = __builtin_bit_cast(float, o.y & 0xFFFF0000u);
+        float sq = fmaf(r0, r0, fmaf(r1, r1, fmaf(r2, r2, r3 * r3)));
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+        if (lane == 0) p.sumsq_out[tileB] = sq;
+    }
 }
 
 // Shape plan: the largest G <= cus with G = tilesA * splitA = tilesB * splitB, whole units per
@@ -448,7 +458,7 @@ size_t ffn_fused_scratch_bytes(int E, int H, const FfnFusedPlan &pl) {
 
 hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int32_t *const qw[3], const int32_t *const qz[3],
                             const uint16_t *const sc[3], const uint16_t *residual, uint16_t *y, uint16_t *h_out, int E, int H,
-                            void *workspace, hipStream_t stream, const FfnFusedNorm *norm) {
+                            void *workspace, hipStream_t stream, const FfnFusedNorm *norm, float *sumsq_out) {
     FfnParams p;
     p.x = x;
     for (int i = 0; i < 3; ++i) {
@@ -463,6 +473,7 @@ hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int
     p.eps = norm ? norm->eps : 0.f;
     p.y = y;
     p.h_out = h_out;
+    p.sumsq_out = sumsq_out;
     p.header = reinterpret_cast<uint32_t *>(workspace);
     char *base = reinterpret_cast<char *>(workspace) + kHeaderBytes;
     p.partialA = reinterpret_cast<float *>(base);

@@ -125,7 +125,8 @@ struct FfnFusedNorm {
 };
 hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int32_t *const qw[3], const int32_t *const qz[3],
                             const uint16_t *const sc[3], const uint16_t *residual, uint16_t *y, uint16_t *h_out, int E, int H,
-                            void *workspace, hipStream_t stream, const FfnFusedNorm *norm = nullptr);
+                            void *workspace, hipStream_t stream, const FfnFusedNorm *norm = nullptr,
+                            float *sumsq_out = nullptr);   // sumsq_out [E / 256]: sum of squares of y per 256-column tile
 
 // Q4NX / Q4_0 block codec (q4nx.hip).  mode: 0 w = s q + m, 1 w = s (q - m), 2 signed q, w = s q.
 hipError_t launch_q4nx_dequant(const void *blocks, uint16_t *out, int M, int K, int mode, hipStream_t stream);

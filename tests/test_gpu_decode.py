@@ -283,3 +283,38 @@ def test_attention_and_block_in_one_call_equal_the_two_calls(ops, n_heads, n_kv,
             assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (pos, fuse)
             assert torch.equal(kb.view(torch.int16), ka.view(torch.int16)) and torch.equal(vb.view(torch.int16), va.view(torch.int16))
         ops.tune("attn_fuse", 1)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,H", [(32, 8, 128, 14336), (32, 8, 64, 8192), (8, 2, 64, 1024)])
+def test_sum_of_squares_chained_into_the_next_norm(ops, n_heads, n_kv, hd, H):
+    """The block's y_sumsq is the sum of squares of its bf16 output per 256-column tile, and w4a16_rms_gemv fed with it
+    equals the plain call up to the summation order of the mean (one-ulp flips of the normalised vector)."""
+    E, pos, max_seq = n_heads * hd, 70, 128
+    rng = np.random.default_rng(E + H)
+    small = lambda w: (w[0], w[1], (w[2].float() * 0.05).to(torch.bfloat16))
+    wo, wg, wu, wd = (small(tuple(map(dev, make_awq(a, b, seed=80 + i)))) for i, (a, b) in enumerate([(E, E), (E, H), (E, H), (H, E)]))
+    wq = tuple(map(dev, make_awq(E, 512, seed=90)))
+    norm_w = dev(f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32)))
+    lut = dev(odec.generate_rope_lut(hd, 500000.0, max_seq))
+    kc = dev(f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32)))
+    vc = dev(f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32)))
+    qkv, x_res = dev(make_x(((n_heads + 2 * n_kv) * hd,), seed=3)), dev(make_x((E,), seed=4))
+    for fused_ffn in (1, 0):   # the persistent FFN kernel and the three streaming launches leave the same pieces
+        ops.tune("ffn_fused", fused_ffn)
+        print(f"chained sum of squares E={E} H={H} ffn_fused={fused_ffn}", flush=True)
+        y, sumsq = ops.decode_attn_o_gemv_ffn(qkv, lut[pos], kc.clone(), vc.clone(), pos, n_heads, x_res, norm_w, wo, wg, wu, wd,
+                                              return_sumsq=True)
+        torch.cuda.synchronize()
+        want = (y.float().double() ** 2).reshape(E // 256, 256).sum(dim=1)
+        assert sumsq.shape == (E // 256,) and torch.allclose(sumsq.double(), want, rtol=1e-5, atol=0)
+        if fused_ffn:
+            first = sumsq.clone()
+        else:
+            assert torch.equal(first, sumsq)
+    ops.tune("ffn_fused", 1)
+    plain = ops.w4a16_rms_gemv(y, norm_w, *wq)
+    chained = ops.w4a16_rms_gemv(y, norm_w, *wq, x_sumsq=sumsq)
+    torch.cuda.synchronize()
+    p64, c64 = plain.float().double().cpu().numpy(), chained.float().double().cpu().numpy()
+    assert np.max(np.abs(p64 - c64)) <= 2 * 2.0**-8 * np.max(np.abs(p64))
+    assert np.mean(p64 != c64) < 0.2

@@ -203,19 +203,25 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.lm_head_gemv_bf16(P, None, 0.0, P, P, None, 100, 512, P, lws - 1, None) == _lib.ERR_WORKSPACE
     aws = lib.w4a16_attention_workspace_bytes(4, 64)
     bws = lib.w4a16_block_workspace_bytes(256, 512)
-    fargs = [P, P, P, P, P, 3, 16, 4, 2, 64, P, aws, P, P, 1e-5] + [P] * 12 + [P, 256, 512, 128, P, bws, None]
+    fargs = [P, P, P, P, P, 3, 16, 4, 2, 64, P, aws, P, P, 1e-5] + [P] * 12 + [P, None, 256, 512, 128, P, bws, None]
     bad = list(fargs); bad[4] = None
     assert lib.w4a16_decode_attn_o_gemv_ffn_bf16(*bad) == _lib.ERR_NULL
-    bad = list(fargs); bad[28] = 512                                        # E != n_heads * head_dim
+    bad = list(fargs); bad[29] = 512                                        # E != n_heads * head_dim
     assert lib.w4a16_decode_attn_o_gemv_ffn_bf16(*bad) == _lib.ERR_SHAPE
     bad = list(fargs); bad[5] = 16                                          # pos == max_seq
     assert lib.w4a16_decode_attn_o_gemv_ffn_bf16(*bad) == _lib.ERR_SHAPE
     bad = list(fargs); bad[11] = aws - 1
     assert lib.w4a16_decode_attn_o_gemv_ffn_bf16(*bad) == _lib.ERR_WORKSPACE
-    bad = list(fargs); bad[32] = bws - 1
+    bad = list(fargs); bad[33] = bws - 1
     assert lib.w4a16_decode_attn_o_gemv_ffn_bf16(*bad) == _lib.ERR_WORKSPACE
     bad = list(fargs); bad[12] = None                                       # x_residual
     assert lib.w4a16_decode_attn_o_gemv_ffn_bf16(*bad) == _lib.ERR_NULL
+    bad = list(fargs); bad[28] = P + 4                                      # y_sumsq misaligned
+    assert lib.w4a16_decode_attn_o_gemv_ffn_bf16(*bad) == _lib.ERR_ALIGN
+    gws = lib.w4a16_gemm_workspace_bytes(1, 256, 64)
+    assert lib.w4a16_rms_gemv_sumsq_bf16(P, None, 1, P, 1e-5, P, P, P, P, 256, 64, 128, P, gws, None) == _lib.ERR_NULL
+    assert lib.w4a16_rms_gemv_sumsq_bf16(P, P, 65, P, 1e-5, P, P, P, P, 256, 64, 128, P, gws, None) == _lib.ERR_SHAPE
+    assert lib.w4a16_rms_gemv_sumsq_bf16(P, P, 1, P, 1e-5, P, P, P, P, 256, 64, 128, P, gws - 1, None) == _lib.ERR_WORKSPACE
     assert lib.rope_halfsplit_bf16(P, P, None, 8, 64, None) == _lib.ERR_NULL
     assert lib.rope_halfsplit_bf16(P, P, P, 8, 24, None) == _lib.ERR_SHAPE        # dim % 16
     assert lib.rope_halfsplit_bf16(P, P, P, 0, 64, None) == _lib.ERR_SHAPE
