@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_1b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_1b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -28,7 +28,10 @@ MALL_BYTES = 256 << 20
 CONFIGS = {
     # name: (M, K, N, bound, description)
     "dequant": dict(M=0, K=4096, N=4096, cfg=0, desc="AWQ dequant K=4096 N=4096 -> bf16"),
-    "gemv": dict(M=1, K=4096, N=11008, cfg=1, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128"),
+    # the weights re-packed once at load time (untimed, as the reference re-packs them) into stream order
+    "gemv": dict(M=1, K=4096, N=11008, cfg=1, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128, stream-order weights"),
+    # the same product on the AutoAWQ checkpoint layout (split-K kernel with a workspace)
+    "gemv_awq": dict(M=1, K=4096, N=11008, cfg=None, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128, checkpoint-layout weights"),
     "gemm16": dict(M=16, K=4096, N=14336, cfg=2, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128"),
     "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128"),
     "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128"),
@@ -49,7 +52,7 @@ LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 204
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
 # scaled by the same counter's reading for a 256 MiB device copy: x2.000 and x1.000); the
 # summaries under profiles/ hold the commands and the raw readings.
-MEASURED_TRAFFIC_BYTES = {"gemv": 24.27e6, "prefill": 342.2e6, "ffn": 97.07e6, "lm_head": 525.9e6}
+MEASURED_TRAFFIC_BYTES = {"gemv_awq": 24.27e6, "prefill": 342.2e6, "ffn": 97.07e6, "lm_head": 525.9e6}
 
 
 def weight_bytes(K, N):
@@ -145,6 +148,16 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             gw = torch.Generator(device="cuda")
             gw.manual_seed(100 + i)
             copies.append(((torch.randn((N, K), device="cuda", generator=gw) * 0.05).to(torch.bfloat16),))
+        elif name == "gemv":
+            # all copies in one arena, as a loader would place a model's layers
+            from air_hip import ops
+            w = make_weights(torch, K, N, 100 + i)
+            sb = int(lib.w4a16_stream_bytes(K, N))
+            if i == 0:
+                arena = torch.empty(ncopies * sb, dtype=torch.uint8, device=dev)
+            arena[i * sb:(i + 1) * sb].copy_(ops.repack_stream(*w).buf)
+            copies.append((arena[i * sb:(i + 1) * sb],) + (w if i == 0 else ()))   # copy 0 keeps its tensors for the CPU baseline
+            del w
         else:
             copies.append(make_weights(torch, K, N, 100 + i))
     gx = torch.Generator(device="cuda")
@@ -216,6 +229,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         elif lm_head:
             rc = lib.lm_head_gemv_bf16(x.data_ptr(), norm_w.data_ptr(), 1e-5, w[0].data_ptr(), outs[0].data_ptr(),
                                        best.data_ptr(), N, K, lm_ws.data_ptr(), lm_ws.numel(), st)
+        elif name == "gemv":
+            rc = lib.w4a16_gemv_stream_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), K, N, 128, st)
         elif q4nx:
             rc = lib.w4a16_q4nx_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), None,
                                           outs[0].data_ptr(), M, K, N, ws.data_ptr(), ws.numel(), st)
@@ -223,6 +238,14 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             rc = lib.w4a16_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
                                      outs[0].data_ptr(), M, K, N, 128, ws.data_ptr(), ws.numel(), st)
         _lib.check(rc)
+
+    def spacers(indices):
+        """Cold runs walk the weight copies cyclically; between two passes over `indices` the cycle is completed
+        with untimed launches, so that the next pass starts on the copy touched longest ago and finds nothing of
+        the previous pass in the Infinity Cache (ncopies x per_copy is 1.5 x its size)."""
+        if len(set(indices)) > 1:
+            for i in range(len(indices) % ncopies, ncopies if len(indices) % ncopies else 0):
+                launch(i, stream.cuda_stream)
 
     def timed_graph(indices):
         """Capture len(indices) launches into one HIP graph, replay it once between events."""
@@ -232,6 +255,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                 for i in indices:
                     launch(i, stream.cuda_stream)
             graph.replay()          # untimed replay: instantiation / first-touch effects
+            spacers(indices)
             stream.synchronize()
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
@@ -244,6 +268,24 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             wall = time.perf_counter() - t0
         return e0.elapsed_time(e1) * 1e-3, wall
 
+    def timed_eager(indices):
+        """The same launches issued one by one behind a spinning kernel: the host queues them while the GPU is
+        still busy, so the interval between the events holds the launches and not the host's launch latency."""
+        with torch.cuda.stream(stream):
+            for i in indices:
+                launch(i, stream.cuda_stream)
+            spacers(indices)
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            torch.cuda._sleep(int(2e5) * max(8, len(indices) // 4))
+            e0.record(stream)
+            for i in indices:
+                launch(i, stream.cuda_stream)
+            e1.record(stream)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3
+
     with torch.cuda.stream(stream):
         for i in range(warmup):
             launch(i, stream.cuda_stream)
@@ -251,6 +293,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
 
     cold_s, cold_wall = timed_graph(list(range(steps)))
     hot_s, _ = timed_graph([0] * steps)
+    eager_s = timed_eager(list(range(steps)))
 
     # one event pair per launch, outside a graph (the reference's harness style,
     # programming_examples/matrix_vector_multiplication/int4_awq/test_packed.cpp:114-150): each figure
@@ -269,6 +312,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         "name": name,
         "cold_us": cold_s / steps * 1e6,
         "hot_us": hot_s / steps * 1e6,
+        "eager_us": eager_s / steps * 1e6,
         "wall_s": cold_wall,
         "bytes": algorithmic_bytes(name),
         "flops": algorithmic_flops(name),
@@ -277,8 +321,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                  "avg": sum(per_launch) / len(per_launch), "max": per_launch[-1]},
     }
 
-    if with_cpu_baseline and name not in ("block", "layer", "lm_head") and not q4nx:
-        res["cpu_baseline"] = cpu_baseline(name, torch, copies[0], x, outs, launch, stream)
+    if with_cpu_baseline and name not in ("block", "layer", "lm_head", "gemv_awq") and not q4nx:
+        res["cpu_baseline"] = cpu_baseline(name, torch, copies[0][1:] if name == "gemv" else copies[0], x, outs, launch, stream)
     return res
 
 
@@ -639,7 +683,8 @@ def main():
         roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": value / HBM_PEAK_GBS, "traffic": None}
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
-    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel", "ffn": "ffn_fused_kernel", "lm_head": "lm_head_kernel"}.get(name, "stream_kernel")
+    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel", "ffn": "ffn_fused_kernel", "lm_head": "lm_head_kernel",
+                      "gemv": "gemv_ws_kernel"}.get(name, "stream_kernel")
     roof["algorithmic_per_launch"] = main_res["flops"] if name == "prefill" else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]
 
@@ -660,6 +705,7 @@ def main():
                    "weight_copies_rotated": main_res["ncopies"], "timing": "HIP graph of K launches, events on the launch stream"},
         "roofline": roof,
         "per_launch_events_us": main_res["per_launch_events_us"],
+        "eager_us_per_step": main_res["eager_us"],
         "hot_cache": {"us_per_step": main_res["hot_us"],
                       "value": (main_res["flops"] / 1e12 if name == "prefill" else main_res["bytes"] / 1e9) / (main_res["hot_us"] * 1e-6),
                       "note": "same buffers every step (Infinity Cache resident for the decode shapes)"},

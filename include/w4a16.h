@@ -151,6 +151,41 @@ int w4a16_gemv_add_bf16(const uint16_t *x,
                         void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Stream order: the device layout of one AWQ matrix for the decode kernels, written once at load
+ * time from the checkpoint tensors.  Counterpart of the reference's load-time re-pack of every
+ * Linear into the order its cores consume it (repack_for_gemv,
+ * programming_examples/llms/llama32_1b_int4/awq_repacker.py:112-135; pack_inputs,
+ * programming_examples/matrix_vector_multiplication/int4_awq/matvec_int4_packed.py:57-103).
+ * Layout: 16-column tiles, each one contiguous slab holding all K rows as 1 KiB cells of
+ * 16 columns x 128 rows (one 128-bit load per lane of a wavefront) with the group's scales and zero
+ * points beside them; mlir-air_amd/csrc/wstream.h states it byte by byte.
+ * w4a16_stream_bytes(K, N) is the size of the buffer (0 for an unsupported shape); K % 128 == 0,
+ * N % 16 == 0, group == 128.
+ */
+size_t w4a16_stream_bytes(int K, int N);
+int w4a16_repack_stream(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                        void *wstream, int K, int N, int group, void *stream);
+
+/*
+ * Decode GEMV on a stream-order matrix, batch 1: y[N] = bf16(x[K] . W), fp32 accumulation, one bf16
+ * rounding.  Stateless: a workgroup owns whole columns, so there is no workspace and no exchange
+ * between workgroups.  Same reference as w4a16_gemv_bf16: matvec_int4_bf16_packed
+ * (programming_examples/matrix_vector_multiplication/int4_awq/mv_int4_bf16.cc:403-411),
+ * matvec_int4_packed.cpu_reference (matvec_int4_packed.py:272-287).
+ * _add: y = bf16(x . W + R), R bf16 [N] (matvec_int4_packed_add.cpu_reference,
+ * matvec_int4_packed_add.py:302-319); y may alias R.
+ * _swiglu: h[H] = bf16(silu(bf16(x . Wg)) * bf16(x . Wu)), both matrices [K, H] in stream order
+ * (matvec_int4_swiglu_rms.cpu_reference, programming_examples/decode_ffn_swiglu/
+ * matvec_int4_swiglu_rms.py:501-516, without the RMSNorm prologue).
+ */
+int w4a16_gemv_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int K, int N, int group,
+                           void *stream);
+int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual,
+                               uint16_t *y, int K, int N, int group, void *stream);
+int w4a16_gemv_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream,
+                                  uint16_t *h, int K, int H, int group, void *stream);
+
+/*
  * RMSNorm prologue + decode GEMV, batch 1:
  *   rstd = 1 / sqrt(mean(x^2) + eps),  n = bf16((x * rstd) * norm_weight),  y = bf16(n . W)
  * The normalisation of matvec_int4_swiglu_rms.cpu_reference

@@ -199,3 +199,82 @@ def unpack_buffer(buf, K, N, gs=GROUP):
     qzeros = buf[lay["z_off"]:lay["z_off"] + lay["z_bytes"]].view(np.int32).reshape(K // gs, N // 8)
     scales = buf[lay["s_off"]:lay["s_off"] + lay["s_bytes"]].view(np.uint16).reshape(K // gs, N).view(bf16.BF16Array)
     return qweight, qzeros, scales
+
+
+# --- stream order: the device layout of the decode kernels ---------------------------------------
+#
+# Counterpart of the reference's load-time re-pack into the order its cores consume the weights
+# (repack_for_gemv, awq_repacker.py:112-135).  Per 16-column tile one contiguous slab of all K rows:
+# blocks of 16 groups, each [1 KiB scales / zero points][one 1 KiB cell per group].  A cell is 64
+# lanes x 4 dwords; lane l = 16 lg + ln, dword t, nibble p holds row 128 g + 32 t + 8 lg +
+# PACK_ORDER[p] of column 16 tile + ln.  Scales / zero points: lane l, dword i belongs to group
+# 16 b + 4 lg + i: bits 0..15 the bf16 scale, bits 16..31 the bf16 value -(128 + z) = 0xC300 | z.
+
+STREAM_TILE_COLS = 16
+STREAM_BLOCK_GROUPS = 16
+
+
+def stream_bytes(K, N):
+    """Size of the stream-order buffer of a [K, N] matrix."""
+    if K % GROUP or N % STREAM_TILE_COLS:
+        raise ValueError("stream order needs K % 128 == 0 and N % 16 == 0")
+    G = K // GROUP
+    return (N // STREAM_TILE_COLS) * (-(-G // STREAM_BLOCK_GROUPS) + G) * 1024
+
+
+def repack_stream(qweight, qzeros, scales):
+    """AWQ layout -> stream order, uint32 [N/16, (NB + G) * 256] (host twin of w4a16_repack_stream)."""
+    q = unpack_int4(qweight)                       # [K, N]
+    z = unpack_int4(qzeros)                        # [G, N]
+    s = bf16.bits_of(scales).astype(np.uint32)     # [G, N]
+    K, N = q.shape
+    G = K // GROUP
+    if K % GROUP or N % STREAM_TILE_COLS or z.shape != (G, N) or s.shape != (G, N):
+        raise ValueError("repack_stream: need K % 128 == 0, N % 16 == 0 and [K/128, N] scales / zeros")
+    NB = -(-G // STREAM_BLOCK_GROUPS)
+    T = N // STREAM_TILE_COLS
+    out = np.zeros((T, (NB + G) * 256), dtype=np.uint32)
+    # cells: q[k, n] with k = 128 g + 32 t + 8 lg + PACK_ORDER[p], n = 16 tile + ln
+    qv = q.reshape(G, 4, 4, 8, T, 16).astype(np.uint32)          # [g, t, lg, j, tile, ln]
+    cells = np.zeros((G, 4, 4, T, 16), dtype=np.uint32)          # [g, t, lg, tile, ln]
+    for p, j in enumerate(PACK_ORDER):
+        cells |= qv[:, :, :, j] << np.uint32(4 * p)
+    cells = cells.transpose(3, 0, 2, 4, 1)                       # [tile, g, lg, ln, t]
+    # scales / zero points: dword (lane, i) of block b <- group 16 b + 4 lg + i
+    md = s | ((np.uint32(0xC300) | z.astype(np.uint32)) << np.uint32(16))     # [G, N]
+    md_pad = np.zeros((NB * STREAM_BLOCK_GROUPS, N), dtype=np.uint32)
+    md_pad[:G] = md
+    md_pad = md_pad.reshape(NB, 4, 4, T, 16).transpose(3, 0, 1, 4, 2)         # [tile, b, lg, ln, i]
+    for b in range(NB):
+        g0 = b * STREAM_BLOCK_GROUPS
+        ng = min(STREAM_BLOCK_GROUPS, G - g0)
+        base = b * (STREAM_BLOCK_GROUPS + 1) * 256
+        out[:, base:base + 256] = md_pad[:, b].reshape(T, 256)
+        out[:, base + 256:base + 256 * (1 + ng)] = cells[:, g0:g0 + ng].reshape(T, ng * 256)
+    return out
+
+
+def unpack_stream(buf, K, N):
+    """Stream order -> (q uint8 [K, N], z uint8 [K/128, N], scale bits uint16 [K/128, N])."""
+    G = K // GROUP
+    NB = -(-G // STREAM_BLOCK_GROUPS)
+    T = N // STREAM_TILE_COLS
+    buf = np.ascontiguousarray(buf).view(np.uint32).reshape(T, (NB + G) * 256)
+    q = np.empty((K, N), dtype=np.uint8)
+    z = np.empty((G, N), dtype=np.uint8)
+    s = np.empty((G, N), dtype=np.uint16)
+    qv = q.reshape(G, 4, 4, 8, T, 16)
+    for b in range(NB):
+        g0 = b * STREAM_BLOCK_GROUPS
+        ng = min(STREAM_BLOCK_GROUPS, G - g0)
+        base = b * (STREAM_BLOCK_GROUPS + 1) * 256
+        md = buf[:, base:base + 256].reshape(T, 4, 16, 4).transpose(1, 3, 0, 2).reshape(16, N)   # [4 lg + i, n]
+        s[g0:g0 + ng] = (md[:ng] & 0xFFFF).astype(np.uint16)
+        hi = md[:ng] >> 16
+        if np.any((hi & 0xFFF0) != 0xC300):
+            raise ValueError("unpack_stream: a zero-point field is not 0xC300 | z")
+        z[g0:g0 + ng] = (hi & 0xF).astype(np.uint8)
+        cells = buf[:, base + 256:base + 256 * (1 + ng)].reshape(T, ng, 4, 16, 4)               # [tile, g, lg, ln, t]
+        for p, j in enumerate(PACK_ORDER):
+            qv[g0:g0 + ng, :, :, j] = ((cells >> np.uint32(4 * p)) & 0xF).transpose(1, 4, 2, 0, 3).astype(np.uint8)
+    return q, z, s

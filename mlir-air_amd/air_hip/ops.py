@@ -139,6 +139,64 @@ def _wptrs(w):
     return [_ptr(w[0]), _ptr(w[1]), _ptr(_bits(w[2]))]
 
 
+class StreamWeight:
+    """One AWQ matrix in stream order (the device layout of the decode kernels), made once at load time
+    by `repack_stream`: the counterpart of the reference's per-layer packed decode buffers
+    (repack_for_gemv, programming_examples/llms/llama32_1b_int4/awq_repacker.py:112-135)."""
+
+    __slots__ = ("buf", "K", "N")
+
+    def __init__(self, buf, K, N):
+        self.buf, self.K, self.N = buf, K, N
+
+
+def repack_stream(qweight, qzeros, scales, group=GROUP):
+    """AWQ tensors on the GPU -> StreamWeight (one kernel, no host round trip)."""
+    lib = _lib.load_library()
+    _need_cuda(qweight, qzeros, scales)
+    K, nb = qweight.shape
+    N = nb * 8
+    nbytes = lib.w4a16_stream_bytes(K, N)
+    if nbytes == 0:
+        raise ValueError(f"stream order needs K % 128 == 0 and N % 16 == 0, got K={K}, N={N}")
+    buf = torch.empty(int(nbytes), dtype=torch.uint8, device=qweight.device)
+    _lib.check(lib.w4a16_repack_stream(_ptr(qweight), _ptr(qzeros), _ptr(_bits(scales)), _ptr(buf), K, N, group, _stream()))
+    return StreamWeight(buf, K, N)
+
+
+def w4a16_gemv_stream(x, w, residual=None, group=GROUP, out=None):
+    """Decode GEMV on a StreamWeight: y[N] = bf16(x[K] . W), with `residual` y = bf16(x . W + R).
+    Stateless (no workspace)."""
+    lib = _lib.load_library()
+    _need_cuda(x, w.buf)
+    if x.numel() != w.K:
+        raise ValueError(f"x has K={x.numel()} but the matrix has {w.K} rows")
+    if out is None:
+        out = torch.empty((w.N,), dtype=torch.bfloat16, device=x.device)
+    if residual is not None:
+        _need_cuda(residual)
+        if residual.numel() != w.N:
+            raise ValueError(f"residual has {residual.numel()} elements, expected N={w.N}")
+        _lib.check(lib.w4a16_gemv_add_stream_bf16(_ptr(_bits(x)), _ptr(w.buf), _ptr(_bits(residual)), _ptr(out), w.K, w.N,
+                                                  group, _stream()))
+    else:
+        _lib.check(lib.w4a16_gemv_stream_bf16(_ptr(_bits(x)), _ptr(w.buf), _ptr(out), w.K, w.N, group, _stream()))
+    return out
+
+
+def w4a16_swiglu_stream(x, gate, up, group=GROUP, out=None):
+    """Decode FFN front half on two StreamWeights: h[H] = bf16(silu(bf16(x Wg)) * bf16(x Wu))."""
+    lib = _lib.load_library()
+    _need_cuda(x, gate.buf, up.buf)
+    if x.numel() != gate.K or (up.K, up.N) != (gate.K, gate.N):
+        raise ValueError("w4a16_swiglu_stream: gate and up must both be [K, H]")
+    if out is None:
+        out = torch.empty((gate.N,), dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.w4a16_gemv_swiglu_stream_bf16(_ptr(_bits(x)), _ptr(gate.buf), _ptr(up.buf), _ptr(out), gate.K, gate.N,
+                                                 group, _stream()))
+    return out
+
+
 def w4a16_gemv_add(x, qweight, qzeros, scales, residual, group=GROUP, out=None):
     """Decode GEMV with residual: y[N] = bf16(x[K] . W + R[N]) (one rounding)."""
     lib = _lib.load_library()

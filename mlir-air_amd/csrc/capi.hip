@@ -4,6 +4,7 @@
 #include "../../include/w4a16.h"
 #include "common.h"
 #include "kernels.h"
+#include "wstream.h"
 
 using namespace w4a16;
 
@@ -382,6 +383,51 @@ int w4a16_rms_gemv_swiglu_bf16(const uint16_t *x, const uint16_t *norm_weight, f
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+size_t w4a16_stream_bytes(int K, int N) {
+    if (K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return 0;
+    return ws_matrix_bytes(K, N);
+}
+
+int w4a16_repack_stream(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *wstream, int K, int N,
+                        int group, void *stream) {
+    if (!wstream) return W4A16_ERR_NULL;
+    int rc = check_quant(qweight, qzeros, scales, K, N, group, kWsTileCols);
+    if (rc) return rc;
+    if (misaligned(wstream)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_repack_ws(qweight, qzeros, scales, wstream, K, N, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+namespace {
+int gemv_stream_impl(const uint16_t *x, const void *w, const void *w_up, const uint16_t *residual, bool need_residual,
+                     uint16_t *y, int K, int N, int group, void *stream) {
+    if (!x || !w || !y || (need_residual && !residual)) return W4A16_ERR_NULL;
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    if (K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(w) || misaligned(y) || (w_up && misaligned(w_up)) || (residual && misaligned(residual)))
+        return W4A16_ERR_ALIGN;
+    GemvWsExtras ex;
+    ex.residual = residual;
+    hipError_t e = launch_gemv_ws(x, w, w_up, y, K, N, static_cast<hipStream_t>(stream), ex);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+}  // namespace
+
+int w4a16_gemv_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int K, int N, int group, void *stream) {
+    return gemv_stream_impl(x, wstream, nullptr, nullptr, false, y, K, N, group, stream);
+}
+
+int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int K, int N,
+                               int group, void *stream) {
+    return gemv_stream_impl(x, wstream, nullptr, residual, true, y, K, N, group, stream);
+}
+
+int w4a16_gemv_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream, uint16_t *h, int K,
+                                  int H, int group, void *stream) {
+    if (!up_wstream) return W4A16_ERR_NULL;
+    return gemv_stream_impl(x, gate_wstream, up_wstream, nullptr, false, h, K, H, group, stream);
+}
+
 size_t w4a16_block_workspace_bytes(int E, int H) {
     if (E <= 0 || H <= 0) return 0;
     const size_t a = stream_partial_bytes(1, H, 2), b = stream_partial_bytes(1, E, 1);
@@ -652,6 +698,12 @@ int w4a16_tune(const char *key, int value) {
         g_stream_tune.no_attn_fuse = value ? 0 : 1;
     } else if (!strcmp(key, "gemm_stream_max_m")) {
         g_stream_tune.stream_max_m = value;
+    } else if (!strcmp(key, "gemv_ws_ct")) {
+        if (value != 0 && value != 4 && value != 8 && value != 16) return W4A16_ERR_TUNE;
+        g_gemv_ws_tune.ct = value;
+    } else if (!strcmp(key, "gemv_ws_waves")) {
+        if (value > 16) return W4A16_ERR_TUNE;
+        g_gemv_ws_tune.waves = value;
     } else if (!strcmp(key, "gemv_ksplit")) {
         if (value > kMaxKSplit) return W4A16_ERR_TUNE;
         g_stream_tune.ksplit = value;

@@ -77,6 +77,9 @@ __device__ __forceinline__ float wave_reduce(float v) {
     return op(v, __shfl_xor(v, 32));
 }
 
+// silu(g) in the reference's tanh form (matvec_int4_swiglu_rms.py:512-514), fp32
+__device__ __forceinline__ float silu_tanh(float g) { return g * 0.5f * (tanhf(g * 0.5f) + 1.0f); }
+
 // "No score yet" of the attention partials: finite, so differences of two of them are 0, not NaN.
 constexpr float kAttnNegBig = -1e30f;
 

@@ -1,0 +1,242 @@
+// Whole-K decode GEMV on the stream-order layout (wstream.h), M = 1, and the re-pack kernel that
+// writes that layout from the AutoAWQ checkpoint tensors.
+//
+// HBM-bound: every packed byte is read once, as 1 KiB global_load_dwordx4 wave loads.  A workgroup
+// owns one 16-column tile for all of K and writes its 16 outputs itself: no partial sums leave the
+// workgroup, so there is no workspace, no cross-workgroup protocol and no state between calls.
+//
+// Arithmetic on the matrix cores (the fp32 VALU cannot keep up with HBM: ~2.5 lane-ops per weight
+// at 8 TB/s, a convert + FMA needs ~2.4; building an MFMA operand costs 7 ops per 8 weights).
+//
+//   task   = up to CT consecutive groups of one block of one tile: all its loads (4 of x, CT cells,
+//            1 of scales / zero points) are issued before anything is consumed, cells are
+//            consumed in arrival order
+//   wave   = tasks w, w + W, ... of the tile's NB * (16 / CT) tasks (W waves per workgroup)
+//
+// M = 1 uses one of the 16 rows of an MFMA product.  Instead of broadcasting x to all rows, row r
+// of the A operand holds the x values of group r of the block (one coalesced load per K-step: lane
+// (lg, ln) reads x[128 (16 b + ln) + 32 t + 8 lg ..+7]).  The product with the cell of group r0 is
+// then wanted in row r0 only; the other rows multiply x of one group with weights of another and
+// are never read.  Row r0 lives in register r0 % 4 of lane group r0 / 4, which is exactly where the
+// block's scales and zero points of group r0 were loaded (wstream.h), and where the ones-product
+// sum_k x[k] of group r0 lands.  So after the 16 cells of a block each lane flushes four groups:
+//        y += s * (sum (128 + q) x  -  (128 + z) * sum x)
+// with 0x4300 | q == bf16(128 + q) exactly, and the lanes of a column are added up at the end.
+#include "common.h"
+#include "kernels.h"
+#include "wstream.h"
+
+namespace w4a16 {
+
+namespace {
+
+constexpr int kMaxWaves = 16;
+
+// (dword >> 4 v) & 0x000F000F | 0x43004300: rows (2 v, 2 v + 1) of the lane's column as bf16 (128 + q)
+__device__ __forceinline__ bf16x8 cell_operand(uint32_t w, uint32_t nib_mask, uint32_t magic) {
+    u32x4 b;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) b[v] = ((w >> (4 * v)) & nib_mask) | magic;
+    return __builtin_bit_cast(bf16x8, b);
+}
+
+// CT   cells per task (4, 8 or 16)
+// NMAT 1, or 2: gate and up matrices with the SwiGLU epilogue h = bf16(silu(bf16 g) * bf16 u)
+template <int CT, int NMAT>
+__global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t *__restrict__ x, const char *__restrict__ w0,
+                                                                 const char *__restrict__ w1, uint16_t *__restrict__ y,
+                                                                 const uint16_t *__restrict__ residual, int G, int NB,
+                                                                 int round_before_add) {
+    constexpr int SUB = kWsBlockGroups / CT;
+    __shared__ float red[NMAT * kMaxWaves * 64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int lg = lane >> 4, ln = lane & 15;
+    const int tile = blockIdx.x;
+    const size_t tile_bytes = (size_t)(NB + G) * kWsCellBytes;
+
+    const uint32_t ones_w = 0x3F803F80u;
+    const u32x4 ones4 = {ones_w, ones_w, ones_w, ones_w};
+    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones4);
+    // Kept opaque so that (v & mask) | magic stays one v_and_or_b32 with register operands.
+    uint32_t nib_mask = 0x000F000Fu, magic = 0x43004300u;
+    asm volatile("" : "+s"(nib_mask));
+    asm volatile("" : "+v"(magic));
+
+    float yv[NMAT];
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) yv[m] = 0.f;
+
+    const int tasks_per_mat = NB * SUB;
+    for (int task = wave; task < NMAT * tasks_per_mat; task += nwaves) {
+        const int mat = NMAT == 1 ? 0 : task / tasks_per_mat;
+        const int tm = task - mat * tasks_per_mat;
+        const int b = tm / SUB, r0 = (tm % SUB) * CT;
+        const int ng = min(kWsBlockGroups, G - kWsBlockGroups * b);   // groups of this block
+        if (r0 >= ng) continue;                                       // wave-uniform
+        const char *blk = (mat ? w1 : w0) + (size_t)tile * tile_bytes + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes);
+
+        // x of the task's groups: A row ln <-> group 16 b + ln; rows outside the task are zero, so that
+        // their (never read) products and their sum x stay finite and contribute nothing
+        const int grow = kWsBlockGroups * b + ln;
+        const bool xvalid = ln >= r0 && ln < r0 + CT && grow < G;
+        const uint16_t *xp = x + (size_t)(xvalid ? grow : 0) * 128 + 8 * lg;
+        u32x4 X[4], cell[CT];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) X[t] = *reinterpret_cast<const u32x4 *>(xp + 32 * t);
+        // scales / zero points next: they sit right in front of the cells (requested after the cells instead: +0.5 us)
+        const u32x4 md = *(reinterpret_cast<const u32x4 *>(blk) + lane);
+#pragma unroll
+        for (int r = 0; r < CT; ++r) {
+            const int rc = r0 + r < ng ? r0 + r : ng - 1;   // a short block re-reads its last cell (x of that row is zero)
+            cell[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)(1 + rc) * kWsCellBytes) + lane);
+        }
+        // every load of the task is requested before the first wait
+        __builtin_amdgcn_sched_barrier(0);
+
+        if (!xvalid) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) X[t] = u32x4{0u, 0u, 0u, 0u};
+        }
+        floatx4 xs = {0.f, 0.f, 0.f, 0.f};   // register i of lane group lg: sum of x over group 16 b + 4 lg + i
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[t]), ones, xs, 0, 0, 0);
+
+        float V[4] = {0.f, 0.f, 0.f, 0.f};   // V[i] of lane group lg: sum (128 + q) x of group 16 b + 4 lg + i
+#pragma unroll
+        for (int r = 0; r < CT; ++r) {
+            floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[t]), cell_operand(cell[r][t], nib_mask, magic),
+                                                              acc, 0, 0, 0);
+            V[r & 3] = (lg == ((r0 + r) >> 2)) ? acc[r & 3] : V[r & 3];
+        }
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float s = __builtin_bit_cast(float, md[i] << 16);
+            const float nz = __builtin_bit_cast(float, md[i] & 0xFFFF0000u);   // -(128 + z)
+            sum = fmaf(s, fmaf(nz, xs[i], V[i]), sum);
+        }
+        if (NMAT == 2 && mat) yv[NMAT - 1] += sum;
+        else yv[0] += sum;
+    }
+
+    // the 4 lane groups x W waves of every column, added by the first 16 threads
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) red[(m * kMaxWaves + wave) * 64 + lane] = yv[m];
+    __syncthreads();
+    if (threadIdx.x < kWsTileCols) {
+        float tot[NMAT];
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) {
+            tot[m] = 0.f;
+            for (int w = 0; w < nwaves; ++w) {
+                const float *src = red + (m * kMaxWaves + w) * 64 + threadIdx.x;
+                tot[m] += (src[0] + src[16]) + (src[32] + src[48]);
+            }
+        }
+        const int col = tile * kWsTileCols + threadIdx.x;
+        float out;
+        if (NMAT == 2) {
+            const float gate = bf16_bits_to_float(float_to_bf16_bits(tot[0]));
+            const float up = bf16_bits_to_float(float_to_bf16_bits(tot[NMAT - 1]));
+            out = silu_tanh(gate) * up;
+        } else {
+            out = tot[0];
+        }
+        if (residual) {
+            if (round_before_add) out = bf16_bits_to_float(float_to_bf16_bits(out));
+            out += bf16_bits_to_float(residual[col]);
+        }
+        y[col] = float_to_bf16_bits(out);
+    }
+}
+
+// One thread per dword of the stream-order buffer.
+__global__ void __launch_bounds__(256) repack_ws_kernel(const uint32_t *__restrict__ qweight, const uint32_t *__restrict__ qzeros,
+                                                        const uint16_t *__restrict__ scales, uint32_t *__restrict__ out, int G,
+                                                        int NB, int N) {
+    const size_t tile_dwords = (size_t)(NB + G) * (kWsCellBytes / 4);
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= tile_dwords * (N / kWsTileCols)) return;
+    const int tile = (int)(idx / tile_dwords);
+    const int off = (int)(idx - (size_t)tile * tile_dwords);
+    constexpr int BLOCK_DWORDS = (kWsBlockGroups + 1) * (int)(kWsCellBytes / 4);
+    const int b = min(off / BLOCK_DWORDS, NB - 1);
+    const int within = off - b * BLOCK_DWORDS;
+    const int l = (within & 255) >> 2, sub = within & 3;   // lane and dword of a 1 KiB piece
+    const int n = tile * kWsTileCols + (l & 15);
+    const int lg = l >> 4;
+    const int nb = N >> 3;
+    const int shift = 4 * unpack_pos(n & 7);               // where column n sits in its checkpoint word
+    uint32_t v = 0;
+    if (within < 256) {                                    // scales and zero points
+        const int g = kWsBlockGroups * b + 4 * lg + sub;
+        if (g < G) {
+            const uint32_t z = (qzeros[(size_t)g * nb + (n >> 3)] >> shift) & 0xFu;
+            v = (uint32_t)scales[(size_t)g * N + n] | ((0xC300u | z) << 16);
+        }
+    } else {
+        const int g = kWsBlockGroups * b + (within >> 8) - 1;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const int k = 128 * g + 32 * sub + 8 * lg + pack_order(p);
+            v |= ((qweight[(size_t)k * nb + (n >> 3)] >> shift) & 0xFu) << (4 * p);
+        }
+    }
+    out[idx] = v;
+}
+
+template <int CT>
+hipError_t launch_ct(int nmat, int waves, const uint16_t *x, const void *w0, const void *w1, uint16_t *y, int K, int N,
+                     const GemvWsExtras &ex, hipStream_t stream) {
+    const int G = K / kGroup, NB = ws_blocks(K);
+    const dim3 grid(N / kWsTileCols), block(waves * 64);
+    if (nmat == 2)
+        hipLaunchKernelGGL((gemv_ws_kernel<CT, 2>), grid, block, 0, stream, x, static_cast<const char *>(w0),
+                           static_cast<const char *>(w1), y, ex.residual, G, NB, ex.round_before_add);
+    else
+        hipLaunchKernelGGL((gemv_ws_kernel<CT, 1>), grid, block, 0, stream, x, static_cast<const char *>(w0),
+                           static_cast<const char *>(w0), y, ex.residual, G, NB, ex.round_before_add);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+GemvWsTune g_gemv_ws_tune;
+
+// Launch shape.  Tasks of 8 cells (16 tasks of a tile in flight at most); one wave per task up to 16 waves.
+GemvWsPlan plan_gemv_ws(int K, int nmat) {
+    GemvWsPlan pl;
+    pl.ct = g_gemv_ws_tune.ct ? g_gemv_ws_tune.ct : 8;
+    const int tasks = nmat * ws_blocks(K) * (kWsBlockGroups / pl.ct);
+    pl.waves = tasks < kMaxWaves ? tasks : kMaxWaves;
+    if (g_gemv_ws_tune.waves && g_gemv_ws_tune.waves < pl.waves) pl.waves = g_gemv_ws_tune.waves;
+    return pl;
+}
+
+hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, uint16_t *y, int K, int N, hipStream_t stream,
+                          const GemvWsExtras &extras) {
+    const int nmat = w_up ? 2 : 1;
+    const GemvWsPlan pl = plan_gemv_ws(K, nmat);
+    switch (pl.ct) {
+        case 4: return launch_ct<4>(nmat, pl.waves, x, w, w_up, y, K, N, extras, stream);
+        case 16: return launch_ct<16>(nmat, pl.waves, x, w, w_up, y, K, N, extras, stream);
+        default: return launch_ct<8>(nmat, pl.waves, x, w, w_up, y, K, N, extras, stream);
+    }
+}
+
+hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *out, int K, int N,
+                            hipStream_t stream) {
+    const size_t dwords = ws_matrix_bytes(K, N) / 4;
+    const size_t blocks = (dwords + 255) / 256;
+    if (blocks > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(repack_ws_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<const uint32_t *>(qweight),
+                       reinterpret_cast<const uint32_t *>(qzeros), scales, static_cast<uint32_t *>(out), K / kGroup, ws_blocks(K), N);
+    return hipGetLastError();
+}
+
+}  // namespace w4a16

@@ -87,6 +87,28 @@ size_t gemm_prefill_splitk_bytes(int M, int K, int N, int cus);
 
 hipError_t launch_fill_workspace(void *ptr, size_t bytes, hipStream_t stream);
 
+// Whole-K decode GEMV on the stream-order layout (gemv_ws.hip, layout in wstream.h): stateless, no workspace.
+struct GemvWsExtras {
+    const uint16_t *residual = nullptr;   // [N] bf16 added to the result before the final rounding
+    int round_before_add = 0;             // 1: y = bf16(bf16(x.W) + R) instead of bf16(x.W + R)
+};
+struct GemvWsTune {
+    int ct = 0;      // cells (groups) per task: 4, 8 or 16 (0 = default)
+    int waves = 0;   // cap on the waves per workgroup (0 = one per task, at most 16)
+};
+extern GemvWsTune g_gemv_ws_tune;
+struct GemvWsPlan {
+    int ct, waves;
+};
+GemvWsPlan plan_gemv_ws(int K, int nmat);
+// y[N] = bf16(x[K] . W) with W in stream order; with `w_up` (second matrix, same shape) the SwiGLU epilogue
+// y = bf16(silu(bf16(x.W)) * bf16(x.W_up)).
+hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, uint16_t *y, int K, int N, hipStream_t stream,
+                          const GemvWsExtras &extras = GemvWsExtras());
+// AutoAWQ checkpoint tensors -> stream order (ws_matrix_bytes(K, N) bytes at `out`).
+hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *out, int K, int N,
+                            hipStream_t stream);
+
 // Prefill O projection + FFN block (prefill_block.hip): five launches, intermediates in the workspace
 // (plain scratch, no initialisation).
 struct PrefillLinear {

@@ -47,6 +47,4 @@ __device__ __forceinline__ bool slot_full(u32x4 v) {
     return v[0] != kEmpty && v[1] != kEmpty && v[2] != kEmpty && v[3] != kEmpty;
 }
 
-__device__ __forceinline__ float silu_tanh(float g) { return g * 0.5f * (tanhf(g * 0.5f) + 1.0f); }
-
 }  // namespace w4a16

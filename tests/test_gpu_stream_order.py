@@ -1,0 +1,164 @@
+"""GPU parity of the stream-order path (through the C ABI): the device re-pack against the host packer bit for
+bit, and the whole-K decode GEMV (plain, + residual, SwiGLU pair) against the float64 oracle.
+
+Tolerance: one bf16 rounding of an fp32-accumulated sum -> within 1 bf16 ulp of the float64 value plus 2e-3
+absolute, and inside the reference's own gate (rtol 0.1, atol 0.05, r >= 0.999)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_bf16_close, dense_f64, make_awq, make_x
+from oracle import awq as oawq, reference as oref
+from oracle.bf16 import bf16_bits_to_f32, f32_to_bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(a).cuda()
+
+
+def bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from air_hip import ops
+    return ops
+
+
+def _stream_weight(ops, qw, qz, s):
+    return ops.repack_stream(dev(qw), dev(qz), dev(s))
+
+
+@pytest.mark.parametrize("K,N", [(128, 16), (256, 48), (2048, 64), (128 * 19, 32), (4096, 4096)])
+def test_device_repack_equals_host_packer(ops, K, N):
+    print(f"repack K={K} N={N}", flush=True)
+    from air_hip import awq, bf16
+    qw, qz, s = make_awq(K, N, seed=K + N)
+    w = _stream_weight(ops, qw, qz, s)
+    torch.cuda.synchronize()
+    want = awq.repack_stream(qw, qz, bf16.from_bits(s))
+    got = w.buf.cpu().numpy().view(np.uint32).reshape(want.shape)
+    assert np.array_equal(got, want)
+
+
+def _gemv_case(ops, K, N, seed, residual=False):
+    print(f"gemv stream K={K} N={N} seed={seed} residual={residual}", flush=True)
+    qw, qz, s = make_awq(K, N, seed=seed)
+    x = make_x((K,), seed=seed + 1)
+    r = make_x((N,), seed=seed + 2) if residual else None
+    w = _stream_weight(ops, qw, qz, s)
+    y = ops.w4a16_gemv_stream(dev(x), w, residual=dev(r) if residual else None)
+    torch.cuda.synchronize()
+    got = bits(y)
+    want = bf16_bits_to_f32(x).astype(np.float64) @ dense_f64(qw, qz, s)
+    if residual:
+        want = want + bf16_bits_to_f32(r).astype(np.float64)
+    assert_bf16_close(got, want, ulps=1.0, atol=2e-3, what=f"gemv stream K={K} N={N}")
+    assert oref.check_outputs(bf16_bits_to_f32(got), bf16_bits_to_f32(f32_to_bf16_bits(want.astype(np.float32))),
+                              rtol=0.1, atol=0.05, min_correlation=0.999 if want.size > 8 else None)
+    return got
+
+
+# K = 128 .. 14336: one short block, whole blocks, a short last block (19 and 86 groups), 7 blocks
+@pytest.mark.parametrize("K,N", [(128, 16), (256, 544), (1024, 512), (128 * 19, 48), (2048, 8192), (4096, 4096),
+                                 (11008, 512), (14336, 4096)])
+def test_gemv_stream_shapes(ops, K, N):
+    _gemv_case(ops, K, N, seed=K + N)
+
+
+def test_gemv_stream_config1(ops):
+    _gemv_case(ops, 4096, 11008, seed=1)
+
+
+@pytest.mark.parametrize("K,N", [(512, 64), (4096, 4096), (14336, 4096)])
+def test_gemv_stream_residual(ops, K, N):
+    _gemv_case(ops, K, N, seed=3 * K + N, residual=True)
+
+
+def test_gemv_stream_zero_weights_return_the_residual_bit_for_bit(ops):
+    K, N = 512, 256
+    qw, qz, s = make_awq(K, N, seed=9)
+    w = _stream_weight(ops, qw, qz, np.zeros_like(s))
+    x, r = make_x((K,), seed=10), make_x((N,), seed=11)
+    y = ops.w4a16_gemv_stream(dev(x), w, residual=dev(r))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), r)
+
+
+def test_gemv_stream_one_hot_x_is_a_dequantised_row(ops):
+    """x = e_k selects row k: (q - z) * s has at most 13 significant bits, so the fp32 sum is exact and the single
+    rounding must reproduce the dense dequant bit for bit - every row position of a cell, both blocks."""
+    K, N = 4096, 64
+    qw, qz, s = make_awq(K, N, seed=3)
+    dense = oawq.dequant_to_bf16(qw, qz, s, 128)
+    w = _stream_weight(ops, qw, qz, s)
+    for k0 in (0, 1, 2, 7, 8, 31, 32, 127, 128, 1000, 2047, 2048, 4095):
+        x = np.zeros(K, np.uint16)
+        x[k0] = 0x3F80
+        y = ops.w4a16_gemv_stream(dev(x), w)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(y), dense[k0]), k0
+
+
+def test_gemv_stream_config1_one_hot_rows(ops):
+    K, N = 4096, 11008
+    qw, qz, s = make_awq(K, N, seed=1)
+    dense = oawq.dequant_to_bf16(qw, qz, s, 128)
+    w = _stream_weight(ops, qw, qz, s)
+    for k0 in (5, 1234, 4095):
+        x = np.zeros(K, np.uint16)
+        x[k0] = 0x3F80
+        y = ops.w4a16_gemv_stream(dev(x), w)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(y), dense[k0]), k0
+
+
+def test_gemv_stream_power_of_two_scaling_is_exact(ops):
+    K, N = 2048, 512
+    qw, qz, s = make_awq(K, N, seed=21)
+    x = make_x((K,), seed=22)
+    w = _stream_weight(ops, qw, qz, s)
+    y1 = bits(ops.w4a16_gemv_stream(dev(x), w))
+    x8 = f32_to_bf16_bits(bf16_bits_to_f32(x) * 8.0)
+    y8 = bits(ops.w4a16_gemv_stream(dev(x8), w))
+    assert np.array_equal(bf16_bits_to_f32(y1) * 8.0, bf16_bits_to_f32(y8))
+
+
+@pytest.mark.parametrize("ct,waves", [(4, 0), (16, 0), (8, 1), (8, 3)])
+def test_gemv_stream_launch_shapes_agree(ops, ct, waves):
+    """Other task sizes and fewer waves than tasks (a wave then walks several tasks) change the summation order only."""
+    base = _gemv_case(ops, 128 * 23, 272, seed=50)
+    ops.tune("gemv_ws_ct", ct)
+    ops.tune("gemv_ws_waves", waves)
+    try:
+        got = _gemv_case(ops, 128 * 23, 272, seed=50)
+    finally:
+        ops.tune("gemv_ws_ct", 0)
+        ops.tune("gemv_ws_waves", 0)
+    d = np.abs(bf16_bits_to_f32(got).astype(np.float64) - bf16_bits_to_f32(base).astype(np.float64))
+    assert np.all(d <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(bf16_bits_to_f32(base)), 1e-30))) - 7) + 2e-3)
+
+
+@pytest.mark.parametrize("K,H", [(256, 64), (2048, 8192), (4096, 14336)])
+def test_swiglu_stream(ops, K, H):
+    print(f"swiglu stream K={K} H={H}", flush=True)
+    g, u = make_awq(K, H, seed=K + 1), make_awq(K, H, seed=K + 2)
+    x = make_x((K,), seed=K + 3)
+    h = ops.w4a16_swiglu_stream(dev(x), _stream_weight(ops, *g), _stream_weight(ops, *u))
+    torch.cuda.synchronize()
+    xf = bf16_bits_to_f32(x).astype(np.float64)
+    gate, up = xf @ dense_f64(*g), xf @ dense_f64(*u)
+    gb = bf16_bits_to_f32(f32_to_bf16_bits(gate.astype(np.float32)))
+    ub = bf16_bits_to_f32(f32_to_bf16_bits(up.astype(np.float32)))
+    want = oref.silu_tanh_f32(gb).astype(np.float64) * ub
+    # gate / up each carry one bf16 rounding that may flip by one ulp against the float64 sum: 1 ulp on each
+    # moves h by up to ~3 ulp (silu' <= 1.1)
+    assert_bf16_close(bits(h), want, ulps=4.0, atol=2e-3, what=f"swiglu stream K={K} H={H}")
+    assert oref.check_outputs(bf16_bits_to_f32(bits(h)), bf16_bits_to_f32(f32_to_bf16_bits(want.astype(np.float32))),
+                              rtol=0.15, atol=0.5, min_correlation=0.99)
