@@ -41,6 +41,7 @@ extern "C" {
 #define W4A16_ERR_HIP (-6)         /* a HIP call failed; see w4a16_last_hip_error() */
 #define W4A16_ERR_TUNE (-7)        /* unknown tuning key or value out of range */
 #define W4A16_ERR_TIMEOUT (-8)     /* w4a16_workspace_check: a split-K reducer timed out */
+#define W4A16_ERR_TOO_LARGE (-9)   /* w4a16_gemv_noalloc_bf16: shape beyond its fixed scratch */
 
 #define W4A16_ABI_VERSION 1
 
@@ -95,6 +96,19 @@ int w4a16_workspace_check(const void *workspace, void *stream);
 int w4a16_gemv_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
                     const uint16_t *scales, uint16_t *y, int K, int N, int group,
                     void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * w4a16_gemv_bf16 without a workspace argument and without any allocation: no counterpart in the
+ * reference; it is for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  The split-K partial slots live in a 4.06 MiB
+ * device array inside the library (one copy per GPU, held until the process ends), so N <= 32768
+ * (W4A16_ERR_TOO_LARGE beyond); other constraints, kernels and results are those of w4a16_gemv_bf16,
+ * bit for bit.  The first call on a GPU prepares the array with a fill kernel on `stream`.  Every
+ * call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * threads) race, exactly as two calls sharing one workspace would.
+ */
+int w4a16_gemv_noalloc_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
+                            const uint16_t *scales, uint16_t *y, int K, int N, int group, void *stream);
 
 /*
  * GEMM, any M >= 1: y[M, N] = bf16(x[M, K] . W).  M <= 16 streams the weights once

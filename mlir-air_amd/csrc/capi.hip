@@ -1,6 +1,8 @@
 // C ABI of libw4a16_hip.so: argument validation (before any HIP call) and dispatch.
 #include <string.h>
 
+#include <mutex>
+
 #include "../../include/w4a16.h"
 #include "common.h"
 #include "kernels.h"
@@ -197,6 +199,7 @@ const char *w4a16_strerror(int code) {
         case W4A16_ERR_HIP: return "HIP call failed";
         case W4A16_ERR_TUNE: return "unknown tuning key or value out of range";
         case W4A16_ERR_TIMEOUT: return "a split-K reducer gave up waiting for a partial result; the output is invalid";
+        case W4A16_ERR_TOO_LARGE: return "shape beyond the fixed scratch of the entry point that allocates nothing (N <= 32768)";
         default: return "unknown error code";
     }
 }
@@ -273,6 +276,61 @@ int w4a16_gemm_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qz
 int w4a16_gemv_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
                     uint16_t *y, int K, int N, int group, void *workspace, size_t workspace_bytes, void *stream) {
     return w4a16_gemm_bf16(x, qweight, qzeros, scales, y, 1, K, N, group, workspace, workspace_bytes, stream);
+}
+
+// ---- entry point that allocates nothing -----------------------------------------------------------
+// The split-K workspace of w4a16_gemv_bf16 as a file-scope device array: every GPU the library runs on holds
+// its own copy until the process ends.  In host code the array's name is a stand-in, not a device address:
+// the address on the current device comes from hipGetSymbolAddress, once per device, and only that pointer
+// is handed to kernels.
+}  // extern "C"
+
+namespace {
+constexpr int kNoAllocMaxN = 32768;
+constexpr size_t kNoAllocScratchBytes = kHeaderBytes + (size_t)kMaxKSplit * (kNoAllocMaxN + 512) * sizeof(float);   // 4.06 MiB
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+void *g_scratch_ptr[64] = {nullptr};   // per device: address of `scratch` there, set once the array is prepared
+std::mutex g_scratch_mutex;
+
+// Address of this device's copy of `scratch`, prepared (header zero, every slot empty) on first use.
+int noalloc_scratch(hipStream_t st, void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    if (dev < 0 || dev >= 64) return W4A16_ERR_SHAPE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e);
+        if (!ptr) return W4A16_ERR_NULL;
+        e = launch_fill_workspace(ptr, kNoAllocScratchBytes, st);   // a fill kernel, not a memset: safe under graph capture
+        if (e != hipSuccess) return hip_fail(e);
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return W4A16_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int w4a16_gemv_noalloc_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales,
+                            uint16_t *y, int K, int N, int group, void *stream) {
+    if (!x || !y) return W4A16_ERR_NULL;
+    int rc = check_quant(qweight, qzeros, scales, K, N, group, 32);
+    if (rc) return rc;
+    if (N > kNoAllocMaxN) return W4A16_ERR_TOO_LARGE;
+    if (misaligned(x) || misaligned(y)) return W4A16_ERR_ALIGN;
+    static_assert(kNoAllocScratchBytes >= kHeaderBytes + (size_t)kMaxKSplit * (kNoAllocMaxN + 512) * sizeof(float), "scratch too small");
+    if (w4a16_gemm_workspace_bytes(1, K, N) > kNoAllocScratchBytes) return W4A16_ERR_TOO_LARGE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    void *ws = nullptr;
+    rc = noalloc_scratch(st, &ws);
+    if (rc) return rc;
+    hipError_t e = launch_stream(x, qweight, qzeros, scales, nullptr, nullptr, nullptr, y, 1, K, N, ws, st);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
 int w4a16_gemv_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
