@@ -8,6 +8,12 @@
 // Arithmetic on the matrix cores (the fp32 VALU cannot keep up with HBM: ~2.5 lane-ops per weight
 // at 8 TB/s, a convert + FMA needs ~2.4; building an MFMA operand costs 7 ops per 8 weights).
 //
+// Launch-shape notes (K = 4096, N = 11008, cold): tasks of 8 cells with one wave each (4 waves per tile) 5.9 us,
+// 16 cells 6.3 us, 4 cells 5.9 us, fewer waves than tasks 6.3-6.8 us.  Tried and not kept: the four K-steps of a
+// cell as four independent MFMAs on an A operand of 4 groups x 4 K-steps (one coalesced x load per four cells instead
+// of four strided ones): the adds of the four results wait out the MFMA latency, 6.1 us; cells in interleaved pairs:
+// 6.0 us; x fetched with coalesced loads and brought into operand order through wave-local LDS rows: 5.9 us, no gain.
+//
 //   task   = up to CT consecutive groups of one block of one tile: all its loads (4 of x, CT cells,
 //            1 of scales / zero points) are issued before anything is consumed, cells are
 //            consumed in arrival order
@@ -46,12 +52,11 @@ template <int CT, int NMAT>
 __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t *__restrict__ x, const char *__restrict__ w0,
                                                                  const char *__restrict__ w1, uint16_t *__restrict__ y,
                                                                  const uint16_t *__restrict__ residual, int G, int NB,
-                                                                 int round_before_add) {
+                                                                 int round_before_add, int nwaves) {
     constexpr int SUB = kWsBlockGroups / CT;
     __shared__ float red[NMAT * kMaxWaves * 64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nwaves = blockDim.x >> 6;
     const int lg = lane >> 4, ln = lane & 15;
     const int tile = blockIdx.x;
     const size_t tile_bytes = (size_t)(NB + G) * kWsCellBytes;
@@ -197,10 +202,10 @@ hipError_t launch_ct(int nmat, int waves, const uint16_t *x, const void *w0, con
     const dim3 grid(N / kWsTileCols), block(waves * 64);
     if (nmat == 2)
         hipLaunchKernelGGL((gemv_ws_kernel<CT, 2>), grid, block, 0, stream, x, static_cast<const char *>(w0),
-                           static_cast<const char *>(w1), y, ex.residual, G, NB, ex.round_before_add);
+                           static_cast<const char *>(w1), y, ex.residual, G, NB, ex.round_before_add, waves);
     else
         hipLaunchKernelGGL((gemv_ws_kernel<CT, 1>), grid, block, 0, stream, x, static_cast<const char *>(w0),
-                           static_cast<const char *>(w0), y, ex.residual, G, NB, ex.round_before_add);
+                           static_cast<const char *>(w0), y, ex.residual, G, NB, ex.round_before_add, waves);
     return hipGetLastError();
 }
 
