@@ -64,6 +64,19 @@ int awq_dequant_bf16(const int32_t *qweight, const int32_t *qzeros, const uint16
                      uint16_t *out_bf16, int K, int N, int group, void *stream);
 
 /*
+ * 1-D dequant on the reference example's own packed buffer: out[i] = bf16_rne((q[i] - z[i / group]) * s[i / group]),
+ * i < n.  `packed` is uint8 [herd_n, tile_bytes] as pack_inputs builds it
+ * (programming_examples/dequant_awq/dequant_awq.py:259-278): per tile of n / herd_n elements
+ * [Q: two elements per byte, the even one in the low nibble][S: bf16 per group][Z: u8 per group], padded to a
+ * multiple of 4 bytes (packed_tile_bytes, dequant_awq.py:59-69); awq_dequant_1d_tile_bytes returns that size (0 for
+ * an unsupported shape).  Same entry as the device kernel dequant_int4_bf16(uint8_t *packed, bfloat16 *out)
+ * (programming_examples/dequant_awq/dequant.cc:77-85), which sees one tile; here one launch covers all tiles.
+ * Any group size that is a multiple of 8 with (n / herd_n) % group == 0.
+ */
+size_t awq_dequant_1d_tile_bytes(int n, int group, int herd_n);
+int awq_dequant_1d_bf16(const uint8_t *packed, uint16_t *out_bf16, int n, int group, int herd_n, void *stream);
+
+/*
  * Workspace for the split-K GEMV / small-M GEMM and the FFN.  The caller allocates
  * `*_workspace_bytes` bytes of device memory once, prepares it once with
  * w4a16_workspace_init, and may then reuse it for any number of calls that do not

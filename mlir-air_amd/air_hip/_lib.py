@@ -16,6 +16,8 @@ SYMBOLS = {
     "w4a16_strerror": (ctypes.c_char_p, [_ci]),
     "w4a16_last_hip_error": (ctypes.c_char_p, []),
     "awq_dequant_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "awq_dequant_1d_tile_bytes": (_sz, [_ci, _ci, _ci]),
+    "awq_dequant_1d_bf16": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_gemm_workspace_bytes": (_sz, [_ci, _ci, _ci]),
     "w4a16_ffn_workspace_bytes": (_sz, [_ci, _ci]),
     "w4a16_workspace_init": (_ci, [_vp, _sz, _vp]),

@@ -201,6 +201,45 @@ def unpack_buffer(buf, K, N, gs=GROUP):
     return qweight, qzeros, scales
 
 
+# --- the 1-D dequant example's tiled buffer ------------------------------------------------------
+
+def packed_tile_bytes_1d(n_tile, group_size):
+    """(q_bytes, s_bytes, z_bytes, tile_bytes) of one tile of the 1-D dequant example: Q two elements per byte,
+    S bf16 per group, Z u8 per group, the tile padded to a multiple of 4 bytes
+    (packed_tile_bytes, programming_examples/dequant_awq/dequant_awq.py:59-69)."""
+    ng = n_tile // group_size
+    q_bytes, s_bytes, z_bytes = n_tile // 2, 2 * ng, ng
+    return q_bytes, s_bytes, z_bytes, -(-(q_bytes + s_bytes + z_bytes) // 4) * 4
+
+
+def pack_inputs_1d(int4_vals, scales, zeros, n, group_size, herd_n):
+    """uint8 [herd_n, tile_bytes]: tile ty holds elements [ty * n / herd_n, (ty + 1) * n / herd_n) as [Q | S | Z | pad],
+    element 2 j of a tile in the low nibble of its byte j (pack_inputs, dequant_awq.py:259-278)."""
+    if n % herd_n or (n // herd_n) % group_size or group_size % 2:
+        raise ValueError("N / herd_n must be divisible by group_size")
+    n_tile = n // herd_n
+    q_bytes, s_bytes, z_bytes, tile_bytes = packed_tile_bytes_1d(n_tile, group_size)
+    q = np.asarray(int4_vals, dtype=np.uint8).reshape(herd_n, n_tile)
+    out = np.zeros((herd_n, tile_bytes), dtype=np.uint8)
+    out[:, :q_bytes] = (q[:, 0::2] & 0xF) | ((q[:, 1::2] & 0xF) << 4)
+    out[:, q_bytes:q_bytes + s_bytes] = np.ascontiguousarray(bf16.bits_of(scales)).reshape(herd_n, -1).view(np.uint8)
+    out[:, q_bytes + s_bytes:q_bytes + s_bytes + z_bytes] = np.asarray(zeros, dtype=np.uint8).reshape(herd_n, -1)
+    return out
+
+
+def unpack_inputs_1d(packed, n, group_size, herd_n):
+    """Inverse of pack_inputs_1d -> (int4_vals u8 [n], scales bf16 [n / gs], zeros u8 [n / gs])."""
+    n_tile = n // herd_n
+    q_bytes, s_bytes, z_bytes, tile_bytes = packed_tile_bytes_1d(n_tile, group_size)
+    packed = np.asarray(packed, dtype=np.uint8).reshape(herd_n, tile_bytes)
+    q = np.empty((herd_n, n_tile), dtype=np.uint8)
+    q[:, 0::2] = packed[:, :q_bytes] & 0xF
+    q[:, 1::2] = packed[:, :q_bytes] >> 4
+    s = np.ascontiguousarray(packed[:, q_bytes:q_bytes + s_bytes]).view(np.uint16).reshape(-1)
+    z = np.ascontiguousarray(packed[:, q_bytes + s_bytes:q_bytes + s_bytes + z_bytes]).reshape(-1)
+    return q.reshape(-1), bf16.from_bits(s), z
+
+
 # --- stream order: the device layout of the decode kernels ---------------------------------------
 #
 # Counterpart of the reference's load-time re-pack into the order its cores consume the weights

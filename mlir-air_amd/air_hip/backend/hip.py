@@ -19,7 +19,7 @@ import numpy as np
 from .. import awq, bf16
 from .abc import AirBackend, AirBackendError
 
-OPS = ("dequant_awq", "matvec_int4", "matvec_int4_add", "matmul_int4", "matvec_int4_swiglu",
+OPS = ("dequant_awq", "dequant_awq_1d", "matvec_int4", "matvec_int4_add", "matmul_int4", "matvec_int4_swiglu",
        "matvec_int4_swiglu_rms", "ffn_swiglu_int4", "o_gemv_ffn_int4")
 # ops whose N is a hidden size that is also the K of a following projection
 _HIDDEN_OPS = ("ffn_swiglu_int4", "o_gemv_ffn_int4")
@@ -59,6 +59,10 @@ class HIPBackend(AirBackend):
             raise AirBackendError(f"HIPBackend.compile expects a HipModule, got {type(module).__name__}")
         if module.op not in OPS:
             raise AirBackendError(f"unknown op '{module.op}' (known: {', '.join(OPS)})")
+        if module.op == "dequant_awq_1d":   # K = n elements, N = herd_n tiles, any even group size that divides a tile
+            if module.K <= 0 or module.N <= 0 or module.gs <= 0 or module.gs % 8 or module.K % module.N or (module.K // module.N) % module.gs:
+                raise AirBackendError(f"dequant_awq_1d: n = {module.K} must split into {module.N} tiles of whole groups of {module.gs} (a multiple of 8)")
+            return module
         if module.gs != awq.GROUP:
             raise AirBackendError(f"group size {module.gs} is not supported (only {awq.GROUP})")
         if module.K <= 0 or module.K % awq.GROUP:
@@ -104,6 +108,8 @@ class HIPBackend(AirBackend):
         def run(dev_in):
             if mod.op == "dequant_awq":
                 return [ops.awq_dequant(*dev_in[0])]
+            if mod.op == "dequant_awq_1d":
+                return [ops.awq_dequant_1d(dev_in[0], mod.K, mod.gs, mod.N)]
             if mod.op == "matvec_int4":
                 return [ops.w4a16_gemv(dev_in[1], *dev_in[0])]
             if mod.op == "matvec_int4_add":
@@ -156,6 +162,13 @@ class HIPBackend(AirBackend):
         if mod.op == "dequant_awq":
             need(1)
             return [weights(inputs[0], K, N)]
+        if mod.op == "dequant_awq_1d":
+            need(1)
+            tile_bytes = awq.packed_tile_bytes_1d(K // N, mod.gs)[3]
+            buf = np.ascontiguousarray(inputs[0], dtype=np.uint8)
+            if buf.size != N * tile_bytes:
+                raise AirBackendError(f"dequant_awq_1d: packed buffer has {buf.size} bytes, expected {N} tiles of {tile_bytes}")
+            return [to_dev(buf.reshape(-1))]
         if mod.op == "matvec_int4":
             need(2)
             return [weights(inputs[0], K, N), to_dev(bf16.bits_of(inputs[1]).reshape(K))]

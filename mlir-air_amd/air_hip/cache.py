@@ -32,6 +32,8 @@ come back in the dtype of the argument they replace, flat, like the reference's 
 
 import dataclasses
 import json
+import collections
+import contextlib
 import time
 from pathlib import Path
 
@@ -120,93 +122,96 @@ def build_attn(lk=2048, lkp=64, lq=2048, lqp=256, dk=64, dv=64, num_q_tiles=4, n
 
 
 class Profiler:
-    """Per-kernel and per-layer wall times with the reference's recording interface
-    (shared/infra/cache.py:70-306).  Disabled by default; every method is then a no-op."""
+    """Timing log of the decode loop behind the method names the reference's drivers call
+    (shared/infra/cache.py:70-306): record_compile / record_kernel / record_cpu / record_breakdown, start_layer /
+    end_layer, time_cpu, report.  One table of samples keyed by (kind, name); a disabled profiler keeps nothing."""
+
+    _BREAKDOWN_FIELDS = ("write_ms", "kernel_ms", "read_ms", "n_written", "bytes_written", "n_readback")
 
     def __init__(self, enabled=False):
-        self.enabled = enabled
-        self.compile_times = {}
-        self.kernel_times = {}
-        self.cpu_times = {}
-        self.layer_times = []
-        self.kernel_breakdowns = {}
+        self.enabled = bool(enabled)
+        self._samples = collections.defaultdict(list)   # (kind, name) -> values in recording order
+        self.layer_times = []                            # (layer index, seconds)
+
+    def _log(self, kind, name, value):
+        if self.enabled:
+            self._samples[(kind, name)].append(value)
+
+    def _table(self, kind):
+        return {name: vals for (k, name), vals in self._samples.items() if k == kind}
+
+    compile_times = property(lambda self: {n: v[-1] for n, v in self._table("compile").items()})
+    kernel_times = property(lambda self: self._table("kernel"))
+    cpu_times = property(lambda self: self._table("cpu"))
+    kernel_breakdowns = property(lambda self: self._table("breakdown"))
 
     def record_compile(self, name, duration):
-        if self.enabled:
-            self.compile_times[name] = duration
+        self._log("compile", name, duration)
 
     def record_kernel(self, name, duration):
-        if self.enabled:
-            self.kernel_times.setdefault(name, []).append(duration)
+        self._log("kernel", name, duration)
 
     def record_cpu(self, name, duration):
-        if self.enabled:
-            self.cpu_times.setdefault(name, []).append(duration)
+        self._log("cpu", name, duration)
 
-    def record_breakdown(self, name, write_ms, kernel_ms, read_ms, n_written, bytes_written, n_readback):
-        if self.enabled:
-            self.kernel_breakdowns.setdefault(name, []).append(
-                dict(write_ms=write_ms, kernel_ms=kernel_ms, read_ms=read_ms, n_written=n_written,
-                     bytes_written=bytes_written, n_readback=n_readback))
+    def record_breakdown(self, name, *fields):
+        self._log("breakdown", name, dict(zip(self._BREAKDOWN_FIELDS, fields)))
 
     def start_layer(self):
         return time.perf_counter() if self.enabled else None
 
     def end_layer(self, layer_idx, t0):
-        if self.enabled and t0 is not None:
+        if t0 is not None and self.enabled:
             self.layer_times.append((layer_idx, time.perf_counter() - t0))
 
+    @contextlib.contextmanager
     def time_cpu(self, name):
-        """`with profiler.time_cpu("decode_attention_cpu"): ...` records the block as a host operation."""
-        prof = self
-
-        class _Timer:
-            def __enter__(self):
-                self.t0 = time.perf_counter() if prof.enabled else None
-                return self
-
-            def __exit__(self, *exc):
-                if self.t0 is not None:
-                    prof.record_cpu(name, time.perf_counter() - self.t0)
-                return False
-
-        return _Timer()
+        """`with profiler.time_cpu("decode_attention_cpu"): ...` logs the block as a host operation."""
+        t0 = time.perf_counter()
+        try:
+            yield self
+        finally:
+            self._log("cpu", name, time.perf_counter() - t0)
 
     def per_token_walls_ms(self, n_layers):
-        if not self.enabled or not self.layer_times or len(self.layer_times) % n_layers:
+        """Wall time of each decoded token: its n_layers consecutive layer samples added up."""
+        secs = [t for _, t in self.layer_times]
+        if not self.enabled or not secs or len(secs) % n_layers:
             return []
-        walls = [t for _, t in self.layer_times]
-        return [sum(walls[i:i + n_layers]) * 1000.0 for i in range(0, len(walls), n_layers)]
+        return [1e3 * sum(secs[i:i + n_layers]) for i in range(0, len(secs), n_layers)]
 
     def report(self):
         if not self.enabled:
             return
+        mean = lambda xs: sum(xs) / len(xs)
         print("Kernel calls (host write + launch + read back):")
         for name, ts in sorted(self.kernel_times.items()):
-            print(f"  {name:24s} n={len(ts):5d} avg={1e3 * sum(ts) / len(ts):8.3f} ms total={sum(ts):7.3f} s")
-            bd = self.kernel_breakdowns.get(name)
-            if bd:
-                avg = lambda k: sum(b[k] for b in bd) / len(bd)
-                print(f"  {'':24s} write {avg('write_ms'):.3f} ms, kernel {avg('kernel_ms'):.3f} ms, read {avg('read_ms'):.3f} ms")
+            print(f"  {name:24s} n={len(ts):5d} avg={1e3 * mean(ts):8.3f} ms total={sum(ts):7.3f} s")
+            parts = self.kernel_breakdowns.get(name)
+            if parts:
+                w, k, r = (mean([b[f] for b in parts]) for f in ("write_ms", "kernel_ms", "read_ms"))
+                print(f"  {'':24s} write {w:.3f} ms, kernel {k:.3f} ms, read {r:.3f} ms")
         if self.cpu_times:
             print("Host operations:")
             for name, ts in sorted(self.cpu_times.items()):
-                print(f"  {name:24s} n={len(ts):5d} avg={1e3 * sum(ts) / len(ts):8.3f} ms")
+                print(f"  {name:24s} n={len(ts):5d} avg={1e3 * mean(ts):8.3f} ms")
 
 
 def _check_shared_alias(shared_alias, static_input_indices, n_args):
-    """The reference validates the alias map before it touches the device (cache.py:576-603)."""
-    static = set(static_input_indices or [])
-    clash = sorted(set(shared_alias) & static)
-    if clash:
-        raise ValueError(f"shared_alias must not target static_input_indices {clash}: "
-                         f"static BOs are per-bo_key, aliases are process-wide")
-    oob = sorted(i for i in shared_alias if not 0 <= i < n_args)
-    if oob:
-        raise ValueError(f"shared_alias indices {oob} out of range for {n_args} args")
-    unnamed = sorted(i for i, n in shared_alias.items() if not isinstance(n, str) or not n)
-    if unnamed:
-        raise ValueError(f"shared_alias pool names must be non-empty strings; bad at arg indices {unnamed}")
+    """Refuse an alias map before anything touches the device (the reference does the same, cache.py:576-603): an
+    aliased argument shares one process-wide buffer by pool name, so it cannot also be a per-bo_key static
+    argument, must name an existing argument, and needs a usable pool name."""
+    static = frozenset(static_input_indices or ())
+    problems = []
+    for idx, pool in shared_alias.items():
+        if not (isinstance(idx, int) and 0 <= idx < n_args):
+            problems.append(f"argument {idx!r} does not exist (the call has {n_args} arguments)")
+        elif idx in static:
+            problems.append(f"argument {idx} is static (kept per bo_key) and cannot join the process-wide pool {pool!r}")
+        if not (isinstance(pool, str) and pool):
+            problems.append(f"argument {idx!r} has no pool name (got {pool!r})")
+    if problems:
+        raise ValueError("shared_alias: " + "; ".join(problems))
 
 
 class KernelCache:

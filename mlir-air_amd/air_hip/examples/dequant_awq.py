@@ -1,8 +1,8 @@
 """AWQ int4 -> bf16 dequant of a 1-D vector: out[i] = (q[i] - z[i // gs]) * s[i // gs]
 (counterpart of programming_examples/dequant_awq/dequant_awq.py).
 
-The GPU kernel dequantises AWQ matrices W[K, N]; the 1-D example maps onto it with K = n and
-one packed word (8 columns) per row that repeats the element, of which column 0 is returned."""
+`pack_inputs` writes the reference's own tiled buffer ([herd_n, tile_bytes] uint8: per tile Q two elements per byte,
+S bf16 per group, Z u8 per group, padded to 4 bytes); the GPU kernel reads that buffer as it is."""
 
 import argparse
 
@@ -12,17 +12,18 @@ from .. import awq, bf16
 from ..backend import HIPBackend, HIPRunner, HipModule
 
 
+def packed_tile_bytes(n_tile, group_size):
+    return awq.packed_tile_bytes_1d(n_tile, group_size)
+
+
 def build_module(n, group_size=128, herd_n=4, **ignored):
-    if n % group_size:
-        raise ValueError("N must be divisible by group_size")
-    return HipModule("dequant_awq", K=n, N=8, gs=group_size)
+    if n % herd_n or (n // herd_n) % group_size:
+        raise ValueError("N / herd_n must be divisible by group_size")
+    return HipModule("dequant_awq_1d", K=n, N=herd_n, gs=group_size)
 
 
 def pack_inputs(int4_vals, scales, zeros, n, group_size, herd_n=4):
-    q = np.repeat(np.asarray(int4_vals, dtype=np.uint8)[:, None], 8, axis=1)
-    z = np.repeat(np.asarray(zeros, dtype=np.uint8)[:, None], 8, axis=1)
-    s = np.repeat(bf16.bits_of(scales)[:, None], 8, axis=1)
-    return awq.pack_buffer(awq.pack_int4(q), awq.pack_int4(z), bf16.from_bits(s))
+    return awq.pack_inputs_1d(int4_vals, scales, zeros, n, group_size, herd_n)
 
 
 def parse_args(argv=None):
@@ -43,20 +44,20 @@ def draw_inputs(args):
     return int4_vals, scales, zeros
 
 
-def dequant(int4_vals, scales, zeros, group_size):
-    """Run the 1-D dequant on the GPU and return bf16 bits [n]."""
+def dequant(int4_vals, scales, zeros, group_size, herd_n=4):
+    """Run the 1-D dequant on the GPU and return bf16 [n]."""
     n = len(int4_vals)
     backend = HIPBackend()
-    invoker = backend.compile_and_load(build_module(n, group_size))
-    out = invoker(pack_inputs(int4_vals, scales, zeros, n, group_size), np.zeros((n, 8), np.uint16).view(bf16.BF16Array))[-1]
+    invoker = backend.compile_and_load(build_module(n, group_size, herd_n))
+    out = invoker(pack_inputs(int4_vals, scales, zeros, n, group_size, herd_n), np.zeros(n, np.uint16).view(bf16.BF16Array))[-1]
     backend.unload()
-    return np.ascontiguousarray(bf16.bits_of(out)[:, 0]).view(bf16.BF16Array)
+    return out
 
 
 def run(args, cpu_reference):
     int4_vals, scales, zeros = draw_inputs(args)
     ref = bf16.from_bits(cpu_reference(int4_vals, bf16.bits_of(scales), zeros, args.group_size))
-    got = dequant(int4_vals, scales, zeros, args.group_size)
+    got = dequant(int4_vals, scales, zeros, args.group_size, args.herd_n)
     ok = HIPRunner(verbose=args.verbose)._check_outputs([got], [ref], rtol=1e-1, atol=5e-2)
     print("PASS!" if ok else "failed.")
     return 0 if ok else -1

@@ -64,6 +64,19 @@ def awq_dequant(qweight, qzeros, scales, group=GROUP, out=None):
     return out
 
 
+def awq_dequant_1d(packed, n, group=GROUP, herd_n=4, out=None):
+    """1-D dequant of the reference example's tiled buffer (uint8 [herd_n * tile_bytes]) -> bf16 [n]."""
+    lib = _lib.load_library()
+    _need_cuda(packed)
+    tile_bytes = lib.awq_dequant_1d_tile_bytes(n, group, herd_n)
+    if tile_bytes == 0 or packed.numel() != herd_n * tile_bytes:
+        raise ValueError(f"awq_dequant_1d: n={n}, group={group}, herd_n={herd_n} needs {herd_n} tiles of {tile_bytes} bytes")
+    if out is None:
+        out = torch.empty((n,), dtype=torch.bfloat16, device=packed.device)
+    _lib.check(lib.awq_dequant_1d_bf16(_ptr(packed), _ptr(out), n, group, herd_n, _stream()))
+    return out
+
+
 def w4a16_gemm(x, qweight, qzeros, scales, group=GROUP, out=None):
     """y[M, N] = bf16(x[M, K] . W); x may also be a vector [K] (returns [N])."""
     lib = _lib.load_library()

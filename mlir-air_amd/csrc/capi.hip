@@ -216,6 +216,20 @@ int awq_dequant_bf16(const int32_t *qweight, const int32_t *qzeros, const uint16
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+size_t awq_dequant_1d_tile_bytes(int n, int group, int herd_n) {
+    if (n <= 0 || group <= 0 || herd_n <= 0 || group % 8 != 0 || n % herd_n != 0 || (n / herd_n) % group != 0) return 0;
+    const int n_tile = n / herd_n, ng = n_tile / group;
+    return (size_t)((n_tile / 2 + 3 * ng + 3) & ~3);
+}
+
+int awq_dequant_1d_bf16(const uint8_t *packed, uint16_t *out_bf16, int n, int group, int herd_n, void *stream) {
+    if (!packed || !out_bf16) return W4A16_ERR_NULL;
+    if (awq_dequant_1d_tile_bytes(n, group, herd_n) == 0) return W4A16_ERR_SHAPE;
+    if (misaligned(packed) || misaligned(out_bf16)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_dequant_1d(packed, out_bf16, n, group, herd_n, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 size_t w4a16_gemm_workspace_bytes(int M, int K, int N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
     return kHeaderBytes + stream_partial_bytes(M, N, 1);

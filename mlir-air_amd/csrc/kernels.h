@@ -35,6 +35,9 @@ StreamPlan plan_stream(int M, int K, int N, bool fixed_shape = false);   // fixe
 hipError_t launch_dequant(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, uint16_t *out,
                           int K, int N, hipStream_t stream);
 
+// 1-D dequant of the reference's tiled [herd_n, tile_bytes] buffer (dequant.hip).
+hipError_t launch_dequant_1d(const uint8_t *packed, uint16_t *out, int n, int gs, int herd_n, hipStream_t stream);
+
 // Optional stages fused into the streaming kernel.
 struct StreamExtras {
     const uint16_t *residual = nullptr;   // [M, N] bf16 added to the result before the final rounding

@@ -131,6 +131,27 @@ def dequant_1d(int4_vals, scales_bits, zeros, group_size):
     return f32_to_bf16_bits(((q - z) * s).astype(np.float32))
 
 
+def pack_inputs_1d_loop(int4_vals, scales_bits, zeros, n, group_size, herd_n):
+    """Scalar restatement of the 1-D dequant example's tiling (pack_inputs, dequant_awq.py:259-278; tile size
+    packed_tile_bytes, :59-69): tile ty = [Q: element pairs, even one in the low nibble][S: bf16 little endian per
+    group][Z: one byte per group][zero padding to a multiple of 4 bytes].  One byte at a time."""
+    n_tile = n // herd_n
+    ng_tile = n_tile // group_size
+    q_bytes, s_bytes, z_bytes = n_tile // 2, 2 * ng_tile, ng_tile
+    tile_bytes = (q_bytes + s_bytes + z_bytes + 3) & ~3
+    out = np.zeros((herd_n, tile_bytes), dtype=np.uint8)
+    for ty in range(herd_n):
+        for j in range(q_bytes):
+            lo, hi = int(int4_vals[ty * n_tile + 2 * j]), int(int4_vals[ty * n_tile + 2 * j + 1])
+            out[ty, j] = lo | (hi << 4)
+        for g in range(ng_tile):
+            bits = int(scales_bits[ty * ng_tile + g])
+            out[ty, q_bytes + 2 * g] = bits & 0xFF
+            out[ty, q_bytes + 2 * g + 1] = bits >> 8
+            out[ty, q_bytes + s_bytes + g] = int(zeros[ty * ng_tile + g])
+    return out
+
+
 def pack_inputs_loop(a_q, a_s_bits, a_z, M, K, GS, M_TILE, K_CHUNK, N_CORES, M_PER_LAUNCH):
     """Scalar restatement of the decode buffer tiling (matvec_int4_packed.py:57-103): one tile per
     (launch, core, M block, K chunk) in that nesting order, each tile

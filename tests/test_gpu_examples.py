@@ -90,6 +90,23 @@ def test_example_dequant_1d_bit_exact(capsys):
     capsys.readouterr()
 
 
+@pytest.mark.parametrize("n,gs,herd_n", [(128, 128, 1), (1024, 128, 4), (4096, 64, 8), (1 << 20, 128, 16), (768, 32, 3)])
+def test_dequant_1d_on_the_reference_tile_buffer(n, gs, herd_n):
+    """The kernel reads the example's [herd_n, tile_bytes] buffer as pack_inputs writes it; random scale bit patterns
+    (finite), every zero point, bit-exact against the oracle."""
+    from air_hip import awq, bf16, ops
+    print(f"dequant 1-D n={n} gs={gs} herd_n={herd_n}", flush=True)
+    rng = np.random.default_rng(n + gs)
+    q = rng.integers(0, 16, n).astype(np.uint8)
+    z = rng.integers(0, 16, n // gs).astype(np.uint8)
+    s = rng.integers(0, 65536, n // gs).astype(np.uint16)
+    s[(s & 0x7F80) == 0x7F80] = 0x3C00
+    packed = awq.pack_inputs_1d(q, bf16.from_bits(s), z, n, gs, herd_n)
+    out = ops.awq_dequant_1d(torch.from_numpy(packed.reshape(-1)).cuda(), n, gs, herd_n)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(out), oawq.dequant_1d(q, s, z, gs))
+
+
 def test_kernels_against_golden_fixtures():
     from air_hip import ops
     print("golden fixtures", flush=True)

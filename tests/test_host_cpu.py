@@ -265,11 +265,11 @@ def test_kernel_cache_host_contract(tmp_path):
         c.load_and_run("attn_gemms", {}, np.zeros(4, np.uint16))
     z = bf16.from_f32(np.zeros(2048))
     args = [z] * 15
-    with pytest.raises(ValueError, match="must not target static_input_indices"):
+    with pytest.raises(ValueError, match="is static"):
         c.load_and_run("o_gemv_ffn_int4", {}, *args, static_input_indices={0, 6}, shared_alias={6: "res"})
-    with pytest.raises(ValueError, match="out of range"):
+    with pytest.raises(ValueError, match="does not exist"):
         c.load_and_run("o_gemv_ffn_int4", {}, *args, shared_alias={15: "res"})
-    with pytest.raises(ValueError, match="non-empty strings"):
+    with pytest.raises(ValueError, match="no pool name"):
         c.load_and_run("o_gemv_ffn_int4", {}, *args, shared_alias={14: ""})
     with pytest.raises(AirBackendError, match="takes 15 arguments"):
         c.load_and_run("o_gemv_ffn_int4", {}, *args[:14])

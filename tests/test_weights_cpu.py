@@ -186,3 +186,37 @@ def test_awq_tensors_to_gemm_tiles_is_the_reference_prefill_packing():
     w_q = (w_nk[:, 0::2] | (w_nk[:, 1::2] << 4)).astype(np.uint8)
     want = oawq.pack_inputs_gemm_loop(w_q, sc, oawq.unpack_awq_int32(qz), K, N, GS, 16, 128)
     assert np.array_equal(got, want)
+
+
+def test_dequant_1d_tile_form_offsets_and_round_trip():
+    """The 1-D dequant example's buffer (dequant_awq.py:59-69, 259-278).  Sizes from the formula by hand: n = 1024,
+    gs = 128, herd_n = 4 -> 256 elements per tile = 128 Q bytes + 2 groups x 2 S bytes + 2 Z bytes = 134 -> 136.  An
+    element followed to its byte: element 777 = tile 3, offset 9 -> byte 4 (high nibble); its group 6 = tile 3, local
+    group 0 -> S at bytes 128..129, Z at byte 132."""
+    from air_hip import awq, bf16
+    from oracle import awq as oawq
+
+    assert awq.packed_tile_bytes_1d(256, 128) == (128, 4, 2, 136)
+    assert awq.packed_tile_bytes_1d(128, 128) == (64, 2, 1, 68)        # 67 -> 68
+    assert awq.packed_tile_bytes_1d(512, 64) == (256, 16, 8, 280)
+    rng = np.random.default_rng(3)
+    n, gs, herd_n = 1024, 128, 4
+    q = rng.integers(0, 16, n).astype(np.uint8)
+    z = rng.integers(0, 16, n // gs).astype(np.uint8)
+    s = rng.integers(0, 65536, n // gs).astype(np.uint16)
+    packed = awq.pack_inputs_1d(q, bf16.from_bits(s), z, n, gs, herd_n)
+    assert packed.shape == (4, 136) and packed.dtype == np.uint8
+    assert packed[3, 4] >> 4 == q[777] and packed[3, 4] & 0xF == q[776]
+    assert int(packed[3, 128]) | (int(packed[3, 129]) << 8) == s[6] and packed[3, 132] == z[6]
+    assert int(packed[3, 130]) | (int(packed[3, 131]) << 8) == s[7] and packed[3, 133] == z[7]
+    assert not packed[:, 134:].any()                                    # padding
+    assert np.array_equal(packed, oawq.pack_inputs_1d_loop(q, s, z, n, gs, herd_n))
+    q2, s2, z2 = awq.unpack_inputs_1d(packed, n, gs, herd_n)
+    assert np.array_equal(q2, q) and np.array_equal(bf16.bits_of(s2), s) and np.array_equal(z2, z)
+    for n2, gs2, h2 in ((512, 64, 8), (128, 128, 1), (4096, 128, 2)):
+        q = rng.integers(0, 16, n2).astype(np.uint8)
+        z = rng.integers(0, 16, n2 // gs2).astype(np.uint8)
+        s = rng.integers(0, 65536, n2 // gs2).astype(np.uint16)
+        assert np.array_equal(awq.pack_inputs_1d(q, bf16.from_bits(s), z, n2, gs2, h2), oawq.pack_inputs_1d_loop(q, s, z, n2, gs2, h2))
+    with pytest.raises(ValueError):
+        awq.pack_inputs_1d(q, bf16.from_bits(s), z, 4096, 128, 3)
