@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|prefill|ffn|block|layer|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_1b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|prefill|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_1b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -35,7 +35,10 @@ CONFIGS = {
     "gemv_awq": dict(M=1, K=4096, N=11008, cfg=None, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128, checkpoint-layout weights"),
     "gemm16": dict(M=16, K=4096, N=14336, cfg=2, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128"),
     "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128"),
-    "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128"),
+    "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128, stream-order weights (2 launches)"),
+    "ffn_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128, checkpoint-layout weights (persistent kernel)"),
+    "block_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode block, checkpoint-layout weights"),
+    "layer_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode layer, checkpoint-layout weights"),
     # beyond the five headline configs: the O projection + RMSNorm + FFN decode block with residuals (3 launches)
     "block": dict(M=1, K=4096, N=14336, cfg=None, desc="decode block O-proj + RMSNorm + SwiGLU FFN W4A16 E=4096 H=14336 g128"),
     # one whole decode layer: RMSNorm + fused QKV GEMV, then RoPE + KV append + GQA attention over 2048 cached
@@ -53,7 +56,7 @@ LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 204
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
 # scaled by the same counter's reading for a 256 MiB device copy: x2.000 and x1.000); the
 # summaries under profiles/ hold the commands and the raw readings.
-MEASURED_TRAFFIC_BYTES = {"gemv": 24.11e6, "gemv_awq": 24.27e6, "prefill": 342.2e6, "ffn": 97.07e6, "lm_head": 525.9e6}
+MEASURED_TRAFFIC_BYTES = {"gemv": 24.11e6, "gemv_awq": 24.27e6, "prefill": 342.2e6, "ffn_awq": 97.07e6, "lm_head": 525.9e6}
 
 
 def weight_bytes(K, N):
@@ -67,6 +70,7 @@ def q4nx_weight_bytes(K, N):
 def algorithmic_bytes(name):
     c = CONFIGS[name]
     M, K, N = c["M"], c["K"], c["N"]
+    name = name[:-4] if name.endswith("_awq") else name
     if name.startswith("q4nx"):
         return q4nx_weight_bytes(K, N) + M * K * 2 + M * N * 2
     if name == "lm_head":   # weights, x and norm weight in, logits out
@@ -86,6 +90,7 @@ def algorithmic_bytes(name):
 
 def algorithmic_flops(name):
     c = CONFIGS[name]
+    name = name[:-4] if name.endswith("_awq") else name
     if name == "ffn":
         return 2 * 3 * c["K"] * c["N"]
     if name in ("block", "layer"):
@@ -126,23 +131,26 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
 
     q4nx = name.startswith("q4nx")
     lm_head = name == "lm_head"
-    per_copy = K * N * 2 if lm_head else q4nx_weight_bytes(K, N) if q4nx else weight_bytes(K, N) * (3 if name in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if name in ("block", "layer") else 0)
+    stream_order = name in ("gemv", "ffn", "block", "layer")     # weights re-packed at load time (untimed)
+    kind = name[:-4] if name.endswith("_awq") else name
+    per_copy = K * N * 2 if lm_head else q4nx_weight_bytes(K, N) if q4nx else weight_bytes(K, N) * (3 if kind in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if kind in ("block", "layer") else 0)
     nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
-    if name == "layer":
+    if kind == "layer":
         per_copy += weight_bytes(K, nqkv)
     if name == "prefill":
         ncopies = 1
     else:
         ncopies = max(2, -(-(MALL_BYTES + MALL_BYTES // 2) // per_copy))
     copies = []
+    awq0 = None   # copy 0 in checkpoint layout, for the CPU baseline of a stream-order workload
     for i in range(ncopies):
-        if name == "ffn":
+        if kind == "ffn":
             copies.append((make_weights(torch, K, N, 100 + 3 * i), make_weights(torch, K, N, 101 + 3 * i),
                            make_weights(torch, N, K, 102 + 3 * i)))
-        elif name in ("block", "layer"):
+        elif kind in ("block", "layer"):
             c4 = (make_weights(torch, K, N, 100 + 5 * i), make_weights(torch, K, N, 101 + 5 * i),
                   make_weights(torch, N, K, 102 + 5 * i), make_weights(torch, K, K, 103 + 5 * i))
-            copies.append(c4 + ((make_weights(torch, K, nqkv, 104 + 5 * i),) if name == "layer" else ()))
+            copies.append(c4 + ((make_weights(torch, K, nqkv, 104 + 5 * i),) if kind == "layer" else ()))
         elif q4nx:
             copies.append(make_q4nx_weights(torch, K, N, 100 + i))
         elif lm_head:
@@ -161,12 +169,17 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             del w
         else:
             copies.append(make_weights(torch, K, N, 100 + i))
+        if stream_order and kind != "gemv":
+            from air_hip import ops
+            if i == 0:
+                awq0 = copies[0]
+            copies[i] = tuple(ops.repack_stream(*m).buf for m in copies[i])
     gx = torch.Generator(device="cuda")
     gx.manual_seed(7)
     x = torch.randn((max(M, 1), K), device="cuda", generator=gx).to(torch.bfloat16)
     if name == "dequant":
         outs = [torch.empty((K, N), dtype=torch.bfloat16, device=dev) for _ in range(min(ncopies, 8))]
-    elif name in ("ffn", "block", "layer"):
+    elif kind in ("ffn", "block", "layer"):
         outs = [torch.empty((K,), dtype=torch.bfloat16, device=dev)]
     else:
         outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev)]
@@ -174,10 +187,10 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         outs = [torch.empty((N,), dtype=torch.bfloat16, device=dev)]
         best = torch.empty((1,), dtype=torch.int32, device=dev)
         lm_ws = torch.empty(int(lib.lm_head_workspace_bytes(N)), dtype=torch.uint8, device=dev)
-    if name in ("block", "layer", "lm_head"):
+    if kind in ("block", "layer", "lm_head"):
         x_residual = torch.randn((K,), device="cuda", generator=gx).to(torch.bfloat16)
         norm_w = (torch.randn((K,), device="cuda", generator=gx) * 0.1 + 1.0).to(torch.bfloat16)
-    if name == "layer":
+    if kind == "layer":
         kv_shape = (LAYER_KV, LAYER_MAXSEQ, LAYER_HD)
         k_cache = torch.randn(kv_shape, device="cuda", generator=gx).to(torch.bfloat16)
         v_cache = torch.randn(kv_shape, device="cuda", generator=gx).to(torch.bfloat16)
@@ -185,12 +198,16 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         qkv = torch.empty((nqkv,), dtype=torch.bfloat16, device=dev)
         attn_out = torch.empty((K,), dtype=torch.bfloat16, device=dev)
         attn_ws = torch.empty(int(lib.w4a16_attention_workspace_bytes(LAYER_HEADS, LAYER_HD)), dtype=torch.uint8, device=dev)
-        x_sumsq = (x_residual.float() ** 2).reshape(K // 256, 256).sum(dim=1).contiguous()
-        y_sumsq = torch.empty((K // 256,), dtype=torch.float32, device=dev)
+        piece = 16 if stream_order else 256
+        x_sumsq = (x_residual.float() ** 2).reshape(K // piece, piece).sum(dim=1).contiguous()
+        y_sumsq = torch.empty((K // piece,), dtype=torch.float32, device=dev)
+    if stream_order and kind in ("ffn", "block", "layer"):
+        h_buf = torch.empty((N,), dtype=torch.bfloat16, device=dev)
+        bws = torch.empty(int(lib.w4a16_block_stream_workspace_bytes(K, N)), dtype=torch.uint8, device=dev)
 
-    if name == "ffn":
+    if kind == "ffn":
         ws_bytes = lib.w4a16_ffn_workspace_bytes(K, N)
-    elif name in ("block", "layer"):
+    elif kind in ("block", "layer"):
         ws_bytes = max(lib.w4a16_block_workspace_bytes(K, N), lib.w4a16_gemm_workspace_bytes(1, K, nqkv))
     else:
         ws_bytes = max(lib.w4a16_gemm_workspace_bytes(max(M, 1), K, N), 16384)
@@ -203,16 +220,33 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             o = outs[i % len(outs)]
             rc = lib.awq_dequant_bf16(w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), o.data_ptr(), K, N, 128, st)
         elif name == "ffn":
+            rc = lib.w4a16_ffn_swiglu_stream_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
+                                                  outs[0].data_ptr(), h_buf.data_ptr(), K, N, 128, st)
+        elif name in ("block", "layer"):
+            g, u, d, o = (t.data_ptr() for t in w[:4])
+            if name == "layer":
+                # the sum of squares of x per 16 columns comes from the block before (here: computed once)
+                _lib.check(lib.w4a16_rms_gemv_stream_bf16(x_residual.data_ptr(), x_sumsq.data_ptr(), x_sumsq.numel(),
+                                                          norm_w.data_ptr(), 1e-5, w[4].data_ptr(), qkv.data_ptr(), K, nqkv, 128, st))
+                _lib.check(lib.w4a16_decode_attn_o_gemv_ffn_stream_bf16(
+                    qkv.data_ptr(), lut_row.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), attn_out.data_ptr(), LAYER_POS,
+                    LAYER_MAXSEQ, LAYER_HEADS, LAYER_KV, LAYER_HD, attn_ws.data_ptr(), attn_ws.numel(), x_residual.data_ptr(),
+                    norm_w.data_ptr(), 1e-5, o, g, u, d, outs[0].data_ptr(), y_sumsq.data_ptr(), K, N, 128, bws.data_ptr(),
+                    bws.numel(), st))
+                return
+            rc = lib.w4a16_o_gemv_ffn_stream_bf16(x.data_ptr(), x_residual.data_ptr(), norm_w.data_ptr(), 1e-5, o, g, u, d,
+                                                  outs[0].data_ptr(), None, None, None, K, N, 128, bws.data_ptr(), bws.numel(), st)
+        elif name == "ffn_awq":
             g, u, d = w
             rc = lib.w4a16_ffn_swiglu_bf16(x.data_ptr(), g[0].data_ptr(), g[1].data_ptr(), g[2].data_ptr(),
                                            u[0].data_ptr(), u[1].data_ptr(), u[2].data_ptr(),
                                            d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(),
                                            outs[0].data_ptr(), None, K, N, 128, ws.data_ptr(), ws.numel(), st)
-        elif name in ("block", "layer"):
+        elif name in ("block_awq", "layer_awq"):
             g, u, d, o = w[:4]
             ptrs = [t.data_ptr() for m in (o, g, u, d) for t in m]
             a_in = x
-            if name == "layer":
+            if name == "layer_awq":
                 qw = w[4]
                 # the sum of squares of x per 256-column tile comes from the block before (here: computed once)
                 _lib.check(lib.w4a16_rms_gemv_sumsq_bf16(x_residual.data_ptr(), x_sumsq.data_ptr(), x_sumsq.numel(),
@@ -322,8 +356,9 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                  "avg": sum(per_launch) / len(per_launch), "max": per_launch[-1]},
     }
 
-    if with_cpu_baseline and name not in ("block", "layer", "lm_head", "gemv_awq") and not q4nx:
-        res["cpu_baseline"] = cpu_baseline(name, torch, copies[0][1:] if name == "gemv" else copies[0], x, outs, launch, stream)
+    if with_cpu_baseline and kind not in ("block", "layer", "lm_head") and not name.endswith("_awq") and not q4nx:
+        w0 = copies[0][1:] if name == "gemv" else awq0 if awq0 is not None else copies[0]
+        res["cpu_baseline"] = cpu_baseline(name, torch, w0, x, outs, launch, stream)
     return res
 
 
@@ -387,7 +422,7 @@ DECODE_MODELS = {
 }
 
 
-def run_decode_model(steps, warmup, model="decode_1b"):
+def run_decode_model(steps, warmup, model="decode_1b", stream_order=True):
     """Greedy decode of a random-weight model in the Llama-3.2-1B shape (16 layers, E=2048, H=8192,
     32/8 heads of 64, vocabulary 128256, tied lm_head) or the Llama-3.1-8B shape, `steps` consecutive
     tokens from position DECODE_1B_POS0 captured as one HIP graph: per token n_layers x (RMSNorm + QKV
@@ -416,6 +451,10 @@ def run_decode_model(steps, warmup, model="decode_1b"):
     layers = [decode.DecodeLayer(attn_norm=norm_w(), ffn_norm=norm_w(), wqkv=lin(E, nqkv, 10 * i), wo=lin(E, E, 10 * i + 1),
                                  w_gate=lin(E, H, 10 * i + 2), w_up=lin(E, H, 10 * i + 3), w_down=lin(H, E, 10 * i + 4))
               for i in range(cfg.n_layers)]
+    if stream_order:
+        for l in layers:   # decode reads stream-order weights; the checkpoint-layout tensors are not needed here
+            l.with_stream()
+            l.wqkv = l.wo = l.w_gate = l.w_up = l.w_down = None
     embed = torch.randn((cfg.vocab_size, E), device="cuda", generator=g).to(torch.bfloat16)
     final_norm = norm_w()
     max_seq = 2048
@@ -684,8 +723,8 @@ def main():
         roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": value / HBM_PEAK_GBS, "traffic": None}
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
-    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel", "ffn": "ffn_fused_kernel", "lm_head": "lm_head_kernel",
-                      "gemv": "gemv_ws_kernel"}.get(name, "stream_kernel")
+    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel", "ffn_awq": "ffn_fused_kernel", "lm_head": "lm_head_kernel",
+                      "gemv": "gemv_ws_kernel", "ffn": "gemv_ws_kernel", "block": "gemv_ws_kernel", "layer": "gemv_ws_kernel"}.get(name, "stream_kernel")
     roof["algorithmic_per_launch"] = main_res["flops"] if name == "prefill" else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]
 

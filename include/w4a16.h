@@ -213,6 +213,44 @@ int w4a16_gemv_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, c
                                   uint16_t *h, int K, int H, int group, void *stream);
 
 /*
+ * The rest of the decode path on stream-order matrices; references and rounding points are those of the
+ * checkpoint-layout entry points of the same name without `_stream` (declared below), none of these keeps state
+ * between calls, and every stage is one whole-K launch.
+ * w4a16_rms_gemv_stream_bf16: y = bf16(bf16((x * rstd) * norm_weight) . W), rstd = 1 / sqrt(mean(x^2) + eps); x_sumsq
+ *   NULL, or n_pieces (<= 4096) partial sums of x^2 left by the call that produced x (then x is not walked for the
+ *   mean; the result agrees up to the summation order of the mean).
+ * w4a16_rms_gemv_swiglu_stream_bf16: RMSNorm + gate / up + SwiGLU (matvec_int4_swiglu_rms.cpu_reference,
+ *   programming_examples/decode_ffn_swiglu/matvec_int4_swiglu_rms.py:490-516).
+ * w4a16_ffn_swiglu_stream_bf16: h = bf16(silu(bf16(x . Wg)) * bf16(x . Wu)), y = bf16(h . Wd); `h` (bf16 [H]) is
+ *   required: it is the intermediate's only home.  Two launches.
+ * w4a16_o_gemv_ffn_stream_bf16: the three stages of o_gemv_ffn_int4
+ *   (programming_examples/llms/llama32_1b_int4/multi_launch_builder/o_gemv_ffn_int4_multi.py:4-37) as three launches;
+ *   res1_out / h_out may be NULL; y_sumsq NULL or E / 16 floats that receive the sum of squares of the bf16 values of y
+ *   per 16 columns, which w4a16_rms_gemv_stream_bf16 of the next layer takes as x_sumsq.  The workspace is plain
+ *   scratch (no initialisation, nothing kept between calls), w4a16_block_stream_workspace_bytes(E, H).
+ * w4a16_decode_attn_o_gemv_ffn_stream_bf16: w4a16_decode_attention_bf16 followed by the block, as one call
+ *   (everything of a decode layer after the Q|K|V projection, llama32_1b_int4_decode.py:270-313).
+ */
+int w4a16_rms_gemv_stream_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
+                               const void *wstream, uint16_t *y, int K, int N, int group, void *stream);
+int w4a16_rms_gemv_swiglu_stream_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const void *gate_wstream,
+                                      const void *up_wstream, uint16_t *h, int K, int H, int group, void *stream);
+int w4a16_ffn_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream,
+                                 const void *down_wstream, uint16_t *y, uint16_t *h, int K, int H, int group, void *stream);
+size_t w4a16_block_stream_workspace_bytes(int E, int H);
+int w4a16_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                                 float eps, const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                 const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, float *y_sumsq,
+                                 int E, int H, int group, void *workspace, size_t workspace_bytes, void *stream);
+int w4a16_decode_attn_o_gemv_ffn_stream_bf16(const uint16_t *qkv, const uint16_t *rope_lut_row, uint16_t *k_cache,
+                                             uint16_t *v_cache, uint16_t *attn_out, int pos, int max_seq, int n_heads,
+                                             int n_kv_heads, int head_dim, void *attn_workspace, size_t attn_workspace_bytes,
+                                             const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                                             const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                             const void *down_wstream, uint16_t *y, float *y_sumsq, int E, int H, int group,
+                                             void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * RMSNorm prologue + decode GEMV, batch 1:
  *   rstd = 1 / sqrt(mean(x^2) + eps),  n = bf16((x * rstd) * norm_weight),  y = bf16(n . W)
  * The normalisation of matvec_int4_swiglu_rms.cpu_reference

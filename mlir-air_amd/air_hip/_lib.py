@@ -54,6 +54,12 @@ SYMBOLS = {
     "w4a16_gemv_stream_bf16": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_gemv_add_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_gemv_swiglu_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a16_rms_gemv_stream_bf16": (_ci, [_vp, _vp, _ci, _vp, _cf, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a16_rms_gemv_swiglu_stream_bf16": (_ci, [_vp, _vp, _cf, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a16_ffn_swiglu_stream_bf16": (_ci, [_vp] * 6 + [_ci, _ci, _ci, _vp]),
+    "w4a16_block_stream_workspace_bytes": (_sz, [_ci, _ci]),
+    "w4a16_o_gemv_ffn_stream_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 8 + [_ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a16_decode_attn_o_gemv_ffn_stream_bf16": (_ci, [_vp] * 5 + [_ci] * 5 + [_vp, _sz, _vp, _vp, _cf] + [_vp] * 6 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_gemv_noalloc_bf16": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_tune": (_ci, [ctypes.c_char_p, _ci]),
 }

@@ -42,6 +42,15 @@ class DecodeLayer:
     w_up: tuple
     w_down: tuple
     codec: str = "awq"   # "awq": triples are (qweight, qzeros, scales); "q4nx": (qweight, scales, mins) from q4nx_repack
+    # AWQ layers: the same five matrices in stream order (ops.StreamWeight), which the decode kernels read; the
+    # checkpoint-layout triples above stay for the prompt pass.  None: decode runs on the triples.
+    stream: dict = None
+
+    def with_stream(self):
+        """Re-pack the layer's matrices into stream order on the GPU (once, at load time)."""
+        if self.codec == "awq" and self.stream is None:
+            self.stream = {name: ops.repack_stream(*getattr(self, name)) for name in ("wqkv", "wo", "w_gate", "w_up", "w_down")}
+        return self
 
 
 def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda") -> DecodeLayer:
@@ -71,8 +80,10 @@ def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda
                        w_down=repack(dev_blocks(blocks["down"]), E, H), codec="q4nx")
 
 
-def prepare_layer(layer: wmod.LayerWeights, device="cuda") -> DecodeLayer:
-    """Host LayerWeights (numpy) -> DecodeLayer: Q, K, V concatenated, everything in HBM."""
+def prepare_layer(layer: wmod.LayerWeights, device="cuda", stream_order=True) -> DecodeLayer:
+    """Host LayerWeights (numpy) -> DecodeLayer: Q, K, V concatenated, everything in HBM, and (stream_order) every
+    matrix re-packed into the decode kernels' stream order, the counterpart of the packed decode buffers the
+    reference attaches per layer at load time (llama32_1b_int4_weights.py:163-216)."""
     def dev(a):
         a = np.ascontiguousarray(a)
         if a.dtype == np.uint16:
@@ -80,9 +91,10 @@ def prepare_layer(layer: wmod.LayerWeights, device="cuda") -> DecodeLayer:
         return torch.from_numpy(a).to(device)
 
     lin = lambda l: tuple(dev(t) for t in l)
-    return DecodeLayer(attn_norm=dev(layer.attn_norm), ffn_norm=dev(layer.ffn_norm),
-                       wqkv=lin(wmod.concat_linears(layer.wq, layer.wk, layer.wv)), wo=lin(layer.wo),
-                       w_gate=lin(layer.w_gate), w_up=lin(layer.w_up), w_down=lin(layer.w_down))
+    out = DecodeLayer(attn_norm=dev(layer.attn_norm), ffn_norm=dev(layer.ffn_norm),
+                      wqkv=lin(wmod.concat_linears(layer.wq, layer.wk, layer.wv)), wo=lin(layer.wo),
+                      w_gate=lin(layer.w_gate), w_up=lin(layer.w_up), w_down=lin(layer.w_down))
+    return out.with_stream() if stream_order else out
 
 
 def new_kv_cache(config, max_seq, device="cuda"):
@@ -98,6 +110,12 @@ def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer
     updated in place at current_pos.  x_sumsq / return_sumsq chain the sum of squares of the block's output into
     the next block's RMSNorm (AWQ layers): with return_sumsq the result is (y, sumsq or None)."""
     q4nx = layer.codec == "q4nx"
+    if layer.stream is not None:   # stream-order weights: stateless whole-K launches, sums of squares per 16 columns
+        sw = layer.stream
+        qkv = ops.w4a16_rms_gemv_stream(x, layer.attn_norm, sw["wqkv"], eps=config.rms_eps, x_sumsq=x_sumsq)
+        return ops.decode_attn_o_gemv_ffn_stream(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos,
+                                                 config.n_heads, x, layer.ffn_norm, sw["wo"], sw["w_gate"], sw["w_up"],
+                                                 sw["w_down"], eps=config.rms_eps, return_sumsq=return_sumsq)
     if not q4nx:   # attention + block as one call: the O projection merges the attention's chunk partials where it can
         qkv = ops.w4a16_rms_gemv(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps, x_sumsq=x_sumsq)
         return ops.decode_attn_o_gemv_ffn(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads,

@@ -356,6 +356,122 @@ def decode_attn_o_gemv_ffn(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, x_
     return (y, sumsq) if return_sumsq else y
 
 
+_block_scratch = {}
+
+
+def _block_stream_scratch(E, H, device):
+    """Plain scratch of the stream-order block (res1, h, sums of squares): nothing is kept in it between calls."""
+    lib = _lib.load_library()
+    key = (device.index, _stream(), E, H)
+    ws = _block_scratch.get(key)
+    if ws is None:
+        ws = torch.empty(int(lib.w4a16_block_stream_workspace_bytes(E, H)), dtype=torch.uint8, device=device)
+        _block_scratch[key] = ws
+    return ws
+
+
+def w4a16_rms_gemv_stream(x, norm_weight, w, eps=1e-5, group=GROUP, x_sumsq=None):
+    """y[N] = bf16(rms_norm(x, norm_weight) . W) on a StreamWeight.  x_sumsq: float32 partial sums of x^2 left by the
+    call that produced x (o_gemv_ffn_stream / decode_attn_o_gemv_ffn_stream with return_sumsq)."""
+    lib = _lib.load_library()
+    _need_cuda(x, norm_weight, w.buf)
+    if x.numel() != w.K or norm_weight.numel() != w.K:
+        raise ValueError("w4a16_rms_gemv_stream: x and norm_weight must have K elements")
+    out = torch.empty((w.N,), dtype=torch.bfloat16, device=x.device)
+    if x_sumsq is not None and (x_sumsq.dtype != torch.float32 or not x_sumsq.is_cuda or not x_sumsq.is_contiguous()):
+        raise ValueError("x_sumsq must be a contiguous float32 GPU tensor")
+    _lib.check(lib.w4a16_rms_gemv_stream_bf16(_ptr(_bits(x)), _ptr(x_sumsq) if x_sumsq is not None else None,
+                                              x_sumsq.numel() if x_sumsq is not None else 0, _ptr(_bits(norm_weight)), float(eps),
+                                              _ptr(w.buf), _ptr(out), w.K, w.N, group, _stream()))
+    return out
+
+
+def w4a16_rms_swiglu_stream(x, norm_weight, gate, up, eps=1e-5, group=GROUP):
+    """h[H] = bf16(silu(bf16(n Wg)) * bf16(n Wu)), n = bf16((x * rstd) * norm_weight), on two StreamWeights."""
+    lib = _lib.load_library()
+    _need_cuda(x, norm_weight, gate.buf, up.buf)
+    if x.numel() != gate.K or (up.K, up.N) != (gate.K, gate.N) or norm_weight.numel() != gate.K:
+        raise ValueError("w4a16_rms_swiglu_stream: gate and up must both be [K, H], x and norm_weight [K]")
+    h = torch.empty((gate.N,), dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.w4a16_rms_gemv_swiglu_stream_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps), _ptr(gate.buf),
+                                                     _ptr(up.buf), _ptr(h), gate.K, gate.N, group, _stream()))
+    return h
+
+
+def ffn_swiglu_stream(x, gate, up, down, group=GROUP, return_h=False):
+    """Decode FFN on StreamWeights: y = Wd(silu(x Wg) * (x Wu)); two whole-K launches, no workspace."""
+    lib = _lib.load_library()
+    _need_cuda(x, gate.buf, up.buf, down.buf)
+    K, H = gate.K, gate.N
+    if x.numel() != K or (up.K, up.N) != (K, H) or (down.K, down.N) != (H, K):
+        raise ValueError("ffn_swiglu_stream: gate/up must be [K, H] and down [H, K]")
+    y = torch.empty((K,), dtype=torch.bfloat16, device=x.device)
+    h = torch.empty((H,), dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.w4a16_ffn_swiglu_stream_bf16(_ptr(_bits(x)), _ptr(gate.buf), _ptr(up.buf), _ptr(down.buf), _ptr(y), _ptr(h),
+                                                K, H, group, _stream()))
+    return (y, h) if return_h else y
+
+
+def _check_block_stream(E, H, wo, gate, up, down, *vectors):
+    if ((wo.K, wo.N) != (E, E) or (gate.K, gate.N) != (E, H) or (up.K, up.N) != (E, H) or (down.K, down.N) != (H, E)
+            or any(v.numel() != E for v in vectors)):
+        raise ValueError("stream-order block: wo must be [E, E], gate/up [E, H], down [H, E], vectors [E]")
+
+
+def o_gemv_ffn_stream(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, group=GROUP,
+                      return_intermediates=False, return_sumsq=False):
+    """Decode block on StreamWeights: res1 = Wo(attn_out) + x_residual; y = Wd(swiglu(rms_norm(res1))) + res1.
+    Returns y, or (y, res1, h); with return_sumsq the sum of squares of y per 16 columns (float32 [E / 16]) is
+    appended for the next layer's w4a16_rms_gemv_stream."""
+    lib = _lib.load_library()
+    _need_cuda(attn_out, x_residual, ffn_norm_weight, wo.buf, gate.buf, up.buf, down.buf)
+    E, H = wo.K, gate.N
+    _check_block_stream(E, H, wo, gate, up, down, attn_out, x_residual, ffn_norm_weight)
+    dev = attn_out.device
+    y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
+    res1 = torch.empty((E,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
+    h = torch.empty((H,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
+    sumsq = torch.empty((E // 16,), dtype=torch.float32, device=dev) if return_sumsq else None
+    ws = _block_stream_scratch(E, H, dev)
+    opt = lambda t: _ptr(t) if t is not None else None
+    _lib.check(lib.w4a16_o_gemv_ffn_stream_bf16(
+        _ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps), _ptr(wo.buf), _ptr(gate.buf),
+        _ptr(up.buf), _ptr(down.buf), _ptr(y), opt(res1), opt(h), opt(sumsq), E, H, group, _ptr(ws), ws.numel(), _stream()))
+    out = (y, res1, h) if return_intermediates else (y,)
+    if return_sumsq:
+        out = out + (sumsq,)
+    return out if len(out) > 1 else y
+
+
+def decode_attn_o_gemv_ffn_stream(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, x_residual, ffn_norm_weight, wo, gate, up,
+                                  down, eps=1e-5, group=GROUP, return_sumsq=False):
+    """decode_attention followed by o_gemv_ffn_stream as one call.  Returns y bf16 [E], with return_sumsq also the sum
+    of squares of y per 16 columns (float32 [E / 16])."""
+    lib = _lib.load_library()
+    _need_cuda(qkv, rope_lut_row, k_cache, v_cache, x_residual, ffn_norm_weight, wo.buf, gate.buf, up.buf, down.buf)
+    n_kv, max_seq, hd = k_cache.shape
+    E, H = n_heads * hd, gate.N
+    if v_cache.shape != k_cache.shape or qkv.numel() != (n_heads + 2 * n_kv) * hd or rope_lut_row.numel() != hd:
+        raise ValueError("decode_attn_o_gemv_ffn_stream: qkv must be [(n_heads + 2 n_kv) * hd], caches [n_kv, max_seq, hd], lut row [hd]")
+    _check_block_stream(E, H, wo, gate, up, down, x_residual, ffn_norm_weight)
+    dev = qkv.device
+    y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
+    attn_out = torch.empty((E,), dtype=torch.bfloat16, device=dev)
+    key = (dev.index, _stream(), n_heads, hd)
+    aws = _attn_ws.get(key)
+    if aws is None:
+        aws = torch.empty(int(lib.w4a16_attention_workspace_bytes(n_heads, hd)), dtype=torch.uint8, device=dev)
+        _attn_ws[key] = aws
+    ws = _block_stream_scratch(E, H, dev)
+    sumsq = torch.empty((E // 16,), dtype=torch.float32, device=dev) if return_sumsq else None
+    _lib.check(lib.w4a16_decode_attn_o_gemv_ffn_stream_bf16(
+        _ptr(_bits(qkv)), _ptr(_bits(rope_lut_row)), _ptr(_bits(k_cache)), _ptr(_bits(v_cache)), _ptr(attn_out), int(pos),
+        max_seq, n_heads, n_kv, hd, _ptr(aws), aws.numel(), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
+        _ptr(wo.buf), _ptr(gate.buf), _ptr(up.buf), _ptr(down.buf), _ptr(y), _ptr(sumsq) if sumsq is not None else None, E, H,
+        group, _ptr(ws), ws.numel(), _stream()))
+    return (y, sumsq) if return_sumsq else y
+
+
 def rope_halfsplit(x, lut):
     """Half-split RoPE of x bf16 [rows, dim] with one LUT row (cos then sin) per row: lut bf16 [rows, dim]."""
     lib = _lib.load_library()

@@ -471,33 +471,150 @@ int w4a16_repack_stream(const int32_t *qweight, const int32_t *qzeros, const uin
 }
 
 namespace {
-int gemv_stream_impl(const uint16_t *x, const void *w, const void *w_up, const uint16_t *residual, bool need_residual,
-                     uint16_t *y, int K, int N, int group, void *stream) {
-    if (!x || !w || !y || (need_residual && !residual)) return W4A16_ERR_NULL;
+// One whole-K launch on stream-order weights: argument checks shared by every stream-order entry point.
+int gemv_stream_call(const uint16_t *x, const void *w, const void *w_up, uint16_t *y, int K, int N, int group, void *stream,
+                     const GemvWsExtras &ex) {
+    if (!x || !w || !y) return W4A16_ERR_NULL;
     if (group != kGroup) return W4A16_ERR_GROUP;
     if (K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
-    if (misaligned(x) || misaligned(w) || misaligned(y) || (w_up && misaligned(w_up)) || (residual && misaligned(residual)))
+    if (ex.norm_w && !(ex.eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (ex.sumsq_in && (ex.sumsq_n < 1 || ex.sumsq_n > 4096)) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(w) || misaligned(y) || (w_up && misaligned(w_up)) || (ex.residual && misaligned(ex.residual)) ||
+        (ex.norm_w && misaligned(ex.norm_w)) || (ex.sumsq_in && misaligned(ex.sumsq_in)) || (ex.sumsq_out && misaligned(ex.sumsq_out)))
         return W4A16_ERR_ALIGN;
-    GemvWsExtras ex;
-    ex.residual = residual;
     hipError_t e = launch_gemv_ws(x, w, w_up, y, K, N, static_cast<hipStream_t>(stream), ex);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+// [res1 bf16 E][h bf16 H][sum of squares of res1, one float per 16 columns]
+struct BlockStreamScratch {
+    uint16_t *res1, *h;
+    float *res1_sumsq;
+};
+BlockStreamScratch block_stream_scratch(void *workspace, int E, int H) {
+    char *p = static_cast<char *>(workspace);
+    BlockStreamScratch s;
+    s.res1 = reinterpret_cast<uint16_t *>(p);
+    s.h = reinterpret_cast<uint16_t *>(p + round256((size_t)E * sizeof(uint16_t)));
+    s.res1_sumsq = reinterpret_cast<float *>(p + round256((size_t)E * sizeof(uint16_t)) + round256((size_t)H * sizeof(uint16_t)));
+    return s;
+}
+
+int o_gemv_ffn_stream_impl(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                           const void *wo, const void *wg, const void *wu, const void *wd, uint16_t *y, uint16_t *res1_out,
+                           uint16_t *h_out, float *y_sumsq, int E, int H, int group, void *workspace, size_t workspace_bytes,
+                           void *stream, bool check_only) {
+    if (!attn_out || !x_residual || !ffn_norm_weight || !wo || !wg || !wu || !wd || !y) return W4A16_ERR_NULL;
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    if (E <= 0 || H <= 0 || E % kGroup != 0 || H % kGroup != 0) return W4A16_ERR_SHAPE;
+    if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if ((res1_out && misaligned(res1_out)) || (h_out && misaligned(h_out)) || (y_sumsq && misaligned(y_sumsq))) return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_block_stream_workspace_bytes(E, H)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    if (check_only) return W4A16_OK;
+    const BlockStreamScratch sc = block_stream_scratch(workspace, E, H);
+    uint16_t *res1 = res1_out ? res1_out : sc.res1;
+    uint16_t *h = h_out ? h_out : sc.h;
+    // stage 1: res1 = bf16(attn_out . Wo + x_residual), leaving sum(res1^2) per tile for the norm of stage 2
+    GemvWsExtras s1;
+    s1.residual = x_residual;
+    s1.sumsq_out = sc.res1_sumsq;
+    int rc = gemv_stream_call(attn_out, wo, nullptr, res1, E, E, group, stream, s1);
+    if (rc) return rc;
+    // stage 2: h = swiglu(rms_norm(res1) . Wgate, rms_norm(res1) . Wup)
+    GemvWsExtras s2;
+    s2.norm_w = ffn_norm_weight;
+    s2.eps = eps;
+    s2.sumsq_in = sc.res1_sumsq;
+    s2.sumsq_n = E / kWsTileCols;
+    rc = gemv_stream_call(res1, wg, wu, h, E, H, group, stream, s2);
+    if (rc) return rc;
+    // stage 3: y = bf16(h . Wdown + res1)
+    GemvWsExtras s3;
+    s3.residual = res1;
+    s3.sumsq_out = y_sumsq;
+    return gemv_stream_call(h, wd, nullptr, y, H, E, group, stream, s3);
 }
 }  // namespace
 
 int w4a16_gemv_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int K, int N, int group, void *stream) {
-    return gemv_stream_impl(x, wstream, nullptr, nullptr, false, y, K, N, group, stream);
+    return gemv_stream_call(x, wstream, nullptr, y, K, N, group, stream, GemvWsExtras());
 }
 
 int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int K, int N,
                                int group, void *stream) {
-    return gemv_stream_impl(x, wstream, nullptr, residual, true, y, K, N, group, stream);
+    if (!residual) return W4A16_ERR_NULL;
+    GemvWsExtras ex;
+    ex.residual = residual;
+    return gemv_stream_call(x, wstream, nullptr, y, K, N, group, stream, ex);
 }
 
 int w4a16_gemv_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream, uint16_t *h, int K,
                                   int H, int group, void *stream) {
     if (!up_wstream) return W4A16_ERR_NULL;
-    return gemv_stream_impl(x, gate_wstream, up_wstream, nullptr, false, h, K, H, group, stream);
+    return gemv_stream_call(x, gate_wstream, up_wstream, h, K, H, group, stream, GemvWsExtras());
+}
+
+int w4a16_rms_gemv_stream_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
+                               const void *wstream, uint16_t *y, int K, int N, int group, void *stream) {
+    if (!norm_weight) return W4A16_ERR_NULL;
+    GemvWsExtras ex;
+    ex.norm_w = norm_weight;
+    ex.eps = eps;
+    ex.sumsq_in = x_sumsq;
+    ex.sumsq_n = x_sumsq ? n_pieces : 0;
+    return gemv_stream_call(x, wstream, nullptr, y, K, N, group, stream, ex);
+}
+
+int w4a16_rms_gemv_swiglu_stream_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const void *gate_wstream,
+                                      const void *up_wstream, uint16_t *h, int K, int H, int group, void *stream) {
+    if (!norm_weight || !up_wstream) return W4A16_ERR_NULL;
+    GemvWsExtras ex;
+    ex.norm_w = norm_weight;
+    ex.eps = eps;
+    return gemv_stream_call(x, gate_wstream, up_wstream, h, K, H, group, stream, ex);
+}
+
+int w4a16_ffn_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream, const void *down_wstream,
+                                 uint16_t *y, uint16_t *h, int K, int H, int group, void *stream) {
+    if (!up_wstream || !down_wstream || !h) return W4A16_ERR_NULL;
+    if (H <= 0 || H % kGroup != 0) return W4A16_ERR_SHAPE;
+    int rc = gemv_stream_call(x, gate_wstream, up_wstream, h, K, H, group, stream, GemvWsExtras());
+    if (rc) return rc;
+    return gemv_stream_call(h, down_wstream, nullptr, y, H, K, group, stream, GemvWsExtras());
+}
+
+size_t w4a16_block_stream_workspace_bytes(int E, int H) {
+    if (E <= 0 || H <= 0) return 0;
+    return round256((size_t)E * sizeof(uint16_t)) + round256((size_t)H * sizeof(uint16_t)) +
+           round256((size_t)(E / kWsTileCols + 1) * sizeof(float));
+}
+
+int w4a16_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                                 float eps, const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                 const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, float *y_sumsq,
+                                 int E, int H, int group, void *workspace, size_t workspace_bytes, void *stream) {
+    return o_gemv_ffn_stream_impl(attn_out, x_residual, ffn_norm_weight, eps, o_wstream, gate_wstream, up_wstream, down_wstream,
+                                  y, res1_out, h_out, y_sumsq, E, H, group, workspace, workspace_bytes, stream, false);
+}
+
+int w4a16_decode_attn_o_gemv_ffn_stream_bf16(const uint16_t *qkv, const uint16_t *rope_lut_row, uint16_t *k_cache,
+                                             uint16_t *v_cache, uint16_t *attn_out, int pos, int max_seq, int n_heads,
+                                             int n_kv_heads, int head_dim, void *attn_workspace, size_t attn_workspace_bytes,
+                                             const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                                             const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                             const void *down_wstream, uint16_t *y, float *y_sumsq, int E, int H, int group,
+                                             void *workspace, size_t workspace_bytes, void *stream) {
+    if (n_heads <= 0 || head_dim <= 0 || n_heads * head_dim != E) return W4A16_ERR_SHAPE;
+    int rc = o_gemv_ffn_stream_impl(attn_out, x_residual, ffn_norm_weight, eps, o_wstream, gate_wstream, up_wstream,
+                                    down_wstream, y, nullptr, nullptr, y_sumsq, E, H, group, workspace, workspace_bytes, stream,
+                                    true);
+    if (rc) return rc;
+    rc = w4a16_decode_attention_bf16(qkv, rope_lut_row, k_cache, v_cache, attn_out, pos, max_seq, n_heads, n_kv_heads, head_dim,
+                                     attn_workspace, attn_workspace_bytes, stream);
+    if (rc) return rc;
+    return o_gemv_ffn_stream_impl(attn_out, x_residual, ffn_norm_weight, eps, o_wstream, gate_wstream, up_wstream, down_wstream,
+                                  y, nullptr, nullptr, y_sumsq, E, H, group, workspace, workspace_bytes, stream, false);
 }
 
 size_t w4a16_block_workspace_bytes(int E, int H) {

@@ -46,13 +46,38 @@ __device__ __forceinline__ bf16x8 cell_operand(uint32_t w, uint32_t nib_mask, ui
     return __builtin_bit_cast(bf16x8, b);
 }
 
+// Arguments that only some launches read; they follow the ones every wave needs at once, which fit the SGPRs
+// that arrive with the wave.
+struct GemvWsTail {
+    const uint16_t *norm_w;    // RMS: bf16 [K]
+    const float *sumsq_in;     // RMS: partial sums of x^2 left by the launch that produced x, or null (the wave walks x)
+    float *sumsq_out;          // sum of squares of this launch's bf16 outputs, one float per 16-column tile, or null
+    float eps;
+    int sumsq_n;
+    int K;
+};
+
+// a0 += sum of squares of the low bf16 halves of v, a1 += of the high halves
+__device__ __forceinline__ void sumsq8(const u32x4 v, float &a0, float &a1) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = __builtin_bit_cast(float, v[j] << 16);
+        const float hi = __builtin_bit_cast(float, v[j] & 0xFFFF0000u);
+        a0 = fmaf(lo, lo, a0);
+        a1 = fmaf(hi, hi, a1);
+    }
+}
+
 // CT   cells per task (4, 8 or 16)
 // NMAT 1, or 2: gate and up matrices with the SwiGLU epilogue h = bf16(silu(bf16 g) * bf16 u)
-template <int CT, int NMAT>
+// RMS  x is RMS-normalised on the fly: every wave obtains rstd = 1 / sqrt(mean(x^2) + eps) itself (from the partial
+//      sums the producer of x left behind, else by walking x, which is K bf16 values and L2-resident) and feeds
+//      bf16((x * rstd) * norm_w) to the matrix cores
+template <int CT, int NMAT, bool RMS>
 __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t *__restrict__ x, const char *__restrict__ w0,
                                                                  const char *__restrict__ w1, uint16_t *__restrict__ y,
                                                                  const uint16_t *__restrict__ residual, int G, int NB,
-                                                                 int round_before_add, int nwaves) {
+                                                                 int round_before_add, int nwaves, const GemvWsTail tail) {
     constexpr int SUB = kWsBlockGroups / CT;
     __shared__ float red[NMAT * kMaxWaves * 64];
     const int lane = threadIdx.x & 63;
@@ -73,6 +98,25 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
 #pragma unroll
     for (int m = 0; m < NMAT; ++m) yv[m] = 0.f;
 
+    float rstd = 0.f;
+    if constexpr (RMS) {
+        float a0 = 0.f, a1 = 0.f;
+        if (tail.sumsq_in) {
+            for (int i = lane; i < tail.sumsq_n; i += 64) a0 += tail.sumsq_in[i];
+        } else {
+            const u32x4 *xv = reinterpret_cast<const u32x4 *>(x);
+            const int nchunks = tail.K >> 3;
+            for (int c0 = lane; c0 < nchunks; c0 += 512) {   // 8 loads in flight
+                u32x4 v[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = c0 + 64 * i < nchunks ? xv[c0 + 64 * i] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sumsq8(v[i], a0, a1);
+            }
+        }
+        rstd = 1.0f / sqrtf(wave_reduce<false>(a0 + a1) / (float)tail.K + tail.eps);
+    }
+
     const int tasks_per_mat = NB * SUB;
     for (int task = wave; task < NMAT * tasks_per_mat; task += nwaves) {
         const int mat = NMAT == 1 ? 0 : task / tasks_per_mat;
@@ -88,8 +132,14 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
         const bool xvalid = ln >= r0 && ln < r0 + CT && grow < G;
         const uint16_t *xp = x + (size_t)(xvalid ? grow : 0) * 128 + 8 * lg;
         u32x4 X[4], cell[CT];
+        u32x4 NW[RMS ? 4 : 1];
 #pragma unroll
         for (int t = 0; t < 4; ++t) X[t] = *reinterpret_cast<const u32x4 *>(xp + 32 * t);
+        if constexpr (RMS) {
+            const uint16_t *np = tail.norm_w + (size_t)(xvalid ? grow : 0) * 128 + 8 * lg;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) NW[t] = *reinterpret_cast<const u32x4 *>(np + 32 * t);
+        }
         // scales / zero points next: they sit right in front of the cells (requested after the cells instead: +0.5 us)
         const u32x4 md = *(reinterpret_cast<const u32x4 *>(blk) + lane);
 #pragma unroll
@@ -100,6 +150,17 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
         // every load of the task is requested before the first wait
         __builtin_amdgcn_sched_barrier(0);
 
+        if constexpr (RMS) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float x_lo = __builtin_bit_cast(float, X[t][j] << 16), x_hi = __builtin_bit_cast(float, X[t][j] & 0xFFFF0000u);
+                    const float w_lo = __builtin_bit_cast(float, NW[t][j] << 16), w_hi = __builtin_bit_cast(float, NW[t][j] & 0xFFFF0000u);
+                    X[t][j] = pack_bf16x2((x_lo * rstd) * w_lo, (x_hi * rstd) * w_hi);
+                }
+            }
+        }
         if (!xvalid) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) X[t] = u32x4{0u, 0u, 0u, 0u};
@@ -156,7 +217,15 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
             if (round_before_add) out = bf16_bits_to_float(float_to_bf16_bits(out));
             out += bf16_bits_to_float(residual[col]);
         }
-        y[col] = float_to_bf16_bits(out);
+        const uint16_t ob = float_to_bf16_bits(out);
+        y[col] = ob;
+        if (tail.sumsq_out) {   // the 16 outputs of the tile as the next RMSNorm will read them
+            const float r = bf16_bits_to_float(ob);
+            float sq = r * r;
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+            if (threadIdx.x == 0) tail.sumsq_out[tile] = sq;
+        }
     }
 }
 
@@ -200,12 +269,19 @@ hipError_t launch_ct(int nmat, int waves, const uint16_t *x, const void *w0, con
                      const GemvWsExtras &ex, hipStream_t stream) {
     const int G = K / kGroup, NB = ws_blocks(K);
     const dim3 grid(N / kWsTileCols), block(waves * 64);
-    if (nmat == 2)
-        hipLaunchKernelGGL((gemv_ws_kernel<CT, 2>), grid, block, 0, stream, x, static_cast<const char *>(w0),
-                           static_cast<const char *>(w1), y, ex.residual, G, NB, ex.round_before_add, waves);
-    else
-        hipLaunchKernelGGL((gemv_ws_kernel<CT, 1>), grid, block, 0, stream, x, static_cast<const char *>(w0),
-                           static_cast<const char *>(w0), y, ex.residual, G, NB, ex.round_before_add, waves);
+    const GemvWsTail tail = {ex.norm_w, ex.sumsq_in, ex.sumsq_out, ex.eps, ex.sumsq_n, K};
+    const char *a = static_cast<const char *>(w0), *b = static_cast<const char *>(w1 ? w1 : w0);
+#define W4A16_GEMV_WS_LAUNCH(NMAT, RMS)                                                                               \
+    hipLaunchKernelGGL((gemv_ws_kernel<CT, NMAT, RMS>), grid, block, 0, stream, x, a, b, y, ex.residual, G, NB,      \
+                       ex.round_before_add, waves, tail)
+    if (ex.norm_w) {
+        if (nmat == 2) W4A16_GEMV_WS_LAUNCH(2, true);
+        else W4A16_GEMV_WS_LAUNCH(1, true);
+    } else {
+        if (nmat == 2) W4A16_GEMV_WS_LAUNCH(2, false);
+        else W4A16_GEMV_WS_LAUNCH(1, false);
+    }
+#undef W4A16_GEMV_WS_LAUNCH
     return hipGetLastError();
 }
 

@@ -94,6 +94,14 @@ hipError_t launch_fill_workspace(void *ptr, size_t bytes, hipStream_t stream);
 struct GemvWsExtras {
     const uint16_t *residual = nullptr;   // [N] bf16 added to the result before the final rounding
     int round_before_add = 0;             // 1: y = bf16(bf16(x.W) + R) instead of bf16(x.W + R)
+    const uint16_t *norm_w = nullptr;     // [K] bf16: x is replaced by bf16((x * rstd) * norm_w)
+    float eps = 1e-5f;
+    // A launch with `sumsq_out` leaves the sum of squares of its (rounded) outputs there, one float per
+    // 16-column tile (N / 16 floats); a following RMS launch on that vector passes them as `sumsq_in`
+    // (`sumsq_n` pieces) and skips its own pass over x.
+    const float *sumsq_in = nullptr;
+    int sumsq_n = 0;
+    float *sumsq_out = nullptr;
 };
 struct GemvWsTune {
     int ct = 0;      // cells (groups) per task: 4, 8 or 16 (0 = default)
