@@ -197,6 +197,21 @@ def w4a16_gemv_stream(x, w, residual=None, group=GROUP, out=None):
     return out
 
 
+def w4a16_gemm_stream(x, w, group=GROUP, out=None):
+    """y[M, N] = bf16(x[M, K] . W) on a StreamWeight; x may be a vector [K]."""
+    lib = _lib.load_library()
+    _need_cuda(x, w.buf)
+    vec = x.dim() == 1
+    x2 = x.unsqueeze(0) if vec else x
+    M, K = x2.shape
+    if K != w.K:
+        raise ValueError(f"x has K={K} but the matrix has {w.K} rows")
+    if out is None:
+        out = torch.empty((M, w.N), dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.w4a16_gemm_stream_bf16(_ptr(_bits(x2)), _ptr(w.buf), _ptr(out), M, K, w.N, group, _stream()))
+    return out.squeeze(0) if vec else out
+
+
 def w4a16_swiglu_stream(x, gate, up, group=GROUP, out=None):
     """Decode FFN front half on two StreamWeights: h[H] = bf16(silu(bf16(x Wg)) * bf16(x Wu))."""
     lib = _lib.load_library()

@@ -541,6 +541,16 @@ int w4a16_gemv_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, 
     return gemv_stream_call(x, wstream, nullptr, y, K, N, group, stream, GemvWsExtras());
 }
 
+int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int M, int K, int N, int group, void *stream) {
+    if (M == 1) return gemv_stream_call(x, wstream, nullptr, y, K, N, group, stream, GemvWsExtras());
+    if (!x || !wstream || !y) return W4A16_ERR_NULL;
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    if (M <= 0 || K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(wstream) || misaligned(y)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_gemm_ws(x, wstream, y, nullptr, M, K, N, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int K, int N,
                                int group, void *stream) {
     if (!residual) return W4A16_ERR_NULL;
@@ -890,6 +900,9 @@ int w4a16_tune(const char *key, int value) {
     } else if (!strcmp(key, "gemv_ws_ct")) {
         if (value != 0 && value != 4 && value != 8 && value != 16) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.ct = value;
+    } else if (!strcmp(key, "gemm_ws_cb")) {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return W4A16_ERR_TUNE;
+        g_gemv_ws_tune.cb = value;
     } else if (!strcmp(key, "gemv_ws_waves")) {
         if (value > 16) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.waves = value;

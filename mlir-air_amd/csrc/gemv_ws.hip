@@ -321,3 +321,146 @@ hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const
 }
 
 }  // namespace w4a16
+
+// ---- batched decode, 2 <= M <= 16, on the same layout ------------------------------------------------------------
+//
+// The 16 rows of the A operand are the rows of x (row m <-> lane ln = m), so a cell's product is the whole
+// [16 x 16] block of y for its 16 columns and the group flush applies to all four accumulator registers.  A workgroup
+// owns CB adjacent tiles (16 CB columns) for all of K, so that the x operands of a group (four gathered loads of
+// 16 rows x 64 bytes) are built once for CB cells; its waves take the groups round-robin, four groups per task with
+// every load of the task (16 of x, 4 CB cells, 4 CB scale words) requested up front.  The waves' [16 x 16 CB] partial
+// sums meet in LDS and leave as bf16.  No workspace, nothing exchanged between workgroups.
+namespace w4a16 {
+namespace {
+
+constexpr int kGemmWsWaves = 8;
+constexpr int kGemmWsGroups = 4;   // groups per task
+
+template <int CB>
+__global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16_t *__restrict__ x, const char *__restrict__ w,
+                                                                    uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
+                                                                    int M, int K, int N, int G, int NB) {
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [wave][cb][reg][lane]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lg = lane >> 4, ln = lane & 15;
+    const size_t tile_bytes = (size_t)(NB + G) * kWsCellBytes;
+    const char *tile0 = w + (size_t)blockIdx.x * CB * tile_bytes;
+
+    const uint32_t ones_w = 0x3F803F80u;
+    const u32x4 ones4 = {ones_w, ones_w, ones_w, ones_w};
+    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones4);
+    uint32_t nib_mask = 0x000F000Fu, magic = 0x43004300u;
+    asm volatile("" : "+s"(nib_mask));
+    asm volatile("" : "+v"(magic));
+
+    floatx4 Y[CB];
+#pragma unroll
+    for (int c = 0; c < CB; ++c) Y[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const bool row_valid = ln < M;
+    const uint16_t *xrow = x + (size_t)(row_valid ? ln : 0) * K + 8 * lg;
+    const int ntasks = (G + kGemmWsGroups - 1) / kGemmWsGroups;
+    for (int task = wave; task < ntasks; task += kGemmWsWaves) {
+        const int g0 = task * kGemmWsGroups;
+        u32x4 X[kGemmWsGroups][4], cell[kGemmWsGroups][CB];
+        uint32_t md[kGemmWsGroups][CB];
+#pragma unroll
+        for (int j = 0; j < kGemmWsGroups; ++j) {
+            const int g = g0 + j < G ? g0 + j : G - 1;   // a short last task re-reads the last group (its x is zeroed below)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) X[j][t] = *reinterpret_cast<const u32x4 *>(xrow + 128 * g + 32 * t);
+        }
+#pragma unroll
+        for (int j = 0; j < kGemmWsGroups; ++j) {
+            const int g = g0 + j < G ? g0 + j : G - 1;
+            const int b = g >> 4, gl = g & 15;
+            const char *blk = tile0 + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes);
+            // the scale word of (group g, column ln) sits in lane 16 (gl / 4) + ln, dword gl % 4 of the block's first KiB
+            // (one 16-byte load per tile for the task's four groups needs 3 more registers per tile at the 256 limit
+            // and spills: 10.6 -> 14.0 us at M = 16, K = 4096, N = 14336)
+#pragma unroll
+            for (int c = 0; c < CB; ++c)
+                md[j][c] = *reinterpret_cast<const uint32_t *>(blk + (size_t)c * tile_bytes + (16 * (gl >> 2) + ln) * 16 + 4 * (gl & 3));
+#pragma unroll
+            for (int c = 0; c < CB; ++c)
+                cell[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)c * tile_bytes + (size_t)(1 + gl) * kWsCellBytes) + lane);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < kGemmWsGroups; ++j) {
+            const bool valid = row_valid && g0 + j < G;
+            floatx4 xs = {0.f, 0.f, 0.f, 0.f};   // register i: sum of x[4 lg + i] over the group
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                if (!valid) X[j][t] = u32x4{0u, 0u, 0u, 0u};
+                xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[j][t]), ones, xs, 0, 0, 0);
+            }
+#pragma unroll
+            for (int c = 0; c < CB; ++c) {
+                floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[j][t]),
+                                                                  cell_operand(cell[j][c][t], nib_mask, magic), acc, 0, 0, 0);
+                const float sf = __builtin_bit_cast(float, md[j][c] << 16);
+                const float nz = __builtin_bit_cast(float, md[j][c] & 0xFFFF0000u);   // -(128 + z)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) Y[c][i] = fmaf(sf, fmaf(nz, xs[i], acc[i]), Y[c][i]);
+            }
+        }
+    }
+
+    // cross-wave sum: red[wave][c][i][lane], then every thread adds the waves for two (row, column) pairs
+#pragma unroll
+    for (int c = 0; c < CB; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[((wave * CB + c) * 4 + i) * 64 + lane] = Y[c][i];
+    __syncthreads();
+    constexpr int PER_WAVE = CB * 4 * 64;
+    for (int e = threadIdx.x; e < PER_WAVE; e += kGemmWsWaves * 64) {
+        // e = (m * CB + c) * 16 + col: consecutive threads write consecutive columns of one row
+        const int col = e & 15, c = (e >> 4) % CB, m = e / (16 * CB);
+        const int src = (c * 4 + (m & 3)) * 64 + 16 * (m >> 2) + col;   // row m lives in lane group m / 4, register m % 4
+        float s = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < kGemmWsWaves; ++wv) s += red[wv * PER_WAVE + src];
+        if (m < M) {
+            const size_t o = (size_t)m * N + (size_t)blockIdx.x * (16 * CB) + 16 * c + col;
+            if (residual) s += bf16_bits_to_float(residual[o]);
+            y[o] = float_to_bf16_bits(s);
+        }
+    }
+}
+
+template <int CB>
+hipError_t launch_gemm_ws_cb(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
+                             hipStream_t stream) {
+    const size_t lds = (size_t)kGemmWsWaves * CB * 4 * 64 * sizeof(float);
+    hipLaunchKernelGGL((gemm_ws_kernel<CB>), dim3(N / (16 * CB)), dim3(kGemmWsWaves * 64), lds, stream, x,
+                       static_cast<const char *>(w), y, residual, M, K, N, K / kGroup, ws_blocks(K));
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// y[M, N] = bf16(x[M, K] . W (+ residual)), 2 <= M <= 16 per launch; more rows run as launches of 16.
+hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
+                          hipStream_t stream) {
+    const int tiles = N / kWsTileCols;
+    int cb = g_gemv_ws_tune.cb;
+    if (!cb) cb = tiles % 4 == 0 && tiles / 4 >= 200 ? 4 : (tiles % 2 == 0 && tiles / 2 >= 200 ? 2 : 1);
+    if (tiles % cb) cb = 1;
+    hipError_t e = hipSuccess;
+    for (int m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
+        const int rows = M - m0 < 16 ? M - m0 : 16;
+        const uint16_t *xr = x + (size_t)m0 * K, *rr = residual ? residual + (size_t)m0 * N : nullptr;
+        uint16_t *yr = y + (size_t)m0 * N;
+        e = cb == 4 ? launch_gemm_ws_cb<4>(xr, w, yr, rr, rows, K, N, stream)
+          : cb == 2 ? launch_gemm_ws_cb<2>(xr, w, yr, rr, rows, K, N, stream)
+                    : launch_gemm_ws_cb<1>(xr, w, yr, rr, rows, K, N, stream);
+    }
+    return e;
+}
+
+}  // namespace w4a16

@@ -106,6 +106,7 @@ struct GemvWsExtras {
 struct GemvWsTune {
     int ct = 0;      // cells (groups) per task: 4, 8 or 16 (0 = default)
     int waves = 0;   // cap on the waves per workgroup (0 = one per task, at most 16)
+    int cb = 0;      // batched kernel: 16-column tiles per workgroup, 1, 2 or 4 (0 = by the number of tiles)
 };
 extern GemvWsTune g_gemv_ws_tune;
 struct GemvWsPlan {
@@ -116,6 +117,9 @@ GemvWsPlan plan_gemv_ws(int K, int nmat);
 // y = bf16(silu(bf16(x.W)) * bf16(x.W_up)).
 hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, uint16_t *y, int K, int N, hipStream_t stream,
                           const GemvWsExtras &extras = GemvWsExtras());
+// y[M, N] = bf16(x[M, K] . W (+ residual [M, N])) with W in stream order, any M >= 2 (launches of up to 16 rows).
+hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
+                          hipStream_t stream);
 // AutoAWQ checkpoint tensors -> stream order (ws_matrix_bytes(K, N) bytes at `out`).
 hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *out, int K, int N,
                             hipStream_t stream);

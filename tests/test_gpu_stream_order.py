@@ -162,3 +162,51 @@ def test_swiglu_stream(ops, K, H):
     assert_bf16_close(bits(h), want, ulps=4.0, atol=2e-3, what=f"swiglu stream K={K} H={H}")
     assert oref.check_outputs(bf16_bits_to_f32(bits(h)), bf16_bits_to_f32(f32_to_bf16_bits(want.astype(np.float32))),
                               rtol=0.15, atol=0.5, min_correlation=0.99)
+
+
+def _gemm_case(ops, M, K, N, seed):
+    print(f"gemm stream M={M} K={K} N={N} seed={seed}", flush=True)
+    qw, qz, s = make_awq(K, N, seed=seed)
+    x = make_x((M, K), seed=seed + 1)
+    y = ops.w4a16_gemm_stream(dev(x), _stream_weight(ops, qw, qz, s))
+    torch.cuda.synchronize()
+    got = bits(y)
+    want = bf16_bits_to_f32(x).astype(np.float64) @ dense_f64(qw, qz, s)
+    assert_bf16_close(got, want, ulps=1.0, atol=2e-3, what=f"gemm stream M={M} K={K} N={N}")
+    assert oref.check_outputs(bf16_bits_to_f32(got), bf16_bits_to_f32(f32_to_bf16_bits(want.astype(np.float32))),
+                              rtol=0.1, atol=0.05, max_mismatch_percentage=0.05, min_correlation=0.999)
+    return got
+
+
+# rows 2..16 and beyond (launches of 16), one / two / four tiles per workgroup (N = 14336 and 6400 pick 4 and 2),
+# K with a short last task (19 groups) and more tasks than waves (K = 14336: 28 tasks on 8 waves)
+@pytest.mark.parametrize("M,K,N", [(2, 128, 16), (3, 256, 544), (7, 1152, 544), (16, 512, 1056), (5, 128 * 19, 48),
+                                   (16, 4096, 6400), (9, 14336, 4096), (40, 1024, 512), (16, 2048, 2048)])
+def test_gemm_stream_shapes(ops, M, K, N):
+    _gemm_case(ops, M, K, N, seed=M + K + N)
+
+
+def test_gemm_stream_config2(ops):
+    _gemm_case(ops, 16, 4096, 14336, seed=2)
+
+
+@pytest.mark.parametrize("cb", [1, 2, 4])
+def test_gemm_stream_tiles_per_workgroup_agree(ops, cb):
+    """The number of tiles a workgroup owns changes nothing about a column's arithmetic: same bits."""
+    base = _gemm_case(ops, 11, 1024, 1024, seed=70)
+    ops.tune("gemm_ws_cb", cb)
+    try:
+        assert np.array_equal(_gemm_case(ops, 11, 1024, 1024, seed=70), base)
+    finally:
+        ops.tune("gemm_ws_cb", 0)
+
+
+def test_gemm_stream_rows_equal_the_gemv_up_to_summation_order(ops):
+    K, N = 2048, 1024
+    qw, qz, s = make_awq(K, N, seed=81)
+    x = make_x((6, K), seed=82)
+    w = _stream_weight(ops, qw, qz, s)
+    y = bf16_bits_to_f32(bits(ops.w4a16_gemm_stream(dev(x), w))).astype(np.float64)
+    for m in range(6):
+        v = bf16_bits_to_f32(bits(ops.w4a16_gemv_stream(dev(x[m]), w))).astype(np.float64)
+        assert np.all(np.abs(y[m] - v) <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(v), 1e-30))) - 7) + 2e-3)
