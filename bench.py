@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm16_awq|prefill|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_1b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_1b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -35,7 +35,8 @@ CONFIGS = {
     "gemv_awq": dict(M=1, K=4096, N=11008, cfg=None, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128, checkpoint-layout weights"),
     "gemm16": dict(M=16, K=4096, N=14336, cfg=2, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128, stream-order weights"),
     "gemm16_awq": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128, checkpoint-layout weights"),
-    "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128"),
+    "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128, stream-order weights"),
+    "prefill_awq": dict(M=2048, K=4096, N=14336, cfg=None, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128, checkpoint-layout weights"),
     "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128, stream-order weights (2 launches)"),
     "ffn_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128, checkpoint-layout weights (persistent kernel)"),
     "block_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode block, checkpoint-layout weights"),
@@ -57,7 +58,7 @@ LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 204
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
 # scaled by the same counter's reading for a 256 MiB device copy: x2.000 and x1.000); the
 # summaries under profiles/ hold the commands and the raw readings.
-MEASURED_TRAFFIC_BYTES = {"gemv": 24.11e6, "gemv_awq": 24.27e6, "prefill": 342.2e6, "ffn_awq": 97.07e6, "lm_head": 525.9e6}
+MEASURED_TRAFFIC_BYTES = {"gemv": 24.11e6, "gemv_awq": 24.27e6, "prefill_awq": 342.2e6, "ffn_awq": 97.07e6, "lm_head": 525.9e6}
 
 
 def weight_bytes(K, N):
@@ -132,13 +133,13 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
 
     q4nx = name.startswith("q4nx")
     lm_head = name == "lm_head"
-    stream_order = name in ("gemv", "gemm16", "ffn", "block", "layer")     # weights re-packed at load time (untimed)
+    stream_order = name in ("gemv", "gemm16", "prefill", "ffn", "block", "layer")     # weights re-packed at load time (untimed)
     kind = name[:-4] if name.endswith("_awq") else name
     per_copy = K * N * 2 if lm_head else q4nx_weight_bytes(K, N) if q4nx else weight_bytes(K, N) * (3 if kind in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if kind in ("block", "layer") else 0)
     nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
     if kind == "layer":
         per_copy += weight_bytes(K, nqkv)
-    if name == "prefill":
+    if kind == "prefill":
         ncopies = 1
     else:
         ncopies = max(2, -(-(MALL_BYTES + MALL_BYTES // 2) // per_copy))
@@ -174,7 +175,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             from air_hip import ops
             if i == 0:
                 awq0 = copies[0]
-            mats = (copies[i],) if kind == "gemm16" else copies[i]
+            mats = (copies[i],) if kind in ("gemm16", "prefill") else copies[i]
             copies[i] = tuple(ops.repack_stream(*m).buf for m in mats)
     gx = torch.Generator(device="cuda")
     gx.manual_seed(7)
@@ -268,7 +269,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                        best.data_ptr(), N, K, lm_ws.data_ptr(), lm_ws.numel(), st)
         elif name == "gemv":
             rc = lib.w4a16_gemv_stream_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), K, N, 128, st)
-        elif name == "gemm16":
+        elif name in ("gemm16", "prefill"):
             rc = lib.w4a16_gemm_stream_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), M, K, N, 128, st)
         elif q4nx:
             rc = lib.w4a16_q4nx_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), None,
@@ -716,7 +717,7 @@ def main():
     main_res = run_workload(a.workload, a.steps, a.warmup, not a.no_cpu_baseline)
     name = a.workload
     sec = main_res["cold_us"] * 1e-6
-    if name == "prefill":
+    if name in ("prefill", "prefill_awq"):
         metric, unit = "W4A16 prefill GEMM TFLOP/s", "TFLOP/s"
         value = main_res["flops"] / sec / 1e12
         roof = {"bound": "mfma", "achieved": value, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -727,9 +728,9 @@ def main():
         roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": value / HBM_PEAK_GBS, "traffic": None}
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
-    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_kernel", "ffn_awq": "ffn_fused_kernel", "lm_head": "lm_head_kernel",
+    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_wsp_kernel", "prefill_awq": "gemm_kernel", "ffn_awq": "ffn_fused_kernel", "lm_head": "lm_head_kernel",
                       "gemv": "gemv_ws_kernel", "gemm16": "gemm_ws_kernel", "ffn": "gemv_ws_kernel", "block": "gemv_ws_kernel", "layer": "gemv_ws_kernel"}.get(name, "stream_kernel")
-    roof["algorithmic_per_launch"] = main_res["flops"] if name == "prefill" else main_res["bytes"]
+    roof["algorithmic_per_launch"] = main_res["flops"] if name in ("prefill", "prefill_awq") else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]
 
     out = {
@@ -753,7 +754,7 @@ def main():
         "per_launch_events_us": main_res["per_launch_events_us"],
         "graph_us_per_step": main_res["graph_us"],
         "hot_cache": {"us_per_step": main_res["hot_us"],
-                      "value": (main_res["flops"] / 1e12 if name == "prefill" else main_res["bytes"] / 1e9) / (main_res["hot_us"] * 1e-6),
+                      "value": (main_res["flops"] / 1e12 if name in ("prefill", "prefill_awq") else main_res["bytes"] / 1e9) / (main_res["hot_us"] * 1e-6),
                       "note": "same buffers every step (Infinity Cache resident for the decode shapes)"},
     }
     if "cpu_baseline" in main_res:
@@ -764,9 +765,9 @@ def main():
         for other in CONFIGS:
             if other == name:
                 continue
-            r = run_workload(other, 20 if other == "prefill" else 100, 5, False)
+            r = run_workload(other, 20 if other.startswith("prefill") else 100, 5, False)
             s = r["cold_us"] * 1e-6
-            if other == "prefill":
+            if other.startswith("prefill"):
                 extra[other] = {"us": r["cold_us"], "TFLOP/s": r["flops"] / s / 1e12,
                                 "frac_mfma_peak": r["flops"] / s / 1e12 / MFMA_BF16_PEAK_TFLOPS}
             else:

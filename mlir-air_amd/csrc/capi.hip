@@ -547,7 +547,12 @@ int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, 
     if (group != kGroup) return W4A16_ERR_GROUP;
     if (M <= 0 || K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
     if (misaligned(x) || misaligned(wstream) || misaligned(y)) return W4A16_ERR_ALIGN;
-    hipError_t e = launch_gemm_ws(x, wstream, y, nullptr, M, K, N, static_cast<hipStream_t>(stream));
+    // up to here the weights are streamed once per 16 rows (exact weights); from here on the tiled kernel that
+    // multiplies bf16-rounded weights (the crossover of the two kernels at K = 4096, N = 14336 is near M = 100)
+    const int prefill_min_m = g_gemv_ws_tune.prefill_min_m > 16 ? g_gemv_ws_tune.prefill_min_m : kStreamMaxM + 1;
+    hipError_t e = M >= prefill_min_m && gemm_prefill_ws_supported(M, K, N)
+                       ? launch_gemm_prefill_ws(x, wstream, y, M, K, N, static_cast<hipStream_t>(stream))
+                       : launch_gemm_ws(x, wstream, y, nullptr, M, K, N, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
@@ -900,6 +905,11 @@ int w4a16_tune(const char *key, int value) {
     } else if (!strcmp(key, "gemv_ws_ct")) {
         if (value != 0 && value != 4 && value != 8 && value != 16) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.ct = value;
+    } else if (!strcmp(key, "prefill_tile")) {
+        if (value > 2) return W4A16_ERR_TUNE;
+        g_gemv_ws_tune.prefill_tile = value;
+    } else if (!strcmp(key, "prefill_min_m")) {
+        g_gemv_ws_tune.prefill_min_m = value;
     } else if (!strcmp(key, "gemm_ws_cb")) {
         if (value != 0 && value != 1 && value != 2 && value != 4) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.cb = value;

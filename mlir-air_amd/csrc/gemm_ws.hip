@@ -1,0 +1,470 @@
+// Prefill W4A16 GEMM on stream-order weights (wstream.h): y[M, N] = bf16(x[M, K] . W), W = bf16_rne((q - z) * s).
+//
+// Compute-bound.  The weights never pass through LDS: a stream-order cell is the B operand of
+// v_mfma_f32_16x16x32_bf16 for four K-steps of 16 columns, so a wave loads the cells of its own columns straight
+// into registers (one 128-bit load per cell and lane), dequantises them there to the bf16 values of the dense
+// dequant, and multiplies.  Only x goes through LDS.
+//
+//   workgroup = 4 waves side by side: 256 rows x 4 * 16 NCB columns; every wave owns all 256 rows (16 row tiles)
+//               and its own 16 NCB columns, so each weight is dequantised exactly once per workgroup and the x
+//               tile is shared.  16 NCB * 4 fp32 accumulators per lane live in AGPRs (NCB = 4: all 256).
+//   K loop    = one quantisation group (128 rows of W) per step: the x tile [256][128] is copied global -> LDS
+//               (global_load_lds_dwordx4, double buffered) while the previous group multiplies; the cells and
+//               scale words of the next group are requested a step ahead; one barrier per group
+//   tiles     = column tiles of two widths in one launch, 256-wide ones first, then 192-wide ones
+//               (pick_widths()): M = 2048, N = 14336 becomes 8 x (32 tiles of 256 + 32 tiles of 192), and each of
+//               the 256 CUs gets one wide and one narrow tile, 1.75 tile times instead of the two full rounds
+//               that 448 tiles of 256 x 256 take.
+//
+// Issue budget (measured with a loop of this kernel's instruction pattern): the MFMA occupies the matrix pipe for
+// 16 cycles and the issue port for 8; a wave issues in order, so exactly two VALU instructions fit behind an
+// MFMA for free, a third costs 4 cycles, and two dependent VALU instructions back to back stall on top of that.
+// Dequantising 8 weights takes 23 instructions, and with 16 row tiles one B operand feeds 16 MFMAs: the 23
+// instructions are cut into 12 slots of two independent instructions (DequantSlots), one slot behind each of the
+// first 12 MFMAs of the previous operand.  With 8 row tiles (2.9 instructions per MFMA) the same loop is bound by
+// the VALU: 128 x 448 tiles measured 288 us against 257 us for 256 x 256 with the same inner loop.
+//
+// Everything in the inner loop is volatile asm: MFMAs with the accumulator tied to one AGPR quad (through the
+// builtin the register allocator gives some MFMAs a destination other than their accumulator input and rotates
+// tiles through spare registers, copies via VGPRs behind s_nop stalls), and the dequant slots, because volatile
+// asm statements keep their source order, which is the only way to hold an exact MFMA / VALU interleaving
+// (scheduling barriers do not stop instruction selection from clustering plain arithmetic).  The compiler does not
+// know these are MFMAs, so the wait states it would insert are the kernel's business: a B operand is complete 4
+// MFMAs before its first use, an accumulator is revisited 16 NCB MFMAs later, and s_nop covers the read of the
+// accumulators after the loop.
+//
+// LDS layout of the x tile: rows of 128 bf16 (256 B, 16 chunks of 16 bytes), chunk c of row r at slot c ^ r % 16.
+// One copy instruction of a wave fills 1 KiB linearly (4 rows); lane l = (row l / 16, slot l % 16) fetches chunk
+// slot ^ row % 16.  The A operand read of K-step t (lane (lg, ln): row 16 rt + ln, chunk 4 t + lg) then touches 16
+// distinct slots over 16 consecutive rows: conflict-free without padding.
+//
+// Dequant in registers: e = w & 0x0F0F0F0F and o = (w >> 4) & 0x0F0F0F0F put the eight nibbles of a dword into bytes,
+// v_cvt_f32_ubyteN converts each, fma(q, s, -z s) equals (q - z) * s exactly ((q - z) has 5 significant bits, s has 8),
+// v_cvt_pk_bf16_f32 rounds once.
+#include <algorithm>
+#include <functional>
+#include <mutex>
+#include <type_traits>
+#include <vector>
+
+#include "common.h"
+#include "kernels.h"
+#include "wstream.h"
+
+namespace w4a16 {
+
+namespace {
+
+constexpr int kPfThreads = 256;
+constexpr int kPfRowTiles = 16;              // row tiles of 16 per wave
+constexpr int kPfRows = 16 * kPfRowTiles;    // rows per workgroup tile
+
+// eight weights of one dword (rows 8 lg .. 8 lg + 7 of the lane's column) as the four registers of a B operand
+__device__ __forceinline__ bf16x8 dequant_operand(uint32_t w, float sf, float c0) {
+    uint32_t e = w & 0x0F0F0F0Fu;          // nibbles 0, 2, 4, 6 -> rows 0, 4, 1, 5
+    uint32_t o = (w >> 4) & 0x0F0F0F0Fu;   // nibbles 1, 3, 5, 7 -> rows 2, 6, 3, 7
+    // kept opaque: the compiler would otherwise fold the masks into one v_bfe_u32 per nibble in front of every
+    // convert (two instructions per weight) instead of the byte-select converts v_cvt_f32_ubyte0..3 (one)
+    asm volatile("" : "+v"(e), "+v"(o));
+    const float k0 = fmaf(static_cast<float>(e & 0xFFu), sf, c0), k4 = fmaf(static_cast<float>((e >> 8) & 0xFFu), sf, c0);
+    const float k1 = fmaf(static_cast<float>((e >> 16) & 0xFFu), sf, c0), k5 = fmaf(static_cast<float>(e >> 24), sf, c0);
+    const float k2 = fmaf(static_cast<float>(o & 0xFFu), sf, c0), k6 = fmaf(static_cast<float>((o >> 8) & 0xFFu), sf, c0);
+    const float k3 = fmaf(static_cast<float>((o >> 16) & 0xFFu), sf, c0), k7 = fmaf(static_cast<float>(o >> 24), sf, c0);
+    const u32x4 b = {pack_bf16x2(k0, k1), pack_bf16x2(k2, k3), pack_bf16x2(k4, k5), pack_bf16x2(k6, k7)};
+    return __builtin_bit_cast(bf16x8, b);
+}
+
+// Four MFMAs of one B operand (row tiles 4 Q .. 4 Q + 3) with, behind each of them, one slot of the NEXT operand's
+// dequant: dequant_operand cut into 12 slots of two instructions that do not depend on each other (quarters 0..2;
+// quarter 3 is MFMAs only).  Two temporaries per parity (a: registers 0 and 2 of the operand, b: 1 and 3) let the
+// converts of one register pair overlap the fmas of the other.  One asm statement per quarter: between separate
+// asm statements that pass a register on the compiler inserts an s_nop, and with one wave per SIMD every
+// instruction, s_nop included, takes one of the four issue slots of an MFMA.
+struct DequantSlots {
+    uint32_t w;
+    float sf, c0;
+    uint32_t e, o;
+    float a0, a1, b0, b1;
+    uint32_t p0, p1, p2, p3;
+    __device__ __forceinline__ bf16x8 operand() const { return __builtin_bit_cast(bf16x8, u32x4{p0, p1, p2, p3}); }
+};
+
+#define PF_MFMA(c, a, b) "v_mfma_f32_16x16x32_bf16 %" #c ", %" #a ", %" #b ", %" #c "\n\t"
+
+template <int Q>
+__device__ __forceinline__ void mfma_quarter(floatx4 &c0, floatx4 &c1, floatx4 &c2, floatx4 &c3, const bf16x8 &a0, const bf16x8 &a1,
+                                             const bf16x8 &a2, const bf16x8 &a3, const bf16x8 &b, DequantSlots &d) {
+    if constexpr (Q == 3) {
+        asm volatile(PF_MFMA(0, 4, 8) PF_MFMA(1, 5, 8) PF_MFMA(2, 6, 8) "v_mfma_f32_16x16x32_bf16 %3, %7, %8, %3"
+                     : "+a"(c0), "+a"(c1), "+a"(c2), "+a"(c3)
+                     : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b));
+    } else if constexpr (Q == 0) {
+        // %4 e, %5 o, %6 a0, %7 a1, %8 b0 | %9..%12 A, %13 B, %14 w, %15 s, %16 -z s
+        asm volatile(PF_MFMA(0, 9, 13) "v_and_b32 %4, 0x0f0f0f0f, %14\n\tv_lshrrev_b32 %5, 4, %14\n\t"
+                     PF_MFMA(1, 10, 13) "v_and_b32 %5, 0x0f0f0f0f, %5\n\tv_cvt_f32_ubyte0 %6, %4\n\t"
+                     PF_MFMA(2, 11, 13) "v_cvt_f32_ubyte2 %7, %4\n\tv_fma_f32 %6, %6, %15, %16\n\t"
+                     PF_MFMA(3, 12, 13) "v_fma_f32 %7, %7, %15, %16\n\tv_cvt_f32_ubyte0 %8, %5"
+                     : "+a"(c0), "+a"(c1), "+a"(c2), "+a"(c3), "=&v"(d.e), "=&v"(d.o), "=&v"(d.a0), "=&v"(d.a1), "=&v"(d.b0)
+                     : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b), "v"(d.w), "v"(d.sf), "v"(d.c0));
+    } else if constexpr (Q == 1) {
+        // %4 a0, %5 a1, %6 b0, %7 b1, %8 p0, %9 p1 | %10..%13 A, %14 B, %15 e, %16 o, %17 s, %18 -z s
+        asm volatile(PF_MFMA(0, 10, 14) "v_cvt_pk_bf16_f32 %8, %4, %5\n\tv_cvt_f32_ubyte2 %7, %16\n\t"
+                     PF_MFMA(1, 11, 14) "v_fma_f32 %6, %6, %17, %18\n\tv_fma_f32 %7, %7, %17, %18\n\t"
+                     PF_MFMA(2, 12, 14) "v_cvt_pk_bf16_f32 %9, %6, %7\n\tv_cvt_f32_ubyte1 %4, %15\n\t"
+                     PF_MFMA(3, 13, 14) "v_cvt_f32_ubyte3 %5, %15\n\tv_fma_f32 %4, %4, %17, %18"
+                     : "+a"(c0), "+a"(c1), "+a"(c2), "+a"(c3), "+v"(d.a0), "+v"(d.a1), "+v"(d.b0), "=&v"(d.b1), "=&v"(d.p0), "=&v"(d.p1)
+                     : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b), "v"(d.e), "v"(d.o), "v"(d.sf), "v"(d.c0));
+    } else {
+        // %4 a1, %5 b0, %6 b1, %7 p2, %8 p3 | %9..%12 A, %13 B, %14 a0, %15 o, %16 s, %17 -z s
+        asm volatile(PF_MFMA(0, 9, 13) "v_fma_f32 %4, %4, %16, %17\n\tv_cvt_f32_ubyte1 %5, %15\n\t"
+                     PF_MFMA(1, 10, 13) "v_cvt_pk_bf16_f32 %7, %14, %4\n\tv_cvt_f32_ubyte3 %6, %15\n\t"
+                     PF_MFMA(2, 11, 13) "v_fma_f32 %5, %5, %16, %17\n\tv_fma_f32 %6, %6, %16, %17\n\t"
+                     PF_MFMA(3, 12, 13) "v_cvt_pk_bf16_f32 %8, %5, %6"
+                     : "+a"(c0), "+a"(c1), "+a"(c2), "+a"(c3), "+v"(d.a1), "=&v"(d.b0), "=&v"(d.b1), "=&v"(d.p2), "=&v"(d.p3)
+                     : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b), "v"(d.a0), "v"(d.o), "v"(d.sf), "v"(d.c0));
+    }
+}
+
+// A wave-uniform pointer pinned to scalar registers: the loads below then take the form "scalar base + 32-bit lane
+// offset" and the per-lane part stays one loop-invariant VGPR (left alone the compiler folds the lane offset into
+// a 64-bit VGPR base per stream and spends two VGPRs and a 64-bit add on every request).
+using gptr = const __attribute__((address_space(1))) char *;
+__device__ __forceinline__ gptr scalar_ptr(const char *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    asm volatile("" : "+s"(lo), "+s"(hi));
+    return reinterpret_cast<gptr>(((uint64_t)hi << 32) | lo);
+}
+
+// scale word -> scale s and -z * s (exact: (128 + z) - 128 and an 8 x 8 bit product)
+__device__ __forceinline__ void decode_md(uint32_t md, float &sf, float &c0) {
+    sf = __builtin_bit_cast(float, md << 16);
+    const float nz = __builtin_bit_cast(float, md & 0xFFFF0000u);   // -(128 + z)
+    c0 = (nz + 128.0f) * sf;
+}
+
+struct PfArgs {
+    const uint16_t *x;
+    const char *w;
+    uint16_t *y;
+    int M, K, N, G, NB;
+    int tiles_m;
+    int n_wide, n_narrow;   // column tiles of each width
+};
+
+// One output tile: rows m0 .., columns col0 .. col0 + 64 NCB - 1.
+template <int NCB>
+__device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int m0, int col0) {
+    constexpr int RT = kPfRowTiles, TM = kPfRows, WN = 16 * NCB, TN = 4 * WN;
+    constexpr int kStageBytes = TM * 256;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lg = lane >> 4, ln = lane & 15;
+    const int M = p.M, K = p.K, N = p.N, G = p.G;
+    const int n0 = col0 + wave * WN;
+
+    // x tile copy: instruction i of wave w fills rows 4 (4 i + w) .. + 3 of the stage
+    const int c_row = lane >> 4, c_slot = lane & 15;
+    uint32_t a_voff[RT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) {
+        int row = 4 * (4 * i + wave) + c_row;
+        const int chunk = c_slot ^ (row & 15);
+        if (m0 + row >= M) row = M - 1 - m0;   // ragged M: copy a row in range, never stored
+        a_voff[i] = (uint32_t)((size_t)row * K * sizeof(uint16_t) + chunk * 16);
+    }
+    const char *a_base = reinterpret_cast<const char *>(p.x + (size_t)m0 * K);
+    auto copy_x = [&](int stage, int g) {
+        const gptr src = scalar_ptr(a_base + (size_t)g * 256);
+#pragma unroll
+        for (int i = 0; i < RT; ++i) {
+            // the zero extension must sit next to the request for it to fold into the instruction's 32-bit offset
+            asm volatile("" : "+v"(a_voff[i]));
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + a_voff[i]),
+                                             (__attribute__((address_space(3))) void *)(lds + stage * kStageBytes + (4 * i + wave) * 1024),
+                                             16, 0, 0);
+        }
+    };
+
+    // this wave's NCB tiles of the stream-order buffer
+    const size_t tile_bytes = (size_t)(p.NB + G) * kWsCellBytes;
+    const char *wt = p.w + (size_t)(n0 / kWsTileCols) * tile_bytes;
+    u32x4 cell[2][NCB];
+    uint32_t md[2][NCB];
+    uint32_t lane16 = (uint32_t)lane * 16, ln16 = (uint32_t)ln * 16;
+    auto load_w = [&](int set, int g) {
+        const int gl = g & 15;
+        const char *blk = wt + (size_t)(g >> 4) * ((kWsBlockGroups + 1) * kWsCellBytes);
+        asm volatile("" : "+v"(lane16), "+v"(ln16));
+#pragma unroll
+        for (int c = 0; c < NCB; ++c) {
+            // scale word of (group g, column ln): lane 16 (gl / 4) + ln, dword gl % 4 of the block's first KiB
+            const gptr tc = scalar_ptr(blk + (size_t)c * tile_bytes);
+            md[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(tc + (256 * (gl >> 2) + 4 * (gl & 3)) + ln16);
+            cell[set][c] = __builtin_nontemporal_load(
+                reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(tc + (size_t)(1 + gl) * kWsCellBytes + lane16));
+        }
+    };
+    // The compiler does not see the explicit s_waitcnt below: with loads in flight it would wait for vmcnt(0) at the
+    // first use of a register loaded a group earlier, i.e. right behind the requests for the next group, and expose
+    // their whole latency.  Taking the registers over right behind the explicit wait puts the compiler's wait where
+    // the counter is already zero.
+    auto take_w = [&](int set) {
+#pragma unroll
+        for (int c = 0; c < NCB; ++c) {
+            asm volatile("" : "+v"(md[set][c]));
+#pragma unroll
+            for (int t = 0; t < 4; ++t) asm volatile("" : "+v"(cell[set][c][t]));
+        }
+    };
+
+    floatx4 acc[RT][NCB];
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int c = 0; c < NCB; ++c) acc[r][c] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // per-lane LDS byte offsets of the A operand of row tile 0
+    // of each (stage, K-step); the row tile is the instruction's offset field
+    uint32_t a_addr[2][4];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            a_addr[st][t] = (uint32_t)(st * kStageBytes + ln * 256 + (((4 * t + lg) ^ ln) << 4));
+            asm volatile("" : "+v"(a_addr[st][t]));   // kept in a register: recomputing it costs issue slots in the loop
+        }
+    auto read_a = [&](int stage, int t, int r) {
+        return *reinterpret_cast<const bf16x8 *>(lds + a_addr[stage][t] + r * 4096);
+    };
+
+    // State carried from group to group: the A operands of K-step 0, the first B operand, the decoded scale words.
+    bf16x8 a[RT];
+    bf16x8 b_cur;
+    float sf[NCB], c0[NCB];
+
+    // One quantisation group, software-pipelined over (K-step t, tile c, row tile r): behind MFMA r of one B operand
+    // sits slot r of the next operand's dequant; on the last tile of a K-step every A operand is refilled from LDS
+    // for the next K-step right behind its last MFMA, 16 MFMAs ahead of its first use.  The last tile of the group
+    // prepares the next group the same way (its x tile and cells were requested at the top of this group and are
+    // waited for just before that tile), so the groups follow each other without a bubble.
+    //
+    // The step after the last one has nothing to request, and that is the only difference: it still prepares a "next
+    // group" from whatever the registers and the other stage hold, and nobody uses it.  One copy of the code for all
+    // groups matters: the accumulators must stay in the same AGPRs from the first MFMA to the last, and in a second
+    // copy of the loop body the register allocator moves them, through VGPRs, right behind MFMAs it does not know of.
+    auto group_step = [&](int g, int stage, int set, bool request_next) {
+        if (request_next) {
+            copy_x(stage ^ 1, g + 1);
+            load_w(set ^ 1, g + 1);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+#pragma unroll
+            for (int c = 0; c < NCB; ++c) {
+                const bool last = t == 3 && c == NCB - 1;
+                const int cn = c + 1 < NCB ? c + 1 : 0, tn = c + 1 < NCB ? t : (t + 1) & 3;
+                if (last) {
+                    // The next group's x tile and cells have landed.  Every wave has consumed its LDS reads of this
+                    // stage (those of K-step 3 were issued during K-step 2), so after the barrier the other stage is
+                    // complete and this one may be overwritten at the top of the next group.
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    __syncthreads();
+                    take_w(set ^ 1);
+                    decode_md(md[set ^ 1][0], sf[0], c0[0]);
+                }
+                DequantSlots dq;
+                dq.w = last ? cell[set ^ 1][0][0] : cell[set][cn][tn];
+                dq.sf = sf[cn];
+                dq.c0 = c0[cn];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    const int r = 4 * q;
+                    auto quarter = [&](auto Q) {
+                        mfma_quarter<decltype(Q)::value>(acc[r][c], acc[r + 1][c], acc[r + 2][c], acc[r + 3][c], a[r], a[r + 1], a[r + 2], a[r + 3], b_cur, dq);
+                    };
+                    if (q == 0) quarter(std::integral_constant<int, 0>{});
+                    else if (q == 1) quarter(std::integral_constant<int, 1>{});
+                    else if (q == 2) quarter(std::integral_constant<int, 2>{});
+                    else quarter(std::integral_constant<int, 3>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (c == NCB - 1) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            if (t < 3) a[r + k] = read_a(stage, t + 1, r + k);
+                            else a[r + k] = read_a(stage ^ 1, 0, r + k);
+                        }
+                    }
+                    // scale words of the next group's other tiles, behind the last quarter of the group
+                    if (last && q == 3) {
+#pragma unroll
+                        for (int k = 1; k < NCB; ++k) decode_md(md[set ^ 1][k], sf[k], c0[k]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                b_cur = dq.operand();
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    copy_x(0, 0);
+    load_w(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the x tile copy writes LDS behind the compiler's back
+    __syncthreads();
+    take_w(0);
+#pragma unroll
+    for (int c = 0; c < NCB; ++c) decode_md(md[0][c], sf[c], c0[c]);
+#pragma unroll
+    for (int r = 0; r < RT; ++r) a[r] = read_a(0, 0, r);
+    b_cur = dequant_operand(cell[0][0][0], sf[0], c0[0]);
+
+    // two groups per trip (G is even): stage / register set 0, then 1
+    for (int g = 0; g < G; g += 2) {
+        group_step(g, 0, 0, true);
+        group_step(g + 1, 1, 1, g + 2 < G);
+    }
+
+    // The bf16 tile leaves through LDS (the K loop is done with it): a lane holds 4 rows of one column, so stores
+    // straight from the registers would be 2-byte stores in 32-byte runs; rows padded by 16 bytes, read back as
+    // 16-byte chunks so that a wave instruction stores whole rows.
+    constexpr int LDC = TN + 8;   // bf16 elements per padded row
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int c = 0; c < NCB; ++c) asm volatile("" : "+a"(acc[r][c]));   // and no read of them moves above that wait
+    __syncthreads();                                      // every wave is done reading the last x tile
+    uint16_t *ct = reinterpret_cast<uint16_t *>(lds);
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int c = 0; c < NCB; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                ct[(16 * r + 4 * lg + i) * LDC + wave * WN + 16 * c + ln] = float_to_bf16_bits(acc[r][c][i]);
+    __syncthreads();
+    constexpr int CPR = TN / 8;   // 16-byte chunks per row
+    for (int chunk = threadIdx.x; chunk < TM * CPR; chunk += kPfThreads) {
+        const int row = chunk / CPR, cc = chunk % CPR;
+        if (m0 + row >= M) continue;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(&ct[row * LDC + 8 * cc]);
+        *reinterpret_cast<u32x4 *>(p.y + (size_t)(m0 + row) * N + col0 + 8 * cc) = v;
+    }
+}
+
+// blockIdx -> tile.  The wide tiles come first in dispatch order, so that the narrow ones fill in behind them.  Each
+// XCD (blockIdx % 8) takes a contiguous range of the tiles of either width with N fastest: the workgroups that run
+// together on an XCD share one x panel in its L2 while the weight panels stream by.
+template <int NW, int NN>
+__global__ void __launch_bounds__(kPfThreads, 1) gemm_wsp_kernel(const PfArgs p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int wide_total = p.tiles_m * p.n_wide, narrow_total = p.tiles_m * p.n_narrow;
+    const int wide_per_xcd = (wide_total + 7) / 8, narrow_per_xcd = (narrow_total + 7) / 8;
+    if (slot < wide_per_xcd) {
+        const int tile = xcd * wide_per_xcd + slot;
+        if (tile >= wide_total) return;
+        pf_tile<NW>(p, lds, (tile / p.n_wide) * kPfRows, (tile % p.n_wide) * 64 * NW);
+    } else if constexpr (NN > 0) {
+        const int tile = xcd * narrow_per_xcd + (slot - wide_per_xcd);
+        if (tile >= narrow_total) return;
+        pf_tile<NN>(p, lds, (tile / p.n_narrow) * kPfRows, p.n_wide * 64 * NW + (tile % p.n_narrow) * 64 * NN);
+    }
+}
+
+// Column tiling of N = 64 U columns into a tiles of 256 and b tiles of 192 (4 a + 3 b = U): the split that finishes
+// first when tiles_m * (a + b) tiles are handed, wide ones first, to `cus` CUs as they fall free (tile time taken
+// as proportional to its width).
+struct Widths {
+    int wide, narrow;
+};
+
+long split_cost(long n_wide_tiles, long n_narrow_tiles, int cus) {
+    // greedy list scheduling of two task sizes, big first, on identical machines: the finishing times after the
+    // wide tiles are 4 q (+ 4 on r machines); every narrow tile goes to the machine that falls free first
+    std::vector<long> load(cus);
+    const long q = n_wide_tiles / cus, r = n_wide_tiles % cus;
+    for (int i = 0; i < cus; ++i) load[i] = 4 * (q + (i < r ? 1 : 0));
+    std::make_heap(load.begin(), load.end(), std::greater<long>());
+    for (long i = 0; i < n_narrow_tiles; ++i) {
+        std::pop_heap(load.begin(), load.end(), std::greater<long>());
+        load.back() += 3;
+        std::push_heap(load.begin(), load.end(), std::greater<long>());
+    }
+    return *std::max_element(load.begin(), load.end());
+}
+
+Widths pick_widths(int tiles_m, int U, int cus) {
+    struct Entry {
+        int tiles_m, U, cus;
+        Widths w;
+    };
+    static std::mutex mu;
+    static Entry cache[8] = {};
+    static int next = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    for (const Entry &e : cache)
+        if (e.U == U && e.tiles_m == tiles_m && e.cus == cus) return e.w;
+    Widths best{-1, -1};
+    long best_cost = -1;
+    for (int a = U / 4; a >= 0; --a) {   // ties go to the split with more wide tiles
+        if ((U - 4 * a) % 3) continue;
+        const int b = (U - 4 * a) / 3;
+        const long cost = split_cost((long)tiles_m * a, (long)tiles_m * b, cus);
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best = Widths{a, b};
+        }
+    }
+    cache[next] = Entry{tiles_m, U, cus, best};
+    next = (next + 1) % 8;
+    return best;
+}
+
+template <int NW, int NN>
+hipError_t launch_wsp(const PfArgs &p, hipStream_t stream) {
+    constexpr size_t kStages = 2 * (size_t)kPfRows * 256, kOut = (size_t)kPfRows * (64 * NW + 8) * sizeof(uint16_t);
+    constexpr size_t kLds = kStages > kOut ? kStages : kOut;
+    static_assert(kLds <= 160 * 1024, "tile does not fit LDS");
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wsp_kernel<NW, NN>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
+    if (e != hipSuccess) return e;
+    const int wide_per_xcd = (p.tiles_m * p.n_wide + 7) / 8, narrow_per_xcd = (p.tiles_m * p.n_narrow + 7) / 8;
+    const int grid = 8 * (wide_per_xcd + narrow_per_xcd);
+    hipLaunchKernelGGL((gemm_wsp_kernel<NW, NN>), dim3(grid), dim3(kPfThreads), kLds, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool gemm_prefill_ws_supported(int M, int K, int N) {
+    if (M <= 0 || K <= 0 || K % (2 * kGroup) || N % 64) return false;
+    const int U = N / 64;
+    return U == 3 || U == 4 || U >= 6;   // 4 a + 3 b = U has a solution
+}
+
+hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream) {
+    if (!gemm_prefill_ws_supported(M, K, N)) return hipErrorInvalidValue;
+    PfArgs p{};
+    p.x = x;
+    p.w = static_cast<const char *>(w);
+    p.y = y;
+    p.M = M, p.K = K, p.N = N, p.G = K / kGroup, p.NB = ws_blocks(K);
+    p.tiles_m = (M + kPfRows - 1) / kPfRows;
+    const int U = N / 64;
+    Widths wd = pick_widths(p.tiles_m, U, 256);
+    if (g_gemv_ws_tune.prefill_tile == 1 && U % 4 == 0) wd = Widths{U / 4, 0};   // tuning: 256-wide tiles only
+    if (g_gemv_ws_tune.prefill_tile == 2 && U % 3 == 0) wd = Widths{0, U / 3};   // tuning: 192-wide tiles only
+    p.n_wide = wd.wide, p.n_narrow = wd.narrow;
+    if (wd.wide == 0) {
+        p.n_wide = wd.narrow, p.n_narrow = 0;
+        return launch_wsp<3, 0>(p, stream);
+    }
+    if (wd.narrow == 0) return launch_wsp<4, 0>(p, stream);
+    return launch_wsp<4, 3>(p, stream);
+}
+
+}  // namespace w4a16

@@ -107,6 +107,8 @@ struct GemvWsTune {
     int ct = 0;      // cells (groups) per task: 4, 8 or 16 (0 = default)
     int waves = 0;   // cap on the waves per workgroup (0 = one per task, at most 16)
     int cb = 0;      // batched kernel: 16-column tiles per workgroup, 1, 2 or 4 (0 = by the number of tiles)
+    int prefill_tile = 0;    // prefill kernel: 0 = by shape, 1 = 128 x 448 tiles, 2 = 256 x 256 tiles
+    int prefill_min_m = 0;   // smallest M that w4a16_gemm_stream_bf16 gives to the prefill kernel (0 = default)
 };
 extern GemvWsTune g_gemv_ws_tune;
 struct GemvWsPlan {
@@ -120,6 +122,9 @@ hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, ui
 // y[M, N] = bf16(x[M, K] . W (+ residual [M, N])) with W in stream order, any M >= 2 (launches of up to 16 rows).
 hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
                           hipStream_t stream);
+// Prefill GEMM on stream-order weights (gemm_ws.hip): bf16-rounded weights dequantised in registers, x through LDS.
+bool gemm_prefill_ws_supported(int M, int K, int N);   // N % 448 == 0 or N % 256 == 0
+hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream);
 // AutoAWQ checkpoint tensors -> stream order (ws_matrix_bytes(K, N) bytes at `out`).
 hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *out, int K, int N,
                             hipStream_t stream);

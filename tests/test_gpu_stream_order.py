@@ -210,3 +210,66 @@ def test_gemm_stream_rows_equal_the_gemv_up_to_summation_order(ops):
     for m in range(6):
         v = bf16_bits_to_f32(bits(ops.w4a16_gemv_stream(dev(x[m]), w))).astype(np.float64)
         assert np.all(np.abs(y[m] - v) <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(v), 1e-30))) - 7) + 2e-3)
+
+
+def _prefill_case(ops, M, K, N, seed):
+    """The tiled prefill kernel multiplies bf16-rounded weights W = bf16_rne((q - z) * s): within 1 bf16 ulp of the
+    float64 product on those weights, and inside the reference's gate against the unrounded product
+    (matmul_int4_packed.cpu_reference, matmul_int4_packed.py:89-105: rtol 0.1, atol 0.05, 0.05 % budget, r >= 0.999)."""
+    print(f"prefill stream M={M} K={K} N={N} seed={seed}", flush=True)
+    qw, qz, s = make_awq(K, N, seed=seed)
+    x = make_x((M, K), seed=seed + 1)
+    y = ops.w4a16_gemm_stream(dev(x), _stream_weight(ops, qw, qz, s))
+    torch.cuda.synchronize()
+    got = bits(y)
+    xf = bf16_bits_to_f32(x).astype(np.float64)
+    assert_bf16_close(got, xf @ dense_f64(qw, qz, s, rounded=True), ulps=1.0, atol=2e-3, what=f"prefill stream M={M} K={K} N={N}")
+    want_u = xf @ dense_f64(qw, qz, s)
+    assert oref.check_outputs(bf16_bits_to_f32(got), bf16_bits_to_f32(f32_to_bf16_bits(want_u.astype(np.float32))),
+                              rtol=0.1, atol=0.05, max_mismatch_percentage=0.05, min_correlation=0.999)
+    return got
+
+
+# N = 64 U is cut into 256-wide and 192-wide column tiles (4 a + 3 b = U): wide only (U = 4, 16), narrow only (3, 6),
+# mixed (7, 14, 28), ragged M, one row tile and several, two groups (no steady-state trip of the K loop) and many
+@pytest.mark.parametrize("M,K,N", [(128, 256, 448), (200, 512, 896), (97, 1024, 256), (300, 512, 1024), (512, 2048, 1792),
+                                   (100, 256, 192), (257, 768, 384)])
+def test_prefill_stream_shapes(ops, M, K, N):
+    _prefill_case(ops, M, K, N, seed=M + K + N)
+
+
+@pytest.mark.parametrize("tile,N", [(1, 1024), (2, 768)])
+def test_prefill_stream_forced_tile_width_agrees(ops, tile, N):
+    """The same product through one tile width only (tuning knob) and through the width chosen by shape: same bits
+    (a column's sum does not depend on the tile it sits in)."""
+    want = _prefill_case(ops, 300, 512, N, seed=N)
+    ops.tune("prefill_tile", tile)
+    try:
+        got = _prefill_case(ops, 300, 512, N, seed=N)
+    finally:
+        ops.tune("prefill_tile", 0)
+    assert np.array_equal(got, want)
+
+
+def test_prefill_stream_small_m_through_the_tiled_kernel(ops):
+    ops.tune("prefill_min_m", 17)
+    try:
+        _prefill_case(ops, 17, 256, 448, seed=5)
+        _prefill_case(ops, 40, 512, 512, seed=6)
+    finally:
+        ops.tune("prefill_min_m", 0)
+
+
+def test_prefill_stream_config3(ops):
+    _prefill_case(ops, 2048, 4096, 14336, seed=3)
+
+
+def test_prefill_stream_one_hot_rows_reproduce_the_dequant(ops):
+    """x = e_k in every row k of a 256-row tile: row k of y is the dense dequant's row k bit for bit."""
+    K, N = 256, 448
+    qw, qz, s = make_awq(K, N, seed=9)
+    x = np.zeros((K, K), np.uint16)
+    x[np.arange(K), np.arange(K)] = 0x3F80
+    y = ops.w4a16_gemm_stream(dev(x), _stream_weight(ops, qw, qz, s))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), oawq.dequant_to_bf16(qw, qz, s, 128))
