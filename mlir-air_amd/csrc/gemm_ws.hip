@@ -175,17 +175,15 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
         a_voff[i] = (uint32_t)((size_t)row * K * sizeof(uint16_t) + chunk * 16);
     }
     const char *a_base = reinterpret_cast<const char *>(p.x + (size_t)m0 * K);
-    auto copy_x = [&](int stage, int g) {
-        const gptr src = scalar_ptr(a_base + (size_t)g * 256);
-#pragma unroll
-        for (int i = 0; i < RT; ++i) {
-            // the zero extension must sit next to the request for it to fold into the instruction's 32-bit offset
-            asm volatile("" : "+v"(a_voff[i]));
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + a_voff[i]),
-                                             (__attribute__((address_space(3))) void *)(lds + stage * kStageBytes + (4 * i + wave) * 1024),
-                                             16, 0, 0);
-        }
+    // request i (of 16) of the x tile copy of one group; src = this workgroup's rows at the group's 128 columns
+    auto copy_x_part = [&](int stage, gptr src, int i) {
+        // the zero extension must sit next to the request for it to fold into the instruction's 32-bit offset
+        asm volatile("" : "+v"(a_voff[i]));
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + a_voff[i]),
+                                         (__attribute__((address_space(3))) void *)(lds + stage * kStageBytes + (4 * i + wave) * 1024),
+                                         16, 0, 0);
     };
+    auto x_src = [&](int g) { return scalar_ptr(a_base + (size_t)g * 256); };
 
     // this wave's NCB tiles of the stream-order buffer
     const size_t tile_bytes = (size_t)(p.NB + G) * kWsCellBytes;
@@ -193,18 +191,16 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     u32x4 cell[2][NCB];
     uint32_t md[2][NCB];
     uint32_t lane16 = (uint32_t)lane * 16, ln16 = (uint32_t)ln * 16;
-    auto load_w = [&](int set, int g) {
+    // scale word and cell of tile c for group g: lane 16 (gl / 4) + ln, dword gl % 4 of the block's first KiB, and
+    // the (1 + gl)-th KiB of the block
+    auto load_w_tile = [&](int set, int g, int c) {
         const int gl = g & 15;
         const char *blk = wt + (size_t)(g >> 4) * ((kWsBlockGroups + 1) * kWsCellBytes);
         asm volatile("" : "+v"(lane16), "+v"(ln16));
-#pragma unroll
-        for (int c = 0; c < NCB; ++c) {
-            // scale word of (group g, column ln): lane 16 (gl / 4) + ln, dword gl % 4 of the block's first KiB
-            const gptr tc = scalar_ptr(blk + (size_t)c * tile_bytes);
-            md[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(tc + (256 * (gl >> 2) + 4 * (gl & 3)) + ln16);
-            cell[set][c] = __builtin_nontemporal_load(
-                reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(tc + (size_t)(1 + gl) * kWsCellBytes + lane16));
-        }
+        const gptr tc = scalar_ptr(blk + (size_t)c * tile_bytes);
+        md[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(tc + (256 * (gl >> 2) + 4 * (gl & 3)) + ln16);
+        cell[set][c] = __builtin_nontemporal_load(
+            reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(tc + (size_t)(1 + gl) * kWsCellBytes + lane16));
     };
     // The compiler does not see the explicit s_waitcnt below: with loads in flight it would wait for vmcnt(0) at the
     // first use of a register loaded a group earlier, i.e. right behind the requests for the next group, and expose
@@ -240,40 +236,44 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     };
 
     // State carried from group to group: the A operands of K-step 0, the first B operand, the decoded scale words.
-    bf16x8 a[RT];
+    // The A operands are double buffered: K-step t multiplies from a[t % 2] while a[(t + 1) % 2] is refilled.
+    bf16x8 a[2][RT];
     bf16x8 b_cur;
     float sf[NCB], c0[NCB];
 
-    // One quantisation group, software-pipelined over (K-step t, tile c, row tile r): behind MFMA r of one B operand
-    // sits slot r of the next operand's dequant; on the last tile of a K-step every A operand is refilled from LDS
-    // for the next K-step right behind its last MFMA, 16 MFMAs ahead of its first use.  The last tile of the group
-    // prepares the next group the same way (its x tile and cells were requested at the top of this group and are
-    // waited for just before that tile), so the groups follow each other without a bubble.
+    // One quantisation group, software-pipelined over (K-step t, tile c, quarter q of the 16 row tiles): behind every
+    // MFMA of one B operand sits a slot of the next operand's dequant, and behind every quarter a share of the memory
+    // requests, spread evenly, because a wave that issues a burst of them waits in the request queue with no MFMA in
+    // flight (all 24 requests of a group at its top cost a third of the run time), and the four waves asking for
+    // their 16 A operands at once want twice what the LDS delivers:
+    //   - the 16 LDS reads that fetch the A operands of the next K-step (K-step 3: of the next group's K-step 0, from
+    //     the other stage);
+    //   - K-step 0: the next group's cells and scale words, one tile per quarter 0; K-steps 1 and 2: the 16 requests
+    //     of its x tile copy.  Before K-step 3 everything has landed (s_waitcnt, then the barrier: every wave also has
+    //     its LDS reads of this stage behind it, K-step 3's operands were fetched during K-step 2), so the other stage
+    //     is complete and this one may be overwritten from K-step 1 of the next group on.
+    // The last tile dequantises the next group's first operand, so the groups follow each other without a bubble.
     //
-    // The step after the last one has nothing to request, and that is the only difference: it still prepares a "next
-    // group" from whatever the registers and the other stage hold, and nobody uses it.  One copy of the code for all
-    // groups matters: the accumulators must stay in the same AGPRs from the first MFMA to the last, and in a second
-    // copy of the loop body the register allocator moves them, through VGPRs, right behind MFMAs it does not know of.
-    auto group_step = [&](int g, int stage, int set, bool request_next) {
-        if (request_next) {
-            copy_x(stage ^ 1, g + 1);
-            load_w(set ^ 1, g + 1);
-        }
+    // The last group requests its own data once more and prepares a "next group" nobody uses: one copy of the code
+    // for all groups matters, because the accumulators must stay in the same AGPRs from the first MFMA to the last,
+    // and in a second copy of the loop body the register allocator moves them, through VGPRs, right behind MFMAs it
+    // does not know of.
+    auto group_step = [&](int g, int stage, int set) {
+        const int gn = g + 1 < G ? g + 1 : g;
+        const gptr xs = x_src(gn);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
+            if (t == 3) {
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                take_w(set ^ 1);
+            }
 #pragma unroll
             for (int c = 0; c < NCB; ++c) {
                 const bool last = t == 3 && c == NCB - 1;
                 const int cn = c + 1 < NCB ? c + 1 : 0, tn = c + 1 < NCB ? t : (t + 1) & 3;
-                if (last) {
-                    // The next group's x tile and cells have landed.  Every wave has consumed its LDS reads of this
-                    // stage (those of K-step 3 were issued during K-step 2), so after the barrier the other stage is
-                    // complete and this one may be overwritten at the top of the next group.
-                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-                    __syncthreads();
-                    take_w(set ^ 1);
-                    decode_md(md[set ^ 1][0], sf[0], c0[0]);
-                }
+                if (last) decode_md(md[set ^ 1][0], sf[0], c0[0]);
                 DequantSlots dq;
                 dq.w = last ? cell[set ^ 1][0][0] : cell[set][cn][tn];
                 dq.sf = sf[cn];
@@ -282,20 +282,26 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
                 for (int q = 0; q < 4; ++q) {
                     __builtin_amdgcn_sched_barrier(0);
                     const int r = 4 * q;
+                    const bf16x8(&ac)[RT] = a[t & 1];
                     auto quarter = [&](auto Q) {
-                        mfma_quarter<decltype(Q)::value>(acc[r][c], acc[r + 1][c], acc[r + 2][c], acc[r + 3][c], a[r], a[r + 1], a[r + 2], a[r + 3], b_cur, dq);
+                        mfma_quarter<decltype(Q)::value>(acc[r][c], acc[r + 1][c], acc[r + 2][c], acc[r + 3][c], ac[r], ac[r + 1], ac[r + 2], ac[r + 3], b_cur, dq);
                     };
                     if (q == 0) quarter(std::integral_constant<int, 0>{});
                     else if (q == 1) quarter(std::integral_constant<int, 1>{});
                     else if (q == 2) quarter(std::integral_constant<int, 2>{});
                     else quarter(std::integral_constant<int, 3>{});
                     __builtin_amdgcn_sched_barrier(0);
-                    if (c == NCB - 1) {
+                    // this quarter's share of the next K-step's A operands
+                    const int i = 4 * c + q;
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            if (t < 3) a[r + k] = read_a(stage, t + 1, r + k);
-                            else a[r + k] = read_a(stage ^ 1, 0, r + k);
-                        }
+                    for (int k = i * RT / (4 * NCB); k < (i + 1) * RT / (4 * NCB); ++k)
+                        a[(t + 1) & 1][k] = t < 3 ? read_a(stage, t + 1, k) : read_a(stage ^ 1, 0, k);
+                    // and of the next group's memory requests
+                    if (t == 0 && q == 0) load_w_tile(set ^ 1, gn, c);
+                    if (t == 1 || t == 2) {
+                        const int j = (t - 1) * 4 * NCB + i;
+#pragma unroll
+                        for (int k = j * RT / (8 * NCB); k < (j + 1) * RT / (8 * NCB); ++k) copy_x_part(stage ^ 1, xs, k);
                     }
                     // scale words of the next group's other tiles, behind the last quarter of the group
                     if (last && q == 3) {
@@ -310,21 +316,23 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    copy_x(0, 0);
-    load_w(0, 0);
+#pragma unroll
+    for (int i = 0; i < RT; ++i) copy_x_part(0, x_src(0), i);
+#pragma unroll
+    for (int c = 0; c < NCB; ++c) load_w_tile(0, 0, c);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the x tile copy writes LDS behind the compiler's back
     __syncthreads();
     take_w(0);
 #pragma unroll
     for (int c = 0; c < NCB; ++c) decode_md(md[0][c], sf[c], c0[c]);
 #pragma unroll
-    for (int r = 0; r < RT; ++r) a[r] = read_a(0, 0, r);
+    for (int r = 0; r < RT; ++r) a[0][r] = read_a(0, 0, r);
     b_cur = dequant_operand(cell[0][0][0], sf[0], c0[0]);
 
     // two groups per trip (G is even): stage / register set 0, then 1
     for (int g = 0; g < G; g += 2) {
-        group_step(g, 0, 0, true);
-        group_step(g + 1, 1, 1, g + 2 < G);
+        group_step(g, 0, 0);
+        group_step(g + 1, 1, 1);
     }
 
     // The bf16 tile leaves through LDS (the K loop is done with it): a lane holds 4 rows of one column, so stores
