@@ -10,7 +10,8 @@
 //               tile is shared.  16 NCB * 4 fp32 accumulators per lane live in AGPRs (NCB = 4: all 256).
 //   K loop    = one quantisation group (128 rows of W) per step: the x tile [256][128] is copied global -> LDS
 //               (global_load_lds_dwordx4, double buffered) while the previous group multiplies; the cells and
-//               scale words of the next group are requested a step ahead; one barrier per group
+//               scale words of the next group are requested a step ahead; one barrier per group; the A operands
+//               are double buffered in registers, one K-step ahead
 //   tiles     = column tiles of two widths in one launch, 256-wide ones first, then 192-wide ones
 //               (pick_widths()): M = 2048, N = 14336 becomes 8 x (32 tiles of 256 + 32 tiles of 192), and each of
 //               the 256 CUs gets one wide and one narrow tile, 1.75 tile times instead of the two full rounds
@@ -23,6 +24,11 @@
 // instructions are cut into 12 slots of two independent instructions (DequantSlots), one slot behind each of the
 // first 12 MFMAs of the previous operand.  With 8 row tiles (2.9 instructions per MFMA) the same loop is bound by
 // the VALU: 128 x 448 tiles measured 288 us against 257 us for 256 x 256 with the same inner loop.
+// Every other instruction (LDS read, memory request, s_add, s_nop, s_waitcnt) takes a slot of its own as well.
+//
+// Where the time goes at M = 2048, K = 4096, N = 14336 (same box, kernel parts compiled out one at a time): MFMAs alone
+// 143 us (the accumulators' pro- and epilogue included), with the dequant 153 us, with LDS reads, x tile copy and
+// cell loads 203 - 213 us; without the x tile copy 169 us, without the LDS reads 192 us, without the cell loads 194 us.
 //
 // Everything in the inner loop is volatile asm: MFMAs with the accumulator tied to one AGPR quad (through the
 // builtin the register allocator gives some MFMAs a destination other than their accumulator input and rotates
@@ -123,6 +129,10 @@ __device__ __forceinline__ void mfma_quarter(floatx4 &c0, floatx4 &c1, floatx4 &
                      : "+a"(c0), "+a"(c1), "+a"(c2), "+a"(c3), "+v"(d.a1), "=&v"(d.b0), "=&v"(d.b1), "=&v"(d.p2), "=&v"(d.p3)
                      : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b), "v"(d.a0), "v"(d.o), "v"(d.sf), "v"(d.c0));
     }
+}
+
+__device__ __forceinline__ void mfma_one(floatx4 &acc, const bf16x8 &a, const bf16x8 &b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
 // A wave-uniform pointer pinned to scalar registers: the loads below then take the form "scalar base + 32-bit lane
@@ -241,17 +251,21 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     bf16x8 b_cur;
     float sf[NCB], c0[NCB];
 
-    // One quantisation group, software-pipelined over (K-step t, tile c, quarter q of the 16 row tiles): behind every
-    // MFMA of one B operand sits a slot of the next operand's dequant, and behind every quarter a share of the memory
-    // requests, spread evenly, because a wave that issues a burst of them waits in the request queue with no MFMA in
-    // flight (all 24 requests of a group at its top cost a third of the run time), and the four waves asking for
-    // their 16 A operands at once want twice what the LDS delivers:
-    //   - the 16 LDS reads that fetch the A operands of the next K-step (K-step 3: of the next group's K-step 0, from
-    //     the other stage);
-    //   - K-step 0: the next group's cells and scale words, one tile per quarter 0; K-steps 1 and 2: the 16 requests
-    //     of its x tile copy.  Before K-step 3 everything has landed (s_waitcnt, then the barrier: every wave also has
-    //     its LDS reads of this stage behind it, K-step 3's operands were fetched during K-step 2), so the other stage
-    //     is complete and this one may be overwritten from K-step 1 of the next group on.
+    // One quantisation group, software-pipelined over (K-step t, tile c, quarter of the 16 row tiles).  Behind every
+    // MFMA of quarters 0..2 sits a slot of the next operand's dequant; those MFMAs have no issue slot to spare.  The
+    // memory requests are spread over the group, between the quarters and behind the MFMAs of quarter 3 (two free
+    // slots each): issued as a burst at the top of the group they leave the wave in the request queue with no MFMA
+    // in flight (a third of the run time), and the four waves asking for their 16 A operands at once want twice what
+    // the LDS delivers.
+    //   - every K-step: the 16 LDS reads that fetch the A operands of the next K-step (K-step 3: of the next group's
+    //     K-step 0, from the other stage);
+    //   - K-steps 0 and 1: the 16 requests of the next group's x tile copy (in K-steps 1 and 2 the last of them is a
+    //     few hundred cycles old when K-step 3 waits for it: 213 us instead of 203 us); K-step 0: its cells and scale
+    //     words.
+    // Before K-step 3 everything has landed (s_waitcnt vmcnt(0), then the barrier).  Every wave has by then issued
+    // all its LDS reads of this stage (K-step 3's operands are fetched during K-step 2) and consumes them within
+    // K-step 3; the stage is overwritten from K-step 0 of the next group on, which a wave reaches a whole K-step of
+    // MFMAs behind the barrier, so the copy cannot overtake those reads.
     // The last tile dequantises the next group's first operand, so the groups follow each other without a bubble.
     //
     // The last group requests its own data once more and prepares a "next group" nobody uses: one copy of the code
@@ -264,7 +278,7 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             if (t == 3) {
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
                 take_w(set ^ 1);
@@ -278,35 +292,47 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
                 dq.w = last ? cell[set ^ 1][0][0] : cell[set][cn][tn];
                 dq.sf = sf[cn];
                 dq.c0 = c0[cn];
+                const bf16x8(&ac)[RT] = a[t & 1];
+                // This tile's share of the LDS reads that fetch the next K-step's A operands: operands n0 .. n1 - 1.
+                // The first three go between the quarters, where the compiler would otherwise put an s_nop (it
+                // separates asm statements that hand a register on), the rest behind the MFMAs of quarter 3.
+                constexpr int kPerTile = (RT + NCB - 1) / NCB;
+                const int n0 = c * RT / NCB, n1 = (c + 1) * RT / NCB;
+                auto fetch_a = [&](int n) {
+                    if (n < n1) a[(t + 1) & 1][n] = t < 3 ? read_a(stage, t + 1, n) : read_a(stage ^ 1, 0, n);
+                };
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_quarter<0>(acc[0][c], acc[1][c], acc[2][c], acc[3][c], ac[0], ac[1], ac[2], ac[3], b_cur, dq);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch_a(n0);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_quarter<1>(acc[4][c], acc[5][c], acc[6][c], acc[7][c], ac[4], ac[5], ac[6], ac[7], b_cur, dq);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch_a(n0 + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_quarter<2>(acc[8][c], acc[9][c], acc[10][c], acc[11][c], ac[8], ac[9], ac[10], ac[11], b_cur, dq);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch_a(n0 + 2);
+                // quarter 3: the dequant is done, two issue slots are free behind each MFMA: the other requests
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
+                for (int k = 0; k < 4; ++k) {
                     __builtin_amdgcn_sched_barrier(0);
-                    const int r = 4 * q;
-                    const bf16x8(&ac)[RT] = a[t & 1];
-                    auto quarter = [&](auto Q) {
-                        mfma_quarter<decltype(Q)::value>(acc[r][c], acc[r + 1][c], acc[r + 2][c], acc[r + 3][c], ac[r], ac[r + 1], ac[r + 2], ac[r + 3], b_cur, dq);
-                    };
-                    if (q == 0) quarter(std::integral_constant<int, 0>{});
-                    else if (q == 1) quarter(std::integral_constant<int, 1>{});
-                    else if (q == 2) quarter(std::integral_constant<int, 2>{});
-                    else quarter(std::integral_constant<int, 3>{});
+                    mfma_one(acc[12 + k][c], ac[12 + k], b_cur);
                     __builtin_amdgcn_sched_barrier(0);
-                    // this quarter's share of the next K-step's A operands
-                    const int i = 4 * c + q;
 #pragma unroll
-                    for (int k = i * RT / (4 * NCB); k < (i + 1) * RT / (4 * NCB); ++k)
-                        a[(t + 1) & 1][k] = t < 3 ? read_a(stage, t + 1, k) : read_a(stage ^ 1, 0, k);
-                    // and of the next group's memory requests
-                    if (t == 0 && q == 0) load_w_tile(set ^ 1, gn, c);
-                    if (t == 1 || t == 2) {
-                        const int j = (t - 1) * 4 * NCB + i;
+                    for (int n = n0 + 3 + k * (kPerTile - 3) / 4; n < n0 + 3 + (k + 1) * (kPerTile - 3) / 4; ++n) fetch_a(n);
+                    // the next group's x tile (K-steps 0 and 1: early enough to have landed before K-step 3) ...
+                    if (t == 0 || t == 1) {
+                        const int j = (t * NCB + c) * 4 + k;
 #pragma unroll
-                        for (int k = j * RT / (8 * NCB); k < (j + 1) * RT / (8 * NCB); ++k) copy_x_part(stage ^ 1, xs, k);
+                        for (int n = j * RT / (8 * NCB); n < (j + 1) * RT / (8 * NCB); ++n) copy_x_part(stage ^ 1, xs, n);
                     }
-                    // scale words of the next group's other tiles, behind the last quarter of the group
-                    if (last && q == 3) {
+                    // ... its cells and scale words (K-step 0) ...
+                    if (t == 0 && k == 3) load_w_tile(set ^ 1, gn, c);
+                    // ... and the scale words of its other tiles, behind the last MFMA of the group
+                    if (last && k == 3) {
 #pragma unroll
-                        for (int k = 1; k < NCB; ++k) decode_md(md[set ^ 1][k], sf[k], c0[k]);
+                        for (int n = 1; n < NCB; ++n) decode_md(md[set ^ 1][n], sf[n], c0[n]);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
