@@ -139,7 +139,7 @@ class HIPBackend(AirBackend):
                 iters = max(self.n_perf_iters, 1)
                 for _ in range(iters):
                     outs = run(dev_in)
-                torch.cuda.synchronize()
+                ops.check_health()   # synchronises; a reducer that timed out surfaces here
                 if self.n_perf_iters > 0:
                     self.last_latency_us = (time.perf_counter() - t0) / iters * 1e6
             except _lib.W4A16Error as e:

@@ -290,7 +290,7 @@ class KernelCache:
 
         import torch
 
-        from . import _lib
+        from . import _lib, ops
 
         try:
             _lib.load_library()
@@ -373,7 +373,7 @@ class KernelCache:
             t_write_ms = (time.perf_counter() - t_write) * 1e3
             t_kernel = time.perf_counter()
             produced = run(readback)
-            torch.cuda.synchronize()
+            ops.check_health()   # synchronises; a reducer that timed out surfaces here
             t_kernel_ms = (time.perf_counter() - t_kernel) * 1e3
         except _lib.W4A16Error as e:
             raise AirBackendError(str(e))

@@ -208,6 +208,7 @@ def generate(prompt_tokens, layers, embed_table, final_norm, lm_head, config, ro
     eos = set(int(t) for t in eos_token_ids)
     if on_token is None:
         rest = decode_greedy(first, n_tokens, layers, embed_table, final_norm, lm_head, config, kv_cache, seq_len, rope_lut)
+        ops.check_health()
         out = [int(first.item())] + [int(t) for t in rest.cpu().tolist()]
         for i in range(1, len(out)):
             if out[i] in eos:
@@ -219,6 +220,7 @@ def generate(prompt_tokens, layers, embed_table, final_norm, lm_head, config, ro
     for i in range(n_tokens):
         _, best = decode_token(tok, layers, embed_table, final_norm, lm_head, config, kv_cache, seq_len + i, rope_lut,
                                return_argmax=True)
+        ops.check_health()
         tok = int(best.item())
         out.append(tok)
         on_token(tok)

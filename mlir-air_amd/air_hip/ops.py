@@ -11,6 +11,7 @@ from . import _lib
 
 GROUP = 128
 _workspaces = {}
+_checked = False
 
 
 def _ptr(t):
@@ -50,6 +51,38 @@ def workspace(nbytes, device, use="gemm"):
         _lib.check(lib.w4a16_workspace_init(_ptr(ws), ws.numel(), _stream()))
         _workspaces[key] = ws
     return ws
+
+
+def check_health():
+    """Synchronise the device and look at every split-K workspace that this module handed out: if a reducer of an
+    earlier call gave up waiting for a partial result (its output is then invalid), re-initialise that workspace, so
+    that the next call works, and raise W4A16Error(ERR_TIMEOUT).  The launches themselves never synchronise, so this is
+    the place where such a failure becomes visible: callers that read results back on the host (the backends, the
+    token loop) call it there (counterpart of the run-state check after a kernel run,
+    python/air/backend/xrt.py:204-218).  The stream-order entry points keep no such state and cannot time out."""
+    lib = _lib.load_library()
+    torch.cuda.synchronize()
+    failed = []
+    for key, ws in _workspaces.items():
+        if lib.w4a16_workspace_check(_ptr(ws), None) == _lib.ERR_TIMEOUT:
+            _lib.check(lib.w4a16_workspace_init(_ptr(ws), ws.numel(), None))
+            failed.append(key)
+    if failed:
+        torch.cuda.synchronize()
+        raise _lib.W4A16Error(_lib.ERR_TIMEOUT, "a split-K reducer gave up waiting for a partial result; the outputs of the calls "
+                              f"since the last check are invalid (workspaces {[k[2] for k in failed]} re-initialised)")
+
+
+def set_checked(on):
+    """Checked mode: every call that uses a split-K workspace synchronises and runs check_health() before it returns
+    (for tests and for hunting a failure down to one call; off by default)."""
+    global _checked
+    _checked = bool(on)
+
+
+def _after_workspace_call():
+    if _checked:
+        check_health()
 
 
 def awq_dequant(qweight, qzeros, scales, group=GROUP, out=None):
@@ -93,6 +126,7 @@ def w4a16_gemm(x, qweight, qzeros, scales, group=GROUP, out=None):
     ws = workspace(nbytes, x.device)
     _lib.check(lib.w4a16_gemm_bf16(_ptr(_bits(x2)), _ptr(qweight), _ptr(qzeros), _ptr(_bits(scales)), _ptr(out),
                                    M, K, N, group, _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return out.squeeze(0) if vec else out
 
 
@@ -109,6 +143,7 @@ def w4a16_gemv(x, qweight, qzeros, scales, group=GROUP, out=None):
     ws = workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
     _lib.check(lib.w4a16_gemv_bf16(_ptr(_bits(x)), _ptr(qweight), _ptr(qzeros), _ptr(_bits(scales)), _ptr(out),
                                    K, N, group, _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return out
 
 
@@ -125,6 +160,7 @@ def w4a16_swiglu(x, gate, up, group=GROUP):
     _lib.check(lib.w4a16_gemv_swiglu_bf16(
         _ptr(_bits(x)), _ptr(gate[0]), _ptr(gate[1]), _ptr(_bits(gate[2])),
         _ptr(up[0]), _ptr(up[1]), _ptr(_bits(up[2])), _ptr(h), K, H, group, _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return h
 
 
@@ -145,6 +181,7 @@ def ffn_swiglu(x, gate, up, down, group=GROUP, return_h=False):
         _ptr(up[0]), _ptr(up[1]), _ptr(_bits(up[2])),
         _ptr(down[0]), _ptr(down[1]), _ptr(_bits(down[2])),
         _ptr(y), _ptr(h) if h is not None else None, K, H, group, _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return (y, h) if return_h else y
 
 
@@ -240,6 +277,7 @@ def w4a16_gemv_add(x, qweight, qzeros, scales, residual, group=GROUP, out=None):
     ws = workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
     _lib.check(lib.w4a16_gemv_add_bf16(_ptr(_bits(x)), *_wptrs((qweight, qzeros, scales)), _ptr(_bits(residual)),
                                        _ptr(out), K, N, group, _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return out
 
 
@@ -265,6 +303,7 @@ def w4a16_rms_gemv(x, norm_weight, qweight, qzeros, scales, eps=1e-5, group=GROU
     _lib.check(lib.w4a16_rms_gemv_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
                                        *_wptrs((qweight, qzeros, scales)), _ptr(out), K, N, group,
                                        _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return out
 
 
@@ -281,6 +320,7 @@ def w4a16_rms_swiglu(x, norm_weight, gate, up, eps=1e-5, group=GROUP):
     _lib.check(lib.w4a16_rms_gemv_swiglu_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
                                               *_wptrs(gate), *_wptrs(up), _ptr(h), K, H, group,
                                               _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return h
 
 
@@ -308,6 +348,7 @@ def o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e
         *_wptrs(wo), *_wptrs(gate), *_wptrs(up), *_wptrs(down), _ptr(y),
         _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
         E, H, group, _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return (y, res1, h) if return_intermediates else y
 
 
@@ -368,6 +409,7 @@ def decode_attn_o_gemv_ffn(qkv, rope_lut_row, k_cache, v_cache, pos, n_heads, x_
         max_seq, n_heads, n_kv, hd, _ptr(aws), aws.numel(), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
         *_wptrs(wo), *_wptrs(gate), *_wptrs(up), *_wptrs(down), _ptr(y), _ptr(sumsq) if sumsq is not None else None, E, H, group,
         _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return (y, sumsq) if return_sumsq else y
 
 
@@ -638,6 +680,7 @@ def q4nx_gemm(x, qweight, scales, mins, residual=None, out=None):
     _lib.check(lib.w4a16_q4nx_gemm_bf16(_ptr(_bits(x2)), _ptr(qweight), _ptr(_bits(scales)), _ptr(_bits(mins)),
                                         _ptr(_bits(residual)) if residual is not None else None, _ptr(out),
                                         M, K, N, _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return out.squeeze(0) if vec else out
 
 
@@ -659,6 +702,7 @@ def q4nx_rms_gemv(x, norm_weight, qweight, scales, mins, eps=1e-5):
     _lib.check(lib.w4a16_q4nx_rms_gemv_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
                                             *_qptrs((qweight, scales, mins)), _ptr(out), K, N,
                                             _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return out
 
 
@@ -682,6 +726,7 @@ def q4nx_o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, e
         *_qptrs(wo), *_qptrs(gate), *_qptrs(up), *_qptrs(down), _ptr(y),
         _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
         E, H, _ptr(ws), ws.numel(), _stream()))
+    _after_workspace_call()
     return (y, res1, h) if return_intermediates else y
 
 

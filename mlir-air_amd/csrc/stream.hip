@@ -434,11 +434,13 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     // The reducer's first polling round is issued before the LDS combine, so that its latency
     // (one trip to L2 per slot) is hidden behind the combine and its barriers.
     u32x4 va[8], vb[8];   // the two polling rounds a reducer thread keeps in flight
-    const bool prefetched = reducer && (int)threadIdx.x < nquads;
+    const bool prefetched = reducer && nprod > 0 && (int)threadIdx.x < nquads;
     if (prefetched) {
+        // every round issues all eight loads (a slot index past the last producer is clamped to it and the copy
+        // ignored): no load of a round is predicated, so no register of a round can hold a stale value
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            if (j < nprod) va[j] = slot_load_planes(tile_partial + (size_t)threadIdx.x * 2 + j * slice_stride, plane);
+            va[j] = slot_load_planes(tile_partial + (size_t)threadIdx.x * 2 + (j < nprod ? j : nprod - 1) * slice_stride, plane);
     }
 
     // ---- cross-wave combine in LDS: red[slot][m][ln][LC], moved as 16-byte chunks (4 columns).  Chunk jj
@@ -487,7 +489,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         floatx4 sum0 = floatx4{0.f, 0.f, 0.f, 0.f}, sum1 = floatx4{0.f, 0.f, 0.f, 0.f};
         for (int s0 = 0; s0 < nprod; s0 += 8) {
 #define W4A16_POLL_ISSUE(dst)                                                                 \
-    _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < nprod) dst[j] = slot_load_planes(slot0 + (s0 + j) * slice_stride, plane)
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) dst[j] = slot_load_planes(slot0 + (s0 + j < nprod ? s0 + j : nprod - 1) * slice_stride, plane)
 #define W4A16_POLL_FULL(src, ok)                                                              \
     ok = true;                                                                                \
     _Pragma("unroll") for (int j = 0; j < 8; ++j) if (s0 + j < nprod) ok = ok && slot_full(src[j])

@@ -182,12 +182,45 @@ def test_reducer_timeout_is_reported_and_workspace_recovers():
         ops.tune("gemv_spin_limit", 8)
         ops.w4a16_gemv(x, *w)
         assert lib.w4a16_workspace_check(ws.data_ptr(), stream) == _lib.ERR_TIMEOUT
+        # the host-side check reports it, names the code, and leaves the workspace usable
+        with pytest.raises(_lib.W4A16Error) as e:
+            ops.check_health()
+        assert e.value.code == _lib.ERR_TIMEOUT
+        assert lib.w4a16_workspace_check(ws.data_ptr(), stream) == 0
+        # checked mode: the call itself raises
+        ops.set_checked(True)
+        with pytest.raises(_lib.W4A16Error):
+            ops.w4a16_gemv(x, *w)
+    finally:
+        ops.set_checked(False)
+        ops.tune("gemv_skip_publish", 0)
+        ops.tune("gemv_spin_limit", 0)
+    ops.check_health()
+    assert torch.equal(ops.w4a16_gemv(x, *w).view(torch.int16), good.view(torch.int16))
+
+
+def test_reducer_timeout_surfaces_as_backend_error():
+    """Through the backend interface the same failure is an AirBackendError at the invoker's read-back."""
+    from air_hip import awq, bf16, ops
+    from air_hip.backend import AirBackendError, HIPBackend, HipModule
+    print("reducer timeout through HIPBackend", flush=True)
+    K, N = 4096, 1024
+    qw, qz, s = make_awq(K, N, seed=23)
+    x = make_x((K,), seed=24)
+    backend = HIPBackend()
+    invoker = backend.compile_and_load(HipModule("matvec_int4", K=K, N=N, gs=128))
+    args = (awq.pack_buffer(qw, qz, bf16.from_bits(s)), bf16.from_bits(x), np.zeros(N, np.uint16).view(bf16.BF16Array))
+    good = invoker(*args)[-1]
+    try:
+        ops.tune("gemv_skip_publish", 1)
+        ops.tune("gemv_spin_limit", 8)
+        with pytest.raises(AirBackendError):
+            invoker(*args)
     finally:
         ops.tune("gemv_skip_publish", 0)
         ops.tune("gemv_spin_limit", 0)
-    _lib.check(lib.w4a16_workspace_init(ws.data_ptr(), ws.numel(), stream))
-    assert lib.w4a16_workspace_check(ws.data_ptr(), stream) == 0
-    assert torch.equal(ops.w4a16_gemv(x, *w).view(torch.int16), good.view(torch.int16))
+    assert np.array_equal(np.asarray(invoker(*args)[-1]).view(np.uint16), np.asarray(good).view(np.uint16))
+    backend.unload()
 
 
 def test_hip_graph_replay_matches_eager():
