@@ -38,7 +38,7 @@ CONFIGS = {
     "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128, stream-order weights"),
     "prefill_awq": dict(M=2048, K=4096, N=14336, cfg=None, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128, checkpoint-layout weights"),
     "ffn": dict(M=1, K=4096, N=14336, cfg=4, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128, stream-order weights (2 launches)"),
-    "ffn_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128, checkpoint-layout weights (persistent kernel)"),
+    "ffn_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode SwiGLU FFN W4A16 K=4096 H=14336 g128, checkpoint-layout weights (two split-K launches)"),
     "block_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode block, checkpoint-layout weights"),
     "layer_awq": dict(M=1, K=4096, N=14336, cfg=None, desc="decode layer, checkpoint-layout weights"),
     # beyond the five headline configs: the O projection + RMSNorm + FFN decode block with residuals (3 launches)
@@ -728,7 +728,7 @@ def main():
         roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": value / HBM_PEAK_GBS, "traffic": None}
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
-    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_wsp_kernel", "prefill_awq": "gemm_kernel", "ffn_awq": "ffn_fused_kernel", "lm_head": "lm_head_kernel",
+    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_wsp_kernel", "prefill_awq": "gemm_kernel", "lm_head": "lm_head_kernel",
                       "gemv": "gemv_ws_kernel", "gemm16": "gemm_ws_kernel", "ffn": "gemv_ws_kernel", "block": "gemv_ws_kernel", "layer": "gemv_ws_kernel"}.get(name, "stream_kernel")
     roof["algorithmic_per_launch"] = main_res["flops"] if name in ("prefill", "prefill_awq") else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]

@@ -84,10 +84,11 @@ int awq_dequant_1d_bf16(const uint8_t *packed, uint16_t *out_bf16, int n, int gr
  * (different streams) need separate workspaces.  The FFN and block entry points keep plain
  * intermediates (h, res1) behind the prepared area, at an offset that depends on their shapes: share
  * a workspace only between calls of one entry point with the same shapes, or prepare it again
- * before a call of another kind.  w4a16_ffn_swiglu_bf16 and w4a16_o_gemv_ffn_bf16 run a persistent
- * kernel whose workgroups wait for one another; two such calls running at the same time on one
- * GPU can starve each other into the timeout path (w4a16_workspace_check), so keep them on one stream
- * or switch the kernel off with w4a16_tune("ffn_fused", 0).
+ * before a call of another kind.  With w4a16_tune("ffn_fused", 1) (off by default) w4a16_ffn_swiglu_bf16
+ * and w4a16_o_gemv_ffn_bf16 run a persistent kernel whose workgroups wait for one another: it needs
+ * all of them resident at once, so two such calls running at the same time on one GPU (two streams,
+ * two processes) can starve each other into the timeout path (w4a16_workspace_check); keep them on
+ * one stream, one process per GPU.
  */
 size_t w4a16_gemm_workspace_bytes(int M, int K, int N);
 size_t w4a16_ffn_workspace_bytes(int K, int H);
@@ -521,8 +522,10 @@ int w4a16_q4nx_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_resid
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic),
  * "gemm_stream_max_m" (largest M given to the streaming kernel, 0 = default 96, otherwise >= 16) and
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the
- * timeout test: split-K producers do not publish), "ffn_fused" (1 = default: w4a16_ffn_swiglu_bf16
- * runs as one persistent kernel when the shape allows, 0 = always two launches).  Process-wide.
+ * timeout test: split-K producers do not publish), "ffn_fused" (0 = default: w4a16_ffn_swiglu_bf16
+ * runs two streaming launches; 1 = one persistent kernel when the shape allows), "gemv_ws_ct", "gemv_ws_waves",
+ * "gemm_ws_cb" (stream-order GEMV / small-batch shapes), "prefill_tile" (1: 256-column tiles only, 2: 192-column
+ * tiles only, 0: by shape) and "prefill_min_m" (smallest M given to the tiled prefill kernel).  Process-wide.
  */
 int w4a16_tune(const char *key, int value);
 

@@ -137,7 +137,7 @@ int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_res
                                                        round256((size_t)H * sizeof(uint16_t)));
     // stage 1: res1 = bf16(attn_out . Wo + x_residual); its reducers also leave sum(res1^2) per column
     // tile, so that stage 2 does not have to read res1 again for the norm
-    const int res1_tiles = plan_stream(1, E, E, affine).ntiles;
+    const int res1_tiles = plan_stream(1, E, E, true).ntiles;   // a launch that leaves sums of squares keeps 256-column tiles
     const bool chain_norm = res1_tiles <= 64;
     StreamExtras add;
     add.residual = x_residual;

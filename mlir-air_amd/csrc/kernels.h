@@ -22,7 +22,7 @@ struct StreamTune {
     int stream_max_m = 0;   // largest M that w4a16_gemm_bf16 gives to the streaming kernel (0 = kStreamMaxM; at least 16)
     int skip_publish = 0; // tests only: producers do not publish, so reducers run into their poll bound
     int spin_limit = 0;   // reducer poll bound (0 = default); tiny values force the timeout path in tests
-    int no_ffn_fused = 0; // 1: w4a16_ffn_swiglu_bf16 always runs its two streaming launches
+    int no_ffn_fused = 1; // 1 (default): w4a16_ffn_swiglu_bf16 runs its two streaming launches; 0: the one-launch persistent kernel (opt-in)
     int no_attn_fuse = 0; // 1: w4a16_decode_attn_o_gemv_ffn_bf16 always runs the attention merge launch
 };
 extern StreamTune g_stream_tune;

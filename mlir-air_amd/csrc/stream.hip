@@ -674,7 +674,8 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
                          const int32_t *up_qweight, const int32_t *up_qzeros, const uint16_t *up_scales,
                          uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream,
                          const StreamExtras &extras) {
-    const StreamPlan pl = plan_stream(M, K, N, extras.mins != nullptr);
+    // the chained sums of squares count one float per 256-column tile: those launches keep that shape whatever the tune keys say
+    const StreamPlan pl = plan_stream(M, K, N, extras.mins != nullptr || extras.sumsq_out != nullptr || extras.sumsq_in != nullptr);
     StreamParams p;
     p.x = x;
     p.qw[0] = reinterpret_cast<const uint32_t *>(qweight);

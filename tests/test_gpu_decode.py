@@ -311,10 +311,22 @@ def test_sum_of_squares_chained_into_the_next_norm(ops, n_heads, n_kv, hd, H):
             first = sumsq.clone()
         else:
             assert torch.equal(first, sumsq)
-    ops.tune("ffn_fused", 1)
+    ops.tune("ffn_fused", 0)
+    # 128-column tiles (tuning key) must not change the chain: launches that leave or take sums of squares keep
+    # their 256-column tiles, one float per tile in a buffer of E / 256
+    ops.tune("gemv_lw", 1)
+    try:
+        y_lw, sumsq_lw = ops.decode_attn_o_gemv_ffn(qkv, lut[pos], kc.clone(), vc.clone(), pos, n_heads, x_res, norm_w, wo, wg, wu, wd,
+                                                    return_sumsq=True)
+        chained_lw = ops.w4a16_rms_gemv(y_lw, norm_w, *wq, x_sumsq=sumsq_lw)
+        torch.cuda.synchronize()
+    finally:
+        ops.tune("gemv_lw", 0)
+    assert torch.equal(y_lw.view(torch.int16), y.view(torch.int16)) and torch.equal(sumsq_lw, sumsq)
     plain = ops.w4a16_rms_gemv(y, norm_w, *wq)
     chained = ops.w4a16_rms_gemv(y, norm_w, *wq, x_sumsq=sumsq)
     torch.cuda.synchronize()
+    assert torch.equal(chained_lw.view(torch.int16), chained.view(torch.int16))
     p64, c64 = plain.float().double().cpu().numpy(), chained.float().double().cpu().numpy()
     assert np.max(np.abs(p64 - c64)) <= 2 * 2.0**-8 * np.max(np.abs(p64))
     assert np.mean(p64 != c64) < 0.2
