@@ -58,7 +58,8 @@ LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 204
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
 # scaled by the same counter's reading for a 256 MiB device copy: x2.000 and x1.000); the
 # summaries under profiles/ hold the commands and the raw readings.
-MEASURED_TRAFFIC_BYTES = {"gemv": 24.11e6, "gemv_awq": 24.27e6, "prefill_awq": 342.2e6, "ffn_awq": 97.07e6, "lm_head": 525.9e6}
+MEASURED_TRAFFIC_BYTES = {"gemv": 24.11e6, "gemm16": 32.83e6, "prefill": 347.4e6, "ffn": 94.07e6,
+                          "gemv_awq": 24.26e6, "gemm16_awq": 41.9e6, "prefill_awq": 351.7e6, "ffn_awq": 94.4e6, "lm_head": 525.9e6}
 
 
 def weight_bytes(K, N):
