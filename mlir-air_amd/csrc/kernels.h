@@ -114,7 +114,7 @@ extern GemvWsTune g_gemv_ws_tune;
 struct GemvWsPlan {
     int ct, waves;
 };
-GemvWsPlan plan_gemv_ws(int K, int nmat);
+GemvWsPlan plan_gemv_ws(int K, int nmat, int N, bool rms);
 // y[N] = bf16(x[K] . W) with W in stream order; with `w_up` (second matrix, same shape) the SwiGLU epilogue
 // y = bf16(silu(bf16(x.W)) * bf16(x.W_up)).
 hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, uint16_t *y, int K, int N, hipStream_t stream,
