@@ -213,9 +213,10 @@ int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uin
 /* Batched decode on a stream-order matrix: y[M, N] = bf16(x[M, K] . W), unrounded weights, fp32 accumulation
  * (matmul_int4_packed.cpu_reference, programming_examples/matrix_multiplication/int4_awq/matmul_int4_packed.py:89-105;
  * device kernel matmul_int4_bf16_packed_f32, mv_int4_bf16.cc:430-448).  Up to 16 rows per launch stream the weights
- * once (M <= 96: launches of 16 rows over the then cache-resident weights); stateless like the GEMV.  Larger M with
- * N % 448 == 0 or N % 256 == 0 runs the tiled prefill kernel, which dequantises the weights to bf16 in registers
- * (W = bf16_rne((q - z) * s), the dense dequant's values) and feeds bf16 MFMA with fp32 accumulation. */
+ * once (M <= 96: launches of 16 rows over the then cache-resident weights); stateless like the GEMV.  From M = 97 on,
+ * with K % 256 == 0 and N % 64 == 0 (N / 64 = 3, 4 or >= 6), the tiled prefill kernel runs instead: it dequantises the
+ * weights to bf16 in registers (W = bf16_rne((q - z) * s), the dense dequant's values) and feeds bf16 MFMA with fp32
+ * accumulation; other shapes stay with the launches of 16 rows.  K % 128 == 0, N % 16 == 0. */
 int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int M, int K, int N, int group,
                            void *stream);
 int w4a16_gemv_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream,

@@ -273,3 +273,38 @@ def test_prefill_stream_one_hot_rows_reproduce_the_dequant(ops):
     y = ops.w4a16_gemm_stream(dev(x), _stream_weight(ops, qw, qz, s))
     torch.cuda.synchronize()
     assert np.array_equal(bits(y), oawq.dequant_to_bf16(qw, qz, s, 128))
+
+
+def test_prefill_sized_m_on_a_shape_the_tiled_kernel_does_not_take(ops):
+    """K = 384 (an odd number of groups) and N = 80: M = 128 runs the batched kernel in launches of 16 rows."""
+    M, K, N = 128, 384, 80
+    qw, qz, s = make_awq(K, N, seed=31)
+    x = make_x((M, K), seed=32)
+    y = ops.w4a16_gemm_stream(dev(x), _stream_weight(ops, qw, qz, s))
+    torch.cuda.synchronize()
+    want = bf16_bits_to_f32(x).astype(np.float64) @ dense_f64(qw, qz, s)
+    assert_bf16_close(bits(y), want, ulps=1.0, atol=2e-3, what="gemm stream fallback")
+
+
+def test_stream_entry_points_reject_bad_arguments(ops):
+    """Argument checks come before the first launch: negative codes, nothing written."""
+    from air_hip import _lib
+    lib = _lib.load_library()
+    K, N = 256, 64
+    qw, qz, s = make_awq(K, N, seed=33)
+    w = _stream_weight(ops, qw, qz, s)
+    x = dev(make_x((K,), seed=34))
+    y = torch.zeros((N,), dtype=torch.bfloat16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+    assert lib.w4a16_gemv_stream_bf16(None, p(w.buf), p(y), K, N, 128, st) == _lib.ERR_NULL
+    assert lib.w4a16_gemv_stream_bf16(p(x), p(w.buf), p(y), K, N, 64, st) == _lib.ERR_GROUP
+    assert lib.w4a16_gemv_stream_bf16(p(x), p(w.buf), p(y), K + 64, N, 128, st) == _lib.ERR_SHAPE
+    assert lib.w4a16_gemv_stream_bf16(p(x), p(w.buf), p(y), K, N + 8, 128, st) == _lib.ERR_SHAPE
+    assert lib.w4a16_gemv_stream_bf16(p(x) + 2, p(w.buf), p(y), K, N, 128, st) == _lib.ERR_ALIGN
+    assert lib.w4a16_gemm_stream_bf16(p(x), p(w.buf), p(y), 0, K, N, 128, st) == _lib.ERR_SHAPE
+    assert lib.w4a16_gemv_add_stream_bf16(p(x), p(w.buf), None, p(y), K, N, 128, st) == _lib.ERR_NULL
+    assert lib.w4a16_repack_stream(p(dev(qw)), p(dev(qz)), p(dev(s)), None, K, N, 128, st) == _lib.ERR_NULL
+    assert lib.w4a16_stream_bytes(K + 1, N) == 0 and lib.w4a16_stream_bytes(K, N) == w.buf.numel()
+    torch.cuda.synchronize()
+    assert not y.any()
