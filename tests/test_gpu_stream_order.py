@@ -308,3 +308,31 @@ def test_stream_entry_points_reject_bad_arguments(ops):
     assert lib.w4a16_stream_bytes(K + 1, N) == 0 and lib.w4a16_stream_bytes(K, N) == w.buf.numel()
     torch.cuda.synchronize()
     assert not y.any()
+
+
+def test_hip_graph_replays_of_the_stream_kernels_match_eager(ops):
+    """The GEMV, the batched kernel and the tiled prefill kernel captured in one HIP graph: every replay, with eager
+    work and synchronisations in between, equals the eager results bit for bit (nothing kept between launches)."""
+    K, N = 1024, 1792
+    qw, qz, s = make_awq(K, N, seed=61)
+    w = _stream_weight(ops, qw, qz, s)
+    shapes = {"gemv": (K,), "gemm": (12, K), "prefill": (300, K)}
+    inputs = {k: [dev(make_x(shp, seed=70 + 3 * i + j)) for j in range(3)] for i, (k, shp) in enumerate(shapes.items())}
+    cur = {k: v[0].clone() for k, v in inputs.items()}
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        outs = {k: ops.w4a16_gemm_stream(cur[k], w) for k in shapes}   # warm-up: outputs allocated outside the graph
+        st.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            for k in shapes:
+                ops.w4a16_gemm_stream(cur[k], w, out=outs[k] if cur[k].dim() == 2 else outs[k].unsqueeze(0))
+        for j in range(3):
+            for k in shapes:
+                cur[k].copy_(inputs[k][j])
+            g.replay()
+            st.synchronize()
+            for k in shapes:
+                want = ops.w4a16_gemm_stream(inputs[k][j], w)
+                st.synchronize()
+                assert torch.equal(outs[k].view(torch.int16), want.view(torch.int16)), (k, j)
