@@ -202,16 +202,26 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     u32x4 cell[2][NCB];
     uint32_t md[2][NCB];
     uint32_t lane16 = (uint32_t)lane * 16, ln16 = (uint32_t)ln * 16;
-    // scale word and cell of tile c for group g: lane 16 (gl / 4) + ln, dword gl % 4 of the block's first KiB, and
-    // the (1 + gl)-th KiB of the block
-    auto load_w_tile = [&](int set, int g, int c) {
+    // Scale word and cell of tile c for group g: lane 16 (gl / 4) + ln, dword gl % 4 of the block's first KiB, and the
+    // (1 + gl)-th KiB of the block.  The tiles' base addresses stay in scalar registers and the group's offset is
+    // folded into two per-lane offsets once per group (w_offsets), so that a tile costs its two requests and nothing
+    // else in the loop.
+    gptr tile_base[NCB];
+#pragma unroll
+    for (int c = 0; c < NCB; ++c) tile_base[c] = scalar_ptr(wt + (size_t)c * tile_bytes);
+    struct WOffsets {
+        uint32_t md, cell;
+    };
+    auto w_offsets = [&](int g) {
         const int gl = g & 15;
-        const char *blk = wt + (size_t)(g >> 4) * ((kWsBlockGroups + 1) * kWsCellBytes);
-        asm volatile("" : "+v"(lane16), "+v"(ln16));
-        const gptr tc = scalar_ptr(blk + (size_t)c * tile_bytes);
-        md[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(tc + (256 * (gl >> 2) + 4 * (gl & 3)) + ln16);
-        cell[set][c] = __builtin_nontemporal_load(
-            reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(tc + (size_t)(1 + gl) * kWsCellBytes + lane16));
+        const uint32_t blk = (uint32_t)(g >> 4) * (uint32_t)((kWsBlockGroups + 1) * kWsCellBytes);
+        WOffsets o{ln16 + (blk + 256 * (gl >> 2) + 4 * (gl & 3)), lane16 + (blk + (uint32_t)(1 + gl) * (uint32_t)kWsCellBytes)};
+        asm volatile("" : "+v"(o.md), "+v"(o.cell));
+        return o;
+    };
+    auto load_w_tile = [&](int set, const WOffsets &o, int c) {
+        md[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(tile_base[c] + o.md);
+        cell[set][c] = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(tile_base[c] + o.cell));
     };
     // The compiler does not see the explicit s_waitcnt below: with loads in flight it would wait for vmcnt(0) at the
     // first use of a register loaded a group earlier, i.e. right behind the requests for the next group, and expose
@@ -276,6 +286,7 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     auto group_step = [&](int g, int stage, int set) {
         const int gn = g + 1 < G ? g + 1 : g;
         const gptr xs = x_src(gn);
+        const WOffsets wo = w_offsets(gn);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             if (t == 3) {
@@ -294,11 +305,19 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
                 dq.sf = sf[cn];
                 dq.c0 = c0[cn];
                 const bf16x8(&ac)[RT] = a[t & 1];
-                // This tile's share of the LDS reads that fetch the next K-step's A operands: operands n0 .. n1 - 1.
-                // The first three go between the quarters, where the compiler would otherwise put an s_nop (it
-                // separates asm statements that hand a register on), the rest behind the MFMAs of quarter 3.
-                constexpr int kPerTile = (RT + NCB - 1) / NCB;
-                const int n0 = c * RT / NCB, n1 = (c + 1) * RT / NCB;
+                // This tile's share of the LDS reads that fetch the next K-step's A operands: operands n0 .. n1 - 1, all of
+                // them issued by the last tile but one, so that one wait at the head of the next K-step (instead of one
+                // in front of every quarter, each an issue slot) finds them all arrived.  The first three go between
+                // the quarters, where the compiler would otherwise put an s_nop (it separates asm statements that hand
+                // a register on), the rest behind the MFMAs of quarter 3.
+                constexpr int kReadTiles = NCB - 1;
+                constexpr int kPerTile = (RT + kReadTiles - 1) / kReadTiles;
+                const int n0 = c < kReadTiles ? c * RT / kReadTiles : RT, n1 = c < kReadTiles ? (c + 1) * RT / kReadTiles : RT;
+                if (c == 0) {   // two statements: an asm statement takes 30 operands at most
+                    bf16x8(&an)[RT] = a[t & 1];
+                    asm volatile("" : "+v"(an[0]), "+v"(an[1]), "+v"(an[2]), "+v"(an[3]), "+v"(an[4]), "+v"(an[5]), "+v"(an[6]), "+v"(an[7]));
+                    asm volatile("" : "+v"(an[8]), "+v"(an[9]), "+v"(an[10]), "+v"(an[11]), "+v"(an[12]), "+v"(an[13]), "+v"(an[14]), "+v"(an[15]));
+                }
                 auto fetch_a = [&](int n) {
                     if (n < n1) a[(t + 1) & 1][n] = t < 3 ? read_a(stage, t + 1, n) : read_a(stage ^ 1, 0, n);
                 };
@@ -329,7 +348,7 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
                         for (int n = j * RT / (8 * NCB); n < (j + 1) * RT / (8 * NCB); ++n) copy_x_part(stage ^ 1, xs, n);
                     }
                     // ... its cells and scale words (K-step 0) ...
-                    if (t == 0 && k == 3) load_w_tile(set ^ 1, gn, c);
+                    if (t == 0 && k == 3) load_w_tile(set ^ 1, wo, c);
                     // ... and the scale words of its other tiles, behind the last MFMA of the group
                     if (last && k == 3) {
 #pragma unroll
@@ -346,7 +365,7 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
 #pragma unroll
     for (int i = 0; i < RT; ++i) copy_x_part(0, x_src(0), i);
 #pragma unroll
-    for (int c = 0; c < NCB; ++c) load_w_tile(0, 0, c);
+    for (int c = 0; c < NCB; ++c) load_w_tile(0, w_offsets(0), c);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the x tile copy writes LDS behind the compiler's back
     __syncthreads();
     take_w(0);
