@@ -65,6 +65,7 @@ namespace {
 constexpr int kPfThreads = 256;
 constexpr int kPfRowTiles = 16;              // row tiles of 16 per wave
 constexpr int kPfRows = 16 * kPfRowTiles;    // rows per workgroup tile
+constexpr double kPfSlowdown128 = 1.4, kPfSlowdown64 = 2.0;   // time per column of 128- and 64-column tiles against 256
 
 // eight weights of one dword (rows 8 lg .. 8 lg + 7 of the lane's column) as the four registers of a B operand
 __device__ __forceinline__ bf16x8 dequant_operand(uint32_t w, float sf, float c0) {
@@ -338,7 +339,7 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
                 // in front of every quarter, each an issue slot) finds them all arrived.  The first three go between
                 // the quarters, where the compiler would otherwise put an s_nop (it separates asm statements that hand
                 // a register on), the rest behind the MFMAs of quarter 3.
-                constexpr int kReadTiles = NCB - 1;
+                constexpr int kReadTiles = NCB > 1 ? NCB - 1 : 1;   // (one tile per K-step: the reads share it)
                 constexpr int kPerTile = (RT + kReadTiles - 1) / kReadTiles;
                 const int n0 = c < kReadTiles ? c * RT / kReadTiles : RT, n1 = c < kReadTiles ? (c + 1) * RT / kReadTiles : RT;
                 if (c == 0) {   // two statements: an asm statement takes 30 operands at most
@@ -457,11 +458,14 @@ __global__ void __launch_bounds__(kPfThreads, 1) gemm_wsp_kernel(const PfArgs p)
     }
 }
 
-// Column tiling of N = 64 U columns into a tiles of 256 and b tiles of 192 (4 a + 3 b = U): the split that finishes
-// first when tiles_m * (a + b) tiles are handed, wide ones first, to `cus` CUs as they fall free (tile time taken
-// as proportional to its width).
+// Column tiling of N = 64 U columns.  Normally a tiles of 256 and b tiles of 192 (4 a + 3 b = U): the split that
+// finishes first when tiles_m * (a + b) tiles are handed, wide ones first, to `cus` CUs as they fall free (tile time
+// taken as proportional to its width).  A matrix with too few such tiles for the chip (N = 2048, M = 2048: 64) is cut
+// into tiles of 128 or 64 columns instead: those read the x tile from LDS two and four times as often per MFMA (the
+// LDS delivers half of what the 64-column tile asks for), which is still better than idle CUs.
 struct Widths {
-    int wide, narrow;
+    int ncb;            // columns / 64 of the "wide" tiles: 4, or 2 / 1 for the narrow uniform tilings
+    int wide, narrow;   // number of column tiles of ncb * 64 columns and of 192 columns
 };
 
 long split_cost(long n_wide_tiles, long n_narrow_tiles, int cus) {
@@ -490,15 +494,26 @@ Widths pick_widths(int tiles_m, int U, int cus) {
     std::lock_guard<std::mutex> lock(mu);
     for (const Entry &e : cache)
         if (e.U == U && e.tiles_m == tiles_m && e.cus == cus) return e.w;
-    Widths best{-1, -1};
-    long best_cost = -1;
+    Widths best{4, -1, -1};
+    double best_cost = -1;
     for (int a = U / 4; a >= 0; --a) {   // ties go to the split with more wide tiles
         if ((U - 4 * a) % 3) continue;
         const int b = (U - 4 * a) / 3;
-        const long cost = split_cost((long)tiles_m * a, (long)tiles_m * b, cus);
+        const double cost = (double)split_cost((long)tiles_m * a, (long)tiles_m * b, cus);
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;
-            best = Widths{a, b};
+            best = Widths{4, a, b};
+        }
+    }
+    // uniform narrow tilings: rounds x width x (measured) slowdown of the narrower tile's inner loop
+    const struct { int ncb; double slowdown; } narrow[2] = {{2, kPfSlowdown128}, {1, kPfSlowdown64}};
+    for (const auto &nv : narrow) {
+        if (U % nv.ncb) continue;
+        const long tiles = (long)tiles_m * (U / nv.ncb);
+        const double cost = (double)((tiles + cus - 1) / cus) * nv.ncb * nv.slowdown;
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best = Widths{nv.ncb, U / nv.ncb, 0};
         }
     }
     cache[next] = Entry{tiles_m, U, cus, best};
@@ -522,11 +537,7 @@ hipError_t launch_wsp(const PfArgs &p, hipStream_t stream) {
 
 }  // namespace
 
-bool gemm_prefill_ws_supported(int M, int K, int N) {
-    if (M <= 0 || K <= 0 || K % (2 * kGroup) || N % 64) return false;
-    const int U = N / 64;
-    return U == 3 || U == 4 || U >= 6;   // 4 a + 3 b = U has a solution
-}
+bool gemm_prefill_ws_supported(int M, int K, int N) { return M > 0 && K > 0 && K % (2 * kGroup) == 0 && N > 0 && N % 64 == 0; }
 
 hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream) {
     if (!gemm_prefill_ws_supported(M, K, N)) return hipErrorInvalidValue;
@@ -538,9 +549,15 @@ hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y,
     p.tiles_m = (M + kPfRows - 1) / kPfRows;
     const int U = N / 64;
     Widths wd = pick_widths(p.tiles_m, U, 256);
-    if (g_gemv_ws_tune.prefill_tile == 1 && U % 4 == 0) wd = Widths{U / 4, 0};   // tuning: 256-wide tiles only
-    if (g_gemv_ws_tune.prefill_tile == 2 && U % 3 == 0) wd = Widths{0, U / 3};   // tuning: 192-wide tiles only
+    // tuning: one tile width only (1: 256 columns, 2: 192, 3: 128, 4: 64) where it divides N
+    const int force = g_gemv_ws_tune.prefill_tile;
+    if (force == 1 && U % 4 == 0) wd = Widths{4, U / 4, 0};
+    if (force == 2 && U % 3 == 0) wd = Widths{4, 0, U / 3};
+    if (force == 3 && U % 2 == 0) wd = Widths{2, U / 2, 0};
+    if (force == 4) wd = Widths{1, U, 0};
     p.n_wide = wd.wide, p.n_narrow = wd.narrow;
+    if (wd.ncb == 2) return launch_wsp<2, 0>(p, stream);
+    if (wd.ncb == 1) return launch_wsp<1, 0>(p, stream);
     if (wd.wide == 0) {
         p.n_wide = wd.narrow, p.n_narrow = 0;
         return launch_wsp<3, 0>(p, stream);

@@ -238,10 +238,10 @@ def test_prefill_stream_shapes(ops, M, K, N):
     _prefill_case(ops, M, K, N, seed=M + K + N)
 
 
-@pytest.mark.parametrize("tile,N", [(1, 1024), (2, 768)])
+@pytest.mark.parametrize("tile,N", [(1, 1024), (2, 768), (3, 896), (4, 448)])
 def test_prefill_stream_forced_tile_width_agrees(ops, tile, N):
-    """The same product through one tile width only (tuning knob) and through the width chosen by shape: same bits
-    (a column's sum does not depend on the tile it sits in)."""
+    """The same product through one tile width only (tuning knob: 256, 192, 128, 64 columns) and through the width
+    chosen by shape: same bits (a column's sum does not depend on the tile it sits in)."""
     want = _prefill_case(ops, 300, 512, N, seed=N)
     ops.tune("prefill_tile", tile)
     try:
@@ -249,6 +249,16 @@ def test_prefill_stream_forced_tile_width_agrees(ops, tile, N):
     finally:
         ops.tune("prefill_tile", 0)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("tile", [1, 2])
+def test_prefill_stream_wide_tiles_on_many_groups(ops, tile):
+    """Small matrices pick the 64-column tiling by themselves; the 256- and 192-column tiles on a long K, forced."""
+    ops.tune("prefill_tile", tile)
+    try:
+        _prefill_case(ops, 257, 2048, 768, seed=40 + tile)
+    finally:
+        ops.tune("prefill_tile", 0)
 
 
 def test_prefill_stream_small_m_through_the_tiled_kernel(ops):
