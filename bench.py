@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_1b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -372,9 +372,10 @@ DECODE_1B_POS0 = 1024
 PREFILL_BLOCK = dict(M=2048, E=2048, H=8192)   # the reference example's dimensions (o_ffn_int4_multi.py:291-293)
 
 
-def run_prefill_block(steps, warmup):
+def run_prefill_block(steps, warmup, stream_order=True):
     """Prefill O projection + residual + RMSNorm + SwiGLU FFN + residual for 2048 tokens at the
-    Llama-3.2-1B widths (w4a16_prefill_o_ffn_bf16), `steps` calls in one HIP graph."""
+    Llama-3.2-1B widths, `steps` calls in one HIP graph: w4a16_prefill_o_ffn_stream_bf16 on stream-order
+    weights, or (stream_order=False) w4a16_prefill_o_ffn_bf16 on the checkpoint tensors."""
     import torch
 
     from air_hip import _lib
@@ -394,10 +395,16 @@ def run_prefill_block(steps, warmup):
     y = torch.empty((M, E), dtype=torch.bfloat16, device=dev)
     scratch = torch.empty(int(lib.w4a16_prefill_block_workspace_bytes(M, E, H)), dtype=torch.uint8, device=dev)
     ptrs = [t.data_ptr() for w in ws for t in w]
+    if stream_order:
+        from air_hip import ops
+        sws = [ops.repack_stream(*w) for w in ws]
+        torch.cuda.synchronize()
+        ptrs = [w.buf.data_ptr() for w in sws]
+    entry = lib.w4a16_prefill_o_ffn_stream_bf16 if stream_order else lib.w4a16_prefill_o_ffn_bf16
 
     def launch(st):
-        _lib.check(lib.w4a16_prefill_o_ffn_bf16(attn.data_ptr(), xres.data_ptr(), nw.data_ptr(), 1e-5, *ptrs, y.data_ptr(),
-                                                None, None, M, E, H, 128, scratch.data_ptr(), scratch.numel(), st))
+        _lib.check(entry(attn.data_ptr(), xres.data_ptr(), nw.data_ptr(), 1e-5, *ptrs, y.data_ptr(),
+                         None, None, M, E, H, 128, scratch.data_ptr(), scratch.numel(), st))
 
     with torch.cuda.stream(stream):
         for _ in range(warmup):
@@ -494,9 +501,10 @@ def run_decode_model(steps, warmup, model="decode_1b", stream_order=True):
             "replays_agree": bool(torch.equal(ref_tokens, tokens))}
 
 
-def run_prefill_model(model="decode_1b", M=2048, reps=3):
+def run_prefill_model(model="decode_1b", M=2048, reps=3, stream_order=True):
     """Prompt pass of M tokens through a random-weight model (air_hip.decode.prefill: per layer RMSNorm + QKV GEMM
-    + RoPE, causal attention, O + FFN block; then the decode tail on the last row), captured as one HIP graph."""
+    + RoPE, causal attention, O + FFN block; then the decode tail on the last row), captured as one HIP graph.
+    stream_order: the layers carry the stream-order re-pack, which the prompt pass then reads (as decode does)."""
     import torch
 
     from air_hip import decode, weights as wmod
@@ -519,6 +527,10 @@ def run_prefill_model(model="decode_1b", M=2048, reps=3):
     layers = [decode.DecodeLayer(attn_norm=norm_w(), ffn_norm=norm_w(), wqkv=lin(E, nqkv, 10 * i), wo=lin(E, E, 10 * i + 1),
                                  w_gate=lin(E, H, 10 * i + 2), w_up=lin(E, H, 10 * i + 3), w_down=lin(H, E, 10 * i + 4))
               for i in range(cfg.n_layers)]
+    if stream_order:
+        for l in layers:
+            l.with_stream()
+            l.wqkv = l.wo = l.w_gate = l.w_up = l.w_down = None
     embed = torch.randn((cfg.vocab_size, E), device="cuda", generator=g).to(torch.bfloat16)
     final_norm = norm_w()
     lut = decode.generate_rope_lut(cfg, M)
@@ -642,7 +654,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b", "decode_8b", "prefill_block", "prefill_1b"])
+    ap.add_argument("--workload", default="gemv", choices=list(CONFIGS) + ["decode_1b", "decode_8b", "prefill_block", "prefill_block_awq", "prefill_1b", "prefill_1b_awq",
+                                                             "prefill_8b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the short runs of the other configs")
     ap.add_argument("--copy-probe", action="store_true",
@@ -669,29 +682,35 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    if a.workload == "prefill_1b":
-        r = run_prefill_model("decode_1b", 2048, max(1, min(a.steps, 5)))
+    if a.workload in ("prefill_1b", "prefill_1b_awq", "prefill_8b"):
+        model = "decode_8b" if a.workload == "prefill_8b" else "decode_1b"
+        r = run_prefill_model(model, 2048, max(1, min(a.steps, 5)), stream_order=not a.workload.endswith("_awq"))
+        c = DECODE_MODELS[model]
+        shape = (f"{c['n_layers']} layers E={c['emb_dim']} H={c['hidden_dim']} {c['n_heads']}/{c['n_kv_heads']} heads "
+                 f"hd={c['head_dim']} V={c['vocab_size']} g128")
+        layout = "checkpoint-layout" if a.workload.endswith("_awq") else "stream-order"
         print(json.dumps({
-            "metric": "int4 prefill tokens/s, Llama-3.2-1B shape, 2048-token prompt", "value": r["tokens_per_s"], "unit": "tokens/s",
+            "metric": f"int4 prefill tokens/s, {'Llama-3.1-8B' if model == 'decode_8b' else 'Llama-3.2-1B'} shape, 2048-token prompt", "value": r["tokens_per_s"], "unit": "tokens/s",
             "n_gpus": 1, "steps": max(1, min(a.steps, 5)), "warmup": 1, "ms_per_step": r["ms"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights (bf16 lm_head), bf16 activations, fp32 accumulate",
             "data": "synthetic (random weights of the architecture, random prompt)",
-            "config": {"workload": "prompt pass, 16 layers E=2048 H=8192 32/8 heads hd=64 V=128256 g128, 2048 tokens, causal attention, KV caches filled",
+            "config": {"workload": f"prompt pass, {shape}, 2048 tokens, causal attention, KV caches filled, {layout} weights",
                        "timing": "one HIP graph of the whole pass, events on the launch stream"},
             "roofline": {"bound": "mfma", "achieved": r["TFLOP/s"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_per_launch": r["flops"],
                          "avg_launch_us": r["ms"] * 1e3},
             "finite": r["finite"]}))
         return
-    if a.workload == "prefill_block":
+    if a.workload in ("prefill_block", "prefill_block_awq"):
         steps = min(a.steps, 20)
-        r = run_prefill_block(steps, min(a.warmup, 3))
+        r = run_prefill_block(steps, min(a.warmup, 3), stream_order=a.workload == "prefill_block")
         print(json.dumps({
             "metric": "W4A16 prefill O + FFN block TFLOP/s", "value": r["TFLOP/s"], "unit": "TFLOP/s", "n_gpus": 1,
             "steps": steps, "warmup": min(a.warmup, 3), "ms_per_step": r["us"] * 1e-3, "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights, bf16 activations, fp32 accumulate",
             "data": "synthetic (uniform uint4 q/z, scales (|N(0,1)|*0.02+1e-3)*0.1, activations ~ N(0,1))",
-            "config": {"workload": "prefill O-proj + residual + RMSNorm + SwiGLU FFN + residual, M=2048 E=2048 H=8192 g128",
+            "config": {"workload": "prefill O-proj + residual + RMSNorm + SwiGLU FFN + residual, M=2048 E=2048 H=8192 g128, "
+                                   + ("stream-order weights" if a.workload == "prefill_block" else "checkpoint-layout weights"),
                        "timing": "HIP graph of K calls (5 to 7 launches each), events on the launch stream"},
             "roofline": {"bound": "mfma", "achieved": r["TFLOP/s"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "algorithmic_per_launch": r["flops"],

@@ -401,6 +401,23 @@ int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residua
                              void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The two prompt-pass blocks on stream-order weights (w4a16_repack_stream of the same matrices; the Q|K|V matrices
+ * concatenated along N before the re-pack): w4a16_prefill_rms_qkv_rope_bf16 and w4a16_prefill_o_ffn_bf16 with the tiled
+ * stream-order GEMM (w4a16_gemm_stream_bf16's kernel for M >= 97) and its fused epilogues in place of the
+ * checkpoint-layout GEMM.  Same references (rms_gemms_rope_int4_multi.py:4-17, 414-436, 543-561;
+ * o_ffn_int4_multi.py:4-17, 644-665), same rounding points, same workspaces (w4a16_prefill_qkv_workspace_bytes,
+ * w4a16_prefill_block_workspace_bytes; plain scratch).  E % 256 == 0, H % 256 == 0, every N % 64 == 0.
+ */
+int w4a16_prefill_rms_qkv_rope_stream_bf16(const uint16_t *x, const uint16_t *attn_norm_weight, float eps, const void *qkv_wstream,
+                                           const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out, int M, int E,
+                                           int n_heads, int n_kv_heads, int head_dim, int group, void *workspace,
+                                           size_t workspace_bytes, void *stream);
+int w4a16_prefill_o_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                                    const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                    const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
+                                    int H, int group, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Prefill counterpart of w4a16_rms_gemv_bf16 + the RoPE of w4a16_decode_attention_bf16 for M tokens at
  * positions pos0 .. pos0 + M - 1: the reference's 6-launch ELF `rms_gemms_rope_int4`
  * (programming_examples/llms/llama32_1b_int4/multi_launch_builder/rms_gemms_rope_int4_multi.py:4-17; CPU reference

@@ -159,6 +159,13 @@ def decode_greedy(token, n_tokens, layers, embed_table, final_norm, lm_head, con
     return out
 
 
+def _prefill_stream_shapes(config):
+    """Shapes the stream-order prompt-pass blocks take: input lengths in whole pairs of groups, widths in whole
+    64-column tiles, attention output as wide as the embedding."""
+    E, H, nq = config.emb_dim, config.hidden_dim, config.n_heads * config.head_dim
+    return E % 256 == 0 and H % 256 == 0 and nq == E and (nq + 2 * config.kv_dim) % 64 == 0
+
+
 def run_prefill_layer(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer, rope_lut):
     """One transformer block over the M prompt tokens at positions 0..M-1 (_run_layer_int4,
     programming_examples/llms/llama32_1b_int4/llama32_1b_int4_prefill.py:241-390): RMSNorm + fused Q|K|V GEMM +
@@ -169,11 +176,18 @@ def run_prefill_layer(x, layer: DecodeLayer, config, k_cache_layer, v_cache_laye
         raise ValueError("the prefill kernels take AWQ layers (the reference prefills its Q4NX models in bf16)")
     M = x.shape[0]
     nh, nkv, hd = config.n_heads, config.n_kv_heads, config.head_dim
-    qkv = ops.prefill_rms_qkv_rope(x, layer.attn_norm, layer.wqkv, rope_lut, 0, nh, nkv, hd, eps=config.rms_eps)
+    # the stream-order copies where the layer has them and the tiled stream-order GEMM takes every matrix
+    sw = layer.stream if layer.stream is not None and _prefill_stream_shapes(config) else None
+    if sw is not None:
+        qkv = ops.prefill_rms_qkv_rope_stream(x, layer.attn_norm, sw["wqkv"], rope_lut, 0, nh, nkv, hd, eps=config.rms_eps)
+    else:
+        qkv = ops.prefill_rms_qkv_rope(x, layer.attn_norm, layer.wqkv, rope_lut, 0, nh, nkv, hd, eps=config.rms_eps)
     nq, nk = nh * hd, nkv * hd
     k_cache_layer[:, :M].copy_(qkv[:, nq:nq + nk].reshape(M, nkv, hd).transpose(0, 1))
     v_cache_layer[:, :M].copy_(qkv[:, nq + nk:].reshape(M, nkv, hd).transpose(0, 1))
     attn_out = ops.prefill_attention(qkv, nh, nkv, hd)
+    if sw is not None:
+        return ops.prefill_o_ffn_stream(attn_out, x, layer.ffn_norm, sw["wo"], sw["w_gate"], sw["w_up"], sw["w_down"], eps=config.rms_eps)
     return ops.prefill_o_ffn(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
 
 

@@ -608,6 +608,51 @@ def prefill_o_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps
     return (y, res1, h) if return_intermediates else y
 
 
+def prefill_rms_qkv_rope_stream(x, attn_norm_weight, wqkv, rope_lut, pos0, n_heads, n_kv_heads, head_dim, eps=1e-5, group=GROUP):
+    """prefill_rms_qkv_rope on a StreamWeight (the re-pack of the concatenated Q|K|V matrix): the tiled stream-order
+    GEMM with the RoPE epilogue in place of the checkpoint-layout GEMM, same rounding points."""
+    lib = _lib.load_library()
+    _need_cuda(x, attn_norm_weight, rope_lut, wqkv.buf)
+    M, E = x.shape
+    N = (n_heads + 2 * n_kv_heads) * head_dim
+    if (wqkv.K, wqkv.N) != (E, N):
+        raise ValueError(f"wqkv is [{wqkv.K}, {wqkv.N}], the block needs [{E}, {N}]")
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    key = (x.device.index, _stream(), "prefill_qkv", M, E)
+    ws = _attn_ws.get(key)
+    if ws is None:
+        ws = torch.empty(int(lib.w4a16_prefill_qkv_workspace_bytes(M, E)), dtype=torch.uint8, device=x.device)
+        _attn_ws[key] = ws
+    _lib.check(lib.w4a16_prefill_rms_qkv_rope_stream_bf16(_ptr(_bits(x)), _ptr(_bits(attn_norm_weight)), float(eps), _ptr(wqkv.buf),
+                                                          _ptr(_bits(rope_lut)), rope_lut.shape[0], int(pos0), _ptr(out), M, E,
+                                                          n_heads, n_kv_heads, head_dim, group, _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def prefill_o_ffn_stream(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, group=GROUP,
+                         return_intermediates=False):
+    """prefill_o_ffn on four StreamWeights: bf16 [M, E] -> [M, E]; with return_intermediates also res1 [M, E] and h [M, H]."""
+    lib = _lib.load_library()
+    _need_cuda(attn_out, x_residual, ffn_norm_weight, wo.buf, gate.buf, up.buf, down.buf)
+    M, E = attn_out.shape
+    H = gate.N
+    if (wo.K, wo.N) != (E, E) or (gate.K, up.K, up.N) != (E, E, H) or (down.K, down.N) != (H, E):
+        raise ValueError("prefill_o_ffn_stream: wo [E, E], gate and up [E, H], down [H, E]")
+    y = torch.empty((M, E), dtype=torch.bfloat16, device=attn_out.device)
+    res1 = torch.empty((M, E), dtype=torch.bfloat16, device=attn_out.device) if return_intermediates else None
+    h = torch.empty((M, H), dtype=torch.bfloat16, device=attn_out.device) if return_intermediates else None
+    key = (attn_out.device.index, _stream(), "prefill_block", M, E, H)
+    ws = _attn_ws.get(key)
+    if ws is None:
+        ws = torch.empty(int(lib.w4a16_prefill_block_workspace_bytes(M, E, H)), dtype=torch.uint8, device=attn_out.device)
+        _attn_ws[key] = ws
+    _lib.check(lib.w4a16_prefill_o_ffn_stream_bf16(_ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)),
+                                                   float(eps), _ptr(wo.buf), _ptr(gate.buf), _ptr(up.buf), _ptr(down.buf), _ptr(y),
+                                                   _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
+                                                   M, E, H, group, _ptr(ws), ws.numel(), _stream()))
+    return (y, res1, h) if return_intermediates else y
+
+
 def lm_head(x, lm_head_weight, norm_weight=None, eps=1e-5, return_argmax=True):
     """Tail of a decode step: logits bf16 [V] = lm_head_weight [V, E] . rms_norm(x) (x itself when
     norm_weight is None), and the index of the largest logit as a device int32 tensor [1]."""

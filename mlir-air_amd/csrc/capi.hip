@@ -733,6 +733,46 @@ int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residua
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+int w4a16_prefill_rms_qkv_rope_stream_bf16(const uint16_t *x, const uint16_t *attn_norm_weight, float eps, const void *qkv_wstream,
+                                           const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out, int M, int E,
+                                           int n_heads, int n_kv_heads, int head_dim, int group, void *workspace,
+                                           size_t workspace_bytes, void *stream) {
+    if (!x || !attn_norm_weight || !qkv_wstream || !rope_lut || !qkv_out) return W4A16_ERR_NULL;
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    if (head_dim != 64 && head_dim != 128) return W4A16_ERR_SHAPE;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads > 1024 || n_kv_heads > 1024) return W4A16_ERR_SHAPE;
+    const int N = (n_heads + 2 * n_kv_heads) * head_dim;
+    if (!prefill_block_supported(M, E, 8) || !gemm_prefill_ws_supported(M, E, N) || !(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (pos0 < 0 || rope_lut_rows <= 0 || pos0 > rope_lut_rows - M) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(attn_norm_weight) || misaligned(qkv_wstream) || misaligned(rope_lut) || misaligned(qkv_out))
+        return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_prefill_qkv_workspace_bytes(M, E)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_prefill_rms_qkv_rope_stream(x, attn_norm_weight, eps, qkv_wstream, rope_lut, pos0, qkv_out, M, E, n_heads,
+                                                      n_kv_heads, head_dim, static_cast<uint16_t *>(workspace),
+                                                      static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_prefill_o_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                                    const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                    const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
+                                    int H, int group, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!attn_out || !x_residual || !ffn_norm_weight || !y || !o_wstream || !gate_wstream || !up_wstream || !down_wstream)
+        return W4A16_ERR_NULL;
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    if (!prefill_block_stream_supported(M, E, H) || !(eps >= 0.f)) return W4A16_ERR_SHAPE;
+    if (misaligned(attn_out) || misaligned(x_residual) || misaligned(ffn_norm_weight) || misaligned(y) || misaligned(o_wstream) ||
+        misaligned(gate_wstream) || misaligned(up_wstream) || misaligned(down_wstream) || (res1_out && misaligned(res1_out)) ||
+        (h_out && misaligned(h_out)))
+        return W4A16_ERR_ALIGN;
+    if (!workspace || workspace_bytes < w4a16_prefill_block_workspace_bytes(M, E, H)) return W4A16_ERR_WORKSPACE;
+    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_prefill_o_ffn_stream(attn_out, x_residual, ffn_norm_weight, eps, o_wstream, gate_wstream, up_wstream,
+                                               down_wstream, y, res1_out, h_out, M, E, H, workspace, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim) {
     if (n_heads <= 0 || head_dim <= 0) return 0;
     return round256(attention_workspace_bytes(n_heads, head_dim));

@@ -170,6 +170,9 @@ struct PfArgs {
     int M, K, N, G, NB;
     int tiles_m;
     int n_wide, n_narrow;   // column tiles of each width
+    const uint16_t *aux;    // operand of the epilogue: residual / gate [M, N], or the RoPE table [positions, head_dim]
+    int epi;                // kEpi*
+    int rope_cols, rope_hd, rope_pos0;
 };
 
 // One output tile: rows m0 .., columns col0 .. col0 + 64 NCB - 1.
@@ -430,12 +433,55 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
                 ct[(16 * r + 4 * lg + i) * LDC + wave * WN + 16 * c + ln] = float_to_bf16_bits(acc[r][c][i]);
     __syncthreads();
     constexpr int CPR = TN / 8;   // 16-byte chunks per row
-    for (int chunk = threadIdx.x; chunk < TM * CPR; chunk += kPfThreads) {
-        const int row = chunk / CPR, cc = chunk % CPR;
-        if (m0 + row >= M) continue;
-        const u32x4 v = *reinterpret_cast<const u32x4 *>(&ct[row * LDC + 8 * cc]);
-        *reinterpret_cast<u32x4 *>(p.y + (size_t)(m0 + row) * N + col0 + 8 * cc) = v;
-    }
+    // Epilogues on the bf16 tile (the same four as the checkpoint-layout kernel's): plain store; residual add of the
+    // bf16 product, y = bf16(bf16(x . W) + aux); SwiGLU with aux = the gate projection, y = bf16(silu(aux) * bf16(x . W)),
+    // silu(g) = g / (1 + exp(-g)) in fp32; half-split RoPE of the bf16 product on columns [0, rope_cols), whose
+    // partner chunk is in the same tile (the tile widths offered to such a launch are whole numbers of heads).
+    auto store_tile = [&](auto EPI) {
+        constexpr int kEpi = decltype(EPI)::value;
+        for (int chunk = threadIdx.x; chunk < TM * CPR; chunk += kPfThreads) {
+            const int row = chunk / CPR, cc = chunk % CPR;
+            if (m0 + row >= M) continue;
+            u32x4 v = *reinterpret_cast<const u32x4 *>(&ct[row * LDC + 8 * cc]);
+            const int grow = m0 + row, gcol = col0 + 8 * cc;
+            const size_t at = (size_t)grow * N + gcol;
+            if constexpr (kEpi == kEpiRope) {
+                if (gcol < p.rope_cols) {
+                    const int hd = p.rope_hd, half = hd >> 1;
+                    const int i = gcol & (hd - 1);
+                    const bool low = i < half;
+                    const u32x4 w2 = *reinterpret_cast<const u32x4 *>(&ct[row * LDC + 8 * cc + (low ? half : -half)]);
+                    const uint16_t *lut = p.aux + (size_t)(p.rope_pos0 + grow) * hd + (low ? i : i - half);
+                    const u32x4 cs = *reinterpret_cast<const u32x4 *>(lut), sn = *reinterpret_cast<const u32x4 *>(lut + half);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t vw = v[e], ww = w2[e], cw = cs[e], sw = sn[e];
+                        const float x0 = bf16_bits_to_float(vw & 0xFFFFu), x1 = bf16_bits_to_float(vw >> 16);
+                        const float y0 = bf16_bits_to_float(ww & 0xFFFFu), y1 = bf16_bits_to_float(ww >> 16);
+                        const float c0 = bf16_bits_to_float(cw & 0xFFFFu), c1 = bf16_bits_to_float(cw >> 16);
+                        const float s0 = bf16_bits_to_float(sw & 0xFFFFu), s1 = bf16_bits_to_float(sw >> 16);
+                        v[e] = low ? pack_bf16x2(x0 * c0 - y0 * s0, x1 * c1 - y1 * s1)
+                                   : pack_bf16x2(x0 * c0 + y0 * s0, x1 * c1 + y1 * s1);
+                    }
+                }
+            } else if constexpr (kEpi != kEpiNone) {
+                const u32x4 a4 = *reinterpret_cast<const u32x4 *>(p.aux + at);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t vw = v[e], aw = a4[e];
+                    const float v0 = bf16_bits_to_float(vw & 0xFFFFu), v1 = bf16_bits_to_float(vw >> 16);
+                    const float a0 = bf16_bits_to_float(aw & 0xFFFFu), a1 = bf16_bits_to_float(aw >> 16);
+                    if constexpr (kEpi == kEpiAddRounded) v[e] = pack_bf16x2(v0 + a0, v1 + a1);
+                    else v[e] = pack_bf16x2(a0 / (1.0f + expf(-a0)) * v0, a1 / (1.0f + expf(-a1)) * v1);
+                }
+            }
+            *reinterpret_cast<u32x4 *>(p.y + at) = v;
+        }
+    };
+    if (p.epi == kEpiAddRounded) store_tile(std::integral_constant<int, kEpiAddRounded>{});
+    else if (p.epi == kEpiSiluGateMul) store_tile(std::integral_constant<int, kEpiSiluGateMul>{});
+    else if (p.epi == kEpiRope) store_tile(std::integral_constant<int, kEpiRope>{});
+    else store_tile(std::integral_constant<int, kEpiNone>{});
 }
 
 // blockIdx -> tile.  The wide tiles come first in dispatch order, so that the narrow ones fill in behind them.  Each
@@ -483,9 +529,11 @@ long split_cost(long n_wide_tiles, long n_narrow_tiles, int cus) {
     return *std::max_element(load.begin(), load.end());
 }
 
-Widths pick_widths(int tiles_m, int U, int cus) {
+// `heads128`: every tile must hold whole heads of 128 columns (RoPE epilogue): no 192- or 64-column tiles.
+Widths pick_widths(int tiles_m, int U, int cus, bool heads128) {
     struct Entry {
         int tiles_m, U, cus;
+        bool heads128;
         Widths w;
     };
     static std::mutex mu;
@@ -493,12 +541,13 @@ Widths pick_widths(int tiles_m, int U, int cus) {
     static int next = 0;
     std::lock_guard<std::mutex> lock(mu);
     for (const Entry &e : cache)
-        if (e.U == U && e.tiles_m == tiles_m && e.cus == cus) return e.w;
+        if (e.U == U && e.tiles_m == tiles_m && e.cus == cus && e.heads128 == heads128) return e.w;
     Widths best{4, -1, -1};
     double best_cost = -1;
     for (int a = U / 4; a >= 0; --a) {   // ties go to the split with more wide tiles
         if ((U - 4 * a) % 3) continue;
         const int b = (U - 4 * a) / 3;
+        if (heads128 && b) continue;
         const double cost = (double)split_cost((long)tiles_m * a, (long)tiles_m * b, cus);
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;
@@ -508,7 +557,7 @@ Widths pick_widths(int tiles_m, int U, int cus) {
     // uniform narrow tilings: rounds x width x (measured) slowdown of the narrower tile's inner loop
     const struct { int ncb; double slowdown; } narrow[2] = {{2, kPfSlowdown128}, {1, kPfSlowdown64}};
     for (const auto &nv : narrow) {
-        if (U % nv.ncb) continue;
+        if (U % nv.ncb || (heads128 && nv.ncb == 1)) continue;
         const long tiles = (long)tiles_m * (U / nv.ncb);
         const double cost = (double)((tiles + cus - 1) / cus) * nv.ncb * nv.slowdown;
         if (best_cost < 0 || cost < best_cost) {
@@ -516,7 +565,7 @@ Widths pick_widths(int tiles_m, int U, int cus) {
             best = Widths{nv.ncb, U / nv.ncb, 0};
         }
     }
-    cache[next] = Entry{tiles_m, U, cus, best};
+    cache[next] = Entry{tiles_m, U, cus, heads128, best};
     next = (next + 1) % 8;
     return best;
 }
@@ -539,22 +588,30 @@ hipError_t launch_wsp(const PfArgs &p, hipStream_t stream) {
 
 bool gemm_prefill_ws_supported(int M, int K, int N) { return M > 0 && K > 0 && K % (2 * kGroup) == 0 && N > 0 && N % 64 == 0; }
 
-hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream) {
+hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream, int epi,
+                                  const uint16_t *aux, const GemmRope *rope) {
     if (!gemm_prefill_ws_supported(M, K, N)) return hipErrorInvalidValue;
+    if ((epi != kEpiNone && !aux) || (epi == kEpiRope && (!rope || (rope->head_dim != 64 && rope->head_dim != 128) ||
+                                                          rope->cols % rope->head_dim || N % rope->head_dim)))
+        return hipErrorInvalidValue;
     PfArgs p{};
     p.x = x;
     p.w = static_cast<const char *>(w);
     p.y = y;
+    p.aux = aux;
+    p.epi = epi;
+    if (epi == kEpiRope) p.rope_cols = rope->cols, p.rope_hd = rope->head_dim, p.rope_pos0 = rope->pos0;
+    const bool heads128 = epi == kEpiRope && rope->head_dim == 128;
     p.M = M, p.K = K, p.N = N, p.G = K / kGroup, p.NB = ws_blocks(K);
     p.tiles_m = (M + kPfRows - 1) / kPfRows;
     const int U = N / 64;
-    Widths wd = pick_widths(p.tiles_m, U, 256);
+    Widths wd = pick_widths(p.tiles_m, U, 256, heads128);
     // tuning: one tile width only (1: 256 columns, 2: 192, 3: 128, 4: 64) where it divides N
     const int force = g_gemv_ws_tune.prefill_tile;
     if (force == 1 && U % 4 == 0) wd = Widths{4, U / 4, 0};
-    if (force == 2 && U % 3 == 0) wd = Widths{4, 0, U / 3};
+    if (force == 2 && U % 3 == 0 && !heads128) wd = Widths{4, 0, U / 3};
     if (force == 3 && U % 2 == 0) wd = Widths{2, U / 2, 0};
-    if (force == 4) wd = Widths{1, U, 0};
+    if (force == 4 && !heads128) wd = Widths{1, U, 0};
     p.n_wide = wd.wide, p.n_narrow = wd.narrow;
     if (wd.ncb == 2) return launch_wsp<2, 0>(p, stream);
     if (wd.ncb == 1) return launch_wsp<1, 0>(p, stream);

@@ -123,8 +123,10 @@ hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, ui
 hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
                           hipStream_t stream);
 // Prefill GEMM on stream-order weights (gemm_ws.hip): bf16-rounded weights dequantised in registers, x through LDS.
-bool gemm_prefill_ws_supported(int M, int K, int N);   // N % 448 == 0 or N % 256 == 0
-hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream);
+bool gemm_prefill_ws_supported(int M, int K, int N);   // K % 256 == 0, N % 64 == 0
+// Epilogues as for launch_gemm_prefill (kEpi*); kEpiRope with heads of 128 needs N % 128 == 0.
+hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream,
+                                  int epi = kEpiNone, const uint16_t *aux = nullptr, const GemmRope *rope = nullptr);
 // AutoAWQ checkpoint tensors -> stream order (ws_matrix_bytes(K, N) bytes at `out`).
 hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *out, int K, int N,
                             hipStream_t stream);
@@ -149,6 +151,15 @@ hipError_t launch_prefill_o_ffn(const uint16_t *attn_out, const uint16_t *x_resi
                                 const PrefillLinear &wo, const PrefillLinear &wg, const PrefillLinear &wu,
                                 const PrefillLinear &wd, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
                                 int H, void *workspace, int cus, hipStream_t stream);
+// The same blocks on stream-order weights (every matrix re-packed with launch_repack_ws).
+bool prefill_block_stream_supported(int M, int E, int H);
+hipError_t launch_prefill_rms_qkv_rope_stream(const uint16_t *x, const uint16_t *norm_w, float eps, const void *wqkv,
+                                              const uint16_t *rope_lut, int pos0, uint16_t *qkv_out, int M, int E, int n_heads,
+                                              int n_kv, int head_dim, uint16_t *normed, hipStream_t stream);
+hipError_t launch_prefill_o_ffn_stream(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_w, float eps,
+                                       const void *wo, const void *wg, const void *wu, const void *wd, uint16_t *y,
+                                       uint16_t *res1_out, uint16_t *h_out, int M, int E, int H, void *workspace,
+                                       hipStream_t stream);
 
 // Decode FFN as one persistent kernel (ffn_fused.hip).  plan_ffn_fused returns false for shapes
 // the kernel does not take (the caller then runs the two streaming launches).

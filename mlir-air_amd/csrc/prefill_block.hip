@@ -137,4 +137,45 @@ hipError_t launch_prefill_o_ffn(const uint16_t *attn_out, const uint16_t *x_resi
     return launch_gemm_prefill(h, wd.qw, wd.qz, wd.sc, y, M, H, E, stream, kEpiAddRounded, res1, sk, cus);
 }
 
+// The same two blocks on stream-order weights (gemm_ws.hip): no split-K scratch, the narrow-tile choice of that kernel
+// covers the projections with few tiles.
+bool prefill_block_stream_supported(int M, int E, int H) {
+    return prefill_block_supported(M, E, H) && gemm_prefill_ws_supported(M, E, E) && gemm_prefill_ws_supported(M, E, H) &&
+           gemm_prefill_ws_supported(M, H, E);
+}
+
+hipError_t launch_prefill_rms_qkv_rope_stream(const uint16_t *x, const uint16_t *norm_w, float eps, const void *wqkv,
+                                              const uint16_t *rope_lut, int pos0, uint16_t *qkv_out, int M, int E, int n_heads,
+                                              int n_kv, int head_dim, uint16_t *normed, hipStream_t stream) {
+    hipError_t e = launch_rmsnorm_rows(x, norm_w, normed, M, E, eps, stream);
+    if (e != hipSuccess) return e;
+    const GemmRope rope = {(n_heads + n_kv) * head_dim, head_dim, pos0};
+    return launch_gemm_prefill_ws(normed, wqkv, qkv_out, M, E, (n_heads + 2 * n_kv) * head_dim, stream, kEpiRope, rope_lut, &rope);
+}
+
+hipError_t launch_prefill_o_ffn_stream(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_w, float eps,
+                                       const void *wo, const void *wg, const void *wu, const void *wd, uint16_t *y,
+                                       uint16_t *res1_out, uint16_t *h_out, int M, int E, int H, void *workspace,
+                                       hipStream_t stream) {
+    char *base = static_cast<char *>(workspace);
+    uint16_t *res1 = reinterpret_cast<uint16_t *>(base);
+    base += round256((size_t)M * E * sizeof(uint16_t));
+    uint16_t *normed = reinterpret_cast<uint16_t *>(base);
+    base += round256((size_t)M * E * sizeof(uint16_t));
+    uint16_t *gate = reinterpret_cast<uint16_t *>(base);
+    base += round256((size_t)M * H * sizeof(uint16_t));
+    uint16_t *h = reinterpret_cast<uint16_t *>(base);
+    if (res1_out) res1 = res1_out;
+    if (h_out) h = h_out;
+    hipError_t e = launch_gemm_prefill_ws(attn_out, wo, res1, M, E, E, stream, kEpiAddRounded, x_residual);
+    if (e != hipSuccess) return e;
+    e = launch_rmsnorm_rows(res1, ffn_norm_w, normed, M, E, eps, stream);
+    if (e != hipSuccess) return e;
+    e = launch_gemm_prefill_ws(normed, wg, gate, M, E, H, stream);
+    if (e != hipSuccess) return e;
+    e = launch_gemm_prefill_ws(normed, wu, h, M, E, H, stream, kEpiSiluGateMul, gate);
+    if (e != hipSuccess) return e;
+    return launch_gemm_prefill_ws(h, wd, y, M, H, E, stream, kEpiAddRounded, res1);
+}
+
 }  // namespace w4a16
