@@ -163,6 +163,11 @@ __device__ __forceinline__ void decode_md(uint32_t md, float &sf, float &c0) {
     c0 = (nz + 128.0f) * sf;
 }
 
+// Gate and up projection in one tile (launch_gemm_prefill_ws_swiglu): a tile of 64 NCB columns holds 32 NCB columns of
+// x . W_gate and the same columns of x . W_up, each wave half and half, and leaves as 32 NCB columns of
+// bf16(silu(bf16 gate) * bf16 up).  N is the width of that output; the tile grid runs over 2 N columns.
+constexpr int kEpiSwigluPair = 16;
+
 struct PfArgs {
     const uint16_t *x;
     const char *w;
@@ -171,7 +176,8 @@ struct PfArgs {
     int tiles_m;
     int n_wide, n_narrow;   // column tiles of each width
     const uint16_t *aux;    // operand of the epilogue: residual / gate [M, N], or the RoPE table [positions, head_dim]
-    int epi;                // kEpi*
+    const char *w_up;       // kEpiSwigluPair: the second matrix (the tile's left half multiplies w, its right half w_up)
+    int epi;                // kEpi*, or kEpiSwigluPair
     int rope_cols, rope_hd, rope_pos0;
 };
 
@@ -226,7 +232,8 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
 
     // this wave's NCB tiles of the stream-order buffer
     const size_t tile_bytes = (size_t)(p.NB + G) * kWsCellBytes;
-    const char *wt = p.w + (size_t)(n0 / kWsTileCols) * tile_bytes;
+    const bool pair = p.epi == kEpiSwigluPair;
+    const char *wt = p.w + (size_t)((pair ? n0 / 2 : n0) / kWsTileCols) * tile_bytes;
     u32x4 cell[2][NCB];
     uint32_t md[2][NCB];
     uint32_t lane16 = (uint32_t)lane * 16, ln16 = (uint32_t)ln * 16;
@@ -236,7 +243,12 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     // else in the loop.
     gptr tile_base[NCB];
 #pragma unroll
-    for (int c = 0; c < NCB; ++c) tile_base[c] = scalar_ptr(wt + (size_t)c * tile_bytes);
+    for (int c = 0; c < NCB; ++c) {
+        const char *t = wt + (size_t)c * tile_bytes;
+        if (pair && NCB % 2 == 0)   // tiles NCB / 2 .. NCB - 1 of the wave: the same columns of the second matrix
+            t = c < NCB / 2 ? t : p.w_up + (t - p.w) - (size_t)(NCB / 2) * tile_bytes;
+        tile_base[c] = scalar_ptr(t);
+    }
     struct WOffsets {
         uint32_t md, cell;
     };
@@ -478,7 +490,26 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
             *reinterpret_cast<u32x4 *>(p.y + at) = v;
         }
     };
-    if (p.epi == kEpiAddRounded) store_tile(std::integral_constant<int, kEpiAddRounded>{});
+    if (pair) {
+        if constexpr (NCB % 2 == 0) {
+            constexpr int HW = WN / 2, OCPR = TN / 16;   // output columns per wave, 16-byte output chunks per row
+            const int Nout = N, ocol0 = col0 / 2;
+            for (int chunk = threadIdx.x; chunk < TM * OCPR; chunk += kPfThreads) {
+                const int row = chunk / OCPR, oc = 8 * (chunk % OCPR);
+                if (m0 + row >= M) continue;
+                const uint16_t *src = &ct[row * LDC + (oc / HW) * WN + oc % HW];
+                const u32x4 gv = *reinterpret_cast<const u32x4 *>(src), uv = *reinterpret_cast<const u32x4 *>(src + HW);
+                u32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float g0 = bf16_bits_to_float(gv[e] & 0xFFFFu), g1 = bf16_bits_to_float(gv[e] >> 16);
+                    const float u0 = bf16_bits_to_float(uv[e] & 0xFFFFu), u1 = bf16_bits_to_float(uv[e] >> 16);
+                    v[e] = pack_bf16x2(g0 / (1.0f + expf(-g0)) * u0, g1 / (1.0f + expf(-g1)) * u1);
+                }
+                *reinterpret_cast<u32x4 *>(p.y + (size_t)(m0 + row) * Nout + ocol0 + oc) = v;
+            }
+        }
+    } else if (p.epi == kEpiAddRounded) store_tile(std::integral_constant<int, kEpiAddRounded>{});
     else if (p.epi == kEpiSiluGateMul) store_tile(std::integral_constant<int, kEpiSiluGateMul>{});
     else if (p.epi == kEpiRope) store_tile(std::integral_constant<int, kEpiRope>{});
     else store_tile(std::integral_constant<int, kEpiNone>{});
@@ -621,6 +652,28 @@ hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y,
     }
     if (wd.narrow == 0) return launch_wsp<4, 0>(p, stream);
     return launch_wsp<4, 3>(p, stream);
+}
+
+// h[M, H] = bf16(silu(bf16(x . W_gate)) * bf16(x . W_up)): both projections in one launch, a tile holding the same
+// 128 (or 64) columns of either; the gate projection never leaves the chip.  H % 64 == 0.
+hipError_t launch_gemm_prefill_ws_swiglu(const uint16_t *x, const void *w_gate, const void *w_up, uint16_t *h, int M, int K, int H,
+                                         hipStream_t stream) {
+    if (!gemm_prefill_ws_supported(M, K, H) || !w_up) return hipErrorInvalidValue;
+    PfArgs p{};
+    p.x = x;
+    p.w = static_cast<const char *>(w_gate);
+    p.w_up = static_cast<const char *>(w_up);
+    p.y = h;
+    p.epi = kEpiSwigluPair;
+    p.M = M, p.K = K, p.N = H, p.G = K / kGroup, p.NB = ws_blocks(K);
+    p.tiles_m = (M + kPfRows - 1) / kPfRows;
+    const int U = 2 * H / 64;   // the tile grid runs over 2 H columns; 192- and 64-column tiles cannot be halved
+    Widths wd = pick_widths(p.tiles_m, U, 256, true);
+    const int force = g_gemv_ws_tune.prefill_tile;
+    if (force == 1 && U % 4 == 0) wd = Widths{4, U / 4, 0};
+    if (force == 3) wd = Widths{2, U / 2, 0};
+    p.n_wide = wd.wide, p.n_narrow = 0;
+    return wd.ncb == 2 ? launch_wsp<2, 0>(p, stream) : launch_wsp<4, 0>(p, stream);
 }
 
 }  // namespace w4a16

@@ -109,6 +109,7 @@ struct GemvWsTune {
     int cb = 0;      // batched kernel: 16-column tiles per workgroup, 1, 2 or 4 (0 = by the number of tiles)
     int prefill_tile = 0;    // prefill kernel: 0 = by shape, 1 = 128 x 448 tiles, 2 = 256 x 256 tiles
     int prefill_min_m = 0;   // smallest M that w4a16_gemm_stream_bf16 gives to the prefill kernel (0 = default)
+    int prefill_swiglu_split = 0;   // 1: the prompt-pass FFN runs gate and up as two launches instead of one
 };
 extern GemvWsTune g_gemv_ws_tune;
 struct GemvWsPlan {
@@ -127,6 +128,10 @@ bool gemm_prefill_ws_supported(int M, int K, int N);   // K % 256 == 0, N % 64 =
 // Epilogues as for launch_gemm_prefill (kEpi*); kEpiRope with heads of 128 needs N % 128 == 0.
 hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream,
                                   int epi = kEpiNone, const uint16_t *aux = nullptr, const GemmRope *rope = nullptr);
+// h[M, H] = bf16(silu(bf16(x . W_gate)) * bf16(x . W_up)) in one launch (H % 64 == 0): bit for bit the gate launch followed
+// by the up launch with kEpiSiluGateMul.
+hipError_t launch_gemm_prefill_ws_swiglu(const uint16_t *x, const void *w_gate, const void *w_up, uint16_t *h, int M, int K, int H,
+                                         hipStream_t stream);
 // AutoAWQ checkpoint tensors -> stream order (ws_matrix_bytes(K, N) bytes at `out`).
 hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *out, int K, int N,
                             hipStream_t stream);

@@ -171,9 +171,13 @@ hipError_t launch_prefill_o_ffn_stream(const uint16_t *attn_out, const uint16_t 
     if (e != hipSuccess) return e;
     e = launch_rmsnorm_rows(res1, ffn_norm_w, normed, M, E, eps, stream);
     if (e != hipSuccess) return e;
-    e = launch_gemm_prefill_ws(normed, wg, gate, M, E, H, stream);
-    if (e != hipSuccess) return e;
-    e = launch_gemm_prefill_ws(normed, wu, h, M, E, H, stream, kEpiSiluGateMul, gate);
+    if (g_gemv_ws_tune.prefill_swiglu_split) {
+        e = launch_gemm_prefill_ws(normed, wg, gate, M, E, H, stream);
+        if (e != hipSuccess) return e;
+        e = launch_gemm_prefill_ws(normed, wu, h, M, E, H, stream, kEpiSiluGateMul, gate);
+    } else {
+        e = launch_gemm_prefill_ws_swiglu(normed, wg, wu, h, M, E, H, stream);
+    }
     if (e != hipSuccess) return e;
     return launch_gemm_prefill_ws(h, wd, y, M, H, E, stream, kEpiAddRounded, res1);
 }

@@ -131,6 +131,27 @@ def test_prefill_block_stream_zero_projections_are_exact(ops):
     assert np.all((bits(h0) & 0x7FFF) == 0)
 
 
+@pytest.mark.parametrize("M,E,H,tile", [(300, 512, 1280, 0), (300, 512, 1024, 1), (130, 256, 768, 3), (2048, 2048, 8192, 0)])
+def test_prefill_block_stream_paired_gate_up_launch_equals_two_launches(ops, M, E, H, tile):
+    """Gate and up in one launch (a tile holds the same columns of both products) against the gate launch followed by
+    the up launch with the SwiGLU epilogue: the same bits in h and y, at the tile width chosen by shape and forced."""
+    ws = _weights(E, H, seed=70 + tile, scale=0.25)
+    sws = [_sw(ops, w) for w in ws]
+    attn, xres, nw = make_x((M, E), seed=71), make_x((M, E), seed=72), _norm_w(E, 73)
+    print(f"prefill block (stream order), one launch for gate and up against two, M={M} E={E} H={H} tile={tile}", flush=True)
+    ops.tune("prefill_tile", tile)
+    try:
+        y1, _, h1 = ops.prefill_o_ffn_stream(dev(attn), dev(xres), dev(nw), *sws, return_intermediates=True)
+        ops.tune("prefill_swiglu_split", 1)
+        y2, _, h2 = ops.prefill_o_ffn_stream(dev(attn), dev(xres), dev(nw), *sws, return_intermediates=True)
+        torch.cuda.synchronize()
+    finally:
+        ops.tune("prefill_swiglu_split", 0)
+        ops.tune("prefill_tile", 0)
+    assert torch.equal(h1.view(torch.int16), h2.view(torch.int16)) and torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+    assert float(h1.float().abs().max()) > 0
+
+
 def test_prefill_block_stream_agrees_with_the_checkpoint_layout_block(ops):
     """The same block on the checkpoint tensors (another kernel, another summation order inside a product): the
     outputs differ by roundings only."""
