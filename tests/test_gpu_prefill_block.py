@@ -244,8 +244,11 @@ def test_prefill_rms_qkv_rope_llama32_1b_size(ops, tiled_gemm):
     assert np.max(np.abs(n_g - n_p)) <= 2.0**-6 * np.max(n_p)
 
 
+# query heads per KV head 1, 2, 3, 4, 8 (a workgroup takes 4, 2 or 1 heads of a group); one item, an odd and an even
+# number of items (the kernel pairs the longest with the shortest), M not a multiple of the 32 queries of a wave
 @pytest.mark.parametrize("M,nh,nkv,hd", [(40, 4, 2, 64), (64, 2, 2, 64), (65, 4, 1, 128), (300, 8, 2, 64), (1, 2, 1, 64),
-                                         (200, 8, 1, 128), (33, 3, 3, 64)])
+                                         (200, 8, 1, 128), (33, 3, 3, 64), (257, 6, 2, 64), (500, 4, 1, 64), (129, 8, 2, 128),
+                                         (700, 2, 1, 128), (96, 4, 1, 64)])
 def test_prefill_attention(ops, M, nh, nkv, hd):
     from oracle import decode as odec
     print(f"prefill attention M={M} heads {nh}/{nkv} hd={hd}", flush=True)
@@ -263,6 +266,28 @@ def test_prefill_attention(ops, M, nh, nkv, hd):
     # the first token attends to itself only: its output is its V row, bit for bit (P = 1)
     v0 = qkv[0, nq + nk:].reshape(nkv, hd).repeat(nh // nkv, axis=0).reshape(-1)
     assert np.array_equal(bits(out)[0], v0)
+
+
+def test_prefill_attention_scores_of_wide_range(ops):
+    """Scores spread over hundreds of log2 units: the kernel's reference maximum, which follows the true one in steps,
+    must not lose the small terms or overflow; and a second call returns the same bits."""
+    from oracle import decode as odec
+    M, nh, nkv, hd = 400, 4, 1, 64
+    rng = np.random.default_rng(11)
+    qkv = rng.standard_normal((M, (nh + 2 * nkv) * hd)).astype(np.float32)
+    qkv[:, :(nh + nkv) * hd] *= 4.0                               # |q . k| / 8 up to ~100
+    qkv[::7, nh * hd:(nh + nkv) * hd] *= 0.05                     # and keys that hardly count
+    qkv = f32_to_bf16_bits(qkv)
+    print("prefill attention, wide score range", flush=True)
+    out = ops.prefill_attention(dev(qkv), nh, nkv, hd)
+    again = ops.prefill_attention(dev(qkv), nh, nkv, hd)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+    nq, nk = nh * hd, nkv * hd
+    want = odec.prefill_attention_reference(qkv[:, :nq], qkv[:, nq:nq + nk], qkv[:, nq + nk:], nh, nkv)
+    got = bf16_bits_to_f32(bits(out)).astype(np.float64)
+    tol = bf16_ulp(want) + 2.0**-8 * np.max(np.abs(bf16_bits_to_f32(qkv[:, nq + nk:]))) + 1e-3
+    assert np.all(np.isfinite(got)) and np.all(np.abs(got - want) <= tol), np.max(np.abs(got - want) - tol)
 
 
 def test_prefill_attention_matches_the_decode_kernel_row_by_row(ops):
