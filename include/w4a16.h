@@ -543,7 +543,7 @@ int w4a16_q4nx_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_resid
  * timeout test: split-K producers do not publish), "ffn_fused" (0 = default: w4a16_ffn_swiglu_bf16
  * runs two streaming launches; 1 = one persistent kernel when the shape allows), "gemv_ws_ct", "gemv_ws_waves",
  * "gemm_ws_cb" (stream-order GEMV / small-batch shapes), "prefill_tile" (one tile width only, 1: 256 columns, 2: 192, 3: 128,
- * 4: 64; 0: by shape), "prefill_min_m" (smallest M given to the tiled prefill kernel) and "prefill_swiglu_split" (1: the
+ * 4: 64; 5: 256 mixed with 128 in the launches that take that mix; 0: by shape), "prefill_min_m" (smallest M given to the tiled prefill kernel) and "prefill_swiglu_split" (1: the
  * stream-order prompt-pass FFN runs its gate and up projections as two launches instead of one; same bits).  Process-wide.
  */
 int w4a16_tune(const char *key, int value);

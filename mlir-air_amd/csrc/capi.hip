@@ -946,7 +946,7 @@ int w4a16_tune(const char *key, int value) {
         if (value != 0 && value != 4 && value != 8 && value != 16) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.ct = value;
     } else if (!strcmp(key, "prefill_tile")) {
-        if (value > 4) return W4A16_ERR_TUNE;
+        if (value > 5) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.prefill_tile = value;
     } else if (!strcmp(key, "prefill_swiglu_split")) {
         if (value != 0 && value != 1) return W4A16_ERR_TUNE;

@@ -542,25 +542,27 @@ __global__ void __launch_bounds__(kPfThreads, 1) gemm_wsp_kernel(const PfArgs p)
 // LDS delivers half of what the 64-column tile asks for), which is still better than idle CUs.
 struct Widths {
     int ncb;            // columns / 64 of the "wide" tiles: 4, or 2 / 1 for the narrow uniform tilings
-    int wide, narrow;   // number of column tiles of ncb * 64 columns and of 192 columns
+    int wide, narrow;   // number of column tiles of ncb * 64 columns and of the narrow width
+    int ncb_narrow = 3; // columns / 64 of the narrow tiles of a mixed launch: 3, or 2 where tiles must be halves or whole heads
 };
 
-long split_cost(long n_wide_tiles, long n_narrow_tiles, int cus) {
+double split_cost(long n_wide_tiles, long n_narrow_tiles, int cus, double narrow_cost) {
     // greedy list scheduling of two task sizes, big first, on identical machines: the finishing times after the
     // wide tiles are 4 q (+ 4 on r machines); every narrow tile goes to the machine that falls free first
-    std::vector<long> load(cus);
+    std::vector<double> load(cus);
     const long q = n_wide_tiles / cus, r = n_wide_tiles % cus;
-    for (int i = 0; i < cus; ++i) load[i] = 4 * (q + (i < r ? 1 : 0));
-    std::make_heap(load.begin(), load.end(), std::greater<long>());
+    for (int i = 0; i < cus; ++i) load[i] = 4.0 * (q + (i < r ? 1 : 0));
+    std::make_heap(load.begin(), load.end(), std::greater<double>());
     for (long i = 0; i < n_narrow_tiles; ++i) {
-        std::pop_heap(load.begin(), load.end(), std::greater<long>());
-        load.back() += 3;
-        std::push_heap(load.begin(), load.end(), std::greater<long>());
+        std::pop_heap(load.begin(), load.end(), std::greater<double>());
+        load.back() += narrow_cost;
+        std::push_heap(load.begin(), load.end(), std::greater<double>());
     }
     return *std::max_element(load.begin(), load.end());
 }
 
-// `heads128`: every tile must hold whole heads of 128 columns (RoPE epilogue): no 192- or 64-column tiles.
+// `heads128`: every tile must hold whole heads of 128 columns (RoPE epilogue) or halve into whole 16-column tiles
+// (gate and up in one tile): no 192- or 64-column tiles; the wide tiles are then mixed with 128-column ones.
 Widths pick_widths(int tiles_m, int U, int cus, bool heads128) {
     struct Entry {
         int tiles_m, U, cus;
@@ -575,14 +577,16 @@ Widths pick_widths(int tiles_m, int U, int cus, bool heads128) {
         if (e.U == U && e.tiles_m == tiles_m && e.cus == cus && e.heads128 == heads128) return e.w;
     Widths best{4, -1, -1};
     double best_cost = -1;
+    const int nn = heads128 ? 2 : 3;
+    const double narrow_cost = heads128 ? 2 * kPfSlowdown128 : 3.0;
     for (int a = U / 4; a >= 0; --a) {   // ties go to the split with more wide tiles
-        if ((U - 4 * a) % 3) continue;
-        const int b = (U - 4 * a) / 3;
-        if (heads128 && b) continue;
-        const double cost = (double)split_cost((long)tiles_m * a, (long)tiles_m * b, cus);
+        if ((U - 4 * a) % nn) continue;
+        const int b = (U - 4 * a) / nn;
+        if (a == 0 && heads128) continue;   // (the uniform 128-column tiling is priced below)
+        const double cost = split_cost((long)tiles_m * a, (long)tiles_m * b, cus, narrow_cost);
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;
-            best = Widths{4, a, b};
+            best = Widths{4, a, b, nn};
         }
     }
     // uniform narrow tilings: rounds x width x (measured) slowdown of the narrower tile's inner loop
@@ -593,7 +597,7 @@ Widths pick_widths(int tiles_m, int U, int cus, bool heads128) {
         const double cost = (double)((tiles + cus - 1) / cus) * nv.ncb * nv.slowdown;
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;
-            best = Widths{nv.ncb, U / nv.ncb, 0};
+            best = Widths{nv.ncb, U / nv.ncb, 0, 3};
         }
     }
     cache[next] = Entry{tiles_m, U, cus, heads128, best};
@@ -637,12 +641,14 @@ hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y,
     p.tiles_m = (M + kPfRows - 1) / kPfRows;
     const int U = N / 64;
     Widths wd = pick_widths(p.tiles_m, U, 256, heads128);
-    // tuning: one tile width only (1: 256 columns, 2: 192, 3: 128, 4: 64) where it divides N
+    // tuning: one tile width only (1: 256 columns, 2: 192, 3: 128, 4: 64) where it divides N; 5: 256 mixed with 128
+    // where the launch takes that mix (RoPE heads of 128, gate and up in one tile)
     const int force = g_gemv_ws_tune.prefill_tile;
     if (force == 1 && U % 4 == 0) wd = Widths{4, U / 4, 0};
     if (force == 2 && U % 3 == 0 && !heads128) wd = Widths{4, 0, U / 3};
     if (force == 3 && U % 2 == 0) wd = Widths{2, U / 2, 0};
     if (force == 4 && !heads128) wd = Widths{1, U, 0};
+    if (force == 5 && heads128 && U % 2 == 0 && U >= 6) wd = Widths{4, (U - 2) / 4, U % 4 == 0 ? 2 : 1, 2};
     p.n_wide = wd.wide, p.n_narrow = wd.narrow;
     if (wd.ncb == 2) return launch_wsp<2, 0>(p, stream);
     if (wd.ncb == 1) return launch_wsp<1, 0>(p, stream);
@@ -651,7 +657,7 @@ hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y,
         return launch_wsp<3, 0>(p, stream);
     }
     if (wd.narrow == 0) return launch_wsp<4, 0>(p, stream);
-    return launch_wsp<4, 3>(p, stream);
+    return wd.ncb_narrow == 2 ? launch_wsp<4, 2>(p, stream) : launch_wsp<4, 3>(p, stream);
 }
 
 // h[M, H] = bf16(silu(bf16(x . W_gate)) * bf16(x . W_up)): both projections in one launch, a tile holding the same
@@ -672,8 +678,10 @@ hipError_t launch_gemm_prefill_ws_swiglu(const uint16_t *x, const void *w_gate, 
     const int force = g_gemv_ws_tune.prefill_tile;
     if (force == 1 && U % 4 == 0) wd = Widths{4, U / 4, 0};
     if (force == 3) wd = Widths{2, U / 2, 0};
-    p.n_wide = wd.wide, p.n_narrow = 0;
-    return wd.ncb == 2 ? launch_wsp<2, 0>(p, stream) : launch_wsp<4, 0>(p, stream);
+    if (force == 5 && U >= 6) wd = Widths{4, (U - 2) / 4, U % 4 == 0 ? 2 : 1, 2};
+    p.n_wide = wd.wide, p.n_narrow = wd.ncb == 4 ? wd.narrow : 0;
+    if (wd.ncb == 2) return launch_wsp<2, 0>(p, stream);
+    return p.n_narrow ? launch_wsp<4, 2>(p, stream) : launch_wsp<4, 0>(p, stream);
 }
 
 }  // namespace w4a16

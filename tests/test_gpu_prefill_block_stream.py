@@ -131,7 +131,8 @@ def test_prefill_block_stream_zero_projections_are_exact(ops):
     assert np.all((bits(h0) & 0x7FFF) == 0)
 
 
-@pytest.mark.parametrize("M,E,H,tile", [(300, 512, 1280, 0), (300, 512, 1024, 1), (130, 256, 768, 3), (2048, 2048, 8192, 0)])
+@pytest.mark.parametrize("M,E,H,tile", [(300, 512, 1280, 0), (300, 512, 1024, 1), (130, 256, 768, 3), (2048, 2048, 8192, 0),
+                                        (300, 512, 1280, 5), (260, 256, 1792, 5)])
 def test_prefill_block_stream_paired_gate_up_launch_equals_two_launches(ops, M, E, H, tile):
     """Gate and up in one launch (a tile holds the same columns of both products) against the gate launch followed by
     the up launch with the SwiGLU epilogue: the same bits in h and y, at the tile width chosen by shape and forced."""
@@ -236,11 +237,12 @@ def _qkv_weights(E, nh, nkv, hd, seed, scale=0.25):
 
 
 # head widths 64 and 128 through every tile width that holds whole heads (tile 0: the width chosen by shape, which for
-# these small matrices is 64 or 128 columns; 1: 256, 2: 192, 3: 128, 4: 64), ragged M, one row tile and two
+# these small matrices is 64 or 128 columns; 1: 256, 2: 192, 3: 128, 4: 64, 5: 256 mixed with 128), ragged M, one row
+# tile and two
 @pytest.mark.parametrize("M,E,nh,nkv,hd,pos0,tile", [(40, 256, 4, 2, 64, 0, 0), (300, 512, 8, 8, 64, 7, 0), (130, 256, 2, 1, 128, 100, 0),
                                                       (17, 256, 3, 1, 64, 1, 0), (270, 512, 1, 1, 128, 3, 0), (300, 256, 4, 2, 64, 5, 1),
                                                       (100, 256, 4, 1, 64, 2, 2), (260, 512, 2, 1, 128, 9, 1), (64, 256, 4, 2, 64, 0, 3),
-                                                      (33, 256, 2, 1, 64, 11, 4)])
+                                                      (33, 256, 2, 1, 64, 11, 4), (270, 256, 4, 1, 128, 6, 5), (100, 512, 3, 2, 128, 0, 5)])
 def test_prefill_rms_qkv_rope_stream(ops, tiled_gemm, M, E, nh, nkv, hd, pos0, tile):
     from oracle import decode as odec
     print(f"prefill qkv rope (stream order) M={M} E={E} heads {nh}/{nkv} hd={hd} pos0={pos0} tile={tile}", flush=True)
