@@ -811,9 +811,10 @@ def main():
                     out["prefill"]["cpu_baseline"] = r["cpu_baseline"]
         r = run_prefill_block(10, 2)
         extra["prefill_block"] = {"us": r["us"], "TFLOP/s": r["TFLOP/s"], "frac_mfma_peak": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS}
-        r = run_prefill_model("decode_1b", 2048, 2)
-        extra["prefill_1b"] = {"ms": r["ms"], "tokens/s": r["tokens_per_s"], "TFLOP/s": r["TFLOP/s"],
-                               "frac_mfma_peak": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS}
+        for name, model in (("prefill_1b", "decode_1b"), ("prefill_8b", "decode_8b")):
+            r = run_prefill_model(model, 2048, 2)
+            extra[name] = {"ms": r["ms"], "tokens/s": r["tokens_per_s"], "TFLOP/s": r["TFLOP/s"],
+                           "frac_mfma_peak": r["TFLOP/s"] / MFMA_BF16_PEAK_TFLOPS}
         for model in DECODE_MODELS:
             r = run_decode_model(32 if model == "decode_1b" else 16, 4, model)
             extra[model] = {"us_per_token": r["us_per_token"], "tokens/s": r["tokens_per_s"],
