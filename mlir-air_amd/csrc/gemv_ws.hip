@@ -379,10 +379,28 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
     const bool row_valid = ln < M;
     const uint16_t *xrow = x + (size_t)(row_valid ? ln : 0) * K + 8 * lg;
     const int ntasks = (G + kGemmWsGroups - 1) / kGemmWsGroups;
+    // The scale words of a task (4 groups x CB tiles x 16 columns: one 16-byte chunk per tile and column, since the
+    // task's groups are one aligned quad of a block) are fetched by one request of the wave, lane (c, ln) taking tile
+    // c's chunk, and handed to the lanes that need them through a KiB of LDS private to the wave.  Fetched as
+    // sixteen 4-byte loads per wave they cost as many address-unit cycles as the task's cells (M = 16, K = 4096,
+    // N = 14336: 9.9 -> 9.2 us on cached weights, 10.4 -> 10.3 us cold); as 16-byte loads of every lane they do not
+    // fit the 256 registers.
+    //
+    // Where the time goes at that shape (requests replaced by constants, cold): 3.6 us without any x or cell request,
+    // +2.9 us for the x requests alone (128 KB per workgroup, L2 hits), +4.0 us for the cells alone (143 KB per
+    // workgroup from HBM), 10.3 us with both: the two streams add up, i.e. a CU takes in ~40 bytes per ns whatever the
+    // source.  Not kept, no gain: x copied to LDS once per workgroup with whole-line requests (10.3 - 10.4 us); the 896
+    // tiles dealt 4 and 3 to 256 workgroups instead of 4 to 224 (10.55 against 10.59 us on one box).
+    u32x4 *mdl = reinterpret_cast<u32x4 *>(red + kGemmWsWaves * CB * 4 * 64) + wave * 64;
     for (int task = wave; task < ntasks; task += kGemmWsWaves) {
         const int g0 = task * kGemmWsGroups;
         u32x4 X[kGemmWsGroups][4], cell[kGemmWsGroups][CB];
-        uint32_t md[kGemmWsGroups][CB];
+        u32x4 mdq;
+        {
+            const int b = g0 >> 4, gl = g0 & 15, c = lg < CB ? lg : CB - 1;
+            mdq = *reinterpret_cast<const u32x4 *>(tile0 + (size_t)c * tile_bytes + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes) +
+                                                   (16 * (gl >> 2) + ln) * 16);
+        }
 #pragma unroll
         for (int j = 0; j < kGemmWsGroups; ++j) {
             const int g = g0 + j < G ? g0 + j : G - 1;   // a short last task re-reads the last group (its x is zeroed below)
@@ -394,17 +412,16 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
             const int g = g0 + j < G ? g0 + j : G - 1;
             const int b = g >> 4, gl = g & 15;
             const char *blk = tile0 + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes);
-            // the scale word of (group g, column ln) sits in lane 16 (gl / 4) + ln, dword gl % 4 of the block's first KiB
-            // (one 16-byte load per tile for the task's four groups needs 3 more registers per tile at the 256 limit
-            // and spills: 10.6 -> 14.0 us at M = 16, K = 4096, N = 14336)
-#pragma unroll
-            for (int c = 0; c < CB; ++c)
-                md[j][c] = *reinterpret_cast<const uint32_t *>(blk + (size_t)c * tile_bytes + (16 * (gl >> 2) + ln) * 16 + 4 * (gl & 3));
 #pragma unroll
             for (int c = 0; c < CB; ++c)
                 cell[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)c * tile_bytes + (size_t)(1 + gl) * kWsCellBytes) + lane);
         }
         __builtin_amdgcn_sched_barrier(0);
+        // the scale word of (group g0 + j, column ln) of tile c: dword j of the chunk that lane 16 c + ln fetched
+        u32x4 md[CB];
+        mdl[lane] = mdq;   // (LDS operations of one wave complete in order; the previous task's reads are done)
+#pragma unroll
+        for (int cc = 0; cc < CB; ++cc) md[cc] = mdl[16 * cc + ln];
 #pragma unroll
         for (int j = 0; j < kGemmWsGroups; ++j) {
             const bool valid = row_valid && g0 + j < G;
@@ -421,8 +438,9 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
                 for (int t = 0; t < 4; ++t)
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[j][t]),
                                                                   cell_operand(cell[j][c][t], nib_mask, magic), acc, 0, 0, 0);
-                const float sf = __builtin_bit_cast(float, md[j][c] << 16);
-                const float nz = __builtin_bit_cast(float, md[j][c] & 0xFFFF0000u);   // -(128 + z)
+                const uint32_t mw = g0 + j < G ? md[c][j] : 0u;   // (a short last task: no such group, s = 0)
+                const float sf = __builtin_bit_cast(float, mw << 16);
+                const float nz = __builtin_bit_cast(float, mw & 0xFFFF0000u);   // -(128 + z)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) Y[c][i] = fmaf(sf, fmaf(nz, xs[i], acc[i]), Y[c][i]);
             }
@@ -454,7 +472,7 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
 template <int CB>
 hipError_t launch_gemm_ws_cb(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
                              hipStream_t stream) {
-    const size_t lds = (size_t)kGemmWsWaves * CB * 4 * 64 * sizeof(float);
+    const size_t lds = (size_t)kGemmWsWaves * CB * 4 * 64 * sizeof(float) + kGemmWsWaves * kWsCellBytes;   // sums, scale words
     hipLaunchKernelGGL((gemm_ws_kernel<CB>), dim3(N / (16 * CB)), dim3(kGemmWsWaves * 64), lds, stream, x,
                        static_cast<const char *>(w), y, residual, M, K, N, K / kGroup, ws_blocks(K));
     return hipGetLastError();
