@@ -154,8 +154,8 @@ def decode_greedy(token, n_tokens, layers, embed_table, final_norm, lm_head, con
         sumsq = None
         for layer, (kc, vc) in zip(layers, kv_cache):
             x, sumsq = run_decode_block(x, layer, config, kc, vc, start_pos + i, rope_lut, x_sumsq=sumsq, return_sumsq=True)
-        _, tok = ops.lm_head(x, lm_head, norm_weight=final_norm, eps=config.rms_eps)
-        out[i:i + 1] = tok
+        tok = out[i:i + 1]   # the argmax lands in the ids buffer; the next embedding lookup reads it from there
+        ops.lm_head(x, lm_head, norm_weight=final_norm, eps=config.rms_eps, argmax_out=tok)
     return out
 
 

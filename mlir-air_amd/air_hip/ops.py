@@ -653,9 +653,10 @@ def prefill_o_ffn_stream(attn_out, x_residual, ffn_norm_weight, wo, gate, up, do
     return (y, res1, h) if return_intermediates else y
 
 
-def lm_head(x, lm_head_weight, norm_weight=None, eps=1e-5, return_argmax=True):
+def lm_head(x, lm_head_weight, norm_weight=None, eps=1e-5, return_argmax=True, argmax_out=None):
     """Tail of a decode step: logits bf16 [V] = lm_head_weight [V, E] . rms_norm(x) (x itself when
-    norm_weight is None), and the index of the largest logit as a device int32 tensor [1]."""
+    norm_weight is None), and the index of the largest logit as a device int32 tensor [1]
+    (`argmax_out`: written there instead of into a new tensor, e.g. a slot of the generated-ids buffer)."""
     lib = _lib.load_library()
     _need_cuda(x, lm_head_weight)
     V, E = lm_head_weight.shape
@@ -664,7 +665,11 @@ def lm_head(x, lm_head_weight, norm_weight=None, eps=1e-5, return_argmax=True):
     if not lm_head_weight.is_contiguous():
         raise ValueError("lm_head must be contiguous [V, E]")
     logits = torch.empty((V,), dtype=torch.bfloat16, device=x.device)
-    best = torch.empty((1,), dtype=torch.int32, device=x.device) if return_argmax else None
+    best = None
+    if return_argmax:
+        best = argmax_out if argmax_out is not None else torch.empty((1,), dtype=torch.int32, device=x.device)
+        if best.dtype != torch.int32 or best.numel() != 1 or not best.is_cuda:
+            raise ValueError("argmax_out must be a device int32 tensor of one element")
     key = (x.device.index, _stream(), "lm_head", V)
     ws = _attn_ws.get(key)
     if ws is None:
