@@ -536,6 +536,28 @@ int w4a16_q4nx_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_resid
                                void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same codec on the fast path: the operands of q4nx_repack re-packed once more, at load time, into the stream order of
+ * the decode kernels (csrc/wstream.h, "Q4NX order": 16-column tiles, 1 KiB cells of 128 rows, and in front of every 16
+ * cells 4 KiB of scale / min words, one pair per 32 rows and column), the counterpart of the reference's own stream
+ * order for these blocks (pack_q4k_cascade, programming_examples/fused_decode/proj_qmm_pack.py:61-140).  The GEMV, the
+ * RMSNorm + GEMV and the O + FFN block then run the whole-K kernels of the AWQ stream order with the per-32-row flush
+ * y += s * (sum q x) + min * (sum x) of _qmm_q4k_bf16 (programming_examples/fused_decode/kernels/q4_k.h:39-45): no
+ * workspace protocol, no state.  `residual` may be NULL; x_sumsq / n_pieces, res1_out, h_out, y_sumsq and the workspace
+ * (w4a16_block_stream_workspace_bytes) as in the AWQ entry points of the same names.  K % 128 == 0, N % 16 == 0.
+ */
+size_t w4a16_q4nx_stream_bytes(int K, int N);
+int w4a16_q4nx_repack_stream(const int32_t *qweight, const uint16_t *scales, const uint16_t *mins, void *wstream, int K, int N,
+                             void *stream);
+int w4a16_q4nx_gemv_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int K, int N,
+                                void *stream);
+int w4a16_q4nx_rms_gemv_stream_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
+                                    const void *wstream, uint16_t *y, int K, int N, void *stream);
+int w4a16_q4nx_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                                      float eps, const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                      const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, float *y_sumsq,
+                                      int E, int H, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Launch-shape override for benchmarking sweeps (not needed for normal use).  Keys:
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic),
  * "gemm_stream_max_m" (largest M given to the streaming kernel, 0 = default 96, otherwise >= 16) and

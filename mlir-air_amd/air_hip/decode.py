@@ -42,22 +42,25 @@ class DecodeLayer:
     w_up: tuple
     w_down: tuple
     codec: str = "awq"   # "awq": triples are (qweight, qzeros, scales); "q4nx": (qweight, scales, mins) from q4nx_repack
-    # AWQ layers: the same five matrices in stream order (ops.StreamWeight), which the decode kernels read; the
-    # checkpoint-layout triples above stay for the prompt pass.  None: decode runs on the triples.
+    # The same five matrices in stream order (ops.StreamWeight; Q4NX order for that codec), which the decode kernels
+    # read; the triples above stay for the checkpoint-layout prompt pass.  None: decode runs on the triples.
     stream: dict = None
 
     def with_stream(self):
         """Re-pack the layer's matrices into stream order on the GPU (once, at load time)."""
-        if self.codec == "awq" and self.stream is None:
-            self.stream = {name: ops.repack_stream(*getattr(self, name)) for name in ("wqkv", "wo", "w_gate", "w_up", "w_down")}
+        if self.stream is None:
+            repack = ops.repack_stream if self.codec == "awq" else ops.q4nx_repack_stream
+            self.stream = {name: repack(*getattr(self, name)) for name in ("wqkv", "wo", "w_gate", "w_up", "w_down")}
         return self
 
 
-def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda") -> DecodeLayer:
+def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda", stream_order=True) -> DecodeLayer:
     """A Q4NX / Q4_0 layer -> DecodeLayer.  `blocks` maps q, k, v, o, gate, up, down to the tensor's
     blocks (uint8 [n_blocks, 5120], numpy or torch) in (row-block, col-block) order as a model.q4nx
     bundle stores them; Q, K, V are fused by concatenating their blocks (whole row-blocks of the output
-    axis), and every matrix is repacked on the GPU once.  Norm weights are bf16 bit patterns or tensors."""
+    axis), and every matrix is repacked on the GPU once (stream_order: and once more into the decode kernels'
+    stream order, as the reference re-packs the blocks into its cascade order, proj_qmm_pack.py:61-140).
+    Norm weights are bf16 bit patterns or tensors."""
     E, H = config.emb_dim, config.hidden_dim
     nq, nkv = config.n_heads * config.head_dim, config.kv_dim
 
@@ -74,10 +77,11 @@ def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda
         return ops.q4nx_repack(t.contiguous(), M, K, mode)
 
     qkv = torch.cat([dev_blocks(blocks[n]) for n in ("q", "k", "v")], dim=0)
-    return DecodeLayer(attn_norm=dev_vec(attn_norm), ffn_norm=dev_vec(ffn_norm),
-                       wqkv=repack(qkv, nq + 2 * nkv, E), wo=repack(dev_blocks(blocks["o"]), E, nq),
-                       w_gate=repack(dev_blocks(blocks["gate"]), H, E), w_up=repack(dev_blocks(blocks["up"]), H, E),
-                       w_down=repack(dev_blocks(blocks["down"]), E, H), codec="q4nx")
+    out = DecodeLayer(attn_norm=dev_vec(attn_norm), ffn_norm=dev_vec(ffn_norm),
+                      wqkv=repack(qkv, nq + 2 * nkv, E), wo=repack(dev_blocks(blocks["o"]), E, nq),
+                      w_gate=repack(dev_blocks(blocks["gate"]), H, E), w_up=repack(dev_blocks(blocks["up"]), H, E),
+                      w_down=repack(dev_blocks(blocks["down"]), E, H), codec="q4nx")
+    return out.with_stream() if stream_order else out
 
 
 def prepare_layer(layer: wmod.LayerWeights, device="cuda", stream_order=True) -> DecodeLayer:
@@ -110,6 +114,12 @@ def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer
     updated in place at current_pos.  x_sumsq / return_sumsq chain the sum of squares of the block's output into
     the next block's RMSNorm (AWQ layers): with return_sumsq the result is (y, sumsq or None)."""
     q4nx = layer.codec == "q4nx"
+    if layer.stream is not None and q4nx:   # Q4NX order: the same whole-K launches, attention as its own call
+        sw = layer.stream
+        qkv = ops.q4nx_rms_gemv_stream(x, layer.attn_norm, sw["wqkv"], eps=config.rms_eps, x_sumsq=x_sumsq)
+        attn_out = ops.decode_attention(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads)
+        return ops.q4nx_o_gemv_ffn_stream(attn_out, x, layer.ffn_norm, sw["wo"], sw["w_gate"], sw["w_up"], sw["w_down"],
+                                          eps=config.rms_eps, return_sumsq=return_sumsq)
     if layer.stream is not None:   # stream-order weights: stateless whole-K launches, sums of squares per 16 columns
         sw = layer.stream
         qkv = ops.w4a16_rms_gemv_stream(x, layer.attn_norm, sw["wqkv"], eps=config.rms_eps, x_sumsq=x_sumsq)

@@ -780,6 +780,73 @@ def q4nx_o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, e
     return (y, res1, h) if return_intermediates else y
 
 
+def q4nx_repack_stream(qweight, scales, mins):
+    """Operands of q4nx_repack (qweight int32 [K, N / 8], scales and mins bf16 [K / 32, N]) -> StreamWeight in Q4NX
+    order, the form the whole-K decode kernels read; once per tensor at load time."""
+    lib = _lib.load_library()
+    _need_cuda(qweight, scales, mins)
+    K, N = qweight.shape[0], qweight.shape[1] * 8
+    if scales.shape != (K // 32, N) or mins.shape != scales.shape:
+        raise ValueError("q4nx_repack_stream: scales and mins must be [K / 32, N]")
+    nbytes = lib.w4a16_q4nx_stream_bytes(K, N)
+    if nbytes == 0:
+        raise ValueError(f"Q4NX stream order needs K % 128 == 0 and N % 16 == 0, got K={K}, N={N}")
+    buf = torch.empty(int(nbytes), dtype=torch.uint8, device=qweight.device)
+    _lib.check(lib.w4a16_q4nx_repack_stream(_ptr(qweight), _ptr(_bits(scales)), _ptr(_bits(mins)), _ptr(buf), K, N, _stream()))
+    return StreamWeight(buf, K, N)
+
+
+def q4nx_gemv_stream(x, w, residual=None, out=None):
+    """y[N] = bf16(x[K] . W (+ residual)) on a Q4NX-order StreamWeight; stateless, no workspace."""
+    lib = _lib.load_library()
+    _need_cuda(x, w.buf)
+    if x.numel() != w.K or (residual is not None and residual.numel() != w.N):
+        raise ValueError("q4nx_gemv_stream: x must have K elements, residual N")
+    if out is None:
+        out = torch.empty((w.N,), dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.w4a16_q4nx_gemv_stream_bf16(_ptr(_bits(x)), _ptr(w.buf), _ptr(_bits(residual)) if residual is not None else None,
+                                               _ptr(out), w.K, w.N, _stream()))
+    return out
+
+
+def q4nx_rms_gemv_stream(x, norm_weight, w, eps=1e-5, x_sumsq=None):
+    """y[N] = bf16(rms_norm(x, norm_weight) . W) on a Q4NX-order StreamWeight (x_sumsq as in w4a16_rms_gemv_stream)."""
+    lib = _lib.load_library()
+    _need_cuda(x, norm_weight, w.buf)
+    if x.numel() != w.K or norm_weight.numel() != w.K:
+        raise ValueError("q4nx_rms_gemv_stream: x and norm_weight must have K elements")
+    out = torch.empty((w.N,), dtype=torch.bfloat16, device=x.device)
+    if x_sumsq is not None and (x_sumsq.dtype != torch.float32 or not x_sumsq.is_cuda or not x_sumsq.is_contiguous()):
+        raise ValueError("x_sumsq must be a contiguous float32 GPU tensor")
+    _lib.check(lib.w4a16_q4nx_rms_gemv_stream_bf16(_ptr(_bits(x)), _ptr(x_sumsq) if x_sumsq is not None else None,
+                                                   x_sumsq.numel() if x_sumsq is not None else 0, _ptr(_bits(norm_weight)),
+                                                   float(eps), _ptr(w.buf), _ptr(out), w.K, w.N, _stream()))
+    return out
+
+
+def q4nx_o_gemv_ffn_stream(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, return_intermediates=False,
+                           return_sumsq=False):
+    """o_gemv_ffn_stream on Q4NX-order StreamWeights: same stages, outputs and scratch."""
+    lib = _lib.load_library()
+    _need_cuda(attn_out, x_residual, ffn_norm_weight, wo.buf, gate.buf, up.buf, down.buf)
+    E, H = wo.K, gate.N
+    _check_block_stream(E, H, wo, gate, up, down, attn_out, x_residual, ffn_norm_weight)
+    dev = attn_out.device
+    y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
+    res1 = torch.empty((E,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
+    h = torch.empty((H,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
+    sumsq = torch.empty((E // 16,), dtype=torch.float32, device=dev) if return_sumsq else None
+    ws = _block_stream_scratch(E, H, dev)
+    opt = lambda t: _ptr(t) if t is not None else None
+    _lib.check(lib.w4a16_q4nx_o_gemv_ffn_stream_bf16(
+        _ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps), _ptr(wo.buf), _ptr(gate.buf),
+        _ptr(up.buf), _ptr(down.buf), _ptr(y), opt(res1), opt(h), opt(sumsq), E, H, _ptr(ws), ws.numel(), _stream()))
+    out = (y, res1, h) if return_intermediates else (y,)
+    if return_sumsq:
+        out = out + (sumsq,)
+    return out if len(out) > 1 else y
+
+
 def tune(key, value):
     lib = _lib.load_library()
     _lib.check(lib.w4a16_tune(key.encode(), int(value)))

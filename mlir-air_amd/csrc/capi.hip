@@ -503,7 +503,7 @@ BlockStreamScratch block_stream_scratch(void *workspace, int E, int H) {
 int o_gemv_ffn_stream_impl(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
                            const void *wo, const void *wg, const void *wu, const void *wd, uint16_t *y, uint16_t *res1_out,
                            uint16_t *h_out, float *y_sumsq, int E, int H, int group, void *workspace, size_t workspace_bytes,
-                           void *stream, bool check_only) {
+                           void *stream, bool check_only, bool q4 = false) {
     if (!attn_out || !x_residual || !ffn_norm_weight || !wo || !wg || !wu || !wd || !y) return W4A16_ERR_NULL;
     if (group != kGroup) return W4A16_ERR_GROUP;
     if (E <= 0 || H <= 0 || E % kGroup != 0 || H % kGroup != 0) return W4A16_ERR_SHAPE;
@@ -517,12 +517,14 @@ int o_gemv_ffn_stream_impl(const uint16_t *attn_out, const uint16_t *x_residual,
     uint16_t *h = h_out ? h_out : sc.h;
     // stage 1: res1 = bf16(attn_out . Wo + x_residual), leaving sum(res1^2) per tile for the norm of stage 2
     GemvWsExtras s1;
+    s1.q4 = q4;
     s1.residual = x_residual;
     s1.sumsq_out = sc.res1_sumsq;
     int rc = gemv_stream_call(attn_out, wo, nullptr, res1, E, E, group, stream, s1);
     if (rc) return rc;
     // stage 2: h = swiglu(rms_norm(res1) . Wgate, rms_norm(res1) . Wup)
     GemvWsExtras s2;
+    s2.q4 = q4;
     s2.norm_w = ffn_norm_weight;
     s2.eps = eps;
     s2.sumsq_in = sc.res1_sumsq;
@@ -531,6 +533,7 @@ int o_gemv_ffn_stream_impl(const uint16_t *attn_out, const uint16_t *x_residual,
     if (rc) return rc;
     // stage 3: y = bf16(h . Wdown + res1)
     GemvWsExtras s3;
+    s3.q4 = q4;
     s3.residual = res1;
     s3.sumsq_out = y_sumsq;
     return gemv_stream_call(h, wd, nullptr, y, H, E, group, stream, s3);
@@ -877,6 +880,48 @@ int q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t
     if (misaligned(blocks) || misaligned(qweight) || misaligned(scales) || misaligned(mins)) return W4A16_ERR_ALIGN;
     hipError_t e = launch_q4nx_repack(blocks, qweight, scales, mins, M, K, mode, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+size_t w4a16_q4nx_stream_bytes(int K, int N) {
+    if (K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return 0;
+    return ws_q4_matrix_bytes(K, N);
+}
+
+int w4a16_q4nx_repack_stream(const int32_t *qweight, const uint16_t *scales, const uint16_t *mins, void *wstream, int K, int N,
+                             void *stream) {
+    if (!qweight || !scales || !mins || !wstream) return W4A16_ERR_NULL;
+    if (K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
+    if (misaligned(qweight) || misaligned(scales) || misaligned(mins) || misaligned(wstream)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_repack_ws_q4(qweight, scales, mins, wstream, K, N, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_q4nx_gemv_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int K, int N,
+                                void *stream) {
+    GemvWsExtras ex;
+    ex.q4 = true;
+    ex.residual = residual;
+    return gemv_stream_call(x, wstream, nullptr, y, K, N, kGroup, stream, ex);
+}
+
+int w4a16_q4nx_rms_gemv_stream_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
+                                    const void *wstream, uint16_t *y, int K, int N, void *stream) {
+    if (!norm_weight) return W4A16_ERR_NULL;
+    GemvWsExtras ex;
+    ex.q4 = true;
+    ex.norm_w = norm_weight;
+    ex.eps = eps;
+    ex.sumsq_in = x_sumsq;
+    ex.sumsq_n = x_sumsq ? n_pieces : 0;
+    return gemv_stream_call(x, wstream, nullptr, y, K, N, kGroup, stream, ex);
+}
+
+int w4a16_q4nx_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                                      float eps, const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                      const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, float *y_sumsq,
+                                      int E, int H, void *workspace, size_t workspace_bytes, void *stream) {
+    return o_gemv_ffn_stream_impl(attn_out, x_residual, ffn_norm_weight, eps, o_wstream, gate_wstream, up_wstream, down_wstream,
+                                  y, res1_out, h_out, y_sumsq, E, H, kGroup, workspace, workspace_bytes, stream, false, true);
 }
 
 int w4a16_q4nx_gemm_bf16(const uint16_t *x, const int32_t *qweight, const uint16_t *scales, const uint16_t *mins,

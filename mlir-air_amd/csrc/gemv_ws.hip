@@ -75,7 +75,9 @@ __device__ __forceinline__ void sumsq8(const u32x4 v, float &a0, float &a1) {
 // RMS  x is RMS-normalised on the fly: every wave obtains rstd = 1 / sqrt(mean(x^2) + eps) itself (from the partial
 //      sums the producer of x left behind, else by walking x, which is K bf16 values and L2-resident) and feeds
 //      bf16((x * rstd) * norm_w) to the matrix cores
-template <int CT, int NMAT, bool RMS>
+// Q4   Q4NX order: a scale and a min per K-step of a cell; the four K-steps of a cell are four products of their own and
+//      the flush is y += s (sum (128 + q) x - 128 sum x) + min' sum x per K-step
+template <int CT, int NMAT, bool RMS, bool Q4>
 __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t *__restrict__ x, const char *__restrict__ w0,
                                                                  const char *__restrict__ w1, uint16_t *__restrict__ y,
                                                                  const uint16_t *__restrict__ residual, int G, int NB,
@@ -86,7 +88,8 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lg = lane >> 4, ln = lane & 15;
     const int tile = blockIdx.x;
-    const size_t tile_bytes = (size_t)(NB + G) * kWsCellBytes;
+    constexpr int MDK = Q4 ? kWsQ4MdKiB : 1;   // KiB of scale words in front of a block's cells
+    const size_t tile_bytes = (size_t)(MDK * NB + G) * kWsCellBytes;
 
     const uint32_t ones_w = 0x3F803F80u;
     const u32x4 ones4 = {ones_w, ones_w, ones_w, ones_w};
@@ -132,7 +135,7 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
         const int b = tm / SUB, r0 = (tm % SUB) * CT;
         const int ng = min(kWsBlockGroups, G - kWsBlockGroups * b);   // groups of this block
         if (r0 >= ng) continue;                                       // wave-uniform
-        const char *blk = (mat ? w1 : w0) + (size_t)tile * tile_bytes + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes);
+        const char *blk = (mat ? w1 : w0) + (size_t)tile * tile_bytes + (size_t)b * ((kWsBlockGroups + MDK) * kWsCellBytes);
 
         // x of the task's groups: A row ln <-> group 16 b + ln; rows outside the task are zero, so that
         // their (never read) products and their sum x stay finite and contribute nothing
@@ -149,11 +152,13 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
             for (int t = 0; t < 4; ++t) NW[t] = *reinterpret_cast<const u32x4 *>(np + 32 * t);
         }
         // scales / zero points next: they sit right in front of the cells (requested after the cells instead: +0.5 us)
-        const u32x4 md = *(reinterpret_cast<const u32x4 *>(blk) + lane);
+        u32x4 md[MDK];
+#pragma unroll
+        for (int t = 0; t < MDK; ++t) md[t] = *(reinterpret_cast<const u32x4 *>(blk + (size_t)t * kWsCellBytes) + lane);
 #pragma unroll
         for (int r = 0; r < CT; ++r) {
             const int rc = r0 + r < ng ? r0 + r : ng - 1;   // a short block re-reads its last cell (x of that row is zero)
-            cell[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)(1 + rc) * kWsCellBytes) + lane);
+            cell[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)(MDK + rc) * kWsCellBytes) + lane);
         }
         // every load of the task is requested before the first wait
         __builtin_amdgcn_sched_barrier(0);
@@ -178,26 +183,56 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
 #pragma unroll
             for (int t = 0; t < 4; ++t) X[t] = u32x4{0u, 0u, 0u, 0u};
         }
-        floatx4 xs = {0.f, 0.f, 0.f, 0.f};   // register i of lane group lg: sum of x over group 16 b + 4 lg + i
+        float sum = 0.f;
+        if constexpr (!Q4) {
+            floatx4 xs = {0.f, 0.f, 0.f, 0.f};   // register i of lane group lg: sum of x over group 16 b + 4 lg + i
 #pragma unroll
-        for (int t = 0; t < 4; ++t) xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[t]), ones, xs, 0, 0, 0);
+            for (int t = 0; t < 4; ++t) xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[t]), ones, xs, 0, 0, 0);
 
-        float V[4] = {0.f, 0.f, 0.f, 0.f};   // V[i] of lane group lg: sum (128 + q) x of group 16 b + 4 lg + i
+            float V[4] = {0.f, 0.f, 0.f, 0.f};   // V[i] of lane group lg: sum (128 + q) x of group 16 b + 4 lg + i
 #pragma unroll
-        for (int r = 0; r < CT; ++r) {
-            floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+            for (int r = 0; r < CT; ++r) {
+                floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[t]), cell_operand(cell[r][t], nib_mask, magic),
+                                                                  acc, 0, 0, 0);
+                V[r & 3] = (lg == ((r0 + r) >> 2)) ? acc[r & 3] : V[r & 3];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float s = __builtin_bit_cast(float, md[0][i] << 16);
+                const float nz = __builtin_bit_cast(float, md[0][i] & 0xFFFF0000u);   // -(128 + z)
+                sum = fmaf(s, fmaf(nz, xs[i], V[i]), sum);
+            }
+        } else {
+            const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+            floatx4 xs[4];                        // xs[t][i]: sum of x over rows 32 t .. 32 t + 31 of group 16 b + 4 lg + i
+#pragma unroll
+            for (int t = 0; t < 4; ++t) xs[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[t]), ones, zero4, 0, 0, 0);
+            float V[4][4];                        // V[t][i]: sum (128 + q) x over the same rows
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[t]), cell_operand(cell[r][t], nib_mask, magic),
-                                                              acc, 0, 0, 0);
-            V[r & 3] = (lg == ((r0 + r) >> 2)) ? acc[r & 3] : V[r & 3];
-        }
-        float sum = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float s = __builtin_bit_cast(float, md[i] << 16);
-            const float nz = __builtin_bit_cast(float, md[i] & 0xFFFF0000u);   // -(128 + z)
-            sum = fmaf(s, fmaf(nz, xs[i], V[i]), sum);
+                for (int i = 0; i < 4; ++i) V[t][i] = 0.f;
+#pragma unroll
+            for (int r = 0; r < CT; ++r) {
+                const bool mine = lg == ((r0 + r) >> 2);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[t]),
+                                                                                cell_operand(cell[r][t], nib_mask, magic), zero4, 0, 0, 0);
+                    V[t][r & 3] = mine ? acc[r & 3] : V[t][r & 3];
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float s = __builtin_bit_cast(float, md[t][i] << 16);
+                    const float mn = __builtin_bit_cast(float, md[t][i] & 0xFFFF0000u);
+                    sum = fmaf(s, fmaf(-128.0f, xs[t][i], V[t][i]), fmaf(mn, xs[t][i], sum));
+                }
         }
         if (NMAT == 2 && mat) yv[NMAT - 1] += sum;
         else yv[0] += sum;
@@ -277,6 +312,42 @@ __global__ void __launch_bounds__(256) repack_ws_kernel(const uint32_t *__restri
     out[idx] = v;
 }
 
+// Q4NX order from the operands of the affine path; one thread per dword of the buffer.
+__global__ void __launch_bounds__(256) repack_ws_q4_kernel(const uint32_t *__restrict__ qweight, const uint16_t *__restrict__ scales,
+                                                           const uint16_t *__restrict__ mins, uint32_t *__restrict__ out, int G, int NB,
+                                                           int N) {
+    const size_t tile_dwords = (size_t)(kWsQ4MdKiB * NB + G) * (kWsCellBytes / 4);
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= tile_dwords * (N / kWsTileCols)) return;
+    const int tile = (int)(idx / tile_dwords);
+    const int off = (int)(idx - (size_t)tile * tile_dwords);
+    constexpr int BLOCK_DWORDS = (kWsBlockGroups + kWsQ4MdKiB) * (int)(kWsCellBytes / 4);
+    const int b = min(off / BLOCK_DWORDS, NB - 1);
+    const int within = off - b * BLOCK_DWORDS;
+    const int l = (within & 255) >> 2, sub = within & 3;   // lane and dword of a 1 KiB piece
+    const int n = tile * kWsTileCols + (l & 15);
+    const int lg = l >> 4;
+    const int nb = N >> 3;
+    const int shift = 4 * unpack_pos(n & 7);               // where column n sits in its packed word
+    uint32_t v = 0;
+    if (within < kWsQ4MdKiB * 256) {                       // scales and mins: KiB t, dword i = group 16 b + 4 lg + i
+        const int t = within >> 8;
+        const int g = kWsBlockGroups * b + 4 * lg + sub;
+        if (g < G) {
+            const size_t at = (size_t)(4 * g + t) * N + n;
+            v = (uint32_t)scales[at] | ((uint32_t)mins[at] << 16);
+        }
+    } else {
+        const int g = kWsBlockGroups * b + (within >> 8) - kWsQ4MdKiB;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const int k = 128 * g + 32 * sub + 8 * lg + pack_order(p);
+            v |= ((qweight[(size_t)k * nb + (n >> 3)] >> shift) & 0xFu) << (4 * p);
+        }
+    }
+    out[idx] = v;
+}
+
 template <int CT>
 hipError_t launch_ct(int nmat, int waves, const uint16_t *x, const void *w0, const void *w1, uint16_t *y, int K, int N,
                      const GemvWsExtras &ex, hipStream_t stream) {
@@ -284,15 +355,27 @@ hipError_t launch_ct(int nmat, int waves, const uint16_t *x, const void *w0, con
     const dim3 grid(N / kWsTileCols), block(waves * 64);
     const GemvWsTail tail = {ex.norm_w, ex.sumsq_in, ex.sumsq_out, ex.eps, ex.sumsq_n, K};
     const char *a = static_cast<const char *>(w0), *b = static_cast<const char *>(w1 ? w1 : w0);
-#define W4A16_GEMV_WS_LAUNCH(NMAT, RMS)                                                                               \
-    hipLaunchKernelGGL((gemv_ws_kernel<CT, NMAT, RMS>), grid, block, 0, stream, x, a, b, y, ex.residual, G, NB,      \
+#define W4A16_GEMV_WS_LAUNCH(NMAT, RMS, Q4)                                                                           \
+    hipLaunchKernelGGL((gemv_ws_kernel<CT, NMAT, RMS, Q4>), grid, block, 0, stream, x, a, b, y, ex.residual, G, NB,  \
                        ex.round_before_add, waves, tail)
-    if (ex.norm_w) {
-        if (nmat == 2) W4A16_GEMV_WS_LAUNCH(2, true);
-        else W4A16_GEMV_WS_LAUNCH(1, true);
+    if (ex.q4) {
+        if constexpr (CT == 8) {   // (the Q4NX plan takes tasks of 8 cells only)
+            if (ex.norm_w) {
+                if (nmat == 2) W4A16_GEMV_WS_LAUNCH(2, true, true);
+                else W4A16_GEMV_WS_LAUNCH(1, true, true);
+            } else {
+                if (nmat == 2) W4A16_GEMV_WS_LAUNCH(2, false, true);
+                else W4A16_GEMV_WS_LAUNCH(1, false, true);
+            }
+        } else {
+            return hipErrorInvalidValue;
+        }
+    } else if (ex.norm_w) {
+        if (nmat == 2) W4A16_GEMV_WS_LAUNCH(2, true, false);
+        else W4A16_GEMV_WS_LAUNCH(1, true, false);
     } else {
-        if (nmat == 2) W4A16_GEMV_WS_LAUNCH(2, false);
-        else W4A16_GEMV_WS_LAUNCH(1, false);
+        if (nmat == 2) W4A16_GEMV_WS_LAUNCH(2, false, false);
+        else W4A16_GEMV_WS_LAUNCH(1, false, false);
     }
 #undef W4A16_GEMV_WS_LAUNCH
     return hipGetLastError();
@@ -320,12 +403,27 @@ GemvWsPlan plan_gemv_ws(int K, int nmat, int N, bool rms) {
 hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, uint16_t *y, int K, int N, hipStream_t stream,
                           const GemvWsExtras &extras) {
     const int nmat = w_up ? 2 : 1;
-    const GemvWsPlan pl = plan_gemv_ws(K, nmat, N, extras.norm_w != nullptr);
+    GemvWsPlan pl = plan_gemv_ws(K, nmat, N, extras.norm_w != nullptr);
+    if (extras.q4 && pl.ct != 8) {   // Q4NX order: tasks of 8 cells
+        pl.ct = 8;
+        const int tasks = nmat * ws_blocks(K) * (kWsBlockGroups / 8);
+        pl.waves = tasks < kMaxWaves ? tasks : kMaxWaves;
+    }
     switch (pl.ct) {
         case 4: return launch_ct<4>(nmat, pl.waves, x, w, w_up, y, K, N, extras, stream);
         case 16: return launch_ct<16>(nmat, pl.waves, x, w, w_up, y, K, N, extras, stream);
         default: return launch_ct<8>(nmat, pl.waves, x, w, w_up, y, K, N, extras, stream);
     }
+}
+
+hipError_t launch_repack_ws_q4(const int32_t *qweight, const uint16_t *scales, const uint16_t *mins, void *out, int K, int N,
+                               hipStream_t stream) {
+    const size_t dwords = ws_q4_matrix_bytes(K, N) / 4;
+    const size_t blocks = (dwords + 255) / 256;
+    if (blocks > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(repack_ws_q4_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<const uint32_t *>(qweight),
+                       scales, mins, static_cast<uint32_t *>(out), K / kGroup, ws_blocks(K), N);
+    return hipGetLastError();
 }
 
 hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *out, int K, int N,

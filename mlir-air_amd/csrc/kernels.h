@@ -102,6 +102,7 @@ struct GemvWsExtras {
     const float *sumsq_in = nullptr;
     int sumsq_n = 0;
     float *sumsq_out = nullptr;
+    bool q4 = false;                      // the matrices are in Q4NX order (a scale and a min per 32 rows)
 };
 struct GemvWsTune {
     int ct = 0;      // cells (groups) per task: 4, 8 or 16 (0 = default)
@@ -132,6 +133,10 @@ hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y,
 // by the up launch with kEpiSiluGateMul.
 hipError_t launch_gemm_prefill_ws_swiglu(const uint16_t *x, const void *w_gate, const void *w_up, uint16_t *h, int M, int K, int H,
                                          hipStream_t stream);
+// Operands of the affine path (q4nx_repack: qweight [K, N / 8], scales and mins [K / 32, N]) -> Q4NX order
+// (ws_q4_matrix_bytes(K, N) bytes at `out`).
+hipError_t launch_repack_ws_q4(const int32_t *qweight, const uint16_t *scales, const uint16_t *mins, void *out, int K, int N,
+                               hipStream_t stream);
 // AutoAWQ checkpoint tensors -> stream order (ws_matrix_bytes(K, N) bytes at `out`).
 hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const uint16_t *scales, void *out, int K, int N,
                             hipStream_t stream);

@@ -25,6 +25,11 @@
 // A matrix takes (N / 16) * (NB + G) KiB: K N / 2 bytes of nibbles plus 4 bytes per (group, column),
 // 1.5 bytes more than the checkpoint's 2.5 (scales bf16 + packed zero points); for G a multiple of
 // 16 that is 1.023 x the checkpoint bytes.
+//
+// Q4NX order (32-row sub-groups with a scale and a min each, w = s q + min'): the same tiles and cells; a block
+// carries 4 KiB of scale / min words instead of 1: KiB t (0..3) belongs to K-step t of the cells, lane l, dword i to
+// group 16 b + 4 lg + i, rows 32 t .. 32 t + 31 of it, column 16 tile + ln: bits 0..15 the bf16 scale, bits 16..31 the
+// bf16 min'.  A tile is (4 NB + G) KiB, block b starts 20 b KiB into it: 5 bits per weight, as in the codec.
 #pragma once
 
 #include <stddef.h>
@@ -39,5 +44,9 @@ constexpr size_t kWsCellBytes = 1024;
 __host__ __device__ constexpr int ws_blocks(int K) { return (K / 128 + kWsBlockGroups - 1) / kWsBlockGroups; }
 __host__ __device__ constexpr size_t ws_tile_bytes(int K) { return (size_t)(ws_blocks(K) + K / 128) * kWsCellBytes; }
 __host__ __device__ constexpr size_t ws_matrix_bytes(int K, int N) { return (size_t)(N / kWsTileCols) * ws_tile_bytes(K); }
+// Q4NX order: KiB of scale / min words per block, bytes of a tile and of a matrix
+constexpr int kWsQ4MdKiB = 4;
+__host__ __device__ constexpr size_t ws_q4_tile_bytes(int K) { return (size_t)(kWsQ4MdKiB * ws_blocks(K) + K / 128) * kWsCellBytes; }
+__host__ __device__ constexpr size_t ws_q4_matrix_bytes(int K, int N) { return (size_t)(N / kWsTileCols) * ws_q4_tile_bytes(K); }
 
 }  // namespace w4a16

@@ -289,3 +289,171 @@ def test_decode_block_q4nx_matches_the_oracle_chain(ops):
         assert np.all(kd <= 2 * bf16_ulp(bf16_bits_to_f32(kc_ref[:, pos])) + 2e-2), kd.max()
         kc[:, pos] = dev(kc_ref[:, pos])
         vc[:, pos] = dev(vc_ref[:, pos])
+
+
+# ---- the same codec in stream order (Q4NX order): whole-K kernels, no workspace ------------------------------------
+
+def _stream_gemv_case(ops, M, K, seed, mode=oq.ADDITIVE, residual=False):
+    print(f"q4nx stream gemv M={M} K={K} mode={mode} residual={residual}", flush=True)
+    q, s, m = make(M, K, seed)
+    rng = np.random.default_rng(seed + 1)
+    x = f32_to_bf16_bits(rng.standard_normal((1, K)).astype(np.float32))
+    qw, sc, mn = ops.q4nx_repack(dev(oq.pack_matrix(q, s, m)), M, K, mode)
+    w = ops.q4nx_repack_stream(qw, sc, mn)
+    res = f32_to_bf16_bits(rng.standard_normal(M).astype(np.float32)) if residual else None
+    y = ops.q4nx_gemv_stream(dev(x[0]), w, residual=dev(res) if residual else None)
+    torch.cuda.synchronize()
+    if mode == oq.SUBTRACTIVE:   # the kernel works on the repacked constant term bf16(-s m)
+        want = oq.gemv_reference(q, s, bits(mn).T.copy(), x, oq.ADDITIVE)[0]
+    else:
+        want = oq.gemv_reference(q, s, m, x, mode)[0]
+    if residual:
+        want = want + bf16_bits_to_f32(res).astype(np.float64)
+    got = bits(y)
+    assert_bf16_close(got, want, ulps=1.0, atol=2e-3, what=f"q4nx stream gemv M={M} K={K}")
+    assert oref.check_outputs(bf16_bits_to_f32(got), bf16_bits_to_f32(f32_to_bf16_bits(want.astype(np.float32))),
+                              rtol=0.1, atol=0.05, min_correlation=0.999)
+    return got, (qw, sc, mn), x
+
+
+# one block of 16 groups and a short one (K = 256), several blocks with a short last one (K = 14336 = 7 blocks,
+# K = 1280 = 10 groups), N from two tiles to the 8B gate width
+@pytest.mark.parametrize("M,K", [(32, 256), (2048, 2048), (1024, 4096), (4096, 14336), (3104, 1280), (14336, 4096)])
+def test_stream_gemv_shapes(ops, M, K):
+    _stream_gemv_case(ops, M, K, seed=M + K)
+
+
+@pytest.mark.parametrize("mode", [oq.SUBTRACTIVE, oq.Q4_0])
+def test_stream_gemv_other_conventions(ops, mode):
+    _stream_gemv_case(ops, 2048, 2048, seed=30 + mode, mode=mode)
+
+
+def test_stream_gemv_with_residual_and_against_the_planar_path(ops):
+    """Residual add; and the stream-order kernel against the kernel on q4nx_repack's own operands: two summation orders
+    of the same fp32 terms, at most an ulp apart, mostly equal."""
+    got, (qw, sc, mn), x = _stream_gemv_case(ops, 4096, 4096, seed=40, residual=False)
+    _stream_gemv_case(ops, 1024, 512, seed=41, residual=True)
+    planar = bits(ops.q4nx_gemm(dev(x), qw, sc, mn))[0]
+    from helpers import bf16_ulp
+    a, b = bf16_bits_to_f32(got).astype(np.float64), bf16_bits_to_f32(planar).astype(np.float64)
+    assert np.all(np.abs(a - b) <= bf16_ulp(b) + 1e-3) and np.mean(got != planar) < 0.2, (np.abs(a - b).max(), np.mean(got != planar))
+
+
+def test_stream_gemv_one_hot_x_is_a_dequantised_row(ops):
+    """x = e_k picks column k of W[M, K]: s q + min of one 32-column group, a single fp32 fma rounded once: bit for bit
+    the dense dequant."""
+    M, K = 256, 512
+    q, s, m = make(M, K, seed=60, wild=True)
+    blocks = dev(oq.pack_matrix(q, s, m))
+    w = ops.q4nx_repack_stream(*ops.q4nx_repack(blocks, M, K, oq.ADDITIVE))
+    dense = bits(ops.q4nx_dequant(blocks, M, K, oq.ADDITIVE))
+    for k in (0, 31, 32, 255, 300, 511):
+        x = np.zeros(K, np.uint16)
+        x[k] = 0x3F80
+        y = bits(ops.q4nx_gemv_stream(dev(x), w))
+        assert np.array_equal(y, dense[:, k]), k
+
+
+@pytest.mark.parametrize("M,K", [(32, 256), (1056, 512), (6144, 4096), (2048, 8192)])
+def test_stream_rms_gemv(ops, M, K):
+    print(f"q4nx stream rms_gemv M={M} K={K}", flush=True)
+    w, wd = _weights(ops, M, K, seed=M + K)
+    sw = ops.q4nx_repack_stream(*wd)
+    x, nw = _vec(K, 70), _norm_w(K, 71)
+    y = ops.q4nx_rms_gemv_stream(dev(x), dev(nw), sw)
+    torch.cuda.synchronize()
+    want = oq.rms_gemv_reference(w, x, nw)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(y)), bf16_bits_to_f32(want), rtol=0.1, atol=0.05, min_correlation=0.999)
+    normed = f32_to_bf16_bits(oref.rms_norm_bf16(x, nw))
+    y2 = ops.q4nx_gemv_stream(dev(normed), sw)     # same GEMV without the prologue, fed the oracle's vector
+    torch.cuda.synchronize()
+    a, b = bf16_bits_to_f32(bits(y)).astype(np.float64), bf16_bits_to_f32(bits(y2)).astype(np.float64)
+    from helpers import bf16_ulp
+    assert np.all(np.abs(a - b) <= 2 * bf16_ulp(b) + 2e-2), np.abs(a - b).max()
+
+
+@pytest.mark.parametrize("E,H", [(256, 512), (2048, 8192), (4096, 14336)])
+def test_stream_o_gemv_ffn_block(ops, E, H):
+    print(f"q4nx stream o_gemv_ffn E={E} H={H}", flush=True)
+    wo, wo_d = _weights(ops, E, E, seed=E)
+    wg, wg_d = _weights(ops, H, E, seed=E + 1)
+    wu, wu_d = _weights(ops, H, E, seed=E + 2)
+    wd, wd_d = _weights(ops, E, H, seed=E + 3)
+    so, sg, su, sd = (ops.q4nx_repack_stream(*t) for t in (wo_d, wg_d, wu_d, wd_d))
+    attn, xres, nw = _vec(E, 80), _vec(E, 81), _norm_w(E, 82)
+    y, res1, h, sumsq = ops.q4nx_o_gemv_ffn_stream(dev(attn), dev(xres), dev(nw), so, sg, su, sd, return_intermediates=True,
+                                                   return_sumsq=True)
+    torch.cuda.synchronize()
+    want1 = oq.gemv_reference(*wo, attn)[0] + bf16_bits_to_f32(xres)
+    assert_bf16_close(bits(res1), want1, ulps=1.0, atol=2e-3, what="res1")
+    want3 = oq.gemv_reference(*wd, bits(h))[0] + bf16_bits_to_f32(bits(res1))
+    assert_bf16_close(bits(y), want3, ulps=1.0, atol=2e-3, what="block y")
+    normed = f32_to_bf16_bits(oref.rms_norm_bf16(bits(res1), nw))
+    gate = bf16_bits_to_f32(f32_to_bf16_bits(oq.gemv_reference(*wg, normed)[0].astype(np.float32)))
+    up = bf16_bits_to_f32(f32_to_bf16_bits(oq.gemv_reference(*wu, normed)[0].astype(np.float32)))
+    h_want = bf16_bits_to_f32(f32_to_bf16_bits(oref.silu_tanh_f32(gate) * up))
+    assert oref.check_outputs(bf16_bits_to_f32(bits(h)), h_want, rtol=0.15, atol=0.5, min_correlation=0.99)
+    r1, hh, yy = oq.block_staged_reference(wo, wg, wu, wd, attn, xres, nw)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(res1)), bf16_bits_to_f32(r1), rtol=0.1, atol=0.05, min_correlation=0.999)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(h)), bf16_bits_to_f32(hh), rtol=0.15, atol=0.5, min_correlation=0.99)
+    assert oref.check_outputs(bf16_bits_to_f32(bits(y)), bf16_bits_to_f32(yy), rtol=0.2, atol=2.0, min_correlation=0.99)
+    # the sums of squares the next layer's norm will use are those of the rounded outputs, 16 columns at a time
+    yf = bf16_bits_to_f32(bits(y)).astype(np.float64)
+    assert np.allclose(sumsq.cpu().numpy(), (yf ** 2).reshape(-1, 16).sum(axis=1), rtol=1e-5)
+    y2 = ops.q4nx_o_gemv_ffn_stream(dev(attn), dev(xres), dev(nw), so, sg, su, sd)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y2), bits(y))
+
+
+def test_stream_entry_points_reject_bad_arguments(ops):
+    from air_hip import _lib
+    lib = _lib.load_library()
+    P = torch.zeros(1 << 16, dtype=torch.int32, device="cuda").data_ptr()
+    assert lib.w4a16_q4nx_stream_bytes(256, 24) == 0 and lib.w4a16_q4nx_stream_bytes(192, 32) == 0
+    assert lib.w4a16_q4nx_stream_bytes(256, 32) == 2 * (4 + 2) * 1024
+    assert lib.w4a16_q4nx_repack_stream(P, P, None, P, 256, 32, None) == _lib.ERR_NULL
+    assert lib.w4a16_q4nx_repack_stream(P, P, P, P, 200, 32, None) == _lib.ERR_SHAPE
+    assert lib.w4a16_q4nx_gemv_stream_bf16(P, P, None, P, 256, 40, None) == _lib.ERR_SHAPE
+    assert lib.w4a16_q4nx_gemv_stream_bf16(P, None, None, P, 256, 32, None) == _lib.ERR_NULL
+    assert lib.w4a16_q4nx_gemv_stream_bf16(P + 2, P, None, P, 256, 32, None) == _lib.ERR_ALIGN
+    assert lib.w4a16_q4nx_rms_gemv_stream_bf16(P, None, 0, None, 1e-5, P, P, 256, 32, None) == _lib.ERR_NULL
+    ws = lib.w4a16_block_stream_workspace_bytes(256, 256)
+    assert lib.w4a16_q4nx_o_gemv_ffn_stream_bf16(P, P, P, 1e-5, P, P, P, P, P, None, None, None, 256, 256, P, ws - 1, None) == _lib.ERR_WORKSPACE
+
+
+def test_decode_block_q4nx_stream_order_agrees_with_the_planar_layer(ops):
+    """run_decode_block on a Q4NX layer with and without the stream-order re-pack: same caches, outputs an ulp or
+    two apart (another summation order in every GEMV)."""
+    from air_hip import decode, weights
+    cfg = weights.LlamaConfig(n_layers=1, emb_dim=512, n_heads=8, head_dim=64, n_kv_heads=2, hidden_dim=1024, vocab_size=32)
+    E, H, nq, nkv = cfg.emb_dim, cfg.hidden_dim, cfg.n_heads * cfg.head_dim, cfg.kv_dim
+
+    def qw(M, K, seed):
+        rng = np.random.default_rng(seed)
+        W = (rng.standard_normal((M, K)) * 0.02).astype(np.float32)
+        q, sc, mn = oq.requant_q4k(W)
+        return q, f32_to_bf16_bits(sc), f32_to_bf16_bits(mn)
+
+    w = {"q": qw(nq, E, 1), "k": qw(nkv, E, 2), "v": qw(nkv, E, 3), "o": qw(E, nq, 4),
+         "gate": qw(H, E, 5), "up": qw(H, E, 6), "down": qw(E, H, 7)}
+    blocks = {k: oq.pack_matrix(*v) for k, v in w.items()}
+    attn_norm, ffn_norm = _norm_w(E, 8), _norm_w(E, 9)
+    planar = decode.prepare_layer_q4nx(blocks, attn_norm, ffn_norm, cfg, stream_order=False)
+    stream = decode.prepare_layer_q4nx(blocks, attn_norm, ffn_norm, cfg)
+    assert stream.stream is not None and planar.stream is None
+    max_seq = 64
+    lut = decode.generate_rope_lut(cfg, max_seq)
+    (kc1, vc1), = decode.new_kv_cache(cfg, max_seq)
+    (kc2, vc2), = decode.new_kv_cache(cfg, max_seq)
+    for pos in range(4):
+        print(f"q4nx decode block, stream order against planar, pos={pos}", flush=True)
+        x = dev(_vec(E, 600 + pos))
+        y1 = decode.run_decode_block(x, planar, cfg, kc1, vc1, pos, lut)
+        y2, sumsq = decode.run_decode_block(x, stream, cfg, kc2, vc2, pos, lut, return_sumsq=True)
+        torch.cuda.synchronize()
+        err = (y1.float() - y2.float()).abs().max().item()
+        assert err <= 4 * 2.0**-8 * y1.float().abs().max().item(), err
+        kerr = (kc1[:, pos].float() - kc2[:, pos].float()).abs().max().item()
+        assert kerr <= 2 * 2.0**-8 * kc1[:, pos].float().abs().max().item() + 1e-2, kerr
+        assert sumsq is not None and sumsq.numel() == E // 16
+        kc2[:, pos], vc2[:, pos] = kc1[:, pos], vc1[:, pos]
