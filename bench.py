@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemv_planar|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemv_planar|q4nx_gemm16|q4nx_gemm16_planar|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -50,7 +50,8 @@ CONFIGS = {
     # projection shape of Llama-3.1-8B (programming_examples/llms/llama31_8b_q4nx)
     "q4nx_gemv": dict(M=1, K=4096, N=14336, cfg=None, desc="decode GEMV Q4NX M=1 K=4096 N=14336 g32, weights in Q4NX stream order"),
     "q4nx_gemv_planar": dict(M=1, K=4096, N=14336, cfg=None, desc="decode GEMV Q4NX M=1 K=4096 N=14336 g32, operands of q4nx_repack (split-K with a workspace)"),
-    "q4nx_gemm16": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM Q4NX M=16 K=4096 N=14336 g32"),
+    "q4nx_gemm16": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM Q4NX M=16 K=4096 N=14336 g32, weights in Q4NX stream order"),
+    "q4nx_gemm16_planar": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM Q4NX M=16 K=4096 N=14336 g32, operands of q4nx_repack (split-K with a workspace)"),
     # the tail of a decode step of Llama-3.2-1B: final RMSNorm + bf16 lm_head GEMV + argmax
     "lm_head": dict(M=1, K=2048, N=128256, cfg=None, desc="decode tail RMSNorm + bf16 lm_head GEMV + argmax E=2048 V=128256"),
 }
@@ -157,7 +158,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             copies.append(c4 + ((make_weights(torch, K, nqkv, 104 + 5 * i),) if kind == "layer" else ()))
         elif q4nx:
             copies.append(make_q4nx_weights(torch, K, N, 100 + i))
-            if name == "q4nx_gemv":   # re-packed at load time (untimed)
+            if name in ("q4nx_gemv", "q4nx_gemm16"):   # re-packed at load time (untimed)
                 from air_hip import ops
                 copies[-1] = (ops.q4nx_repack_stream(*copies[-1]).buf,)
         elif lm_head:
@@ -278,6 +279,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             rc = lib.w4a16_gemm_stream_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), M, K, N, 128, st)
         elif name == "q4nx_gemv":
             rc = lib.w4a16_q4nx_gemv_stream_bf16(x.data_ptr(), w[0].data_ptr(), None, outs[0].data_ptr(), K, N, st)
+        elif name == "q4nx_gemm16":
+            rc = lib.w4a16_q4nx_gemm_stream_bf16(x.data_ptr(), w[0].data_ptr(), None, outs[0].data_ptr(), M, K, N, st)
         elif q4nx:
             rc = lib.w4a16_q4nx_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), None,
                                           outs[0].data_ptr(), M, K, N, ws.data_ptr(), ws.numel(), st)

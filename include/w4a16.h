@@ -550,6 +550,9 @@ int w4a16_q4nx_repack_stream(const int32_t *qweight, const uint16_t *scales, con
                              void *stream);
 int w4a16_q4nx_gemv_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int K, int N,
                                 void *stream);
+/* y[M, N] = bf16(x[M, K] . W + residual [M, N]): the GEMV at M = 1, the batched whole-K kernel in launches of 16 rows else */
+int w4a16_q4nx_gemm_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int M, int K, int N,
+                                void *stream);
 int w4a16_q4nx_rms_gemv_stream_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
                                     const void *wstream, uint16_t *y, int K, int N, void *stream);
 int w4a16_q4nx_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,

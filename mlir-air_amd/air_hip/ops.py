@@ -809,6 +809,22 @@ def q4nx_gemv_stream(x, w, residual=None, out=None):
     return out
 
 
+def q4nx_gemm_stream(x, w, residual=None, out=None):
+    """y[M, N] = bf16(x[M, K] . W (+ residual [M, N])) on a Q4NX-order StreamWeight; x may be a vector [K]."""
+    lib = _lib.load_library()
+    _need_cuda(x, w.buf)
+    vec = x.dim() == 1
+    x2 = x.unsqueeze(0) if vec else x
+    M, K = x2.shape
+    if K != w.K or (residual is not None and residual.numel() != M * w.N):
+        raise ValueError("q4nx_gemm_stream: x must be [M, K], residual [M, N]")
+    if out is None:
+        out = torch.empty((M, w.N), dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.w4a16_q4nx_gemm_stream_bf16(_ptr(_bits(x2)), _ptr(w.buf), _ptr(_bits(residual)) if residual is not None else None,
+                                               _ptr(out), M, K, w.N, _stream()))
+    return out.squeeze(0) if vec else out
+
+
 def q4nx_rms_gemv_stream(x, norm_weight, w, eps=1e-5, x_sumsq=None):
     """y[N] = bf16(rms_norm(x, norm_weight) . W) on a Q4NX-order StreamWeight (x_sumsq as in w4a16_rms_gemv_stream)."""
     lib = _lib.load_library()

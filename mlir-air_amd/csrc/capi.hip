@@ -904,6 +904,16 @@ int w4a16_q4nx_gemv_stream_bf16(const uint16_t *x, const void *wstream, const ui
     return gemv_stream_call(x, wstream, nullptr, y, K, N, kGroup, stream, ex);
 }
 
+int w4a16_q4nx_gemm_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int M, int K, int N,
+                                void *stream) {
+    if (M == 1) return w4a16_q4nx_gemv_stream_bf16(x, wstream, residual, y, K, N, stream);
+    if (!x || !wstream || !y) return W4A16_ERR_NULL;
+    if (M <= 0 || K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
+    if (misaligned(x) || misaligned(wstream) || misaligned(y) || (residual && misaligned(residual))) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_gemm_ws(x, wstream, y, residual, M, K, N, static_cast<hipStream_t>(stream), true);
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_q4nx_rms_gemv_stream_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
                                     const void *wstream, uint16_t *y, int K, int N, void *stream) {
     if (!norm_weight) return W4A16_ERR_NULL;

@@ -452,7 +452,9 @@ namespace {
 constexpr int kGemmWsWaves = 8;
 constexpr int kGemmWsGroups = 4;   // groups per task
 
-template <int CB>
+// Q4: the matrix is in Q4NX order (a scale and a min per 32 rows): every K-step of a cell is a product of its own,
+// folded in at once as y += s sum((128 + q) x) + (min - 128 s) sum(x).
+template <int CB, bool Q4>
 __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16_t *__restrict__ x, const char *__restrict__ w,
                                                                     uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
                                                                     int M, int K, int N, int G, int NB) {
@@ -460,7 +462,8 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lg = lane >> 4, ln = lane & 15;
-    const size_t tile_bytes = (size_t)(NB + G) * kWsCellBytes;
+    constexpr int MDK = Q4 ? kWsQ4MdKiB : 1;   // KiB of scale words in front of a block's cells
+    const size_t tile_bytes = (size_t)(MDK * NB + G) * kWsCellBytes;
     const char *tile0 = w + (size_t)blockIdx.x * CB * tile_bytes;
 
     const uint32_t ones_w = 0x3F803F80u;
@@ -489,15 +492,18 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
     // workgroup from HBM), 10.3 us with both: the two streams add up, i.e. a CU takes in ~40 bytes per ns whatever the
     // source.  Not kept, no gain: x copied to LDS once per workgroup with whole-line requests (10.3 - 10.4 us); the 896
     // tiles dealt 4 and 3 to 256 workgroups instead of 4 to 224 (10.55 against 10.59 us on one box).
-    u32x4 *mdl = reinterpret_cast<u32x4 *>(red + kGemmWsWaves * CB * 4 * 64) + wave * 64;
+    // (Q4NX order: one such request and KiB per K-step, lane (c, ln) of KiB t holding the task's four (scale, min) pairs of
+    // rows 32 t .. 32 t + 31.)
+    u32x4 *mdl = reinterpret_cast<u32x4 *>(red + kGemmWsWaves * CB * 4 * 64) + wave * 64 * MDK;
     for (int task = wave; task < ntasks; task += kGemmWsWaves) {
         const int g0 = task * kGemmWsGroups;
         u32x4 X[kGemmWsGroups][4], cell[kGemmWsGroups][CB];
-        u32x4 mdq;
+        u32x4 mdq[MDK];
         {
             const int b = g0 >> 4, gl = g0 & 15, c = lg < CB ? lg : CB - 1;
-            mdq = *reinterpret_cast<const u32x4 *>(tile0 + (size_t)c * tile_bytes + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes) +
-                                                   (16 * (gl >> 2) + ln) * 16);
+            const char *src = tile0 + (size_t)c * tile_bytes + (size_t)b * ((kWsBlockGroups + MDK) * kWsCellBytes) + (16 * (gl >> 2) + ln) * 16;
+#pragma unroll
+            for (int t = 0; t < MDK; ++t) mdq[t] = *reinterpret_cast<const u32x4 *>(src + (size_t)t * kWsCellBytes);
         }
 #pragma unroll
         for (int j = 0; j < kGemmWsGroups; ++j) {
@@ -509,15 +515,46 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
         for (int j = 0; j < kGemmWsGroups; ++j) {
             const int g = g0 + j < G ? g0 + j : G - 1;
             const int b = g >> 4, gl = g & 15;
-            const char *blk = tile0 + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes);
+            const char *blk = tile0 + (size_t)b * ((kWsBlockGroups + MDK) * kWsCellBytes);
 #pragma unroll
             for (int c = 0; c < CB; ++c)
-                cell[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)c * tile_bytes + (size_t)(1 + gl) * kWsCellBytes) + lane);
+                cell[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)c * tile_bytes + (size_t)(MDK + gl) * kWsCellBytes) + lane);
         }
         __builtin_amdgcn_sched_barrier(0);
+        // (LDS operations of one wave complete in order; the previous task's reads are done)
+#pragma unroll
+        for (int t = 0; t < MDK; ++t) mdl[64 * t + lane] = mdq[t];
+        if constexpr (Q4) {
+            const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < kGemmWsGroups; ++j) {
+                const bool valid = row_valid && g0 + j < G;
+                floatx4 xs[4];   // xs[t][i]: sum of x[4 lg + i] over rows 32 t .. 32 t + 31 of the group
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    if (!valid) X[j][t] = u32x4{0u, 0u, 0u, 0u};
+                    xs[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[j][t]), ones, zero4, 0, 0, 0);
+                }
+#pragma unroll
+                for (int c = 0; c < CB; ++c) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[j][t]),
+                                                                                    cell_operand(cell[j][c][t], nib_mask, magic), zero4, 0, 0, 0);
+                        // the pair of (group g0 + j, K-step t, column ln) of tile c: dword j of the chunk lane 16 c + ln fetched
+                        uint32_t mw = reinterpret_cast<const uint32_t *>(mdl + 64 * t + 16 * c + ln)[j];
+                        if (g0 + j >= G) mw = 0u;   // (a short last task: no such group)
+                        const float sf = __builtin_bit_cast(float, mw << 16);
+                        const float c2 = fmaf(-128.0f, sf, __builtin_bit_cast(float, mw & 0xFFFF0000u));   // min - 128 s
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) Y[c][i] = fmaf(sf, acc[i], fmaf(c2, xs[t][i], Y[c][i]));
+                    }
+                }
+            }
+            continue;
+        }
         // the scale word of (group g0 + j, column ln) of tile c: dword j of the chunk that lane 16 c + ln fetched
         u32x4 md[CB];
-        mdl[lane] = mdq;   // (LDS operations of one wave complete in order; the previous task's reads are done)
 #pragma unroll
         for (int cc = 0; cc < CB; ++cc) md[cc] = mdl[16 * cc + ln];
 #pragma unroll
@@ -567,20 +604,30 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
     }
 }
 
-template <int CB>
-hipError_t launch_gemm_ws_cb(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
-                             hipStream_t stream) {
-    const size_t lds = (size_t)kGemmWsWaves * CB * 4 * 64 * sizeof(float) + kGemmWsWaves * kWsCellBytes;   // sums, scale words
-    hipLaunchKernelGGL((gemm_ws_kernel<CB>), dim3(N / (16 * CB)), dim3(kGemmWsWaves * 64), lds, stream, x,
+template <int CB, bool Q4>
+hipError_t launch_gemm_ws_q(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
+                            hipStream_t stream) {
+    const size_t lds = (size_t)kGemmWsWaves * CB * 4 * 64 * sizeof(float) + kGemmWsWaves * kWsCellBytes * (Q4 ? kWsQ4MdKiB : 1);   // sums, scale words
+    if (lds >= 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_ws_kernel<CB, Q4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((gemm_ws_kernel<CB, Q4>), dim3(N / (16 * CB)), dim3(kGemmWsWaves * 64), lds, stream, x,
                        static_cast<const char *>(w), y, residual, M, K, N, K / kGroup, ws_blocks(K));
     return hipGetLastError();
+}
+
+template <int CB>
+hipError_t launch_gemm_ws_cb(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
+                             hipStream_t stream, bool q4) {
+    return q4 ? launch_gemm_ws_q<CB, true>(x, w, y, residual, M, K, N, stream) : launch_gemm_ws_q<CB, false>(x, w, y, residual, M, K, N, stream);
 }
 
 }  // namespace
 
 // y[M, N] = bf16(x[M, K] . W (+ residual)), 2 <= M <= 16 per launch; more rows run as launches of 16.
 hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
-                          hipStream_t stream) {
+                          hipStream_t stream, bool q4) {
     const int tiles = N / kWsTileCols;
     int cb = g_gemv_ws_tune.cb;
     if (!cb) cb = tiles % 4 == 0 && tiles / 4 >= 200 ? 4 : (tiles % 2 == 0 && tiles / 2 >= 200 ? 2 : 1);
@@ -590,9 +637,9 @@ hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const u
         const int rows = M - m0 < 16 ? M - m0 : 16;
         const uint16_t *xr = x + (size_t)m0 * K, *rr = residual ? residual + (size_t)m0 * N : nullptr;
         uint16_t *yr = y + (size_t)m0 * N;
-        e = cb == 4 ? launch_gemm_ws_cb<4>(xr, w, yr, rr, rows, K, N, stream)
-          : cb == 2 ? launch_gemm_ws_cb<2>(xr, w, yr, rr, rows, K, N, stream)
-                    : launch_gemm_ws_cb<1>(xr, w, yr, rr, rows, K, N, stream);
+        e = cb == 4 ? launch_gemm_ws_cb<4>(xr, w, yr, rr, rows, K, N, stream, q4)
+          : cb == 2 ? launch_gemm_ws_cb<2>(xr, w, yr, rr, rows, K, N, stream, q4)
+                    : launch_gemm_ws_cb<1>(xr, w, yr, rr, rows, K, N, stream, q4);
     }
     return e;
 }

@@ -123,7 +123,7 @@ hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, ui
                           const GemvWsExtras &extras = GemvWsExtras());
 // y[M, N] = bf16(x[M, K] . W (+ residual [M, N])) with W in stream order, any M >= 2 (launches of up to 16 rows).
 hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
-                          hipStream_t stream);
+                          hipStream_t stream, bool q4 = false);   // q4: W in Q4NX order
 // Prefill GEMM on stream-order weights (gemm_ws.hip): bf16-rounded weights dequantised in registers, x through LDS.
 bool gemm_prefill_ws_supported(int M, int K, int N);   // K % 256 == 0, N % 64 == 0
 // Epilogues as for launch_gemm_prefill (kEpi*); kEpiRope with heads of 128 needs N % 128 == 0.

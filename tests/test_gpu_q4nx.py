@@ -339,6 +339,31 @@ def test_stream_gemv_with_residual_and_against_the_planar_path(ops):
     assert np.all(np.abs(a - b) <= bf16_ulp(b) + 1e-3) and np.mean(got != planar) < 0.2, (np.abs(a - b).max(), np.mean(got != planar))
 
 
+@pytest.mark.parametrize("rows,M,K,residual", [(2, 512, 1024, False), (16, 512, 1024, True), (7, 64, 256, False), (17, 1024, 512, True),
+                                               (40, 512, 1280, False), (16, 14336, 4096, False)])
+def test_stream_gemm_rows(ops, rows, M, K, residual):
+    """The batched whole-K kernel on the Q4NX order: 2..16 rows per launch, more rows in launches of 16; the tile count of
+    N decides how many tiles a workgroup takes (1, 2 or 4)."""
+    print(f"q4nx stream gemm rows={rows} M={M} K={K} residual={residual}", flush=True)
+    q, s, m = make(M, K, seed=rows + M)
+    rng = np.random.default_rng(rows + 1)
+    x = f32_to_bf16_bits(rng.standard_normal((rows, K)).astype(np.float32))
+    w = ops.q4nx_repack_stream(*ops.q4nx_repack(dev(oq.pack_matrix(q, s, m)), M, K, oq.ADDITIVE))
+    res = f32_to_bf16_bits(rng.standard_normal((rows, M)).astype(np.float32)) if residual else None
+    y = ops.q4nx_gemm_stream(dev(x), w, residual=dev(res) if residual else None)
+    torch.cuda.synchronize()
+    want = oq.gemv_reference(q, s, m, x, oq.ADDITIVE)
+    if residual:
+        want = want + bf16_bits_to_f32(res).astype(np.float64)
+    got = bits(y)
+    assert_bf16_close(got, want, ulps=1.0, atol=2e-3, what=f"q4nx stream gemm rows={rows} M={M} K={K}")
+    # row r of the batch is the GEMV of row r up to the summation order
+    y0 = bits(ops.q4nx_gemv_stream(dev(x[0]), w, residual=dev(res[0]) if residual else None))
+    from helpers import bf16_ulp
+    a, b = bf16_bits_to_f32(got[0]).astype(np.float64), bf16_bits_to_f32(y0).astype(np.float64)
+    assert np.all(np.abs(a - b) <= bf16_ulp(b) + 1e-3)
+
+
 def test_stream_gemv_one_hot_x_is_a_dequantised_row(ops):
     """x = e_k picks column k of W[M, K]: s q + min of one 32-column group, a single fp32 fma rounded once: bit for bit
     the dense dequant."""
