@@ -293,6 +293,41 @@ def repack_stream(qweight, qzeros, scales):
     return out
 
 
+def repack_stream_q4nx(q, scale_bits, min_bits):
+    """Q4NX stream order, uint32 [N/16, (4 NB + G) * 256], from the values of the affine path: q uint8 [K, N] (unsigned
+    nibbles), scale and min' bit patterns uint16 [K/32, N] with w = s q + min' (host twin of w4a16_q4nx_repack_stream,
+    whose operands are the same values in q4nx_repack's packing).  Cells as in repack_stream; in front of a block's
+    cells 4 KiB of words, KiB t, lane 16 lg + ln, dword i = (scale | min' << 16) of rows 32 t .. 32 t + 31 of group
+    16 b + 4 lg + i, column 16 tile + ln."""
+    q = np.asarray(q)
+    s = np.asarray(scale_bits).astype(np.uint32)
+    m = np.asarray(min_bits).astype(np.uint32)
+    K, N = q.shape
+    G = K // GROUP
+    if K % GROUP or N % STREAM_TILE_COLS or s.shape != (K // 32, N) or m.shape != s.shape:
+        raise ValueError("repack_stream_q4nx: need K % 128 == 0, N % 16 == 0 and [K/32, N] scales / mins")
+    NB = -(-G // STREAM_BLOCK_GROUPS)
+    T = N // STREAM_TILE_COLS
+    MDK = 4
+    out = np.zeros((T, (MDK * NB + G) * 256), dtype=np.uint32)
+    qv = q.reshape(G, 4, 4, 8, T, 16).astype(np.uint32)          # [g, t, lg, j, tile, ln]
+    cells = np.zeros((G, 4, 4, T, 16), dtype=np.uint32)          # [g, t, lg, tile, ln]
+    for p, j in enumerate(PACK_ORDER):
+        cells |= qv[:, :, :, j] << np.uint32(4 * p)
+    cells = cells.transpose(3, 0, 2, 4, 1)                       # [tile, g, lg, ln, t]
+    md = (s | (m << np.uint32(16))).reshape(G, 4, N)             # [g, t, n]
+    md_pad = np.zeros((NB * STREAM_BLOCK_GROUPS, 4, N), dtype=np.uint32)
+    md_pad[:G] = md
+    md_pad = md_pad.reshape(NB, 4, 4, 4, T, 16).transpose(4, 0, 3, 1, 5, 2)   # [tile, b, t, lg, ln, i]
+    for b in range(NB):
+        g0 = b * STREAM_BLOCK_GROUPS
+        ng = min(STREAM_BLOCK_GROUPS, G - g0)
+        base = b * (STREAM_BLOCK_GROUPS + MDK) * 256
+        out[:, base:base + MDK * 256] = md_pad[:, b].reshape(T, MDK * 256)
+        out[:, base + MDK * 256:base + 256 * (MDK + ng)] = cells[:, g0:g0 + ng].reshape(T, ng * 256)
+    return out
+
+
 def unpack_stream(buf, K, N):
     """Stream order -> (q uint8 [K, N], z uint8 [K/128, N], scale bits uint16 [K/128, N])."""
     G = K // GROUP

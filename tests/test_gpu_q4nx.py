@@ -364,6 +364,18 @@ def test_stream_gemm_rows(ops, rows, M, K, residual):
     assert np.all(np.abs(a - b) <= bf16_ulp(b) + 1e-3)
 
 
+@pytest.mark.parametrize("M,K", [(32, 256), (96, 2304), (1024, 4096)])
+def test_stream_device_repack_equals_host_packer(ops, M, K):
+    """w4a16_q4nx_repack_stream on the operands of q4nx_repack against the host packer on the same values."""
+    from air_hip import awq
+    q, s, m = make(M, K, seed=M + K, wild=True)
+    qw, sc, mn = ops.q4nx_repack(dev(oq.pack_matrix(q, s, m)), M, K, oq.ADDITIVE)
+    w = ops.q4nx_repack_stream(qw, sc, mn)
+    torch.cuda.synchronize()
+    want = awq.repack_stream_q4nx(q.T.copy(), s.T.copy(), m.T.copy())     # [K, N = M] values
+    assert np.array_equal(w.buf.cpu().numpy().view(np.uint32).reshape(want.shape), want)
+
+
 def test_stream_gemv_one_hot_x_is_a_dequantised_row(ops):
     """x = e_k picks column k of W[M, K]: s q + min of one 32-column group, a single fp32 fma rounded once: bit for bit
     the dense dequant."""

@@ -68,3 +68,37 @@ def test_rejects_shapes_outside_the_layout():
         awq.stream_bytes(4096, 24)
     with pytest.raises(ValueError):
         awq.stream_bytes(4000, 32)
+
+
+def test_q4nx_order_elements_followed_by_hand():
+    """Q4NX order, K = 2304 (18 groups: one full block and a short one), N = 32: a tile is (4 * 2 + 18) KiB, block b
+    starts 20 b KiB into it; the pair of (row k, column n) sits in KiB t = (k % 128) / 32 of the block's first four,
+    lane 16 lg + ln with 4 lg + i = (k / 128) % 16, dword i; the nibble as in the AWQ order behind those 4 KiB."""
+    K, N = 2304, 32
+    rng = np.random.default_rng(5)
+    q = rng.integers(0, 16, (K, N), dtype=np.uint8)
+    s = rng.integers(0, 65536, (K // 32, N)).astype(np.uint16)
+    m = rng.integers(0, 65536, (K // 32, N)).astype(np.uint16)
+    raw = awq.repack_stream_q4nx(q, s, m)
+    assert raw.nbytes == (N // 16) * (4 * 2 + 18) * 1024
+    by = raw.view(np.uint8).reshape(-1).astype(np.int64)
+    tile_bytes = 26 * 1024
+    for k, n in ((0, 0), (77, 9), (128 * 5 + 33, 17), (128 * 16 + 100, 31), (2303, 16)):
+        tile, ln = n // 16, n % 16
+        g, r = k // 128, k % 128
+        b, gl = g // 16, g % 16
+        t, lg, j = r // 32, (r % 32) // 8, r % 8
+        p = (0, 2, 4, 6, 1, 3, 5, 7).index(j)
+        blk = tile * tile_bytes + b * 20 * 1024
+        # nibble: cell gl of the block, behind the 4 KiB of pairs
+        byte = blk + (4 + gl) * 1024 + (16 * lg + ln) * 16 + 4 * t + p // 2
+        assert ((by[byte] >> (4 * (p % 2))) & 0xF) == q[k, n], (k, n)
+        # pair of this row's 32-row sub-group: KiB t, lane 16 (gl / 4) + ln, dword gl % 4
+        word = blk + t * 1024 + (16 * (gl // 4) + ln) * 16 + 4 * (gl % 4)
+        got = by[word] | (by[word + 1] << 8) | (by[word + 2] << 16) | (by[word + 3] << 24)
+        assert got == (int(s[k // 32, n]) | (int(m[k // 32, n]) << 16)), (k, n)
+    # groups 18 .. 31 of the short block do not exist: their pair words are zero
+    short = raw[0, 20 * 256:20 * 256 + 4 * 256].reshape(4, 4, 16, 4)      # [t, lg, ln, i] of block 1
+    assert np.all(short[:, 1:] == 0) and np.all(short[:, 0, :, 2:] == 0) and np.any(short[:, 0, :, :2] != 0)
+    with pytest.raises(ValueError):
+        awq.repack_stream_q4nx(q[:100], s[:3], m[:3])
