@@ -22,8 +22,9 @@ read back, one result per argument with empty arrays for slots that are not read
 `_run_layer_int4` can be pointed at it unchanged.  The packed weight slots take the reference's
 buffers (decode: uint8 [tiles, tile_bytes], `matvec_int4_packed.pack_inputs`; prefill: uint8
 [N / tile_n, K / 128, tile_bytes], `awq_pack_for_npu`); on the first call of a `bo_key` they are
-unpacked to the AutoAWQ layout the HIP kernels read and stay in HBM, the counterpart of the
-reference's write-once buffer objects.  "Compiling" validates a module description against the
+unpacked, re-packed on the GPU into the stream order the whole-K decode kernels and the tiled prompt-pass
+GEMM read (`KernelCache(stream_order=False)`: left as AutoAWQ triples for the checkpoint-layout kernels)
+and stay in HBM, the counterpart of the reference's write-once buffer objects.  "Compiling" validates a module description against the
 kernels' shape rules; there is nothing to build at run time.
 
 bf16 arrays are `air_hip.bf16.BF16Array` (uint16 bit patterns) or ml_dtypes bfloat16 arrays; results
@@ -219,12 +220,14 @@ class KernelCache:
 
     MANIFEST_FILE = "manifest.json"
 
-    def __init__(self, cache_dir=None, verbose=False, profiler=None):
+    def __init__(self, cache_dir=None, verbose=False, profiler=None, stream_order=True):
         self.cache_dir = Path(cache_dir) if cache_dir is not None else None
         if self.cache_dir is not None:
             self.cache_dir.mkdir(parents=True, exist_ok=True)
         self.verbose = verbose
         self.profiler = profiler or Profiler()
+        # static weight slots are kept in HBM in stream order (False: as AutoAWQ triples, for the checkpoint-layout kernels)
+        self.stream_order = stream_order
         self.artifacts = {}      # name -> DecodeModule
         self._cached_bos = {}    # bo_key -> {arg index or derived name: device tensors}
         self._shared_bos = {}    # (alias, bytes) -> device tensor handed from a producer to a consumer
@@ -340,10 +343,23 @@ class KernelCache:
             stats["bytes"] += int(np.asarray(inputs[i]).size)
             return awq.unpack_gemm_tiles(np.asarray(inputs[i]).view(np.uint8), K, N, mod.gs, mod.tile_n, mod.tile_k)
 
+        # One layout for every matrix of a call: stream order where the call's kernels take all of them (decode:
+        # input lengths in whole groups; prompt pass: whole pairs of groups and 64-column tiles).
+        E, H, n_qkv = mod.emb_dim, mod.hidden_dim, mod.emb_dim + 2 * mod.kv_dim
+        stream_order = self.stream_order and mod.gs == awq.GROUP and {
+            "rms_qkv_int4_rope": E % 128 == 0 and n_qkv % 16 == 0,
+            "o_gemv_ffn_int4": E % 128 == 0 and H % 128 == 0,
+            "rms_gemms_rope_int4": E % 256 == 0 and n_qkv % 64 == 0,
+            "o_ffn_int4": E % 256 == 0 and H % 256 == 0,
+        }.get(mod.kernel, False)
+
         def to_awq_dev(l1):
+            """Kernel-side arrays -> the matrix in HBM: in stream order (ops.StreamWeight, the layout the fast
+            kernels read) where the call takes it, else the AutoAWQ triple for the checkpoint-layout kernels."""
             qw, qz, sc = awq.awq_from_l1(*l1)
             dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-            return dev(qw), dev(qz), dev(bf16.bits_of(sc).view(np.int16)).view(torch.bfloat16)
+            triple = dev(qw), dev(qz), dev(bf16.bits_of(sc).view(np.int16)).view(torch.bfloat16)
+            return ops.repack_stream(*triple, group=mod.gs) if stream_order else triple
 
         def weights(tag, indices, build):
             """Device weights derived from packed slots `indices`; kept while all of them are resident."""
@@ -421,7 +437,10 @@ class KernelCache:
         lut_k = vec(10, (nkv, hd))
 
         def run(readback):
-            qkv = ops.w4a16_rms_gemv(x, norm_w, *wqkv, eps=mod.eps)
+            if isinstance(wqkv, ops.StreamWeight):
+                qkv = ops.w4a16_rms_gemv_stream(x, norm_w, wqkv, eps=mod.eps, group=mod.gs)
+            else:
+                qkv = ops.w4a16_rms_gemv(x, norm_w, *wqkv, eps=mod.eps)
             q, k, v = qkv[:E], qkv[E:E + KV], qkv[E + KV:]
             out = {4: q, 6: k, 8: v}
             if 11 in readback:
@@ -454,8 +473,9 @@ class KernelCache:
         wd = weights("wdown", (12,), lambda: to_awq_dev(linear(12, E, H)))
 
         def run(readback):
-            y, res1, h = ops.o_gemv_ffn(attn_out, x_residual, rms_buf[1].contiguous(), wo, wg, wu, wd, eps=mod.eps,
-                                        return_intermediates=True)
+            block = ops.o_gemv_ffn_stream if all(isinstance(w, ops.StreamWeight) for w in (wo, wg, wu, wd)) else ops.o_gemv_ffn
+            y, res1, h = block(attn_out, x_residual, rms_buf[1].contiguous(), wo, wg, wu, wd, eps=mod.eps,
+                               return_intermediates=True)
             out = {14: y, 11: h}
             if 6 in readback:
                 out[6] = torch.stack([res1, rms_buf[1]])
@@ -485,11 +505,13 @@ class KernelCache:
         lut = vec(9, (M, nh, hd))[:, 0].contiguous()
 
         def run(readback):
-            qkv = ops.prefill_rms_qkv_rope(x, norm_w, wqkv, lut, 0, nh, nkv, hd, eps=mod.eps)
+            stream = isinstance(wqkv, ops.StreamWeight)
+            rms_qkv_rope = ops.prefill_rms_qkv_rope_stream if stream else ops.prefill_rms_qkv_rope
+            qkv = rms_qkv_rope(x, norm_w, wqkv, lut, 0, nh, nkv, hd, eps=mod.eps)
             out = {11: qkv[:, :E], 12: qkv[:, E:E + KV], 8: qkv[:, E + KV:]}
             if readback & {2, 4, 6}:   # the unrotated projections and the normalised input, for diagnosis
                 normed = ops.rms_norm_rows(x, norm_w, eps=mod.eps)
-                plain = ops.w4a16_gemm(normed, *wqkv)
+                plain = ops.w4a16_gemm_stream(normed, wqkv) if stream else ops.w4a16_gemm(normed, *wqkv)
                 out.update({2: normed, 4: plain[:, :E], 6: plain[:, E:E + KV]})
             return out
 
@@ -523,7 +545,9 @@ class KernelCache:
         wd = weights("wdown", (12,), lambda: to_awq_dev(gemm_linear(12, H, E)))
 
         def run(readback):
-            y, res1, h = ops.prefill_o_ffn(attn_out, x_residual, norm_w, wo, wg, wu, wd, eps=mod.eps, return_intermediates=True)
+            stream = all(isinstance(w, ops.StreamWeight) for w in (wo, wg, wu, wd))
+            o_ffn = ops.prefill_o_ffn_stream if stream else ops.prefill_o_ffn
+            y, res1, h = o_ffn(attn_out, x_residual, norm_w, wo, wg, wu, wd, eps=mod.eps, return_intermediates=True)
             return {14: y, 4: res1, 11: h}
 
         return run, (4, 11, 14)

@@ -90,15 +90,18 @@ def _decode_block_through_cache(cache, x, packed, attn_norm, ffn_norm, cfg, k_ca
     return np.asarray(r[14]).view(np.uint16), (q_roped, k_roped, v)
 
 
-def test_decode_blocks_through_the_kernel_cache_match_the_oracle():
-    from air_hip import cache as kc, weights
+@pytest.mark.parametrize("stream_order", [True, False])
+def test_decode_blocks_through_the_kernel_cache_match_the_oracle(stream_order):
+    """stream_order: the static weight slots are kept in stream order and the whole-K launches run (the default);
+    False keeps AutoAWQ triples for the checkpoint-layout kernels."""
+    from air_hip import cache as kc, ops, weights
 
     cfg = weights.LlamaConfig(n_layers=2, emb_dim=512, n_heads=8, head_dim=64, n_kv_heads=2, hidden_dim=1024, vocab_size=32)
     E, H, nh, nkv, hd = cfg.emb_dim, cfg.hidden_dim, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim
     max_seq = 16
     models = [_model(E, H, nh, nkv, hd, seed=500 + 20 * i) for i in range(cfg.n_layers)]
     packed = [weights.reference_decode_buffers(host, k_chunk=E) for host, _ in models]
-    cache = kc.KernelCache(profiler=kc.Profiler(enabled=True))
+    cache = kc.KernelCache(profiler=kc.Profiler(enabled=True), stream_order=stream_order)
     cache.compile_and_cache("rms_qkv_int4_rope", kc.build_rms_qkv_int4_rope_module(E, nkv * hd, nh, nkv, hd, k_chunk=E), {})
     cache.compile_and_cache("o_gemv_ffn_int4", kc.build_o_gemv_ffn_int4_module(E, H, k_chunk=E), {})
     lut_bits = odec.generate_rope_lut(hd, cfg.rope_base, max_seq)
@@ -122,6 +125,9 @@ def test_decode_blocks_through_the_kernel_cache_match_the_oracle():
             caches[li][0][:, pos], caches[li][1][:, pos] = ref_caches[li][0][:, pos], ref_caches[li][1][:, pos]
             x_ref = want
     assert len(cache.profiler.kernel_times["o_gemv_ffn_int4"]) == 8
+    kept = [cache._cached_bos["rms_qkv_int4_rope_L1"]["wqkv"], cache._cached_bos["o_gemv_ffn_int4_L0"]["wdown"],
+            *cache._cached_bos["o_gemv_ffn_int4_L1"]["wgateup"]]
+    assert all(isinstance(w, ops.StreamWeight) == stream_order for w in kept)
     bd = cache.profiler.kernel_breakdowns["o_gemv_ffn_int4"]
     # static slots are written on the first call of a bo_key only: 3 packed buffers + the RMS buffer, then 2 vectors
     assert bd[0]["n_written"] == 6 and bd[1]["n_written"] == 6 and bd[2]["n_written"] == 2 and bd[-1]["n_written"] == 2
@@ -191,10 +197,12 @@ def test_lm_head_partitions_through_the_kernel_cache():
     assert int(np.argmax(bf16_bits_to_f32(logits))) == odec.lm_head_reference(x, None, w)[1]
 
 
-def test_prompt_layer_through_the_kernel_cache_matches_the_oracle():
+@pytest.mark.parametrize("stream_order", [True, False])
+def test_prompt_layer_through_the_kernel_cache_matches_the_oracle(stream_order):
     """The call sequence of _run_layer_int4 (llama32_1b_int4_prefill.py:241-364): rms_gemms_rope_int4, flash_attn,
-    o_ffn_int4, with the packed GEMM buffers awq_pack_for_npu makes, stage by stage against the oracle."""
-    from air_hip import bf16, cache as kc, weights
+    o_ffn_int4, with the packed GEMM buffers awq_pack_for_npu makes, stage by stage against the oracle; on the
+    stream-order copies of the weights (the default) and on the AutoAWQ triples."""
+    from air_hip import bf16, cache as kc, ops, weights
 
     M, E, H, nh, nkv, hd = 72, 256, 512, 4, 2, 64
     kv = nkv * hd
@@ -205,7 +213,7 @@ def test_prompt_layer_through_the_kernel_cache_matches_the_oracle():
         setattr(host, f, big(getattr(host, f)))
         l1[f] = oawq.repack_hf_awq_linear(*getattr(host, f), 128)
     packed = weights.reference_prefill_buffers(host, n_tile=16, k_chunk=128)
-    cache = kc.KernelCache()
+    cache = kc.KernelCache(stream_order=stream_order)
     cache.compile_and_cache("rms_gemms_rope_int4", kc.build_rms_gemms_rope_int4_module(M, E, kv, nh, nkv, hd, tile_n=16), {})
     cache.compile_and_cache("flash_attn", kc.build_attn(lk=M, lkp=hd, lq=M, lqp=256, dk=hd, dv=hd, num_heads=nh,
                                                         num_kv_heads=nkv, causal=True), {})
@@ -251,3 +259,5 @@ def test_prompt_layer_through_the_kernel_cache_matches_the_oracle():
     want_y, _, _ = oref.o_ffn_int4_prefill_reference(l1["wo"], l1["w_gate"], l1["w_up"], l1["w_down"], attn, x, host.ffn_norm)
     assert oref.check_outputs(f(y), f(want_y), rtol=0.2, atol=2.0, min_correlation=0.99)
     assert np.max(np.abs(f(y) - f(want_y))) <= 8 * 2.0**-8 * np.max(np.abs(f(want_y)))
+    kept = [cache._cached_bos["rms_int4_L0"]["wqkv"]] + [cache._cached_bos["offn_int4_L0"][k] for k in ("wo", "wgate", "wup", "wdown")]
+    assert all(isinstance(w, ops.StreamWeight) == stream_order for w in kept)
