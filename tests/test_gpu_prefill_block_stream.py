@@ -324,3 +324,41 @@ def test_prefill_rms_qkv_rope_stream_model_sizes(ops, M, E, nh, nkv, hd):
     p = bf16_bits_to_f32(prod[:, :nq]).reshape(M, nh, 2, hd // 2).astype(np.float64)
     n_g, n_p = np.sqrt((g**2).sum(axis=2)), np.sqrt((p**2).sum(axis=2))
     assert np.max(np.abs(n_g - n_p)) <= 2.0**-6 * np.max(n_p)
+
+
+def test_prompt_layer_on_stream_order_weights_replays_from_a_hip_graph(ops):
+    """RMSNorm + Q|K|V + RoPE, causal attention and the O + FFN block (the tiled kernel raises its LDS limit by a
+    function attribute at every launch) captured in one HIP graph: every replay, with eager work and
+    synchronisations in between, equals the eager results bit for bit."""
+    from oracle import decode as odec
+    M, E, H, nh, nkv, hd = 300, 512, 1280, 8, 2, 64
+    print(f"prompt layer graph M={M} E={E} H={H}", flush=True)
+    _, fused = _qkv_weights(E, nh, nkv, hd, seed=2100)
+    wqkv = _sw(ops, fused)
+    wo, wg, wu, wd = (_sw(ops, w) for w in _weights(E, H, seed=2110, scale=0.5))
+    nw_a, nw_f = dev(_norm_w(E, 2120)), dev(_norm_w(E, 2121))
+    lut = dev(odec.generate_rope_lut(hd, 500000.0, M))
+    xs = [dev(make_x((M, E), seed=2130 + j)) for j in range(3)]
+    cur = xs[0].clone()
+
+    def layer(x):
+        qkv = ops.prefill_rms_qkv_rope_stream(x, nw_a, wqkv, lut, 0, nh, nkv, hd)
+        attn = ops.prefill_attention(qkv, nh, nkv, hd)
+        return qkv, attn, ops.prefill_o_ffn_stream(attn, x, nw_f, wo, wg, wu, wd)
+
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        layer(cur)   # warm-up: workspaces and function attributes outside the graph
+        st.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            outs = layer(cur)
+        for j in range(3):
+            cur.copy_(xs[j])
+            g.replay()
+            st.synchronize()
+            want = layer(xs[j])
+            st.synchronize()
+            for name, a, b in zip(("qkv", "attention", "block"), outs, want):
+                assert torch.isfinite(a.float()).all(), (name, j)
+                assert torch.equal(a.view(torch.int16), b.view(torch.int16)), (name, j)

@@ -442,6 +442,43 @@ def test_stream_o_gemv_ffn_block(ops, E, H):
     assert np.array_equal(bits(y2), bits(y))
 
 
+def test_stream_launches_replay_from_a_hip_graph(ops):
+    """RMSNorm + Q|K|V GEMV, the O + FFN block and the batched kernel (which raises its LDS limit by a function
+    attribute at launch) on Q4NX-order weights, captured in one HIP graph: every replay, with eager work and
+    synchronisations in between, equals the eager results bit for bit."""
+    E, H = 512, 1024
+    print(f"q4nx stream graph E={E} H={H}", flush=True)
+    sw = [ops.q4nx_repack_stream(*_weights(ops, M, K, seed=900 + i)[1]) for i, (M, K) in enumerate([(3 * E, E), (E, E), (H, E), (H, E), (E, H)])]
+    wqkv, so, sg, su, sd = sw
+    nw_a, nw_f = dev(_norm_w(E, 910)), dev(_norm_w(E, 911))
+    rng = np.random.default_rng(912)
+    vecs = [dev(f32_to_bf16_bits(rng.standard_normal((3, E)).astype(np.float32))) for _ in range(3)]   # x, attn, residual per replay
+    rows = [dev(f32_to_bf16_bits(rng.standard_normal((16, E)).astype(np.float32))) for _ in range(3)]
+    cur_v, cur_r = vecs[0].clone(), rows[0].clone()
+
+    def step(v, r):
+        qkv = ops.q4nx_rms_gemv_stream(v[0], nw_a, wqkv)
+        y = ops.q4nx_o_gemv_ffn_stream(v[1], v[2], nw_f, so, sg, su, sd)
+        return qkv, y, ops.q4nx_gemm_stream(r, so)
+
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        step(cur_v, cur_r)   # warm-up: scratch buffers and the function attribute outside the graph
+        st.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            outs = step(cur_v, cur_r)
+        for j in range(3):
+            cur_v.copy_(vecs[j])
+            cur_r.copy_(rows[j])
+            g.replay()
+            st.synchronize()
+            want = step(vecs[j], rows[j])
+            st.synchronize()
+            for name, a, b in zip(("qkv", "block", "gemm16"), outs, want):
+                assert torch.equal(a.view(torch.int16), b.view(torch.int16)), (name, j)
+
+
 def test_stream_entry_points_reject_bad_arguments(ops):
     from air_hip import _lib
     lib = _lib.load_library()
