@@ -212,11 +212,12 @@ int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uin
                                uint16_t *y, int K, int N, int group, void *stream);
 /* Batched decode on a stream-order matrix: y[M, N] = bf16(x[M, K] . W), unrounded weights, fp32 accumulation
  * (matmul_int4_packed.cpu_reference, programming_examples/matrix_multiplication/int4_awq/matmul_int4_packed.py:89-105;
- * device kernel matmul_int4_bf16_packed_f32, mv_int4_bf16.cc:430-448).  Up to 16 rows per launch stream the weights
- * once (M <= 96: launches of 16 rows over the then cache-resident weights); stateless like the GEMV.  From M = 97 on,
+ * device kernel matmul_int4_bf16_packed_f32, mv_int4_bf16.cc:430-448).  Up to 64 rows per launch stream the weights
+ * once (M <= 128: launches of 64 rows and a rest, the second over cache-resident weights); stateless like the GEMV.  From
+ * M = 129 on,
  * with K % 256 == 0 and N % 64 == 0 (N / 64 = 3, 4 or >= 6), the tiled prefill kernel runs instead: it dequantises the
  * weights to bf16 in registers (W = bf16_rne((q - z) * s), the dense dequant's values) and feeds bf16 MFMA with fp32
- * accumulation; other shapes stay with the launches of 16 rows.  K % 128 == 0, N % 16 == 0. */
+ * accumulation; other shapes stay with the launches of 64 rows.  K % 128 == 0, N % 16 == 0. */
 int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int M, int K, int N, int group,
                            void *stream);
 int w4a16_gemv_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream,
@@ -403,7 +404,7 @@ int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residua
 /*
  * The two prompt-pass blocks on stream-order weights (w4a16_repack_stream of the same matrices; the Q|K|V matrices
  * concatenated along N before the re-pack): w4a16_prefill_rms_qkv_rope_bf16 and w4a16_prefill_o_ffn_bf16 with the tiled
- * stream-order GEMM (w4a16_gemm_stream_bf16's kernel for M >= 97) and its fused epilogues in place of the
+ * stream-order GEMM (w4a16_gemm_stream_bf16's kernel for M >= 129) and its fused epilogues in place of the
  * checkpoint-layout GEMM.  Same references (rms_gemms_rope_int4_multi.py:4-17, 414-436, 543-561;
  * o_ffn_int4_multi.py:4-17, 644-665), same rounding points, same workspaces (w4a16_prefill_qkv_workspace_bytes,
  * w4a16_prefill_block_workspace_bytes; plain scratch).  E % 256 == 0, H % 256 == 0, every N % 64 == 0.
@@ -567,7 +568,7 @@ int w4a16_q4nx_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the
  * timeout test: split-K producers do not publish), "ffn_fused" (0 = default: w4a16_ffn_swiglu_bf16
  * runs two streaming launches; 1 = one persistent kernel when the shape allows), "gemv_ws_ct", "gemv_ws_waves",
- * "gemm_ws_cb" (stream-order GEMV / small-batch shapes), "prefill_tile" (one tile width only, 1: 256 columns, 2: 192, 3: 128,
+ * "gemm_ws_cb", "gemm_ws_rows" (stream-order GEMV / small-batch shapes; rows: most rows per batched launch, 16, 32 or 64), "prefill_tile" (one tile width only, 1: 256 columns, 2: 192, 3: 128,
  * 4: 64; 5: 256 mixed with 128 in the launches that take that mix; 0: by shape), "prefill_min_m" (smallest M given to the tiled prefill kernel) and "prefill_swiglu_split" (1: the
  * stream-order prompt-pass FFN runs its gate and up projections as two launches instead of one; same bits).  Process-wide.
  */

@@ -550,9 +550,10 @@ int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, 
     if (group != kGroup) return W4A16_ERR_GROUP;
     if (M <= 0 || K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
     if (misaligned(x) || misaligned(wstream) || misaligned(y)) return W4A16_ERR_ALIGN;
-    // up to here the weights are streamed once per 16 rows (exact weights); from here on the tiled kernel that
-    // multiplies bf16-rounded weights (the crossover of the two kernels at K = 4096, N = 14336 is near M = 100)
-    const int prefill_min_m = g_gemv_ws_tune.prefill_min_m > 16 ? g_gemv_ws_tune.prefill_min_m : kStreamMaxM + 1;
+    // up to here the weights are streamed once per 64 rows (exact weights); from here on the tiled kernel that
+    // multiplies bf16-rounded weights.  The tiled kernel takes the same time for any M <= 256 (K = 4096, N = 14336:
+    // 51 us; N = 4096: 49 us; K = 2048, N = 8192: 27 us), two launches of 64 rows 46, 38 and 24 us, three 67, 56 and 36 us.
+    const int prefill_min_m = g_gemv_ws_tune.prefill_min_m > 16 ? g_gemv_ws_tune.prefill_min_m : kGemmWsMaxM + 1;
     hipError_t e = M >= prefill_min_m && gemm_prefill_ws_supported(M, K, N)
                        ? launch_gemm_prefill_ws(x, wstream, y, M, K, N, static_cast<hipStream_t>(stream))
                        : launch_gemm_ws(x, wstream, y, nullptr, M, K, N, static_cast<hipStream_t>(stream));
@@ -1008,6 +1009,9 @@ int w4a16_tune(const char *key, int value) {
         g_gemv_ws_tune.prefill_swiglu_split = value;
     } else if (!strcmp(key, "prefill_min_m")) {
         g_gemv_ws_tune.prefill_min_m = value;
+    } else if (!strcmp(key, "gemm_ws_rows")) {
+        if (value != 0 && value != 16 && value != 32 && value != 64) return W4A16_ERR_TUNE;
+        g_gemv_ws_tune.gemm_rows = value;
     } else if (!strcmp(key, "gemm_ws_cb")) {
         if (value != 0 && value != 1 && value != 2 && value != 4) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.cb = value;

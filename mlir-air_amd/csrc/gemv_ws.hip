@@ -604,6 +604,150 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
     }
 }
 
+// 17 <= M <= 64 in one launch: RT row tiles of 16.  The same plan as gemm_ws_kernel (a workgroup owns CB tiles for all of
+// K, its waves take the tasks round-robin and meet in LDS), with a cell's B operand built once and multiplied with RT A
+// operands.  A task is 4 / RT groups (RT = 4: one), so that the x operands of a task stay at 64 registers; the scale
+// words are read from the task's KiB one dword at a time, because which dword of a chunk belongs to the task's group
+// depends on the group.  AWQ order only.
+template <int CB, int RT>
+__global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_rows_kernel(const uint16_t *__restrict__ x, const char *__restrict__ w,
+                                                                         uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
+                                                                         int M, int K, int N, int G, int NB) {
+    constexpr int GPT = 4 / RT;   // groups per task
+    static_assert(RT == 2 || RT == 4, "row tiles per launch");
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [wave][row tile][cb][reg][lane]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lg = lane >> 4, ln = lane & 15;
+    const size_t tile_bytes = (size_t)(NB + G) * kWsCellBytes;
+    const char *tile0 = w + (size_t)blockIdx.x * CB * tile_bytes;
+
+    const uint32_t ones_w = 0x3F803F80u;
+    const u32x4 ones4 = {ones_w, ones_w, ones_w, ones_w};
+    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones4);
+    uint32_t nib_mask = 0x000F000Fu, magic = 0x43004300u;
+    asm volatile("" : "+s"(nib_mask));
+    asm volatile("" : "+v"(magic));
+
+    floatx4 Y[RT][CB];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int c = 0; c < CB; ++c) Y[rt][c] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    bool row_valid[RT];
+    const uint16_t *xrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        row_valid[rt] = 16 * rt + ln < M;
+        xrow[rt] = x + (size_t)(row_valid[rt] ? 16 * rt + ln : 0) * K + 8 * lg;
+    }
+    const int ntasks = (G + GPT - 1) / GPT;
+    u32x4 *mdl = reinterpret_cast<u32x4 *>(red + kGemmWsWaves * RT * CB * 4 * 64) + wave * 64;
+    for (int task = wave; task < ntasks; task += kGemmWsWaves) {
+        const int g0 = task * GPT;
+        u32x4 X[GPT][RT][4], cell[GPT][CB];
+        u32x4 mdq;
+        {   // the chunk of the aligned quad of groups that holds the task's: lane (c, ln) takes tile c's
+            const int b = g0 >> 4, gl = g0 & 15, c = lg < CB ? lg : CB - 1;
+            mdq = *reinterpret_cast<const u32x4 *>(tile0 + (size_t)c * tile_bytes + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes) +
+                                                   (16 * (gl >> 2) + ln) * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < GPT; ++j) {
+            const int g = g0 + j < G ? g0 + j : G - 1;   // a short last task re-reads the last group (its x is zeroed below)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) X[j][rt][t] = *reinterpret_cast<const u32x4 *>(xrow[rt] + 128 * g + 32 * t);
+        }
+#pragma unroll
+        for (int j = 0; j < GPT; ++j) {
+            const int g = g0 + j < G ? g0 + j : G - 1;
+            const int b = g >> 4, gl = g & 15;
+            const char *blk = tile0 + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes);
+#pragma unroll
+            for (int c = 0; c < CB; ++c)
+                cell[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)c * tile_bytes + (size_t)(1 + gl) * kWsCellBytes) + lane);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mdl[lane] = mdq;   // (LDS operations of one wave complete in order; the previous task's reads are done)
+#pragma unroll
+        for (int j = 0; j < GPT; ++j) {
+            const bool have = g0 + j < G;
+            floatx4 xs[RT];   // xs[rt][i]: sum of x[16 rt + 4 lg + i] over the group
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                xs[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    if (!(row_valid[rt] && have)) X[j][rt][t] = u32x4{0u, 0u, 0u, 0u};
+                    xs[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[j][rt][t]), ones, xs[rt], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < CB; ++c) {
+                floatx4 acc[RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const bf16x8 bop = cell_operand(cell[j][c][t], nib_mask, magic);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, X[j][rt][t]), bop, acc[rt], 0, 0, 0);
+                }
+                // the scale word of (group g0 + j, column ln) of tile c: dword (g0 + j) % 4 of the chunk lane 16 c + ln fetched
+                uint32_t mw = reinterpret_cast<const uint32_t *>(mdl + 16 * c + ln)[(g0 + j) & 3];
+                if (!have) mw = 0u;   // (a short last task: no such group, s = 0)
+                const float sf = __builtin_bit_cast(float, mw << 16);
+                const float nz = __builtin_bit_cast(float, mw & 0xFFFF0000u);   // -(128 + z)
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) Y[rt][c][i] = fmaf(sf, fmaf(nz, xs[rt][i], acc[rt][i]), Y[rt][c][i]);
+            }
+        }
+    }
+
+    // cross-wave sum: red[wave][rt][c][i][lane], then every thread adds the waves for its (row, column) pairs
+    constexpr int PER_TILE = CB * 4 * 64, PER_WAVE = RT * PER_TILE;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int c = 0; c < CB; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave * PER_WAVE + rt * PER_TILE + (c * 4 + i) * 64 + lane] = Y[rt][c][i];
+    __syncthreads();
+    for (int e = threadIdx.x; e < PER_WAVE; e += kGemmWsWaves * 64) {
+        // e = (m * CB + c) * 16 + col: consecutive threads write consecutive columns of one row
+        const int col = e & 15, c = (e >> 4) % CB, m = e / (16 * CB);
+        const int mt = m & 15;   // row m lives in row tile m / 16, lane group mt / 4, register mt % 4
+        const int src = (m >> 4) * PER_TILE + (c * 4 + (mt & 3)) * 64 + 16 * (mt >> 2) + col;
+        float s = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < kGemmWsWaves; ++wv) s += red[wv * PER_WAVE + src];
+        if (m < M) {
+            const size_t o = (size_t)m * N + (size_t)blockIdx.x * (16 * CB) + 16 * c + col;
+            if (residual) s += bf16_bits_to_float(residual[o]);
+            y[o] = float_to_bf16_bits(s);
+        }
+    }
+}
+
+template <int CB, int RT>
+hipError_t launch_gemm_ws_rows(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
+                               hipStream_t stream) {
+    const size_t lds = (size_t)kGemmWsWaves * RT * CB * 4 * 64 * sizeof(float) + kGemmWsWaves * kWsCellBytes;   // sums, scale words
+    if (lds >= 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_ws_rows_kernel<CB, RT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((gemm_ws_rows_kernel<CB, RT>), dim3(N / (16 * CB)), dim3(kGemmWsWaves * 64), lds, stream, x,
+                       static_cast<const char *>(w), y, residual, M, K, N, K / kGroup, ws_blocks(K));
+    return hipGetLastError();
+}
+
 template <int CB, bool Q4>
 hipError_t launch_gemm_ws_q(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
                             hipStream_t stream) {
@@ -625,7 +769,7 @@ hipError_t launch_gemm_ws_cb(const uint16_t *x, const void *w, uint16_t *y, cons
 
 }  // namespace
 
-// y[M, N] = bf16(x[M, K] . W (+ residual)), 2 <= M <= 16 per launch; more rows run as launches of 16.
+// y[M, N] = bf16(x[M, K] . W (+ residual)): up to 64 rows per launch (Q4NX order: 16), more rows as further launches.
 hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
                           hipStream_t stream, bool q4) {
     const int tiles = N / kWsTileCols;
@@ -633,13 +777,24 @@ hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const u
     if (!cb) cb = tiles % 4 == 0 && tiles / 4 >= 200 ? 4 : (tiles % 2 == 0 && tiles / 2 >= 200 ? 2 : 1);
     if (tiles % cb) cb = 1;
     hipError_t e = hipSuccess;
-    for (int m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
-        const int rows = M - m0 < 16 ? M - m0 : 16;
+    const int max_rows = q4 || g_gemv_ws_tune.gemm_rows == 16 ? 16 : (g_gemv_ws_tune.gemm_rows == 32 ? 32 : 64);
+    for (int m0 = 0; m0 < M && e == hipSuccess;) {
+        const int rows = M - m0 < max_rows ? M - m0 : max_rows;
         const uint16_t *xr = x + (size_t)m0 * K, *rr = residual ? residual + (size_t)m0 * N : nullptr;
         uint16_t *yr = y + (size_t)m0 * N;
-        e = cb == 4 ? launch_gemm_ws_cb<4>(xr, w, yr, rr, rows, K, N, stream, q4)
-          : cb == 2 ? launch_gemm_ws_cb<2>(xr, w, yr, rr, rows, K, N, stream, q4)
-                    : launch_gemm_ws_cb<1>(xr, w, yr, rr, rows, K, N, stream, q4);
+        if (rows > 32)
+            e = cb == 4 ? launch_gemm_ws_rows<4, 4>(xr, w, yr, rr, rows, K, N, stream)
+              : cb == 2 ? launch_gemm_ws_rows<2, 4>(xr, w, yr, rr, rows, K, N, stream)
+                        : launch_gemm_ws_rows<1, 4>(xr, w, yr, rr, rows, K, N, stream);
+        else if (rows > 16)
+            e = cb == 4 ? launch_gemm_ws_rows<4, 2>(xr, w, yr, rr, rows, K, N, stream)
+              : cb == 2 ? launch_gemm_ws_rows<2, 2>(xr, w, yr, rr, rows, K, N, stream)
+                        : launch_gemm_ws_rows<1, 2>(xr, w, yr, rr, rows, K, N, stream);
+        else
+            e = cb == 4 ? launch_gemm_ws_cb<4>(xr, w, yr, rr, rows, K, N, stream, q4)
+              : cb == 2 ? launch_gemm_ws_cb<2>(xr, w, yr, rr, rows, K, N, stream, q4)
+                        : launch_gemm_ws_cb<1>(xr, w, yr, rr, rows, K, N, stream, q4);
+        m0 += rows;
     }
     return e;
 }

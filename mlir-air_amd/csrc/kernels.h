@@ -12,6 +12,7 @@ namespace w4a16 {
 constexpr size_t kHeaderBytes = 256;
 constexpr int kMaxKSplit = 32;
 constexpr int kStreamMaxM = 96;   // up to here w4a16_gemm_bf16 runs the streaming kernel in 16-row launches
+constexpr int kGemmWsMaxM = 128;  // up to here w4a16_gemm_stream_bf16 runs the batched kernel (launches of up to 64 rows)
 
 struct StreamTune {
     int lw = 0;       // packed words per lane per row: 1, 2 or 4 (tile = 128 * lw columns)
@@ -109,6 +110,7 @@ struct GemvWsTune {
     int waves = 0;   // cap on the waves per workgroup (0 = one per task, at most 16)
     int cb = 0;      // batched kernel: 16-column tiles per workgroup, 1, 2 or 4 (0 = by the number of tiles)
     int prefill_tile = 0;    // prefill kernel: 0 = by shape, 1 = 128 x 448 tiles, 2 = 256 x 256 tiles
+    int gemm_rows = 0;       // batched kernel: most rows per launch, 16, 32 or 64 (0 = 64)
     int prefill_min_m = 0;   // smallest M that w4a16_gemm_stream_bf16 gives to the prefill kernel (0 = default)
     int prefill_swiglu_split = 0;   // 1: the prompt-pass FFN runs gate and up as two launches instead of one
 };

@@ -178,12 +178,34 @@ def _gemm_case(ops, M, K, N, seed):
     return got
 
 
-# rows 2..16 and beyond (launches of 16), one / two / four tiles per workgroup (N = 14336 and 6400 pick 4 and 2),
+# rows 2..16 and beyond, one / two / four tiles per workgroup (N = 14336 and 6400 pick 4 and 2),
 # K with a short last task (19 groups) and more tasks than waves (K = 14336: 28 tasks on 8 waves)
 @pytest.mark.parametrize("M,K,N", [(2, 128, 16), (3, 256, 544), (7, 1152, 544), (16, 512, 1056), (5, 128 * 19, 48),
                                    (16, 4096, 6400), (9, 14336, 4096), (40, 1024, 512), (16, 2048, 2048)])
 def test_gemm_stream_shapes(ops, M, K, N):
     _gemm_case(ops, M, K, N, seed=M + K + N)
+
+
+# 17 .. 64 rows run as one launch of two or four row tiles, more rows as launches of 64 and a rest: ragged last row tile,
+# a rest of one row, short last task (19 groups in tasks of two), more tasks than waves, one / two / four tiles per workgroup
+@pytest.mark.parametrize("M,K,N", [(17, 256, 64), (32, 1024, 544), (33, 512, 1056), (48, 128 * 19, 48), (64, 4096, 6400),
+                                   (65, 1024, 512), (96, 2048, 2048), (30, 128 * 19, 528), (64, 2048, 14336), (20, 14336, 4096)])
+def test_gemm_stream_more_than_sixteen_rows(ops, M, K, N):
+    _gemm_case(ops, M, K, N, seed=M + K + N)
+
+
+@pytest.mark.parametrize("rows", [16, 32])
+def test_gemm_stream_rows_per_launch_agree_up_to_summation_order(ops, rows):
+    """The rows a launch takes change only how a column's groups are dealt to the waves: the same sums in another order."""
+    M, K, N = 64, 2048, 1024
+    base = bf16_bits_to_f32(_gemm_case(ops, M, K, N, seed=90)).astype(np.float64)
+    ops.tune("gemm_ws_rows", rows)
+    try:
+        other = bf16_bits_to_f32(_gemm_case(ops, M, K, N, seed=90)).astype(np.float64)
+    finally:
+        ops.tune("gemm_ws_rows", 0)
+    assert np.all(np.abs(base - other) <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(base), 1e-30))) - 7) + 2e-3)
+    assert np.mean(base != other) < 0.02
 
 
 def test_gemm_stream_config2(ops):
@@ -219,8 +241,12 @@ def _prefill_case(ops, M, K, N, seed):
     print(f"prefill stream M={M} K={K} N={N} seed={seed}", flush=True)
     qw, qz, s = make_awq(K, N, seed=seed)
     x = make_x((M, K), seed=seed + 1)
-    y = ops.w4a16_gemm_stream(dev(x), _stream_weight(ops, qw, qz, s))
-    torch.cuda.synchronize()
+    ops.tune("prefill_min_m", 17)   # (by itself the tiled kernel runs from M = 129 on)
+    try:
+        y = ops.w4a16_gemm_stream(dev(x), _stream_weight(ops, qw, qz, s))
+        torch.cuda.synchronize()
+    finally:
+        ops.tune("prefill_min_m", 0)
     got = bits(y)
     xf = bf16_bits_to_f32(x).astype(np.float64)
     assert_bf16_close(got, xf @ dense_f64(qw, qz, s, rounded=True), ulps=1.0, atol=2e-3, what=f"prefill stream M={M} K={K} N={N}")
@@ -262,12 +288,30 @@ def test_prefill_stream_wide_tiles_on_many_groups(ops, tile):
 
 
 def test_prefill_stream_small_m_through_the_tiled_kernel(ops):
+    _prefill_case(ops, 17, 256, 448, seed=5)
+    _prefill_case(ops, 40, 512, 512, seed=6)
+
+
+def test_gemm_stream_hands_over_to_the_tiled_kernel_above_128_rows(ops):
+    """M = 128 is two launches of the batched kernel (unrounded weights), M = 129 the tiled kernel (bf16-rounded
+    weights): row 0 of x gives the batched kernel's bits in the first case and the tiled kernel's in the second."""
+    K, N = 1024, 512
+    qw, qz, s = make_awq(K, N, seed=55)
+    w = _stream_weight(ops, qw, qz, s)
+    x = make_x((129, K), seed=56)
+    y128 = bits(ops.w4a16_gemm_stream(dev(x[:128]), w))
+    y129 = bits(ops.w4a16_gemm_stream(dev(x), w))
     ops.tune("prefill_min_m", 17)
     try:
-        _prefill_case(ops, 17, 256, 448, seed=5)
-        _prefill_case(ops, 40, 512, 512, seed=6)
+        tiled = bits(ops.w4a16_gemm_stream(dev(x[:128]), w))
     finally:
         ops.tune("prefill_min_m", 0)
+    batched = bits(ops.w4a16_gemm_stream(dev(x[:16]), w))
+    torch.cuda.synchronize()
+    assert np.array_equal(y129[:128], tiled) and not np.array_equal(y128, tiled)
+    xf = bf16_bits_to_f32(x).astype(np.float64)
+    assert_bf16_close(y128, xf[:128] @ dense_f64(qw, qz, s), ulps=1.0, atol=2e-3, what="M = 128 on the batched kernel")
+    assert np.mean(y128[:16] != batched) < 0.02   # the same sums in another order
 
 
 def test_prefill_stream_config3(ops):
@@ -286,8 +330,8 @@ def test_prefill_stream_one_hot_rows_reproduce_the_dequant(ops):
 
 
 def test_prefill_sized_m_on_a_shape_the_tiled_kernel_does_not_take(ops):
-    """K = 384 (an odd number of groups) and N = 80: M = 128 runs the batched kernel in launches of 16 rows."""
-    M, K, N = 128, 384, 80
+    """K = 384 (an odd number of groups) and N = 80: M = 200 runs the batched kernel in launches of 64 rows and a rest."""
+    M, K, N = 200, 384, 80
     qw, qz, s = make_awq(K, N, seed=31)
     x = make_x((M, K), seed=32)
     y = ops.w4a16_gemm_stream(dev(x), _stream_weight(ops, qw, qz, s))
