@@ -438,7 +438,7 @@ hipError_t launch_repack_ws(const int32_t *qweight, const int32_t *qzeros, const
 
 }  // namespace w4a16
 
-// ---- batched decode, 2 <= M <= 16, on the same layout ------------------------------------------------------------
+// ---- batched decode, 2 <= M <= 16 (gemm_ws_kernel) and up to 64 rows (gemm_ws_rows_kernel), on the same layout ----
 //
 // The 16 rows of the A operand are the rows of x (row m <-> lane ln = m), so a cell's product is the whole
 // [16 x 16] block of y for its 16 columns and the group flush applies to all four accumulator registers.  A workgroup
