@@ -390,3 +390,41 @@ def test_hip_graph_replays_of_the_stream_kernels_match_eager(ops):
                 want = ops.w4a16_gemm_stream(inputs[k][j], w)
                 st.synchronize()
                 assert torch.equal(outs[k].view(torch.int16), want.view(torch.int16)), (k, j)
+
+
+def test_stream_entry_points_from_two_threads_on_two_streams(ops):
+    """The stream-order entry points keep no state: two host threads, each on its own stream, calling the GEMV, the
+    batched kernel and the SwiGLU front half at the same time get the bits a single thread gets."""
+    import threading
+    K, N = 2048, 1792
+    w = [_stream_weight(ops, *make_awq(K, N, seed=120 + i)) for i in range(2)]
+    xs = [dev(make_x((24, K), seed=130 + i)) for i in range(2)]
+
+    def work(i):
+        return (ops.w4a16_gemv_stream(xs[i][0], w[i]), ops.w4a16_gemm_stream(xs[i], w[i]),
+                ops.w4a16_swiglu_stream(xs[i][1], w[i], w[1 - i]))
+
+    want = [work(i) for i in range(2)]
+    torch.cuda.synchronize()
+    got, errors = [None, None], []
+
+    def run(i):
+        try:
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                for _ in range(50):
+                    got[i] = work(i)
+                st.synchronize()
+        except Exception as e:   # surfaced below: an exception in a thread would otherwise pass silently
+            errors.append(e)
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(2):
+        for a, b in zip(got[i], want[i]):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
