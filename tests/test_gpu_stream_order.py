@@ -365,12 +365,12 @@ def test_stream_entry_points_reject_bad_arguments(ops):
 
 
 def test_hip_graph_replays_of_the_stream_kernels_match_eager(ops):
-    """The GEMV, the batched kernel and the tiled prefill kernel captured in one HIP graph: every replay, with eager
+    """The GEMV, the batched kernels (up to 16 rows, and four row tiles) and the tiled prefill kernel captured in one HIP graph: every replay, with eager
     work and synchronisations in between, equals the eager results bit for bit (nothing kept between launches)."""
     K, N = 1024, 1792
     qw, qz, s = make_awq(K, N, seed=61)
     w = _stream_weight(ops, qw, qz, s)
-    shapes = {"gemv": (K,), "gemm": (12, K), "prefill": (300, K)}
+    shapes = {"gemv": (K,), "gemm": (12, K), "rows": (40, K), "prefill": (300, K)}
     inputs = {k: [dev(make_x(shp, seed=70 + 3 * i + j)) for j in range(3)] for i, (k, shp) in enumerate(shapes.items())}
     cur = {k: v[0].clone() for k, v in inputs.items()}
     st = torch.cuda.Stream()
