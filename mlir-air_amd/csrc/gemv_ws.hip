@@ -611,8 +611,7 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_kernel(const uint16
 // depends on the group.  AWQ order only.
 template <int CB, int RT>
 __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_rows_kernel(const uint16_t *__restrict__ x, const char *__restrict__ w,
-                                                                         uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
-                                                                         int M, int K, int N, int G, int NB) {
+                                                                         uint16_t *__restrict__ y, int M, int K, int N, int G, int NB) {
     constexpr int GPT = 4 / RT;   // groups per task
     static_assert(RT == 2 || RT == 4, "row tiles per launch");
     extern __shared__ __attribute__((aligned(16))) float red[];   // [wave][row tile][cb][reg][lane]
@@ -727,24 +726,19 @@ __global__ void __launch_bounds__(kGemmWsWaves * 64) gemm_ws_rows_kernel(const u
         float s = 0.f;
 #pragma unroll
         for (int wv = 0; wv < kGemmWsWaves; ++wv) s += red[wv * PER_WAVE + src];
-        if (m < M) {
-            const size_t o = (size_t)m * N + (size_t)blockIdx.x * (16 * CB) + 16 * c + col;
-            if (residual) s += bf16_bits_to_float(residual[o]);
-            y[o] = float_to_bf16_bits(s);
-        }
+        if (m < M) y[(size_t)m * N + (size_t)blockIdx.x * (16 * CB) + 16 * c + col] = float_to_bf16_bits(s);
     }
 }
 
 template <int CB, int RT>
-hipError_t launch_gemm_ws_rows(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
-                               hipStream_t stream) {
+hipError_t launch_gemm_ws_rows(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream) {
     const size_t lds = (size_t)kGemmWsWaves * RT * CB * 4 * 64 * sizeof(float) + kGemmWsWaves * kWsCellBytes;   // sums, scale words
     if (lds >= 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_ws_rows_kernel<CB, RT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
     hipLaunchKernelGGL((gemm_ws_rows_kernel<CB, RT>), dim3(N / (16 * CB)), dim3(kGemmWsWaves * 64), lds, stream, x,
-                       static_cast<const char *>(w), y, residual, M, K, N, K / kGroup, ws_blocks(K));
+                       static_cast<const char *>(w), y, M, K, N, K / kGroup, ws_blocks(K));
     return hipGetLastError();
 }
 
@@ -769,7 +763,8 @@ hipError_t launch_gemm_ws_cb(const uint16_t *x, const void *w, uint16_t *y, cons
 
 }  // namespace
 
-// y[M, N] = bf16(x[M, K] . W (+ residual)): up to 64 rows per launch (Q4NX order: 16), more rows as further launches.
+// y[M, N] = bf16(x[M, K] . W (+ residual)): up to 64 rows per launch (Q4NX order, or with a residual: 16), more rows as
+// further launches.
 hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
                           hipStream_t stream, bool q4) {
     const int tiles = N / kWsTileCols;
@@ -777,19 +772,20 @@ hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const u
     if (!cb) cb = tiles % 4 == 0 && tiles / 4 >= 200 ? 4 : (tiles % 2 == 0 && tiles / 2 >= 200 ? 2 : 1);
     if (tiles % cb) cb = 1;
     hipError_t e = hipSuccess;
-    const int max_rows = q4 || g_gemv_ws_tune.gemm_rows == 16 ? 16 : (g_gemv_ws_tune.gemm_rows == 32 ? 32 : 64);
+    // (the launches of several row tiles take the AWQ order and no residual)
+    const int max_rows = q4 || residual || g_gemv_ws_tune.gemm_rows == 16 ? 16 : (g_gemv_ws_tune.gemm_rows == 32 ? 32 : 64);
     for (int m0 = 0; m0 < M && e == hipSuccess;) {
         const int rows = M - m0 < max_rows ? M - m0 : max_rows;
         const uint16_t *xr = x + (size_t)m0 * K, *rr = residual ? residual + (size_t)m0 * N : nullptr;
         uint16_t *yr = y + (size_t)m0 * N;
         if (rows > 32)
-            e = cb == 4 ? launch_gemm_ws_rows<4, 4>(xr, w, yr, rr, rows, K, N, stream)
-              : cb == 2 ? launch_gemm_ws_rows<2, 4>(xr, w, yr, rr, rows, K, N, stream)
-                        : launch_gemm_ws_rows<1, 4>(xr, w, yr, rr, rows, K, N, stream);
+            e = cb == 4 ? launch_gemm_ws_rows<4, 4>(xr, w, yr, rows, K, N, stream)
+              : cb == 2 ? launch_gemm_ws_rows<2, 4>(xr, w, yr, rows, K, N, stream)
+                        : launch_gemm_ws_rows<1, 4>(xr, w, yr, rows, K, N, stream);
         else if (rows > 16)
-            e = cb == 4 ? launch_gemm_ws_rows<4, 2>(xr, w, yr, rr, rows, K, N, stream)
-              : cb == 2 ? launch_gemm_ws_rows<2, 2>(xr, w, yr, rr, rows, K, N, stream)
-                        : launch_gemm_ws_rows<1, 2>(xr, w, yr, rr, rows, K, N, stream);
+            e = cb == 4 ? launch_gemm_ws_rows<4, 2>(xr, w, yr, rows, K, N, stream)
+              : cb == 2 ? launch_gemm_ws_rows<2, 2>(xr, w, yr, rows, K, N, stream)
+                        : launch_gemm_ws_rows<1, 2>(xr, w, yr, rows, K, N, stream);
         else
             e = cb == 4 ? launch_gemm_ws_cb<4>(xr, w, yr, rr, rows, K, N, stream, q4)
               : cb == 2 ? launch_gemm_ws_cb<2>(xr, w, yr, rr, rows, K, N, stream, q4)
