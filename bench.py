@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm64|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemv_planar|q4nx_gemm16|q4nx_gemm16_planar|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm64|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -51,9 +51,7 @@ CONFIGS = {
     # the Q4NX codec (w = q * s + m, 32-column groups) through the same streaming kernel: the gate / up
     # projection shape of Llama-3.1-8B (programming_examples/llms/llama31_8b_q4nx)
     "q4nx_gemv": dict(M=1, K=4096, N=14336, cfg=None, desc="decode GEMV Q4NX M=1 K=4096 N=14336 g32, weights in Q4NX stream order"),
-    "q4nx_gemv_planar": dict(M=1, K=4096, N=14336, cfg=None, desc="decode GEMV Q4NX M=1 K=4096 N=14336 g32, operands of q4nx_repack (split-K with a workspace)"),
     "q4nx_gemm16": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM Q4NX M=16 K=4096 N=14336 g32, weights in Q4NX stream order"),
-    "q4nx_gemm16_planar": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM Q4NX M=16 K=4096 N=14336 g32, operands of q4nx_repack (split-K with a workspace)"),
     # the tail of a decode step of Llama-3.2-1B: final RMSNorm + bf16 lm_head GEMV + argmax
     "lm_head": dict(M=1, K=2048, N=128256, cfg=None, desc="decode tail RMSNorm + bf16 lm_head GEMV + argmax E=2048 V=128256"),
 }
@@ -160,9 +158,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             copies.append(c4 + ((make_weights(torch, K, nqkv, 104 + 5 * i),) if kind == "layer" else ()))
         elif q4nx:
             copies.append(make_q4nx_weights(torch, K, N, 100 + i))
-            if name in ("q4nx_gemv", "q4nx_gemm16"):   # re-packed at load time (untimed)
-                from air_hip import ops
-                copies[-1] = (ops.q4nx_repack_stream(*copies[-1]).buf,)
+            from air_hip import ops
+            copies[-1] = (ops.q4nx_repack_stream(*copies[-1]).buf,)   # re-packed at load time (untimed)
         elif lm_head:
             gw = torch.Generator(device="cuda")
             gw.manual_seed(100 + i)
@@ -283,9 +280,6 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             rc = lib.w4a16_q4nx_gemv_stream_bf16(x.data_ptr(), w[0].data_ptr(), None, outs[0].data_ptr(), K, N, st)
         elif name == "q4nx_gemm16":
             rc = lib.w4a16_q4nx_gemm_stream_bf16(x.data_ptr(), w[0].data_ptr(), None, outs[0].data_ptr(), M, K, N, st)
-        elif q4nx:
-            rc = lib.w4a16_q4nx_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), None,
-                                          outs[0].data_ptr(), M, K, N, ws.data_ptr(), ws.numel(), st)
         else:
             rc = lib.w4a16_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
                                      outs[0].data_ptr(), M, K, N, 128, ws.data_ptr(), ws.numel(), st)
@@ -330,7 +324,13 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
-            torch.cuda._sleep(int(2e5) * max(8, len(indices) // 4))
+            torch.cuda._sleep(int(2e5) * max(16, len(indices) // 2))
+            # one untimed rotation over the copies, continuing the cyclic order, right in front of the timed launches:
+            # the interval then starts in the steady state of a decode loop (memory and fabric clocks up; after the
+            # idle spin the first ~100 us of launches run 5 % slower) and the first event follows a launch of the
+            # same kind instead of the spinning kernel
+            for i in range(ncopies):
+                launch(indices[0] - ncopies + i if len(set(indices)) > 1 else indices[0], stream.cuda_stream)
             e0.record(stream)
             for i in indices:
                 launch(i, stream.cuda_stream)
@@ -478,7 +478,6 @@ def run_decode_model(steps, warmup, model="decode_1b", stream_order=True):
     if stream_order:
         for l in layers:   # decode reads stream-order weights; the checkpoint-layout tensors are not needed here
             l.with_stream()
-            l.wqkv = l.wo = l.w_gate = l.w_up = l.w_down = None
     embed = torch.randn((cfg.vocab_size, E), device="cuda", generator=g).to(torch.bfloat16)
     final_norm = norm_w()
     max_seq = 2048
@@ -541,7 +540,6 @@ def run_prefill_model(model="decode_1b", M=2048, reps=3, stream_order=True):
     if stream_order:
         for l in layers:
             l.with_stream()
-            l.wqkv = l.wo = l.w_gate = l.w_up = l.w_down = None
     embed = torch.randn((cfg.vocab_size, E), device="cuda", generator=g).to(torch.bfloat16)
     final_norm = norm_w()
     lut = decode.generate_rope_lut(cfg, M)
@@ -779,8 +777,9 @@ def main():
         "data": "synthetic (W ~ N(0,1)*0.05 as bf16, x ~ N(0,1))" if name == "lm_head" else "synthetic (uniform uint4 q/z, scales |N(0,1)|*0.02+1e-3, x ~ N(0,1)), random weights",
         "config": {"workload": CONFIGS[name]["desc"], "group": 32 if name.startswith("q4nx") else 128,
                    "weight_copies_rotated": main_res["ncopies"],
-                   "timing": "K launches queued on one stream behind a spinning kernel, HIP events on that stream around them "
-                             "(graph_us_per_step: the same K launches replayed as one HIP graph)"},
+                   "timing": "K launches queued on one stream behind a spinning kernel and one untimed rotation over the weight "
+                             "copies, HIP events on that stream around the K launches (graph_us_per_step: the same K launches "
+                             "replayed as one HIP graph)"},
         "roofline": roof,
         "per_launch_events_us": main_res["per_launch_events_us"],
         "graph_us_per_step": main_res["graph_us"],

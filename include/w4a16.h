@@ -84,11 +84,7 @@ int awq_dequant_1d_bf16(const uint8_t *packed, uint16_t *out_bf16, int n, int gr
  * (different streams) need separate workspaces.  The FFN and block entry points keep plain
  * intermediates (h, res1) behind the prepared area, at an offset that depends on their shapes: share
  * a workspace only between calls of one entry point with the same shapes, or prepare it again
- * before a call of another kind.  With w4a16_tune("ffn_fused", 1) (off by default) w4a16_ffn_swiglu_bf16
- * and w4a16_o_gemv_ffn_bf16 run a persistent kernel whose workgroups wait for one another: it needs
- * all of them resident at once, so two such calls running at the same time on one GPU (two streams,
- * two processes) can starve each other into the timeout path (w4a16_workspace_check); keep them on
- * one stream, one process per GPU.
+ * before a call of another kind.
  */
 size_t w4a16_gemm_workspace_bytes(int M, int K, int N);
 size_t w4a16_ffn_workspace_bytes(int K, int H);
@@ -486,7 +482,7 @@ int lm_head_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps,
  * written above, one rounding to bf16), replacing Q4nxModel.dequant / dequant_q4_0
  * (programming_examples/llms/qwen25_3b_q4/qwen25_3b_q4_weights.py:86-95) followed by the cast to bf16.
  *
- * q4nx_repack turns the blocks into the operands of w4a16_q4nx_gemm_bf16, once at load time (the
+ * q4nx_repack turns the blocks into the operands of w4a16_q4nx_repack_stream, once at load time (the
  * reference re-packs the same blocks into its own device stream order, pack_q4k_cascade,
  * proj_qmm_pack.py:61-140): qweight int32 [K, M / 8] (word (k, j) = rows 8 j .. 8 j + 7 of
  * column k, unsigned nibbles in the AutoAWQ order), scales and mins bf16 [K / 32, M] with
@@ -502,48 +498,15 @@ int q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t
                 int M, int K, int mode, void *stream);
 
 /*
- * y[M, N] = bf16(x[M, K] . W + residual) for the affine 32-row-group codec above, W given by the
- * operands of q4nx_repack (N = that function's M).  In fp32 per group:
- * y += s * sum(q x) + m * sum(x), the arithmetic of _qmm_q4k_bf16
- * (programming_examples/fused_decode/kernels/q4_k.h:39-45: c += (q*b)*scale; c += min*sum(b)).
- * `residual` bf16 [M, N] may be NULL.  Any M >= 1 (16 rows per launch of the streaming kernel;
- * the reference runs the prefill of these models as dense bf16 GEMMs on dequantised weights,
- * so there is no large-M kernel for this codec).  K % 128 == 0, N % 32 == 0.
- * Workspace: w4a16_gemm_workspace_bytes(M, K, N), initialised with w4a16_workspace_init.
- */
-int w4a16_q4nx_gemm_bf16(const uint16_t *x, const int32_t *qweight, const uint16_t *scales, const uint16_t *mins,
-                         const uint16_t *residual, uint16_t *y, int M, int K, int N,
-                         void *workspace, size_t workspace_bytes, void *stream);
-
-/*
- * The decode-layer entry points for the affine codec: w4a16_rms_gemv_bf16 and w4a16_o_gemv_ffn_bf16
- * with every weight triple given as (qweight, scales, mins) from q4nx_repack.  Same arithmetic,
- * stages, workspace sizes and optional outputs as their AWQ counterparts above; they cover the
- * proj / O / FFN phases of the fused decode dispatch
- * (programming_examples/fused_decode/fused_decode.py: proj_qmm, rms_residual, glu kernels) around
- * w4a16_decode_attention_bf16.
- */
-int w4a16_q4nx_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps,
-                             const int32_t *qweight, const uint16_t *scales, const uint16_t *mins,
-                             uint16_t *y, int K, int N,
-                             void *workspace, size_t workspace_bytes, void *stream);
-int w4a16_q4nx_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual,
-                               const uint16_t *ffn_norm_weight, float eps,
-                               const int32_t *o_qweight, const uint16_t *o_scales, const uint16_t *o_mins,
-                               const int32_t *gate_qweight, const uint16_t *gate_scales, const uint16_t *gate_mins,
-                               const int32_t *up_qweight, const uint16_t *up_scales, const uint16_t *up_mins,
-                               const int32_t *down_qweight, const uint16_t *down_scales, const uint16_t *down_mins,
-                               uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int E, int H,
-                               void *workspace, size_t workspace_bytes, void *stream);
-
-/*
- * The same codec on the fast path: the operands of q4nx_repack re-packed once more, at load time, into the stream order of
+ * The products of this codec: the operands of q4nx_repack re-packed once more, at load time, into the stream order of
  * the decode kernels (csrc/wstream.h, "Q4NX order": 16-column tiles, 1 KiB cells of 128 rows, and in front of every 16
  * cells 4 KiB of scale / min words, one pair per 32 rows and column), the counterpart of the reference's own stream
  * order for these blocks (pack_q4k_cascade, programming_examples/fused_decode/proj_qmm_pack.py:61-140).  The GEMV, the
  * RMSNorm + GEMV and the O + FFN block then run the whole-K kernels of the AWQ stream order with the per-32-row flush
- * y += s * (sum q x) + min * (sum x) of _qmm_q4k_bf16 (programming_examples/fused_decode/kernels/q4_k.h:39-45): no
- * workspace protocol, no state.  `residual` may be NULL; x_sumsq / n_pieces, res1_out, h_out, y_sumsq and the workspace
+ * y += s * (sum q x) + min * (sum x) of _qmm_q4k_bf16 (programming_examples/fused_decode/kernels/q4_k.h:39-45: c += (q*b)*scale;
+ * c += min*sum(b)): no workspace protocol, no state.  They cover the proj / O / FFN phases of the fused decode dispatch
+ * (programming_examples/fused_decode/fused_decode.py: proj_qmm, rms_residual, glu kernels) around w4a16_decode_attention_bf16; the
+ * reference runs the prefill of these models as dense bf16 GEMMs on dequantised weights, so there is no large-M kernel for the codec.  `residual` may be NULL; x_sumsq / n_pieces, res1_out, h_out, y_sumsq and the workspace
  * (w4a16_block_stream_workspace_bytes) as in the AWQ entry points of the same names.  K % 128 == 0, N % 16 == 0.
  */
 size_t w4a16_q4nx_stream_bytes(int K, int N);
@@ -566,8 +529,7 @@ int w4a16_q4nx_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *
  * "gemv_lw", "gemv_ksteps", "gemv_waves", "gemv_units", "gemv_ksplit" (0 = built-in heuristic),
  * "gemm_stream_max_m" (largest M given to the streaming kernel, 0 = default 96, otherwise >= 16) and
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the
- * timeout test: split-K producers do not publish), "ffn_fused" (0 = default: w4a16_ffn_swiglu_bf16
- * runs two streaming launches; 1 = one persistent kernel when the shape allows), "gemv_ws_ct", "gemv_ws_waves",
+ * timeout test: split-K producers do not publish), "gemv_ws_ct", "gemv_ws_waves",
  * "gemm_ws_cb", "gemm_ws_rows" (stream-order GEMV / small-batch shapes; rows: most rows per batched launch, 16, 32 or 64), "prefill_tile" (one tile width only, 1: 256 columns, 2: 192, 3: 128,
  * 4: 64; 5: 256 mixed with 128 in the launches that take that mix; 0: by shape), "prefill_min_m" (smallest M given to the tiled prefill kernel) and "prefill_swiglu_split" (1: the
  * stream-order prompt-pass FFN runs its gate and up projections as two launches instead of one; same bits).  Process-wide.

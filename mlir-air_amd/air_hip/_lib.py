@@ -54,9 +54,6 @@ SYMBOLS = {
     "w4a16_q4nx_gemm_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_q4nx_rms_gemv_stream_bf16": (_ci, [_vp, _vp, _ci, _vp, _cf, _vp, _vp, _ci, _ci, _vp]),
     "w4a16_q4nx_o_gemv_ffn_stream_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 8 + [_ci, _ci, _vp, _sz, _vp]),
-    "w4a16_q4nx_gemm_bf16": (_ci, [_vp] * 6 + [_ci, _ci, _ci, _vp, _sz, _vp]),
-    "w4a16_q4nx_rms_gemv_bf16": (_ci, [_vp, _vp, _cf] + [_vp] * 4 + [_ci, _ci, _vp, _sz, _vp]),
-    "w4a16_q4nx_o_gemv_ffn_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 15 + [_ci, _ci, _vp, _sz, _vp]),
     "w4a16_stream_bytes": (_sz, [_ci, _ci]),
     "w4a16_repack_stream": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_gemv_stream_bf16": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),

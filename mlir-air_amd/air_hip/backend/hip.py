@@ -102,8 +102,12 @@ class HIPBackend(AirBackend):
             return torch.from_numpy(a).cuda()
 
         def weights(buf, K, N):
+            """The packed weight buffer of one matrix on the device: the dequant op reads the AutoAWQ tensors, every
+            product reads the stream-order re-pack (made here, where the reference writes the buffer into its BO:
+            staging, outside the timed iterations)."""
             qw, qz, s = awq.unpack_buffer(buf, K, N, mod.gs)
-            return to_dev(qw), to_dev(qz), to_dev(s)
+            triple = to_dev(qw), to_dev(qz), to_dev(s)
+            return triple if mod.op == "dequant_awq" else ops.repack_stream(*triple, group=mod.gs)
 
         def run(dev_in):
             if mod.op == "dequant_awq":
@@ -111,20 +115,20 @@ class HIPBackend(AirBackend):
             if mod.op == "dequant_awq_1d":
                 return [ops.awq_dequant_1d(dev_in[0], mod.K, mod.gs, mod.N)]
             if mod.op == "matvec_int4":
-                return [ops.w4a16_gemv(dev_in[1], *dev_in[0])]
+                return [ops.w4a16_gemv_stream(dev_in[1], dev_in[0])]
             if mod.op == "matvec_int4_add":
-                return [ops.w4a16_gemv_add(dev_in[1], *dev_in[0], dev_in[2])]
+                return [ops.w4a16_gemv_stream(dev_in[1], dev_in[0], residual=dev_in[2])]
             if mod.op == "matmul_int4":
-                return [ops.w4a16_gemm(dev_in[0], *dev_in[1])]
+                return [ops.w4a16_gemm_stream(dev_in[0], dev_in[1])]
             if mod.op == "matvec_int4_swiglu":
-                return [ops.w4a16_swiglu(dev_in[2], dev_in[0], dev_in[1])]
+                return [ops.w4a16_swiglu_stream(dev_in[2], dev_in[0], dev_in[1])]
             if mod.op == "matvec_int4_swiglu_rms":
-                return [ops.w4a16_rms_swiglu(dev_in[2][0], dev_in[2][1], dev_in[0], dev_in[1], eps=mod.eps)]
+                return [ops.w4a16_rms_swiglu_stream(dev_in[2][0], dev_in[2][1], dev_in[0], dev_in[1], eps=mod.eps)]
             if mod.op == "ffn_swiglu_int4":
-                return [ops.ffn_swiglu(dev_in[3], dev_in[0], dev_in[1], dev_in[2])]
+                return [ops.ffn_swiglu_stream(dev_in[3], dev_in[0], dev_in[1], dev_in[2])]
             if mod.op == "o_gemv_ffn_int4":
                 wo, attn_out, x_res, norm_w, gate, up, down = dev_in
-                return [ops.o_gemv_ffn(attn_out, x_res, norm_w, wo, gate, up, down, eps=mod.eps)]
+                return [ops.o_gemv_ffn_stream(attn_out, x_res, norm_w, wo, gate, up, down, eps=mod.eps)]
             raise AirBackendError(f"unknown op {mod.op}")
 
         def invoker(*args):
@@ -139,7 +143,7 @@ class HIPBackend(AirBackend):
                 iters = max(self.n_perf_iters, 1)
                 for _ in range(iters):
                     outs = run(dev_in)
-                ops.check_health()   # synchronises; a reducer that timed out surfaces here
+                torch.cuda.synchronize()   # (the stream-order launches keep no state that could time out)
                 if self.n_perf_iters > 0:
                     self.last_latency_us = (time.perf_counter() - t0) / iters * 1e6
             except _lib.W4A16Error as e:

@@ -43,23 +43,38 @@ class DecodeLayer:
     w_down: tuple
     codec: str = "awq"   # "awq": triples are (qweight, qzeros, scales); "q4nx": (qweight, scales, mins) from q4nx_repack
     # The same five matrices in stream order (ops.StreamWeight; Q4NX order for that codec), which the decode kernels
-    # read; the triples above stay for the checkpoint-layout prompt pass.  None: decode runs on the triples.
+    # and the prompt pass read.  None: an AWQ layer whose widths the stream order does not take runs on the triples.
     stream: dict = None
 
-    def with_stream(self):
-        """Re-pack the layer's matrices into stream order on the GPU (once, at load time)."""
+    def with_stream(self, keep_triples=False):
+        """Re-pack the layer's matrices into stream order on the GPU (once, at load time).  A layer with a matrix the
+        stream order does not take (N % 16 != 0) keeps its triples and runs the checkpoint-layout kernels.  Unless
+        `keep_triples`, the triples are dropped once nothing reads them any more, i.e. when the prompt pass also takes
+        the stream-order copies (Q4NX layers: always), so that the weights are held once."""
+        names = ("wqkv", "wo", "w_gate", "w_up", "w_down")
         if self.stream is None:
+            if self.codec == "awq" and any(getattr(self, n)[0].shape[1] * 8 % 16 for n in names):
+                return self
             repack = ops.repack_stream if self.codec == "awq" else ops.q4nx_repack_stream
-            self.stream = {name: repack(*getattr(self, name)) for name in ("wqkv", "wo", "w_gate", "w_up", "w_down")}
+            self.stream = {name: repack(*getattr(self, name)) for name in names}
+        if not keep_triples and (self.codec != "awq" or _stream_covers_prefill(self.stream)):
+            self.wqkv = self.wo = self.w_gate = self.w_up = self.w_down = None
         return self
 
 
-def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda", stream_order=True) -> DecodeLayer:
+def _stream_covers_prefill(sw):
+    """Whether the prompt pass runs on these stream-order copies (run_prefill_layer): input lengths in whole pairs of
+    groups, widths in whole 64-column tiles, attention output as wide as the embedding."""
+    E, H, nq, nqkv = sw["w_gate"].K, sw["w_gate"].N, sw["wo"].K, sw["wqkv"].N
+    return E % 256 == 0 and H % 256 == 0 and nq == E and nqkv % 64 == 0
+
+
+def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda") -> DecodeLayer:
     """A Q4NX / Q4_0 layer -> DecodeLayer.  `blocks` maps q, k, v, o, gate, up, down to the tensor's
     blocks (uint8 [n_blocks, 5120], numpy or torch) in (row-block, col-block) order as a model.q4nx
     bundle stores them; Q, K, V are fused by concatenating their blocks (whole row-blocks of the output
-    axis), and every matrix is repacked on the GPU once (stream_order: and once more into the decode kernels'
-    stream order, as the reference re-packs the blocks into its cascade order, proj_qmm_pack.py:61-140).
+    axis), and every matrix is repacked on the GPU into the decode kernels' stream order in two steps (as the
+    reference re-packs the blocks into its cascade order, proj_qmm_pack.py:61-140).
     Norm weights are bf16 bit patterns or tensors."""
     E, H = config.emb_dim, config.hidden_dim
     nq, nkv = config.n_heads * config.head_dim, config.kv_dim
@@ -81,13 +96,14 @@ def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda
                       wqkv=repack(qkv, nq + 2 * nkv, E), wo=repack(dev_blocks(blocks["o"]), E, nq),
                       w_gate=repack(dev_blocks(blocks["gate"]), H, E), w_up=repack(dev_blocks(blocks["up"]), H, E),
                       w_down=repack(dev_blocks(blocks["down"]), E, H), codec="q4nx")
-    return out.with_stream() if stream_order else out
+    return out.with_stream()
 
 
-def prepare_layer(layer: wmod.LayerWeights, device="cuda", stream_order=True) -> DecodeLayer:
+def prepare_layer(layer: wmod.LayerWeights, device="cuda", stream_order=True, keep_triples=False) -> DecodeLayer:
     """Host LayerWeights (numpy) -> DecodeLayer: Q, K, V concatenated, everything in HBM, and (stream_order) every
     matrix re-packed into the decode kernels' stream order, the counterpart of the packed decode buffers the
-    reference attaches per layer at load time (llama32_1b_int4_weights.py:163-216)."""
+    reference attaches per layer at load time (llama32_1b_int4_weights.py:163-216).  stream_order=False leaves the
+    AutoAWQ triples for the checkpoint-layout kernels; keep_triples keeps them beside the re-pack."""
     def dev(a):
         a = np.ascontiguousarray(a)
         if a.dtype == np.uint16:
@@ -98,7 +114,7 @@ def prepare_layer(layer: wmod.LayerWeights, device="cuda", stream_order=True) ->
     out = DecodeLayer(attn_norm=dev(layer.attn_norm), ffn_norm=dev(layer.ffn_norm),
                       wqkv=lin(wmod.concat_linears(layer.wq, layer.wk, layer.wv)), wo=lin(layer.wo),
                       w_gate=lin(layer.w_gate), w_up=lin(layer.w_up), w_down=lin(layer.w_down))
-    return out.with_stream() if stream_order else out
+    return out.with_stream(keep_triples) if stream_order else out
 
 
 def new_kv_cache(config, max_seq, device="cuda"):
@@ -126,15 +142,14 @@ def run_decode_block(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer
         return ops.decode_attn_o_gemv_ffn_stream(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos,
                                                  config.n_heads, x, layer.ffn_norm, sw["wo"], sw["w_gate"], sw["w_up"],
                                                  sw["w_down"], eps=config.rms_eps, return_sumsq=return_sumsq)
-    if not q4nx:   # attention + block as one call: the O projection merges the attention's chunk partials where it can
-        qkv = ops.w4a16_rms_gemv(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps, x_sumsq=x_sumsq)
-        return ops.decode_attn_o_gemv_ffn(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads,
-                                          x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps,
-                                          return_sumsq=return_sumsq)
-    qkv = ops.q4nx_rms_gemv(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps)
-    attn_out = ops.decode_attention(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads)
-    y = ops.q4nx_o_gemv_ffn(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
-    return (y, None) if return_sumsq else y
+    if q4nx:
+        raise ValueError("a Q4NX layer runs on its stream-order re-pack (prepare_layer_q4nx / DecodeLayer.with_stream)")
+    # AutoAWQ triples (widths the stream order does not take, or a layer prepared with stream_order=False): attention +
+    # block as one call, the O projection merges the attention's chunk partials where it can
+    qkv = ops.w4a16_rms_gemv(x, layer.attn_norm, *layer.wqkv, eps=config.rms_eps, x_sumsq=x_sumsq)
+    return ops.decode_attn_o_gemv_ffn(qkv, rope_lut[current_pos], k_cache_layer, v_cache_layer, current_pos, config.n_heads,
+                                      x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps,
+                                      return_sumsq=return_sumsq)
 
 
 def decode_token(token_id, layers, embed_table, final_norm, lm_head, config, kv_cache, current_pos, rope_lut,
@@ -169,13 +184,6 @@ def decode_greedy(token, n_tokens, layers, embed_table, final_norm, lm_head, con
     return out
 
 
-def _prefill_stream_shapes(config):
-    """Shapes the stream-order prompt-pass blocks take: input lengths in whole pairs of groups, widths in whole
-    64-column tiles, attention output as wide as the embedding."""
-    E, H, nq = config.emb_dim, config.hidden_dim, config.n_heads * config.head_dim
-    return E % 256 == 0 and H % 256 == 0 and nq == E and (nq + 2 * config.kv_dim) % 64 == 0
-
-
 def run_prefill_layer(x, layer: DecodeLayer, config, k_cache_layer, v_cache_layer, rope_lut):
     """One transformer block over the M prompt tokens at positions 0..M-1 (_run_layer_int4,
     programming_examples/llms/llama32_1b_int4/llama32_1b_int4_prefill.py:241-390): RMSNorm + fused Q|K|V GEMM +
@@ -187,7 +195,7 @@ def run_prefill_layer(x, layer: DecodeLayer, config, k_cache_layer, v_cache_laye
     M = x.shape[0]
     nh, nkv, hd = config.n_heads, config.n_kv_heads, config.head_dim
     # the stream-order copies where the layer has them and the tiled stream-order GEMM takes every matrix
-    sw = layer.stream if layer.stream is not None and _prefill_stream_shapes(config) else None
+    sw = layer.stream if layer.stream is not None and _stream_covers_prefill(layer.stream) else None
     if sw is not None:
         qkv = ops.prefill_rms_qkv_rope_stream(x, layer.attn_norm, sw["wqkv"], rope_lut, 0, nh, nkv, hd, eps=config.rms_eps)
     else:

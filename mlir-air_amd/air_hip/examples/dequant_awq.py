@@ -5,10 +5,12 @@
 S bf16 per group, Z u8 per group, padded to 4 bytes); the GPU kernel reads that buffer as it is."""
 
 import argparse
+import sys
 
 import numpy as np
 
 from .. import awq, bf16
+from . import _common
 from ..backend import HIPBackend, HIPRunner, HipModule
 
 
@@ -32,7 +34,7 @@ def parse_args(argv=None):
     p.add_argument("--n", type=int, default=1024)
     p.add_argument("--group-size", type=int, default=128)
     p.add_argument("--herd-n", type=int, default=4, dest="herd_n")
-    return p.parse_args(argv)
+    return _common.add_reference_cli(p).parse_args(argv)
 
 
 def draw_inputs(args):
@@ -61,3 +63,12 @@ def run(args, cpu_reference):
     ok = HIPRunner(verbose=args.verbose)._check_outputs([got], [ref], rtol=1e-1, atol=5e-2)
     print("PASS!" if ok else "failed.")
     return 0 if ok else -1
+
+
+def main(argv=None):
+    args = parse_args(argv)
+    return _common.cli_main(args, build_module(args.n, args.group_size, args.herd_n), run)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -2,11 +2,13 @@
 (counterpart of programming_examples/matrix_multiplication/int4_awq/matmul_int4_packed.py)."""
 
 import argparse
+import sys
 
 import numpy as np
 
 from .. import awq, bf16
 from ..backend import HIPRunner, HipModule
+from . import _common
 from ._common import draw_l1_weights
 
 
@@ -27,7 +29,7 @@ def parse_args(argv=None):
     p.add_argument("--n", type=int, default=128)
     p.add_argument("--gs", type=int, default=128)
     p.add_argument("-v", "--verbose", action="store_true")
-    return p.parse_args(argv)
+    return _common.add_reference_cli(p).parse_args(argv)
 
 
 def draw_inputs(args):
@@ -44,3 +46,12 @@ def run(args, cpu_reference):
     C_ref = bf16.from_bits(cpu_reference(W_q, bf16.bits_of(W_s), W_z, bf16.bits_of(A)))
     return HIPRunner(verbose=args.verbose).run_test(module, inputs=[A, packed], expected_outputs=[C_ref], rtol=0.1,
                                                     atol=0.05, max_mismatch_percentage=0.05, min_correlation=0.999)
+
+
+def main(argv=None):
+    args = parse_args(argv)
+    return _common.cli_main(args, build_module(args.m, args.k, args.n, args.gs), run)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

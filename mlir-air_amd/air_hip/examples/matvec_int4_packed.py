@@ -2,11 +2,13 @@
 (counterpart of programming_examples/matrix_vector_multiplication/int4_awq/matvec_int4_packed.py)."""
 
 import argparse
+import sys
 
 import numpy as np
 
 from .. import awq, bf16
 from ..backend import HIPRunner, HipModule
+from . import _common
 from ._common import draw_l1_weights
 
 
@@ -31,7 +33,7 @@ def parse_args(argv=None):
     p.add_argument("--m-tile", type=int, default=8, dest="m_tile")
     p.add_argument("--k-chunk", type=int, default=2048, dest="k_chunk")
     p.add_argument("--n-cores", type=int, default=8, dest="n_cores")
-    return p.parse_args(argv)
+    return _common.add_reference_cli(p).parse_args(argv)
 
 
 def draw_inputs(args):
@@ -49,3 +51,12 @@ def run(args, cpu_reference):
     runner = HIPRunner(verbose=args.verbose)
     return runner.run_test(module, inputs=[packed, B], expected_outputs=[D_ref], rtol=0.1, atol=0.05,
                            min_correlation=0.999)
+
+
+def main(argv=None):
+    args = parse_args(argv)
+    return _common.cli_main(args, build_module(args.m, args.k, GS=args.gs), run)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

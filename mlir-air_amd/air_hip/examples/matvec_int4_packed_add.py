@@ -1,11 +1,13 @@
 """int4-AWQ GEMV with residual: D = dequant(A) @ B + R
 (counterpart of .../int4_awq/matvec_int4_packed_add.py)."""
 
+import sys
+
 import numpy as np
 
 from .. import bf16
 from ..backend import HIPRunner, HipModule
-from . import matvec_int4_packed as base
+from . import _common, matvec_int4_packed as base
 
 pack_inputs = base.pack_inputs
 parse_args = base.parse_args
@@ -28,3 +30,12 @@ def run(args, cpu_reference):
     packed = pack_inputs(A_q, A_s, A_z, args.m, args.k, args.gs)
     return HIPRunner(verbose=args.verbose).run_test(module, inputs=[packed, B, R], expected_outputs=[D_ref],
                                                     rtol=0.1, atol=0.05, min_correlation=0.999)
+
+
+def main(argv=None):
+    args = parse_args(argv)
+    return _common.cli_main(args, build_module(args.m, args.k, GS=args.gs), run)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

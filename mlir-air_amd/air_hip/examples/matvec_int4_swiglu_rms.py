@@ -5,11 +5,13 @@ One GPU kernel: every wave normalises the K-slice of x it feeds to the matrix co
 gate and up matrices and the reducer applies SwiGLU in its epilogue."""
 
 import argparse
+import sys
 
 import numpy as np
 
 from .. import awq, bf16
 from ..backend import HIPRunner, HipModule
+from . import _common
 from ._common import draw_l1_weights
 
 
@@ -31,7 +33,7 @@ def parse_args(argv=None):
     p.add_argument("--m", type=int, default=16384)
     p.add_argument("--k", type=int, default=2048)
     p.add_argument("--gs", type=int, default=128)
-    return p.parse_args(argv)
+    return _common.add_reference_cli(p).parse_args(argv)
 
 
 def draw_inputs(args):
@@ -50,3 +52,12 @@ def run(args, cpu_reference):
     gate_buf, up_buf = pack_inputs(A_q, A_s, A_z, args.m, args.k, args.gs)
     return HIPRunner(verbose=args.verbose).run_test(module, inputs=[gate_buf, up_buf, RMS_in], expected_outputs=[D_ref],
                                                     rtol=0.15, atol=0.5, min_correlation=0.99)
+
+
+def main(argv=None):
+    args = parse_args(argv)
+    return _common.cli_main(args, build_module(args.m, args.k, GS=args.gs), run)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

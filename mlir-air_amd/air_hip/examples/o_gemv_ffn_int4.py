@@ -8,10 +8,12 @@
 Three kernel launches behind one C-ABI call; res1 and swiglu stay on the device."""
 
 import argparse
+import sys
 
 import numpy as np
 
 from .. import awq, bf16
+from . import _common
 from ..backend import HIPRunner, HipModule
 
 
@@ -40,7 +42,7 @@ def parse_args(argv=None):
     p.add_argument("--emb-dim", type=int, default=2048)
     p.add_argument("--hidden-dim", type=int, default=8192)
     p.add_argument("--gs", type=int, default=128)
-    return p.parse_args(argv)
+    return _common.add_reference_cli(p).parse_args(argv)
 
 
 def draw_inputs(args):
@@ -69,3 +71,12 @@ def run(args, cpu_reference):
     inputs = [pack_inputs(*wo), attn_out, x_residual, ffn_norm_w, pack_inputs(*gate), pack_inputs(*up), pack_inputs(*wd)]
     return HIPRunner(verbose=args.verbose).run_test(module, inputs=inputs, expected_outputs=[expected],
                                                     rtol=0.2, atol=2.0, min_correlation=0.99)
+
+
+def main(argv=None):
+    args = parse_args(argv)
+    return _common.cli_main(args, build_module(args.emb_dim, args.hidden_dim, gs=args.gs), run)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -696,7 +696,7 @@ def q4nx_dequant(blocks, M, K, mode=0, out=None):
 
 def q4nx_repack(blocks, M, K, mode=0):
     """Blocks -> (qweight int32 [K, M/8], scales bf16 [K/32, M], mins bf16 [K/32, M]), the
-    operands of q4nx_gemm; done once per tensor at load time."""
+    operands of q4nx_repack_stream; done once per tensor at load time."""
     lib = _lib.load_library()
     _need_cuda(blocks)
     if blocks.numel() * blocks.element_size() != (M // 32) * (K // 256) * 5120:
@@ -709,75 +709,22 @@ def q4nx_repack(blocks, M, K, mode=0):
 
 
 def q4nx_gemm(x, qweight, scales, mins, residual=None, out=None):
-    """y = bf16(x . W + residual) for the operands of q4nx_repack; x [rows, K] or a vector [K]."""
-    lib = _lib.load_library()
-    _need_cuda(x, qweight, scales, mins)
-    vec = x.dim() == 1
-    x2 = x.unsqueeze(0) if vec else x
-    M, K = x2.shape
-    if qweight.shape[0] != K:
-        raise ValueError(f"x has K={K} but qweight has {qweight.shape[0]} rows")
-    N = qweight.shape[1] * 8
-    if scales.shape != (K // 32, N) or mins.shape != (K // 32, N):
-        raise ValueError(f"scales / mins must be [{K // 32}, {N}], got {tuple(scales.shape)} / {tuple(mins.shape)}")
-    if residual is not None:
-        _need_cuda(residual)
-        if residual.numel() != M * N:
-            raise ValueError("residual must have the shape of the result")
-    if out is None:
-        out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    ws = workspace(lib.w4a16_gemm_workspace_bytes(M, K, N), x.device)
-    _lib.check(lib.w4a16_q4nx_gemm_bf16(_ptr(_bits(x2)), _ptr(qweight), _ptr(_bits(scales)), _ptr(_bits(mins)),
-                                        _ptr(_bits(residual)) if residual is not None else None, _ptr(out),
-                                        M, K, N, _ptr(ws), ws.numel(), _stream()))
-    _after_workspace_call()
-    return out.squeeze(0) if vec else out
-
-
-def _qptrs(w):
-    """(qweight, scales, mins) of the affine codec as C-ABI pointers."""
-    return [_ptr(w[0]), _ptr(_bits(w[1])), _ptr(_bits(w[2]))]
+    """y = bf16(x . W + residual) for the operands of q4nx_repack; x [rows, K] or a vector [K].  Re-packs W into Q4NX
+    stream order on every call: a caller that multiplies more than once keeps the result of q4nx_repack_stream and
+    calls q4nx_gemm_stream."""
+    return q4nx_gemm_stream(x, q4nx_repack_stream(qweight, scales, mins), residual=residual, out=out)
 
 
 def q4nx_rms_gemv(x, norm_weight, qweight, scales, mins, eps=1e-5):
-    """y[N] = bf16(rms_norm(x, norm_weight) . W) for the operands of q4nx_repack."""
-    lib = _lib.load_library()
-    _need_cuda(x, norm_weight, qweight, scales, mins)
-    K = x.numel()
-    if qweight.shape[0] != K or norm_weight.numel() != K:
-        raise ValueError(f"x has K={K}, qweight {qweight.shape[0]} rows, norm weight {norm_weight.numel()}")
-    N = qweight.shape[1] * 8
-    out = torch.empty((N,), dtype=torch.bfloat16, device=x.device)
-    ws = workspace(lib.w4a16_gemm_workspace_bytes(1, K, N), x.device)
-    _lib.check(lib.w4a16_q4nx_rms_gemv_bf16(_ptr(_bits(x)), _ptr(_bits(norm_weight)), float(eps),
-                                            *_qptrs((qweight, scales, mins)), _ptr(out), K, N,
-                                            _ptr(ws), ws.numel(), _stream()))
-    _after_workspace_call()
-    return out
+    """y[N] = bf16(rms_norm(x, norm_weight) . W) for the operands of q4nx_repack (re-packed on every call, as q4nx_gemm)."""
+    return q4nx_rms_gemv_stream(x, norm_weight, q4nx_repack_stream(qweight, scales, mins), eps=eps)
 
 
 def q4nx_o_gemv_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, return_intermediates=False):
-    """o_gemv_ffn for the affine codec: wo/gate/up/down are (qweight, scales, mins) from q4nx_repack."""
-    lib = _lib.load_library()
-    _need_cuda(attn_out, x_residual, ffn_norm_weight, *wo, *gate, *up, *down)
-    E = attn_out.numel()
-    H = gate[0].shape[1] * 8
-    if (wo[0].shape[0] != E or wo[0].shape[1] * 8 != E or gate[0].shape[0] != E or up[0].shape != gate[0].shape
-            or down[0].shape[0] != H or down[0].shape[1] * 8 != E or x_residual.numel() != E
-            or ffn_norm_weight.numel() != E):
-        raise ValueError("q4nx_o_gemv_ffn: wo must be [E, E/8], gate/up [E, H/8], down [H, E/8], vectors [E]")
-    dev = attn_out.device
-    y = torch.empty((E,), dtype=torch.bfloat16, device=dev)
-    res1 = torch.empty((E,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
-    h = torch.empty((H,), dtype=torch.bfloat16, device=dev) if return_intermediates else None
-    ws = workspace(lib.w4a16_block_workspace_bytes(E, H), dev, ("block", E, H))
-    _lib.check(lib.w4a16_q4nx_o_gemv_ffn_bf16(
-        _ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps),
-        *_qptrs(wo), *_qptrs(gate), *_qptrs(up), *_qptrs(down), _ptr(y),
-        _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
-        E, H, _ptr(ws), ws.numel(), _stream()))
-    _after_workspace_call()
-    return (y, res1, h) if return_intermediates else y
+    """o_gemv_ffn for the affine codec: wo/gate/up/down are (qweight, scales, mins) from q4nx_repack (re-packed on every
+    call, as q4nx_gemm)."""
+    sw = [q4nx_repack_stream(*w) for w in (wo, gate, up, down)]
+    return q4nx_o_gemv_ffn_stream(attn_out, x_residual, ffn_norm_weight, *sw, eps=eps, return_intermediates=return_intermediates)
 
 
 def q4nx_repack_stream(qweight, scales, mins):

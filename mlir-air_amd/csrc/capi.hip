@@ -50,43 +50,25 @@ size_t stream_partial_bytes(int M, int N, int nmat) {
     return round256((size_t)nmat * kMaxKSplit * (size_t)(M < 16 ? M : 16) * ((size_t)N + 512) * sizeof(float));
 }
 
-// One quantised matrix in either codec: AWQ (qweight, qzeros, scales [K / 128, N]) or the affine
-// 32-row-group codec of q4nx_repack (qweight, mins, scales [K / 32, N]).
+// One AWQ matrix in the checkpoint layout (qweight, qzeros, scales [K / 128, N]).
 struct QuantW {
-    const int32_t *qw;
-    const void *aux;   // qzeros int32 or mins bf16
+    const int32_t *qw, *qz;
     const uint16_t *sc;
 };
 
-int check_affine(const QuantW &w, int K, int N) {
-    if (!w.qw || !w.aux || !w.sc) return W4A16_ERR_NULL;
-    if (K <= 0 || N <= 0 || K % kGroup != 0 || N % 32 != 0) return W4A16_ERR_SHAPE;
-    if (misaligned(w.qw) || misaligned(w.aux) || misaligned(w.sc)) return W4A16_ERR_ALIGN;
-    return W4A16_OK;
-}
+int check_w(const QuantW &w, int K, int N, int group) { return check_quant(w.qw, w.qz, w.sc, K, N, group, 32); }
 
-int check_w(bool affine, const QuantW &w, int K, int N, int group) {
-    return affine ? check_affine(w, K, N) : check_quant(w.qw, w.aux, w.sc, K, N, group, 32);
-}
-
-hipError_t stream_w(bool affine, const uint16_t *x, const QuantW &a, const QuantW *up, uint16_t *y, int M, int K, int N,
-                    void *workspace, hipStream_t st, StreamExtras ex) {
-    if (affine) {
-        ex.mins = static_cast<const uint16_t *>(a.aux);
-        ex.up_mins = up ? static_cast<const uint16_t *>(up->aux) : nullptr;
-        return launch_stream(x, a.qw, nullptr, a.sc, up ? up->qw : nullptr, nullptr, up ? up->sc : nullptr, y, M, K, N,
-                             workspace, st, ex);
-    }
-    return launch_stream(x, a.qw, static_cast<const int32_t *>(a.aux), a.sc, up ? up->qw : nullptr,
-                         up ? static_cast<const int32_t *>(up->aux) : nullptr, up ? up->sc : nullptr, y, M, K, N,
+hipError_t stream_w(const uint16_t *x, const QuantW &a, const QuantW *up, uint16_t *y, int M, int K, int N, void *workspace,
+                    hipStream_t st, const StreamExtras &ex) {
+    return launch_stream(x, a.qw, a.qz, a.sc, up ? up->qw : nullptr, up ? up->qz : nullptr, up ? up->sc : nullptr, y, M, K, N,
                          workspace, st, ex);
 }
 
-int rms_gemv_impl(bool affine, const uint16_t *x, const uint16_t *norm_weight, float eps, const QuantW &w, uint16_t *y,
+int rms_gemv_impl(const uint16_t *x, const uint16_t *norm_weight, float eps, const QuantW &w, uint16_t *y,
                   int K, int N, int group, void *workspace, size_t workspace_bytes, void *stream,
                   const float *x_sumsq = nullptr, int n_pieces = 0) {
     if (!x || !y || !norm_weight) return W4A16_ERR_NULL;
-    int rc = check_w(affine, w, K, N, group);
+    int rc = check_w(w, K, N, group);
     if (rc) return rc;
     if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
     if (misaligned(x) || misaligned(y) || misaligned(norm_weight)) return W4A16_ERR_ALIGN;
@@ -97,7 +79,7 @@ int rms_gemv_impl(bool affine, const uint16_t *x, const uint16_t *norm_weight, f
     ex.eps = eps;
     ex.sumsq_in = x_sumsq;
     ex.sumsq_n = x_sumsq ? n_pieces : 0;
-    hipError_t e = stream_w(affine, x, w, nullptr, y, 1, K, N, workspace, static_cast<hipStream_t>(stream), ex);
+    hipError_t e = stream_w(x, w, nullptr, y, 1, K, N, workspace, static_cast<hipStream_t>(stream), ex);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
@@ -107,19 +89,19 @@ struct AttnPartials {
     int nsplit, hd;
 };
 
-int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+int o_gemv_ffn_impl(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
                     float eps, const QuantW &wo, const QuantW &wg, const QuantW &wu, const QuantW &wd, uint16_t *y,
                     uint16_t *res1_out, uint16_t *h_out, int E, int H, int group, void *workspace,
                     size_t workspace_bytes, void *stream, const AttnPartials *partials = nullptr, bool check_only = false,
                     float *y_sumsq = nullptr) {
     if (!attn_out || !x_residual || !ffn_norm_weight || !y) return W4A16_ERR_NULL;
-    int rc = check_w(affine, wo, E, E, group);
+    int rc = check_w(wo, E, E, group);
     if (rc) return rc;
-    rc = check_w(affine, wg, E, H, group);
+    rc = check_w(wg, E, H, group);
     if (rc) return rc;
-    rc = check_w(affine, wu, E, H, group);
+    rc = check_w(wu, E, H, group);
     if (rc) return rc;
-    rc = check_w(affine, wd, H, E, group);
+    rc = check_w(wd, H, E, group);
     if (rc) return rc;
     if (!(eps >= 0.f)) return W4A16_ERR_SHAPE;
     if (misaligned(attn_out) || misaligned(x_residual) || misaligned(ffn_norm_weight) || misaligned(y) ||
@@ -148,23 +130,9 @@ int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_res
         add.attn_nsplit = partials->nsplit;
         add.attn_hd = partials->hd;
     }
-    hipError_t e = stream_w(affine, attn_out, wo, nullptr, res1, 1, E, E, workspace, st, add);
+    hipError_t e = stream_w(attn_out, wo, nullptr, res1, 1, E, E, workspace, st, add);
     add.attn_ml = add.attn_acc = nullptr;   // stage 3 reuses `add` for the down projection
     if (e != hipSuccess) return hip_fail(e);
-    // stages 2 and 3 as one persistent kernel when the shape fits it (AWQ codec): h = swiglu(rms_norm(res1) . Wgate,
-    // rms_norm(res1) . Wup), y = bf16(h . Wdown + res1)
-    FfnFusedPlan fpl;
-    if (!affine && chain_norm && !g_stream_tune.no_ffn_fused && plan_ffn_fused(E, H, current_cus(), &fpl) &&
-        kHeaderBytes + ffn_fused_scratch_bytes(E, H, fpl) + 256 + round256((size_t)E * sizeof(uint16_t)) +
-                round256((size_t)H * sizeof(uint16_t)) <= w4a16_block_workspace_bytes(E, H)) {
-        const int32_t *const qw[3] = {wg.qw, wu.qw, wd.qw};
-        const int32_t *const qz[3] = {static_cast<const int32_t *>(wg.aux), static_cast<const int32_t *>(wu.aux),
-                                      static_cast<const int32_t *>(wd.aux)};
-        const uint16_t *const sc[3] = {wg.sc, wu.sc, wd.sc};
-        const FfnFusedNorm norm = {ffn_norm_weight, res1_sumsq, res1_tiles, eps};
-        e = launch_ffn_fused(fpl, res1, qw, qz, sc, res1, y, h_out, E, H, workspace, st, &norm, y_sumsq);
-        return e == hipSuccess ? W4A16_OK : hip_fail(e);
-    }
     // stage 2: h = swiglu(rms_norm(res1) . Wgate, rms_norm(res1) . Wup)
     StreamExtras rms;
     rms.norm_w = ffn_norm_weight;
@@ -173,12 +141,12 @@ int o_gemv_ffn_impl(bool affine, const uint16_t *attn_out, const uint16_t *x_res
         rms.sumsq_in = res1_sumsq;
         rms.sumsq_n = res1_tiles;
     }
-    e = stream_w(affine, res1, wg, &wu, h, 1, E, H, workspace, st, rms);
+    e = stream_w(res1, wg, &wu, h, 1, E, H, workspace, st, rms);
     if (e != hipSuccess) return hip_fail(e);
     // stage 3: y = bf16(h . Wdown + res1)
     add.sumsq_out = y_sumsq;
     add.residual = res1;
-    e = stream_w(affine, h, wd, nullptr, y, 1, H, E, workspace, st, add);
+    e = stream_w(h, wd, nullptr, y, 1, H, E, workspace, st, add);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
@@ -380,16 +348,6 @@ int w4a16_ffn_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const 
     if (!workspace || workspace_bytes < w4a16_ffn_workspace_bytes(K, H)) return W4A16_ERR_WORKSPACE;
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // One persistent kernel when the shape fits it (every workgroup resident at once), else two launches.
-    FfnFusedPlan fpl;
-    if (!g_stream_tune.no_ffn_fused && plan_ffn_fused(K, H, current_cus(), &fpl) &&
-        kHeaderBytes + ffn_fused_scratch_bytes(K, H, fpl) <= w4a16_ffn_workspace_bytes(K, H)) {
-        const int32_t *const qw[3] = {gate_qweight, up_qweight, down_qweight};
-        const int32_t *const qz[3] = {gate_qzeros, up_qzeros, down_qzeros};
-        const uint16_t *const sc[3] = {gate_scales, up_scales, down_scales};
-        hipError_t ef = launch_ffn_fused(fpl, x, qw, qz, sc, nullptr, y, h_out, K, H, workspace, st);
-        return ef == hipSuccess ? W4A16_OK : hip_fail(ef);
-    }
     uint16_t *h = h_out;
     if (!h) h = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + w4a16_ffn_workspace_bytes(K, H) -
                                              round256((size_t)H * sizeof(uint16_t)));
@@ -419,7 +377,7 @@ int w4a16_gemv_add_bf16(const uint16_t *x, const int32_t *qweight, const int32_t
 int w4a16_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const int32_t *qweight,
                         const int32_t *qzeros, const uint16_t *scales, uint16_t *y, int K, int N, int group,
                         void *workspace, size_t workspace_bytes, void *stream) {
-    return rms_gemv_impl(false, x, norm_weight, eps, QuantW{qweight, qzeros, scales}, y, K, N, group, workspace,
+    return rms_gemv_impl(x, norm_weight, eps, QuantW{qweight, qzeros, scales}, y, K, N, group, workspace,
                          workspace_bytes, stream);
 }
 
@@ -429,7 +387,7 @@ int w4a16_rms_gemv_sumsq_bf16(const uint16_t *x, const float *x_sumsq, int n_pie
     if (!x_sumsq) return W4A16_ERR_NULL;
     if (n_pieces < 1 || n_pieces > 64) return W4A16_ERR_SHAPE;
     if (misaligned(x_sumsq)) return W4A16_ERR_ALIGN;
-    return rms_gemv_impl(false, x, norm_weight, eps, QuantW{qweight, qzeros, scales}, y, K, N, group, workspace,
+    return rms_gemv_impl(x, norm_weight, eps, QuantW{qweight, qzeros, scales}, y, K, N, group, workspace,
                          workspace_bytes, stream, x_sumsq, n_pieces);
 }
 
@@ -651,7 +609,7 @@ int w4a16_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, 
                           const int32_t *down_qweight, const int32_t *down_qzeros, const uint16_t *down_scales,
                           uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int E, int H, int group, void *workspace,
                           size_t workspace_bytes, void *stream) {
-    return o_gemv_ffn_impl(false, attn_out, x_residual, ffn_norm_weight, eps, QuantW{o_qweight, o_qzeros, o_scales},
+    return o_gemv_ffn_impl(attn_out, x_residual, ffn_norm_weight, eps, QuantW{o_qweight, o_qzeros, o_scales},
                            QuantW{gate_qweight, gate_qzeros, gate_scales}, QuantW{up_qweight, up_qzeros, up_scales},
                            QuantW{down_qweight, down_qzeros, down_scales}, y, res1_out, h_out, E, H, group, workspace,
                            workspace_bytes, stream);
@@ -831,7 +789,7 @@ int w4a16_decode_attn_o_gemv_ffn_bf16(const uint16_t *qkv, const uint16_t *rope_
     if (misaligned(attn_workspace)) return W4A16_ERR_ALIGN;
     const QuantW wo{o_qweight, o_qzeros, o_scales}, wg{gate_qweight, gate_qzeros, gate_scales},
         wu{up_qweight, up_qzeros, up_scales}, wd{down_qweight, down_qzeros, down_scales};
-    int rc = o_gemv_ffn_impl(false, attn_out, x_residual, ffn_norm_weight, eps, wo, wg, wu, wd, y, nullptr, nullptr, E, H,
+    int rc = o_gemv_ffn_impl(attn_out, x_residual, ffn_norm_weight, eps, wo, wg, wu, wd, y, nullptr, nullptr, E, H,
                              group, workspace, workspace_bytes, stream, nullptr, true);
     if (rc) return rc;
     // With several sequence chunks and an O projection whose units lie inside one head, the projection merges the
@@ -844,7 +802,7 @@ int w4a16_decode_attn_o_gemv_ffn_bf16(const uint16_t *qkv, const uint16_t *rope_
     hipError_t e = launch_decode_attention(qkv, rope_lut_row, k_cache, v_cache, attn_out, pos, max_seq, n_heads, n_kv_heads,
                                            head_dim, attn_workspace, static_cast<hipStream_t>(stream), !fuse);
     if (e != hipSuccess) return hip_fail(e);
-    return o_gemv_ffn_impl(false, attn_out, x_residual, ffn_norm_weight, eps, wo, wg, wu, wd, y, nullptr, nullptr, E, H,
+    return o_gemv_ffn_impl(attn_out, x_residual, ffn_norm_weight, eps, wo, wg, wu, wd, y, nullptr, nullptr, E, H,
                            group, workspace, workspace_bytes, stream, fuse ? &ap : nullptr, false, y_sumsq);
 }
 
@@ -935,48 +893,6 @@ int w4a16_q4nx_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *
                                   y, res1_out, h_out, y_sumsq, E, H, kGroup, workspace, workspace_bytes, stream, false, true);
 }
 
-int w4a16_q4nx_gemm_bf16(const uint16_t *x, const int32_t *qweight, const uint16_t *scales, const uint16_t *mins,
-                         const uint16_t *residual, uint16_t *y, int M, int K, int N, void *workspace,
-                         size_t workspace_bytes, void *stream) {
-    if (!x || !y || !qweight || !scales || !mins) return W4A16_ERR_NULL;
-    if (M <= 0 || K <= 0 || N <= 0 || K % 128 != 0 || N % 32 != 0) return W4A16_ERR_SHAPE;
-    if (misaligned(x) || misaligned(y) || misaligned(qweight) || misaligned(scales) || misaligned(mins) ||
-        misaligned(residual))
-        return W4A16_ERR_ALIGN;
-    if (!workspace || workspace_bytes < w4a16_gemm_workspace_bytes(M, K, N)) return W4A16_ERR_WORKSPACE;
-    if (misaligned(workspace)) return W4A16_ERR_ALIGN;
-    hipError_t e = hipSuccess;
-    for (int m0 = 0; m0 < M && e == hipSuccess; m0 += 16) {
-        const int rows = M - m0 < 16 ? M - m0 : 16;
-        StreamExtras extras;
-        extras.mins = mins;
-        extras.residual = residual ? residual + (size_t)m0 * N : nullptr;
-        e = launch_stream(x + (size_t)m0 * K, qweight, nullptr, scales, nullptr, nullptr, nullptr, y + (size_t)m0 * N,
-                          rows, K, N, workspace, static_cast<hipStream_t>(stream), extras);
-    }
-    return e == hipSuccess ? W4A16_OK : hip_fail(e);
-}
-
-int w4a16_q4nx_rms_gemv_bf16(const uint16_t *x, const uint16_t *norm_weight, float eps, const int32_t *qweight,
-                             const uint16_t *scales, const uint16_t *mins, uint16_t *y, int K, int N, void *workspace,
-                             size_t workspace_bytes, void *stream) {
-    return rms_gemv_impl(true, x, norm_weight, eps, QuantW{qweight, mins, scales}, y, K, N, 32, workspace,
-                         workspace_bytes, stream);
-}
-
-int w4a16_q4nx_o_gemv_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
-                               float eps, const int32_t *o_qweight, const uint16_t *o_scales, const uint16_t *o_mins,
-                               const int32_t *gate_qweight, const uint16_t *gate_scales, const uint16_t *gate_mins,
-                               const int32_t *up_qweight, const uint16_t *up_scales, const uint16_t *up_mins,
-                               const int32_t *down_qweight, const uint16_t *down_scales, const uint16_t *down_mins,
-                               uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int E, int H, void *workspace,
-                               size_t workspace_bytes, void *stream) {
-    return o_gemv_ffn_impl(true, attn_out, x_residual, ffn_norm_weight, eps, QuantW{o_qweight, o_mins, o_scales},
-                           QuantW{gate_qweight, gate_mins, gate_scales}, QuantW{up_qweight, up_mins, up_scales},
-                           QuantW{down_qweight, down_mins, down_scales}, y, res1_out, h_out, E, H, 32, workspace,
-                           workspace_bytes, stream);
-}
-
 int w4a16_tune(const char *key, int value) {
     if (!key || value < 0) return W4A16_ERR_TUNE;
     if (!strcmp(key, "gemv_lw")) {
@@ -992,8 +908,6 @@ int w4a16_tune(const char *key, int value) {
         g_stream_tune.skip_publish = value ? 1 : 0;
     } else if (!strcmp(key, "gemv_spin_limit")) {
         g_stream_tune.spin_limit = value;
-    } else if (!strcmp(key, "ffn_fused")) {
-        g_stream_tune.no_ffn_fused = value ? 0 : 1;
     } else if (!strcmp(key, "attn_fuse")) {
         g_stream_tune.no_attn_fuse = value ? 0 : 1;
     } else if (!strcmp(key, "gemm_stream_max_m")) {

@@ -23,7 +23,6 @@ struct StreamTune {
     int stream_max_m = 0;   // largest M that w4a16_gemm_bf16 gives to the streaming kernel (0 = kStreamMaxM; at least 16)
     int skip_publish = 0; // tests only: producers do not publish, so reducers run into their poll bound
     int spin_limit = 0;   // reducer poll bound (0 = default); tiny values force the timeout path in tests
-    int no_ffn_fused = 1; // 1 (default): w4a16_ffn_swiglu_bf16 runs its two streaming launches; 0: the one-launch persistent kernel (opt-in)
     int no_attn_fuse = 0; // 1: w4a16_decode_attn_o_gemv_ffn_bf16 always runs the attention merge launch
 };
 extern StreamTune g_stream_tune;
@@ -51,10 +50,6 @@ struct StreamExtras {
     const float *sumsq_in = nullptr;
     int sumsq_n = 0;
     float *sumsq_out = nullptr;
-    // Affine codec with 32-row groups (w = q * s + m): per-group minimum [K / 32, N] bf16.  `scales` is then
-    // [K / 32, N] too and `qzeros` is not read.  `up_mins` belongs to the second matrix of a SwiGLU launch.
-    const uint16_t *mins = nullptr;
-    const uint16_t *up_mins = nullptr;
     // M == 1: x is not read; it is the merge of the decode attention's per-chunk partials (attention_partials below),
     // computed by every wave for the rows of its units exactly as the attention merge kernel computes it.  Only where
     // stream_attn_fusable says so.
@@ -172,26 +167,6 @@ hipError_t launch_prefill_o_ffn_stream(const uint16_t *attn_out, const uint16_t 
                                        const void *wo, const void *wg, const void *wu, const void *wd, uint16_t *y,
                                        uint16_t *res1_out, uint16_t *h_out, int M, int E, int H, void *workspace,
                                        hipStream_t stream);
-
-// Decode FFN as one persistent kernel (ffn_fused.hip).  plan_ffn_fused returns false for shapes
-// the kernel does not take (the caller then runs the two streaming launches).
-struct FfnFusedPlan {
-    int G, tilesA, splitA, upsA, tilesB, splitB, upsB;
-};
-bool plan_ffn_fused(int E, int H, int cus, FfnFusedPlan *pl);
-size_t ffn_fused_scratch_bytes(int E, int H, const FfnFusedPlan &pl);   // bytes after the workspace header
-// RMSNorm prologue of the fused kernel: x is the output of a launch that left sum(x^2) in `sumsq_in`
-// (`sumsq_n` <= 64 pieces, StreamExtras::sumsq_out).
-struct FfnFusedNorm {
-    const uint16_t *norm_w;
-    const float *sumsq_in;
-    int sumsq_n;
-    float eps;
-};
-hipError_t launch_ffn_fused(const FfnFusedPlan &pl, const uint16_t *x, const int32_t *const qw[3], const int32_t *const qz[3],
-                            const uint16_t *const sc[3], const uint16_t *residual, uint16_t *y, uint16_t *h_out, int E, int H,
-                            void *workspace, hipStream_t stream, const FfnFusedNorm *norm = nullptr,
-                            float *sumsq_out = nullptr);   // sumsq_out [E / 256]: sum of squares of y per 256-column tile
 
 // Q4NX / Q4_0 block codec (q4nx.hip).  mode: 0 w = s q + m, 1 w = s (q - m), 2 signed q, w = s q.
 hipError_t launch_q4nx_dequant(const void *blocks, uint16_t *out, int M, int K, int mode, hipStream_t stream);

@@ -51,7 +51,6 @@ struct StreamParams {
     const uint32_t *qw[2];
     const uint32_t *qz[2];
     const uint16_t *sc[2];
-    const uint16_t *mn[2];   // affine codec: per-group minimum [K / 32, N] bf16 of each matrix (qz unused), else null
     uint16_t *y;
     uint32_t *header;   // workspace header: word 0 = poll timeouts seen
     float *partial;     // [nmat * ksplit][ntiles][2 planes][M * tile columns / 2]: a quad's words 0, 1 and words 2, 3
@@ -102,13 +101,10 @@ struct Words<1> { typedef uint32_t type __attribute__((ext_vector_type(1))); };
 // RMS    x is RMS-normalised on the fly: every wave computes 1/sqrt(mean(x^2) + eps) of its
 //        rows itself (x is K bf16 values, L2-resident) while its weight loads are in
 //        flight, and feeds bf16((x * rstd) * norm_w) to the matrix cores.  M <= 4.
-// AFF    affine codec with groups of 32 rows (one K-step): w = q * s + m with unsigned q, s and m
-//        bf16 [K / 32, N].  Every K-step is flushed on its own:
-//        y += s * sum (128 + q) x  +  (m - 128 s) * sum x.
 // ATT    M == 1: x is the merge of the decode attention's chunk partials, computed by every wave for the 64 rows of
 //        its unit (KSTEPS == 2, inside one head) with the merge kernel's arithmetic in the merge kernel's order,
 //        so the result is the same bit for bit; the partials are requested ahead of the weights.
-template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS, bool AFF, bool ATT = false>
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS, bool ATT = false>
 __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParams p) {
     constexpr int SLOTS = WAVES;   // one LDS slot per wave: a single write round, no read-modify-write
     typedef typename Words<LW>::type wvec;
@@ -153,7 +149,6 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
     const char *qw_s = reinterpret_cast<const char *>(p.qw[mat]);
     const char *qz_s = reinterpret_cast<const char *>(p.qz[mat]);
     const char *sc_s = reinterpret_cast<const char *>(p.sc[mat]);
-    const char *mn_s = reinterpret_cast<const char *>(p.mn[mat]);
     const uint32_t qw_lane = (uint32_t)(((size_t)chunk_c * LW + (size_t)(8 * lg) * p.nb) * sizeof(uint32_t));
     const uint32_t qz_lane = (uint32_t)((size_t)chunk_c * LW * sizeof(uint32_t));
     const uint32_t sc_lane = (uint32_t)((size_t)chunk_c * LC * sizeof(uint16_t));
@@ -233,7 +228,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         float attn_a[ATT ? kMaxAttnSplit : 1];
         float attn_m = kAttnNegBig, attn_l = 0.f;
         if constexpr (ATT) {
-            static_assert(!ATT || (KSTEPS == 2 && MI == 1 && NMAT == 1 && !RMS && !AFF), "attention merge prologue: plain M = 1 units of 64 rows");
+            static_assert(!ATT || (KSTEPS == 2 && MI == 1 && NMAT == 1 && !RMS), "attention merge prologue: plain M = 1 units of 64 rows");
             const int head = (kstep0 * 32) / p.attn_hd;                 // scalar: the unit lies inside one head
             const int e = kstep0 * 32 - head * p.attn_hd + lane;        // this lane's element of the head
             const float *src = p.attn_acc + (size_t)head * p.attn_nsplit * p.attn_hd + e;
@@ -259,18 +254,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
         }
         wvec zw;
         u32x4 sv[LW];
-        u32x4 gs[AFF ? KSTEPS : 1][LW], gm[AFF ? KSTEPS : 1][LW];   // affine codec: scales and minima of each K-step
-        if constexpr (AFF) {
-#pragma unroll
-            for (int s = 0; s < KSTEPS; ++s) {
-#pragma unroll
-                for (int c = 0; c < LW; ++c) {
-                    const size_t off = ((size_t)(kstep0 + s) * p.N + 8 * c) * sizeof(uint16_t) + sc_lane;
-                    gs[s][c] = *reinterpret_cast<const u32x4 *>(sc_s + off);
-                    gm[s][c] = *reinterpret_cast<const u32x4 *>(mn_s + off);
-                }
-            }
-        } else {
+        {
             zw = *reinterpret_cast<const wvec *>(qz_s + (size_t)g * row_bytes + qz_lane);
 #pragma unroll
             for (int c = 0; c < LW; ++c)
@@ -322,45 +306,7 @@ __global__ void __launch_bounds__(WAVES * 64, 2) stream_kernel(const StreamParam
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s)
             if (!a_valid) av[s] = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (AFF) {
-            // One group per K-step: the MFMA tiles of a K-step start from zero and are folded into
-            // yacc right away.  Column mapping as in the group flush below.
-            const floatx4 zero4 = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < KSTEPS; ++s) {
-                const bf16x8 a = __builtin_bit_cast(bf16x8, av[s]);
-                const floatx4 xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ones, zero4, 0, 0, 0);
-#pragma unroll
-                for (int c = 0; c < LW; ++c) {
-                    floatx4 acc[8];
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        const uint32_t sel = 0x0C000C00u | ((4u + b) << 16) | (uint32_t)b;
-                        u32x4 lo, hi;
-#pragma unroll
-                        for (int v = 0; v < 4; ++v) {
-                            const uint32_t pr = __builtin_amdgcn_perm(w[s][2 * v + 1][c], w[s][2 * v][c], sel);
-                            lo[v] = (pr & nib_mask) | magic;
-                            hi[v] = ((pr >> 4) & nib_mask) | magic;
-                        }
-                        acc[2 * b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, lo), zero4, 0, 0, 0);
-                        acc[2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, hi), zero4, 0, 0, 0);
-                    }
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const uint32_t sw = gs[s][c][q], mw = gm[s][c][q];
-                        const float s_lo = __builtin_bit_cast(float, sw << 16), s_hi = __builtin_bit_cast(float, sw & 0xFFFF0000u);
-                        const float m_lo = __builtin_bit_cast(float, mw << 16), m_hi = __builtin_bit_cast(float, mw & 0xFFFF0000u);
-                        const float c_lo = fmaf(-128.f, s_lo, m_lo), c_hi = fmaf(-128.f, s_hi, m_hi);
-#pragma unroll
-                        for (int i = 0; i < MI; ++i) {
-                            yacc[c * 8 + 2 * q][i] = fmaf(s_lo, acc[q][i], fmaf(c_lo, xs[i], yacc[c * 8 + 2 * q][i]));
-                            yacc[c * 8 + 2 * q + 1][i] = fmaf(s_hi, acc[q + 4][i], fmaf(c_hi, xs[i], yacc[c * 8 + 2 * q + 1][i]));
-                        }
-                    }
-                }
-            }
-        } else {
+        {
             floatx4 xs = floatx4{0.f, 0.f, 0.f, 0.f};
     #pragma unroll
             for (int s = 0; s < KSTEPS; ++s)
@@ -620,35 +566,20 @@ bool stream_attn_fusable(int K, int N, int head_dim, int nsplit) {
     return pl.lw == 2 && pl.ksteps == 2 && pl.waves == 8;   // units of 64 rows: a unit never straddles two heads
 }
 
-template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false, bool AFF = false, bool ATT = false>
+template <int LW, int WB, int KSTEPS, int WAVES, int MI, int NMAT, bool RMS = false, bool ATT = false>
 static hipError_t launch_one(const StreamParams &p, dim3 grid, hipStream_t stream) {
     const size_t lds = (size_t)WAVES * p.M * 8 * LW * 16 * sizeof(float);   // 128 KB at M = 16, LW = 2, 8 waves
     if (lds > 64 * 1024) {   // more than 64 KB of dynamic LDS needs the attribute (per device, so set it every time)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF, ATT>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, ATT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, AFF, ATT>), grid, dim3(WAVES * 64), lds, stream, p);
+    hipLaunchKernelGGL((stream_kernel<LW, WB, KSTEPS, WAVES, MI, NMAT, RMS, ATT>), grid, dim3(WAVES * 64), lds, stream, p);
     return hipGetLastError();
 }
 
 template <int LW, int WB, int KSTEPS, int WAVES>
 static hipError_t launch_mi(int mi, const StreamParams &p, dim3 grid, hipStream_t stream) {
-    if (p.mn[0]) {   // affine codec: only the default launch shape is instantiated
-        if constexpr (LW == 2 && WAVES == 8) {
-            if (p.norm_w)   // M <= 4 checked by the caller
-                return p.nmat == 2 ? launch_one<LW, WB, KSTEPS, WAVES, 1, 2, true, true>(p, grid, stream)
-                                   : launch_one<LW, WB, KSTEPS, WAVES, 1, 1, true, true>(p, grid, stream);
-            if (p.nmat == 2) return launch_one<LW, WB, KSTEPS, WAVES, 1, 2, false, true>(p, grid, stream);
-            switch (mi) {
-                case 1: return launch_one<LW, WB, KSTEPS, WAVES, 1, 1, false, true>(p, grid, stream);
-                case 2: return launch_one<LW, WB, KSTEPS, WAVES, 2, 1, false, true>(p, grid, stream);
-                default: return launch_one<LW, WB, KSTEPS, WAVES, 4, 1, false, true>(p, grid, stream);
-            }
-        } else {
-            return hipErrorInvalidValue;
-        }
-    }
     if (p.norm_w)   // M <= 4 checked by the caller
         return p.nmat == 2 ? launch_one<LW, WB, KSTEPS, WAVES, 1, 2, true>(p, grid, stream)
                            : launch_one<LW, WB, KSTEPS, WAVES, 1, 1, true>(p, grid, stream);
@@ -675,7 +606,7 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
                          uint16_t *y, int M, int K, int N, void *workspace, hipStream_t stream,
                          const StreamExtras &extras) {
     // the chained sums of squares count one float per 256-column tile: those launches keep that shape whatever the tune keys say
-    const StreamPlan pl = plan_stream(M, K, N, extras.mins != nullptr || extras.sumsq_out != nullptr || extras.sumsq_in != nullptr);
+    const StreamPlan pl = plan_stream(M, K, N, extras.sumsq_out != nullptr || extras.sumsq_in != nullptr);
     StreamParams p;
     p.x = x;
     p.qw[0] = reinterpret_cast<const uint32_t *>(qweight);
@@ -685,8 +616,6 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.qw[1] = reinterpret_cast<const uint32_t *>(up_qweight ? up_qweight : qweight);
     p.qz[1] = reinterpret_cast<const uint32_t *>(up_qzeros ? up_qzeros : qzeros);
     p.sc[1] = up_scales ? up_scales : scales;
-    p.mn[0] = extras.mins;
-    p.mn[1] = extras.up_mins ? extras.up_mins : extras.mins;
     p.y = y;
     p.header = reinterpret_cast<uint32_t *>(workspace);
     p.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + kHeaderBytes);
@@ -714,10 +643,10 @@ hipError_t launch_stream(const uint16_t *x, const int32_t *qweight, const int32_
     p.spin_limit = g_stream_tune.spin_limit > 0 ? g_stream_tune.spin_limit : (1 << 18);
     const dim3 grid(((pl.ntiles + 7) / 8) * 8, pl.ksplit, p.nmat);
     if (extras.attn_acc) {   // x comes from the attention partials: one instantiation, shapes checked by stream_attn_fusable
-        if (M != 1 || up_qweight || extras.norm_w || extras.mins || !extras.attn_ml ||
+        if (M != 1 || up_qweight || extras.norm_w || !extras.attn_ml ||
             !stream_attn_fusable(K, N, extras.attn_hd, extras.attn_nsplit))
             return hipErrorInvalidValue;
-        return launch_one<2, 2, 2, 8, 1, 1, false, false, true>(p, grid, stream);
+        return launch_one<2, 2, 2, 8, 1, 1, false, true>(p, grid, stream);
     }
     return pl.lw == 1 ? launch_ksteps<1, 1>(pl.ksteps, pl.waves, pl.mi, p, grid, stream)
                       : launch_ksteps<2, 2>(pl.ksteps, pl.waves, pl.mi, p, grid, stream);

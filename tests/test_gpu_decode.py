@@ -299,19 +299,12 @@ def test_sum_of_squares_chained_into_the_next_norm(ops, n_heads, n_kv, hd, H):
     kc = dev(f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32)))
     vc = dev(f32_to_bf16_bits(rng.standard_normal((n_kv, max_seq, hd)).astype(np.float32)))
     qkv, x_res = dev(make_x(((n_heads + 2 * n_kv) * hd,), seed=3)), dev(make_x((E,), seed=4))
-    for fused_ffn in (1, 0):   # the persistent FFN kernel and the three streaming launches leave the same pieces
-        ops.tune("ffn_fused", fused_ffn)
-        print(f"chained sum of squares E={E} H={H} ffn_fused={fused_ffn}", flush=True)
-        y, sumsq = ops.decode_attn_o_gemv_ffn(qkv, lut[pos], kc.clone(), vc.clone(), pos, n_heads, x_res, norm_w, wo, wg, wu, wd,
-                                              return_sumsq=True)
-        torch.cuda.synchronize()
-        want = (y.float().double() ** 2).reshape(E // 256, 256).sum(dim=1)
-        assert sumsq.shape == (E // 256,) and torch.allclose(sumsq.double(), want, rtol=1e-5, atol=0)
-        if fused_ffn:
-            first = sumsq.clone()
-        else:
-            assert torch.equal(first, sumsq)
-    ops.tune("ffn_fused", 0)
+    print(f"chained sum of squares E={E} H={H}", flush=True)
+    y, sumsq = ops.decode_attn_o_gemv_ffn(qkv, lut[pos], kc.clone(), vc.clone(), pos, n_heads, x_res, norm_w, wo, wg, wu, wd,
+                                          return_sumsq=True)
+    torch.cuda.synchronize()
+    want = (y.float().double() ** 2).reshape(E // 256, 256).sum(dim=1)
+    assert sumsq.shape == (E // 256,) and torch.allclose(sumsq.double(), want, rtol=1e-5, atol=0)
     # 128-column tiles (tuning key) must not change the chain: launches that leave or take sums of squares keep
     # their 256-column tiles, one float per tile in a buffer of E / 256
     ops.tune("gemv_lw", 1)

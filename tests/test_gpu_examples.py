@@ -1,6 +1,7 @@
 """GPU: the example entry points end to end (PASS! harness), the golden fixtures, full-size
 properties, and the host-forced failure path of the split-K reducer."""
 import os
+import sys
 
 import numpy as np
 import pytest
@@ -199,28 +200,68 @@ def test_reducer_timeout_is_reported_and_workspace_recovers():
     assert torch.equal(ops.w4a16_gemv(x, *w).view(torch.int16), good.view(torch.int16))
 
 
-def test_reducer_timeout_surfaces_as_backend_error():
-    """Through the backend interface the same failure is an AirBackendError at the invoker's read-back."""
+def test_backend_runs_the_stream_order_kernels_and_reports_library_errors():
+    """HIPBackend re-packs its weight buffers into stream order and runs the whole-K / tiled stream-order kernels: its
+    outputs equal the stream-order ops bit for bit; an error code from the library is an AirBackendError."""
     from air_hip import awq, bf16, ops
     from air_hip.backend import AirBackendError, HIPBackend, HipModule
-    print("reducer timeout through HIPBackend", flush=True)
+    print("HIPBackend on stream-order kernels", flush=True)
     K, N = 4096, 1024
     qw, qz, s = make_awq(K, N, seed=23)
     x = make_x((K,), seed=24)
     backend = HIPBackend()
     invoker = backend.compile_and_load(HipModule("matvec_int4", K=K, N=N, gs=128))
     args = (awq.pack_buffer(qw, qz, bf16.from_bits(s)), bf16.from_bits(x), np.zeros(N, np.uint16).view(bf16.BF16Array))
-    good = invoker(*args)[-1]
-    try:
-        ops.tune("gemv_skip_publish", 1)
-        ops.tune("gemv_spin_limit", 8)
-        with pytest.raises(AirBackendError):
-            invoker(*args)
-    finally:
-        ops.tune("gemv_skip_publish", 0)
-        ops.tune("gemv_spin_limit", 0)
-    assert np.array_equal(np.asarray(invoker(*args)[-1]).view(np.uint16), np.asarray(good).view(np.uint16))
+    got = np.asarray(invoker(*args)[-1]).view(np.uint16)
+    want = bits(ops.w4a16_gemv_stream(dev(x), ops.repack_stream(dev(qw), dev(qz), dev(s))))
+    assert np.array_equal(got, want)
     backend.unload()
+    xm = make_x((32, K), seed=25)
+    invoker = backend.compile_and_load(HipModule("matmul_int4", M=32, K=K, N=N, gs=128))
+    got = np.asarray(invoker(bf16.from_bits(xm), args[0], np.zeros((32, N), np.uint16).view(bf16.BF16Array))[-1]).view(np.uint16)
+    want = bits(ops.w4a16_gemm_stream(dev(xm), ops.repack_stream(dev(qw), dev(qz), dev(s))))
+    assert np.array_equal(got, want)
+    with pytest.raises(AirBackendError):
+        invoker(bf16.from_bits(xm), args[0])   # no output placeholder
+    backend.unload()
+
+
+@pytest.mark.parametrize("example,argv", [
+    ("matvec_int4_packed", ["--m", "2048", "--k", "2048"]),
+    ("matvec_int4_packed_add", ["--m", "1024", "--k", "2048"]),
+    ("matmul_int4_packed", ["--m", "2048", "--k", "2048", "--n", "2048"]),
+    ("matmul_int4_packed", []),
+    ("matvec_int4_swiglu_rms", ["--m", "4096", "--k", "2048"]),
+    ("o_gemv_ffn_int4", ["--emb-dim", "1024", "--hidden-dim", "4096"]),
+    ("dequant_awq", []),
+])
+def test_examples_run_as_scripts(example, argv, tmp_path, capsys, monkeypatch):
+    """`python -m air_hip.examples.<name> <the reference's flags> --expected file.npz` prints PASS! and exits 0, the
+    expected output written beforehand by tests/golden/make_expected.py (the reference's examples end in
+    exit(runner.run_test(...)), matvec_int4_packed.py:376)."""
+    import runpy
+    sys.path.insert(0, G)
+    try:
+        import make_expected
+    finally:
+        sys.path.remove(G)
+    print("script", example, argv, flush=True)
+    path = make_expected.write_expected(example, argv, str(tmp_path / "expected.npz"))
+    monkeypatch.setattr(sys, "argv", [example + ".py", *argv, "--expected", path])
+    with pytest.raises(SystemExit) as e:
+        runpy.run_module(f"air_hip.examples.{example}", run_name="__main__")
+    assert e.value.code == 0
+    assert "PASS!" in capsys.readouterr().out
+    # a file computed for other arguments is refused
+    import importlib
+    from air_hip.examples import _common
+    ex = importlib.import_module(f"air_hip.examples.{example}")
+    if _common.params_of(ex.parse_args(argv)) != _common.params_of(ex.parse_args([])):
+        monkeypatch.setattr(sys, "argv", [example + ".py", "--expected", path])
+        with pytest.raises(SystemExit) as e:
+            runpy.run_module(f"air_hip.examples.{example}", run_name="__main__")
+        assert e.value.code == 2
+        capsys.readouterr()
 
 
 def test_hip_graph_replay_matches_eager():

@@ -172,8 +172,7 @@ def test_argument_errors(ops):
     lib = _lib.load_library()
     assert lib.q4nx_repack(None, None, None, None, 32, 256, 0, None) == _lib.ERR_NULL
     assert lib.q4nx_dequant_bf16(blocks.data_ptr(), blocks.data_ptr(), 48, 256, 0, None) == _lib.ERR_SHAPE
-    assert lib.w4a16_q4nx_gemm_bf16(blocks.data_ptr(), blocks.data_ptr(), blocks.data_ptr(), blocks.data_ptr(), None,
-                                    blocks.data_ptr(), 1, 128, 32, None, 0, None) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_q4nx_gemm_stream_bf16(blocks.data_ptr(), blocks.data_ptr(), None, blocks.data_ptr(), 1, 128, 24, None) == _lib.ERR_SHAPE
 
 
 # ---- decode-layer entry points on the affine codec ----
@@ -263,7 +262,7 @@ def test_decode_block_q4nx_matches_the_oracle_chain(ops):
          "gate": qw(H, E, 5), "up": qw(H, E, 6), "down": qw(E, H, 7)}
     attn_norm, ffn_norm = _norm_w(E, 8), _norm_w(E, 9)
     layer = decode.prepare_layer_q4nx({k: oq.pack_matrix(*v) for k, v in w.items()}, attn_norm, ffn_norm, cfg)
-    assert layer.codec == "q4nx" and layer.wqkv[0].shape == (E, (nq + 2 * nkv) // 8)
+    assert layer.codec == "q4nx" and layer.wqkv is None and (layer.stream["wqkv"].K, layer.stream["wqkv"].N) == (E, nq + 2 * nkv)
     lut_bits = odec.generate_rope_lut(cfg.head_dim, cfg.rope_base, max_seq)
     lut = decode.generate_rope_lut(cfg, max_seq)
     (kc, vc), = decode.new_kv_cache(cfg, max_seq)
@@ -328,15 +327,9 @@ def test_stream_gemv_other_conventions(ops, mode):
     _stream_gemv_case(ops, 2048, 2048, seed=30 + mode, mode=mode)
 
 
-def test_stream_gemv_with_residual_and_against_the_planar_path(ops):
-    """Residual add; and the stream-order kernel against the kernel on q4nx_repack's own operands: two summation orders
-    of the same fp32 terms, at most an ulp apart, mostly equal."""
-    got, (qw, sc, mn), x = _stream_gemv_case(ops, 4096, 4096, seed=40, residual=False)
+def test_stream_gemv_with_residual(ops):
+    _stream_gemv_case(ops, 4096, 4096, seed=40, residual=False)
     _stream_gemv_case(ops, 1024, 512, seed=41, residual=True)
-    planar = bits(ops.q4nx_gemm(dev(x), qw, sc, mn))[0]
-    from helpers import bf16_ulp
-    a, b = bf16_bits_to_f32(got).astype(np.float64), bf16_bits_to_f32(planar).astype(np.float64)
-    assert np.all(np.abs(a - b) <= bf16_ulp(b) + 1e-3) and np.mean(got != planar) < 0.2, (np.abs(a - b).max(), np.mean(got != planar))
 
 
 @pytest.mark.parametrize("rows,M,K,residual", [(2, 512, 1024, False), (16, 512, 1024, True), (7, 64, 256, False), (17, 1024, 512, True),
@@ -493,41 +486,3 @@ def test_stream_entry_points_reject_bad_arguments(ops):
     assert lib.w4a16_q4nx_rms_gemv_stream_bf16(P, None, 0, None, 1e-5, P, P, 256, 32, None) == _lib.ERR_NULL
     ws = lib.w4a16_block_stream_workspace_bytes(256, 256)
     assert lib.w4a16_q4nx_o_gemv_ffn_stream_bf16(P, P, P, 1e-5, P, P, P, P, P, None, None, None, 256, 256, P, ws - 1, None) == _lib.ERR_WORKSPACE
-
-
-def test_decode_block_q4nx_stream_order_agrees_with_the_planar_layer(ops):
-    """run_decode_block on a Q4NX layer with and without the stream-order re-pack: same caches, outputs an ulp or
-    two apart (another summation order in every GEMV)."""
-    from air_hip import decode, weights
-    cfg = weights.LlamaConfig(n_layers=1, emb_dim=512, n_heads=8, head_dim=64, n_kv_heads=2, hidden_dim=1024, vocab_size=32)
-    E, H, nq, nkv = cfg.emb_dim, cfg.hidden_dim, cfg.n_heads * cfg.head_dim, cfg.kv_dim
-
-    def qw(M, K, seed):
-        rng = np.random.default_rng(seed)
-        W = (rng.standard_normal((M, K)) * 0.02).astype(np.float32)
-        q, sc, mn = oq.requant_q4k(W)
-        return q, f32_to_bf16_bits(sc), f32_to_bf16_bits(mn)
-
-    w = {"q": qw(nq, E, 1), "k": qw(nkv, E, 2), "v": qw(nkv, E, 3), "o": qw(E, nq, 4),
-         "gate": qw(H, E, 5), "up": qw(H, E, 6), "down": qw(E, H, 7)}
-    blocks = {k: oq.pack_matrix(*v) for k, v in w.items()}
-    attn_norm, ffn_norm = _norm_w(E, 8), _norm_w(E, 9)
-    planar = decode.prepare_layer_q4nx(blocks, attn_norm, ffn_norm, cfg, stream_order=False)
-    stream = decode.prepare_layer_q4nx(blocks, attn_norm, ffn_norm, cfg)
-    assert stream.stream is not None and planar.stream is None
-    max_seq = 64
-    lut = decode.generate_rope_lut(cfg, max_seq)
-    (kc1, vc1), = decode.new_kv_cache(cfg, max_seq)
-    (kc2, vc2), = decode.new_kv_cache(cfg, max_seq)
-    for pos in range(4):
-        print(f"q4nx decode block, stream order against planar, pos={pos}", flush=True)
-        x = dev(_vec(E, 600 + pos))
-        y1 = decode.run_decode_block(x, planar, cfg, kc1, vc1, pos, lut)
-        y2, sumsq = decode.run_decode_block(x, stream, cfg, kc2, vc2, pos, lut, return_sumsq=True)
-        torch.cuda.synchronize()
-        err = (y1.float() - y2.float()).abs().max().item()
-        assert err <= 4 * 2.0**-8 * y1.float().abs().max().item(), err
-        kerr = (kc1[:, pos].float() - kc2[:, pos].float()).abs().max().item()
-        assert kerr <= 2 * 2.0**-8 * kc1[:, pos].float().abs().max().item() + 1e-2, kerr
-        assert sumsq is not None and sumsq.numel() == E // 16
-        kc2[:, pos], vc2[:, pos] = kc1[:, pos], vc1[:, pos]

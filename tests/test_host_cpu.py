@@ -101,6 +101,37 @@ def test_examples_draw_order_and_packing():
     assert np.array_equal(wo[0], q[:, 0::2] | (q[:, 1::2] << 4))
 
 
+def test_example_scripts_cli_without_a_gpu(tmp_path, capsys):
+    """The stand-alone entry points: -p prints the module, compile-only validates it, a run without --expected or with
+    a file written for other arguments returns 2 before anything touches the GPU."""
+    import json
+    import sys
+    from air_hip.examples import _common
+    assert matvec_int4_packed.main(["-p", "--m", "256", "--k", "512"]) == 0
+    assert "hip.module @matvec_int4 {M = 1, K = 512, N = 256, gs = 128}" in capsys.readouterr().out
+    assert matmul_int4_packed.main(["--compile-mode", "compile-only", "--output-format", "xclbin"]) == 0
+    with pytest.raises(AirBackendError):
+        matvec_int4_packed.main(["--compile-mode", "compile-only", "--k", "100"])
+    assert o_gemv_ffn_int4.main([]) == 2
+    assert "--expected" in capsys.readouterr().err
+    args = dequant_awq.parse_args(["--n", "256"])
+    path = str(tmp_path / "e.npz")
+    _common.save_expected(path, args, np.zeros(256, np.uint16))
+    with np.load(path) as f:
+        assert json.loads(str(f["params"])) == {"group_size": 128, "herd_n": 4, "n": 256}
+    assert dequant_awq.main(["--n", "512", "--expected", path]) == 2
+    assert "was computed for" in capsys.readouterr().err
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
+    try:
+        import make_expected
+    finally:
+        sys.path.pop(0)
+    path = make_expected.write_expected("matvec_int4_packed", ["--m", "64", "--k", "256"], str(tmp_path / "m.npz"))
+    a_q, a_s, a_z, b = matvec_int4_packed.draw_inputs(matvec_int4_packed.parse_args(["--m", "64", "--k", "256"]))
+    with np.load(path) as f:
+        assert np.array_equal(f["expected"], oref.matvec_cpu_reference_loop(a_q, bf16.bits_of(a_s), a_z, bf16.bits_of(b)))
+
+
 def test_runner_comparator_semantics_match_reference_restatement(capsys):
     r = HIPRunner()
     e = np.linspace(1, 2, 1000)
