@@ -294,7 +294,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                 launch(i, stream.cuda_stream)
 
     def timed_graph(indices):
-        """Capture len(indices) launches into one HIP graph, replay it once between events."""
+        """Capture len(indices) launches into one HIP graph; behind a spinning kernel, replay it twice and time the
+        second replay (the first is the warm-up that the eager timing gets from its untimed rotation)."""
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(stream):
             with torch.cuda.graph(graph, stream=stream):
@@ -307,6 +308,9 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             e1 = torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
+            torch.cuda._sleep(int(2e5) * 16)
+            graph.replay()
+            spacers(indices)
             e0.record(stream)
             graph.replay()
             e1.record(stream)

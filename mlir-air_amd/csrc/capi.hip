@@ -921,6 +921,9 @@ int w4a16_tune(const char *key, int value) {
     } else if (!strcmp(key, "prefill_swiglu_split")) {
         if (value != 0 && value != 1) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.prefill_swiglu_split = value;
+    } else if (!strcmp(key, "prefill_band")) {
+        if (value > 64) return W4A16_ERR_TUNE;
+        g_gemv_ws_tune.prefill_band = value;
     } else if (!strcmp(key, "prefill_min_m")) {
         g_gemv_ws_tune.prefill_min_m = value;
     } else if (!strcmp(key, "gemm_ws_rows")) {

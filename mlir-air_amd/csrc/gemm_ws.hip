@@ -179,6 +179,7 @@ struct PfArgs {
     const char *w_up;       // kEpiSwigluPair: the second matrix (the tile's left half multiplies w, its right half w_up)
     int epi;                // kEpi*, or kEpiSwigluPair
     int rope_cols, rope_hd, rope_pos0;
+    int band;               // row panels per band of the tile order (pf_tile_of)
 };
 
 // One output tile: rows m0 .., columns col0 .. col0 + 64 NCB - 1.
@@ -261,7 +262,8 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     };
     auto load_w_tile = [&](int set, const WOffsets &o, int c) {
         md[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(tile_base[c] + o.md);
-        cell[set][c] = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(tile_base[c] + o.cell));
+        // (a plain load: the workgroups of the same band and column tile on this XCD read the same cells out of its L2)
+        cell[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(tile_base[c] + o.cell);
     };
     // The compiler does not see the explicit s_waitcnt below: with loads in flight it would wait for vmcnt(0) at the
     // first use of a register loaded a group earlier, i.e. right behind the requests for the next group, and expose
@@ -487,7 +489,7 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
                     else v[e] = pack_bf16x2(a0 / (1.0f + expf(-a0)) * v0, a1 / (1.0f + expf(-a1)) * v1);
                 }
             }
-            *reinterpret_cast<u32x4 *>(p.y + at) = v;
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p.y + at));   // y is not read again here: keep x and W in L2
         }
     };
     if (pair) {
@@ -515,9 +517,19 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     else store_tile(std::integral_constant<int, kEpiNone>{});
 }
 
+// Tile order of one width: the row panels are cut into bands of `band` panels; inside a band the order runs down the
+// band's panels first, then to the next column tile.  An XCD takes a contiguous range of that order, so the
+// workgroups that run together on it cover band x (32 / band) tiles: they share `band` x panels and 32 / band weight
+// slabs in its L2, and over the launch a weight slab is fetched by tiles_m / band XCDs instead of by every one.
+__device__ __forceinline__ void pf_tile_of(int idx, int tiles_m, int n_cols, int band, int &row, int &col) {
+    const int per_band = band * n_cols, b = idx / per_band, r = idx - b * per_band;
+    const int rows = min(band, tiles_m - b * band);   // (the last band may be short)
+    row = b * band + r % rows;
+    col = r / rows;
+}
+
 // blockIdx -> tile.  The wide tiles come first in dispatch order, so that the narrow ones fill in behind them.  Each
-// XCD (blockIdx % 8) takes a contiguous range of the tiles of either width with N fastest: the workgroups that run
-// together on an XCD share one x panel in its L2 while the weight panels stream by.
+// XCD (blockIdx % 8) takes a contiguous range of the tiles of either width in the order of pf_tile_of.
 template <int NW, int NN>
 __global__ void __launch_bounds__(kPfThreads, 1) gemm_wsp_kernel(const PfArgs p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -527,11 +539,15 @@ __global__ void __launch_bounds__(kPfThreads, 1) gemm_wsp_kernel(const PfArgs p)
     if (slot < wide_per_xcd) {
         const int tile = xcd * wide_per_xcd + slot;
         if (tile >= wide_total) return;
-        pf_tile<NW>(p, lds, (tile / p.n_wide) * kPfRows, (tile % p.n_wide) * 64 * NW);
+        int row, col;
+        pf_tile_of(tile, p.tiles_m, p.n_wide, p.band, row, col);
+        pf_tile<NW>(p, lds, row * kPfRows, col * 64 * NW);
     } else if constexpr (NN > 0) {
         const int tile = xcd * narrow_per_xcd + (slot - wide_per_xcd);
         if (tile >= narrow_total) return;
-        pf_tile<NN>(p, lds, (tile / p.n_narrow) * kPfRows, p.n_wide * 64 * NW + (tile % p.n_narrow) * 64 * NN);
+        int row, col;
+        pf_tile_of(tile, p.tiles_m, p.n_narrow, p.band, row, col);
+        pf_tile<NN>(p, lds, row * kPfRows, p.n_wide * 64 * NW + col * 64 * NN);
     }
 }
 
@@ -605,6 +621,15 @@ Widths pick_widths(int tiles_m, int U, int cus, bool heads128) {
     return best;
 }
 
+// Row panels per band.  Fetch traffic of a launch over 8 XCDs is about (tiles_m / band) x the weights + 2 band x the
+// activations (a wide and a narrow pass): least at band 2 to 4 for M = 2048, N = 14336.  Measured there (us per launch,
+// two boxes): band 1 205 / -, 2 198 / 192, 4 194 / 191, 8 196 / -; with plain instead of non-temporal cell loads and
+// non-temporal stores of y on top: band 2 182, band 4 183 - 187.
+int pf_band(int tiles_m) {
+    const int want = g_gemv_ws_tune.prefill_band ? g_gemv_ws_tune.prefill_band : 2;
+    return want < tiles_m ? want : tiles_m;
+}
+
 template <int NW, int NN>
 hipError_t launch_wsp(const PfArgs &p, hipStream_t stream) {
     constexpr size_t kStages = 2 * (size_t)kPfRows * 256, kOut = (size_t)kPfRows * (64 * NW + 8) * sizeof(uint16_t);
@@ -639,6 +664,7 @@ hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y,
     const bool heads128 = epi == kEpiRope && rope->head_dim == 128;
     p.M = M, p.K = K, p.N = N, p.G = K / kGroup, p.NB = ws_blocks(K);
     p.tiles_m = (M + kPfRows - 1) / kPfRows;
+    p.band = pf_band(p.tiles_m);
     const int U = N / 64;
     Widths wd = pick_widths(p.tiles_m, U, 256, heads128);
     // tuning: one tile width only (1: 256 columns, 2: 192, 3: 128, 4: 64) where it divides N; 5: 256 mixed with 128
@@ -673,6 +699,7 @@ hipError_t launch_gemm_prefill_ws_swiglu(const uint16_t *x, const void *w_gate, 
     p.epi = kEpiSwigluPair;
     p.M = M, p.K = K, p.N = H, p.G = K / kGroup, p.NB = ws_blocks(K);
     p.tiles_m = (M + kPfRows - 1) / kPfRows;
+    p.band = pf_band(p.tiles_m);
     const int U = 2 * H / 64;   // the tile grid runs over 2 H columns; 192- and 64-column tiles cannot be halved
     Widths wd = pick_widths(p.tiles_m, U, 256, true);
     const int force = g_gemv_ws_tune.prefill_tile;

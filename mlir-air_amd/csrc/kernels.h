@@ -107,6 +107,7 @@ struct GemvWsTune {
     int prefill_tile = 0;    // prefill kernel: 0 = by shape, 1 = 128 x 448 tiles, 2 = 256 x 256 tiles
     int gemm_rows = 0;       // batched kernel: most rows per launch, 16, 32 or 64 (0 = 64)
     int prefill_min_m = 0;   // smallest M that w4a16_gemm_stream_bf16 gives to the prefill kernel (0 = default)
+    int prefill_band = 0;    // prefill kernel: row panels per band of the tile order (0 = default)
     int prefill_swiglu_split = 0;   // 1: the prompt-pass FFN runs gate and up as two launches instead of one
 };
 extern GemvWsTune g_gemv_ws_tune;
