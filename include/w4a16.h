@@ -42,6 +42,7 @@ extern "C" {
 #define W4A16_ERR_TUNE (-7)        /* unknown tuning key or value out of range */
 #define W4A16_ERR_TIMEOUT (-8)     /* w4a16_workspace_check: a split-K reducer timed out */
 #define W4A16_ERR_TOO_LARGE (-9)   /* w4a16_gemv_noalloc_bf16: shape beyond its fixed scratch */
+#define W4A16_ERR_NOT_PREPARED (-10) /* w4a16_gemv_noalloc_bf16: first use on this GPU under stream capture */
 
 #define W4A16_ABI_VERSION 1
 
@@ -113,12 +114,20 @@ int w4a16_gemv_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qz
  * tight serving loops, harnesses that forbid hipMalloc).  The split-K partial slots live in a 4.06 MiB
  * device array inside the library (one copy per GPU, held until the process ends), so N <= 32768
  * (W4A16_ERR_TOO_LARGE beyond); other constraints, kernels and results are those of w4a16_gemv_bf16,
- * bit for bit.  The first call on a GPU prepares the array with a fill kernel on `stream`.  Every
- * call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two
- * threads) race, exactly as two calls sharing one workspace would.
+ * bit for bit.  The first use on a GPU prepares the array (a fill kernel on `stream`, waited for before
+ * anything else may see the array), which a capturing stream cannot do: a first use under stream capture
+ * returns W4A16_ERR_NOT_PREPARED and launches nothing; call w4a16_noalloc_check once per GPU outside
+ * capture beforehand.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU
+ * (two streams, two threads) race, exactly as two calls sharing one workspace would.
+ *
+ * w4a16_noalloc_check(stream) is w4a16_workspace_check for that array (it synchronises `stream`, so not
+ * under capture): it prepares the array if this GPU has not used it yet, returns W4A16_ERR_TIMEOUT if a
+ * reducer of an earlier w4a16_gemv_noalloc_bf16 call gave up waiting (that call's output is invalid) and
+ * then empties the array again, so that the next call is sound; W4A16_OK otherwise.  Allocates nothing.
  */
 int w4a16_gemv_noalloc_bf16(const uint16_t *x, const int32_t *qweight, const int32_t *qzeros,
                             const uint16_t *scales, uint16_t *y, int K, int N, int group, void *stream);
+int w4a16_noalloc_check(void *stream);
 
 /*
  * GEMM, any M >= 1: y[M, N] = bf16(x[M, K] . W).  M <= 16 streams the weights once

@@ -7,7 +7,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libw4a16_hip.so")
 
 OK = 0
-ERR_NULL, ERR_SHAPE, ERR_GROUP, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_TUNE, ERR_TIMEOUT, ERR_TOO_LARGE = -1, -2, -3, -4, -5, -6, -7, -8, -9
+ERR_NULL, ERR_SHAPE, ERR_GROUP, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_TUNE, ERR_TIMEOUT, ERR_TOO_LARGE, ERR_NOT_PREPARED = -1, -2, -3, -4, -5, -6, -7, -8, -9, -10
 
 # every symbol include/w4a16.h declares: name -> (restype, argtypes)
 _vp, _ci, _sz, _cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_float
@@ -67,6 +67,7 @@ SYMBOLS = {
     "w4a16_o_gemv_ffn_stream_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 8 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_decode_attn_o_gemv_ffn_stream_bf16": (_ci, [_vp] * 5 + [_ci] * 5 + [_vp, _sz, _vp, _vp, _cf] + [_vp] * 6 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_gemv_noalloc_bf16": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a16_noalloc_check": (_ci, [_vp]),
     "w4a16_tune": (_ci, [ctypes.c_char_p, _ci]),
 }
 

@@ -67,10 +67,33 @@ def check_health():
         if lib.w4a16_workspace_check(_ptr(ws), None) == _lib.ERR_TIMEOUT:
             _lib.check(lib.w4a16_workspace_init(_ptr(ws), ws.numel(), None))
             failed.append(key)
+    if _noalloc_used and lib.w4a16_noalloc_check(None) == _lib.ERR_TIMEOUT:   # (the array inside the library)
+        failed.append((None, None, "no-alloc array"))
     if failed:
         torch.cuda.synchronize()
         raise _lib.W4A16Error(_lib.ERR_TIMEOUT, "a split-K reducer gave up waiting for a partial result; the outputs of the calls "
                               f"since the last check are invalid (workspaces {[k[2] for k in failed]} re-initialised)")
+
+
+_noalloc_used = False
+
+
+def w4a16_gemv_noalloc(x, qweight, qzeros, scales, group=GROUP, out=None):
+    """w4a16_gemv on the library's own split-K array (w4a16_gemv_noalloc_bf16): no workspace from this module.
+    check_health() looks at that array as well once this has been called."""
+    global _noalloc_used
+    lib = _lib.load_library()
+    _need_cuda(x, qweight, qzeros, scales)
+    K, N = x.numel(), qweight.shape[1] * 8
+    if qweight.shape[0] != K:
+        raise ValueError(f"x has K={K} but qweight has {qweight.shape[0]} rows")
+    if out is None:
+        out = torch.empty((N,), dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.w4a16_gemv_noalloc_bf16(_ptr(_bits(x)), _ptr(qweight), _ptr(qzeros), _ptr(_bits(scales)), _ptr(out), K, N,
+                                           group, _stream()))
+    _noalloc_used = True
+    _after_workspace_call()
+    return out
 
 
 def set_checked(on):

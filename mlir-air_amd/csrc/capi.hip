@@ -168,6 +168,8 @@ const char *w4a16_strerror(int code) {
         case W4A16_ERR_TUNE: return "unknown tuning key or value out of range";
         case W4A16_ERR_TIMEOUT: return "a split-K reducer gave up waiting for a partial result; the output is invalid";
         case W4A16_ERR_TOO_LARGE: return "shape beyond the fixed scratch of the entry point that allocates nothing (N <= 32768)";
+        case W4A16_ERR_NOT_PREPARED:
+            return "first use of the entry point that allocates nothing on this GPU under stream capture: call w4a16_noalloc_check outside capture first";
         default: return "unknown error code";
     }
 }
@@ -272,10 +274,13 @@ constexpr int kNoAllocMaxN = 32768;
 constexpr size_t kNoAllocScratchBytes = kHeaderBytes + (size_t)kMaxKSplit * (kNoAllocMaxN + 512) * sizeof(float);   // 4.06 MiB
 static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 
-void *g_scratch_ptr[64] = {nullptr};   // per device: address of `scratch` there, set once the array is prepared
+void *g_scratch_ptr[64] = {nullptr};   // per device: address of `scratch` there, published once the array is prepared
 std::mutex g_scratch_mutex;
 
-// Address of this device's copy of `scratch`, prepared (header zero, every slot empty) on first use.
+// Address of this device's copy of `scratch`.  On first use the array is prepared (header zero, every slot empty) and
+// the fill has FINISHED before the address is published: a zero-initialised array is not an empty one, so no launch
+// on any stream may see it earlier.  That needs a synchronisation, which a capturing stream cannot give: the first
+// use under capture returns W4A16_ERR_NOT_PREPARED instead (w4a16_noalloc_check prepares the array ahead of it).
 int noalloc_scratch(hipStream_t st, void **out) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -283,16 +288,29 @@ int noalloc_scratch(hipStream_t st, void **out) {
     if (dev < 0 || dev >= 64) return W4A16_ERR_SHAPE;
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (!g_scratch_ptr[dev]) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(st, &cap);
+        if (e != hipSuccess) return hip_fail(e);
+        if (cap != hipStreamCaptureStatusNone) return W4A16_ERR_NOT_PREPARED;
         void *ptr = nullptr;
         e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return hip_fail(e);
         if (!ptr) return W4A16_ERR_NULL;
-        e = launch_fill_workspace(ptr, kNoAllocScratchBytes, st);   // a fill kernel, not a memset: safe under graph capture
+        e = launch_fill_workspace(ptr, kNoAllocScratchBytes, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return hip_fail(e);
         g_scratch_ptr[dev] = ptr;
     }
     *out = g_scratch_ptr[dev];
     return W4A16_OK;
+}
+
+// tests only (w4a16_tune("noalloc_forget", 1)): the next use on the current device prepares the array again
+void noalloc_forget() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    g_scratch_ptr[dev] = nullptr;
 }
 }  // namespace
 
@@ -313,6 +331,20 @@ int w4a16_gemv_noalloc_bf16(const uint16_t *x, const int32_t *qweight, const int
     if (rc) return rc;
     hipError_t e = launch_stream(x, qweight, qzeros, scales, nullptr, nullptr, nullptr, y, 1, K, N, ws, st);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
+int w4a16_noalloc_check(void *stream) {
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    void *ws = nullptr;
+    int rc = noalloc_scratch(st, &ws);   // prepares the array on first use (not under capture)
+    if (rc) return rc;
+    rc = w4a16_workspace_check(ws, stream);
+    if (rc == W4A16_ERR_TIMEOUT) {   // slots filled late are dirty: empty the array again before the next call
+        hipError_t e = launch_fill_workspace(ws, kNoAllocScratchBytes, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess) return hip_fail(e);
+    }
+    return rc;
 }
 
 int w4a16_gemv_swiglu_bf16(const uint16_t *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
@@ -935,6 +967,8 @@ int w4a16_tune(const char *key, int value) {
     } else if (!strcmp(key, "gemv_ws_waves")) {
         if (value > 16) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.waves = value;
+    } else if (!strcmp(key, "noalloc_forget")) {
+        noalloc_forget();
     } else if (!strcmp(key, "gemv_ksplit")) {
         if (value > kMaxKSplit) return W4A16_ERR_TUNE;
         g_stream_tune.ksplit = value;
