@@ -675,7 +675,7 @@ def main():
                     help="also launch one device copy of 256 MiB (a dispatch of known traffic that calibrates "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
-                    help="set a library tuning key (w4a16_tune) before the run, e.g. --tune colgemv=1; repeatable")
+                    help="set a library tuning key (w4a16_tune) before the run, e.g. --tune gemv_ws_ct=16; repeatable")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures the single-GPU W4A16 kernels; --gpus must be 1 "

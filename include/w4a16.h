@@ -222,7 +222,11 @@ int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uin
  * M = 129 on,
  * with K % 256 == 0 and N % 64 == 0 (N / 64 = 3, 4 or >= 6), the tiled prefill kernel runs instead: it dequantises the
  * weights to bf16 in registers (W = bf16_rne((q - z) * s), the dense dequant's values) and feeds bf16 MFMA with fp32
- * accumulation; other shapes stay with the launches of 64 rows.  K % 128 == 0, N % 16 == 0. */
+ * accumulation; other shapes stay with the launches of 64 rows.  So the numerics change between M = 128 and M = 129:
+ * below, y is one rounding of the fp32 sum over exact weights (q - z) s, as the reference's cpu_reference computes it;
+ * above, the weights carry one more bf16 rounding each (relative 2^-9), which moves y by at most 2^-9 sum |x w| and
+ * stays inside the reference's gate (rtol 0.1, atol 0.05, 0.05 % budget, r >= 0.999); a caller that needs the same
+ * bits for every M keeps M <= 128 per call.  K % 128 == 0, N % 16 == 0. */
 int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int M, int K, int N, int group,
                            void *stream);
 int w4a16_gemv_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream,

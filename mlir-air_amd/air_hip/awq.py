@@ -65,6 +65,32 @@ def l1_from_awq(qweight, qzeros, scales):
     return A_q, bf16.from_bits(bf16.bits_of(scales)), z
 
 
+def fake_quantize_awq_int4(W_bf16, gs=GROUP):
+    """Asymmetric uint4 quantisation per group of `gs` input features of a weight [M, K] (bf16 bits or floats),
+    the quantiser of the stand-alone GEMM example (fake_quantize_awq_int4,
+    programming_examples/llms/llama32_1b_int4/awq_pack.py:287-316): per (row, group) scale = (max - min) / 15 in
+    float32 (1e-7 for a constant group), zero = round(-min / scale) clipped to 0..15, q = round(w / scale + zero)
+    clipped likewise.  Returns the kernel-side arrays pack_inputs takes: W_q u8 [M, K / 2] (even k in the low nibble),
+    W_s bf16 [K / gs, M], W_z u8 [K / gs, M]."""
+    W = bf16.to_f32(bf16.bits_of(W_bf16)) if bf16.is_bf16(W_bf16) or np.asarray(W_bf16).dtype == np.uint16 else np.asarray(W_bf16, np.float32)
+    M, K = W.shape
+    if K % gs:
+        raise ValueError(f"K={K} not divisible by gs={gs}")
+    grouped = W.reshape(M, K // gs, gs)
+    lo, hi = grouped.min(axis=2), grouped.max(axis=2)
+    scale = ((hi - lo) / np.float32(15.0)).astype(np.float32)
+    scale[scale == 0] = np.float32(1e-7)
+    zero = np.clip(np.round(-lo / scale), 0, 15).astype(np.uint8)
+    q = np.clip(np.round(grouped / scale[:, :, None] + zero.astype(np.float32)[:, :, None]), 0, 15).astype(np.uint8).reshape(M, K)
+    return pack_l1_nibbles(q), bf16.from_f32(scale.T), np.ascontiguousarray(zero.T)
+
+
+def pack_l1_nibbles(q):
+    """nibbles u8 [M, K] -> u8 [M, K / 2], even k in the low nibble (the kernel-side A_q of the examples)."""
+    q = np.asarray(q, dtype=np.uint8)
+    return (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)
+
+
 def interleave_rows(gate, up):
     """Row-interleave two kernel-side weight triples (row 2i = gate[i], 2i+1 = up[i]),
     the layout of the decode FFN front half (llama32_1b_int4_weights.py:173-207)."""

@@ -123,16 +123,17 @@ def load_weights_awq(model_name_or_path, config: Optional[LlamaConfig] = None, g
     if config is None:
         config = LlamaConfig()
     files = resolve_safetensor_files(model_name_or_path)
-    key_to_file = {}
+    shard_of = {}   # tensor name -> the shard that holds it
     for path in files:
         with safe_open(path, framework="pt") as f:
-            for key in f.keys():
-                key_to_file[key] = path
+            shard_of.update((key, path) for key in f.keys())
 
     def tensor(key, what="weight"):
-        if key not in key_to_file:
-            raise KeyError(f"Missing {what}: {key}" + (" (is this an AutoAWQ checkpoint?)" if what == "AWQ tensor" else ""))
-        with safe_open(key_to_file[key], framework="pt") as f:
+        path = shard_of.get(key)
+        if path is None:
+            hint = "; the directory holds no qweight / qzeros / scales triple under that name, so it was not written by AutoAWQ" if what == "AWQ tensor" else ""
+            raise KeyError(f"{what} {key} is in none of the {len(files)} safetensors shard(s){hint}")
+        with safe_open(path, framework="pt") as f:
             return f.get_tensor(key)
 
     embed_table = _bf16_bits(tensor("model.embed_tokens.weight"))
@@ -163,7 +164,7 @@ def load_weights_awq(model_name_or_path, config: Optional[LlamaConfig] = None, g
         layers.append(LayerWeights(**fields))
 
     final_norm = _bf16_bits(tensor("model.norm.weight"))
-    lm_head = _bf16_bits(tensor("lm_head.weight")) if "lm_head.weight" in key_to_file else embed_table
+    lm_head = _bf16_bits(tensor("lm_head.weight")) if "lm_head.weight" in shard_of else embed_table
     return LlamaWeights(embed_table=embed_table, layers=layers, final_norm=final_norm, lm_head=lm_head)
 
 

@@ -121,6 +121,36 @@ def l1_to_awq(a_q, a_s_bits, a_z):
     return qweight, qzeros, np.ascontiguousarray(a_s_bits).astype(np.uint16)
 
 
+def fake_quantize_awq_int4_loop(w_f32, gs):
+    """Scalar restatement of fake_quantize_awq_int4 (programming_examples/llms/llama32_1b_int4/awq_pack.py:287-316) on a
+    float32 matrix [M, K], one (row, group) at a time: scale = (max - min) / 15 in float32 (1e-7 if zero),
+    zero = clip(round(-min / scale), 0, 15), q = clip(round(w / scale + zero), 0, 15), rounding half to even as
+    np.round does.  Returns (A_q u8 [M, K / 2], scale bf16 bits [K / gs, M], zero u8 [K / gs, M]).
+    Pinned in tests/test_oracle_awq.py by a ramp whose quantisation is exact by hand (scale 1/4, zero 8, q = the ramp
+    index), the end points (min -> 0, max -> 15 when the group straddles zero), the error bound |w - (q - z) s| <= s / 2
+    inside the representable range, and constant groups."""
+    w = np.asarray(w_f32, dtype=np.float32)
+    M, K = w.shape
+    G = K // gs
+    q = np.zeros((M, K), np.uint8)
+    scale = np.zeros((G, M), np.float32)
+    zero = np.zeros((G, M), np.uint8)
+    f = np.float32
+    for m in range(M):
+        for g in range(G):
+            grp = w[m, g * gs:(g + 1) * gs]
+            lo, hi = f(min(grp)), f(max(grp))
+            sc = f(f(hi - lo) / f(15.0))
+            if sc == 0:
+                sc = f(1e-7)
+            z = min(max(float(np.round(f(-lo) / sc)), 0.0), 15.0)
+            scale[g, m], zero[g, m] = sc, int(z)
+            for i in range(gs):
+                q[m, g * gs + i] = int(min(max(float(np.round(f(f(grp[i] / sc) + f(z)))), 0.0), 15.0))
+    a_q = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)
+    return a_q, f32_to_bf16_bits(scale), zero
+
+
 def dequant_1d(int4_vals, scales_bits, zeros, group_size):
     """1-D form of the dequant example: out[i] = bf16((q[i] - z[g]) * s[g])
     evaluated in double as the reference's Python floats do."""

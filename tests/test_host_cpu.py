@@ -317,3 +317,22 @@ def test_kernel_cache_host_contract(tmp_path):
     off = kc.Profiler()
     off.record_kernel("k", 1.0)
     assert off.start_layer() is None and off.kernel_times == {} and off.per_token_walls_ms(1) == []
+
+
+def test_fake_quantize_matches_the_oracle_loop():
+    """The vectorised host quantiser against the oracle's scalar restatement, bit for bit, on groups with outliers,
+    constant groups and one-sided groups; accepts bf16 bits or floats."""
+    rng = np.random.default_rng(9)
+    w = (rng.standard_normal((12, 512)) * 10.0 ** rng.uniform(-3, 1, (12, 1))).astype(np.float32)
+    w[3, 128:256] = 0.25
+    w[4, :128] = np.abs(w[4, :128]) + 1.0
+    w[5, 17] = 40.0
+    wb = bf16.from_f32(w)
+    got = awq.fake_quantize_awq_int4(wb, 128)
+    want = oawq.fake_quantize_awq_int4_loop(bf16.to_f32(bf16.bits_of(wb)), 128)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(bf16.bits_of(got[1]), want[1]) and np.array_equal(got[2], want[2])
+    got_f = awq.fake_quantize_awq_int4(bf16.to_f32(bf16.bits_of(wb)), 128)
+    assert all(np.array_equal(np.asarray(a), np.asarray(b)) for a, b in zip(got, got_f))
+    assert got[0].shape == (12, 256) and got[1].shape == (4, 12) and got[2].dtype == np.uint8
+    with pytest.raises(ValueError):
+        awq.fake_quantize_awq_int4(w[:, :100], 128)

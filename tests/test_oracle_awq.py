@@ -155,3 +155,45 @@ def test_dequant_1d_matches_dense_form_and_c_restatement():
     got = np.zeros((K, N), np.uint16)
     lib.oracle_dequant_awq(qw.ctypes.data, qz.ctypes.data, sc.ctypes.data, K, N, gs, got.ctypes.data)
     assert np.array_equal(got, w)
+
+
+def test_fake_quantize_known_answers_and_bounds():
+    """fake_quantize_awq_int4 (awq_pack.py:287-316).  A ramp w_i = (i % 16 - 8) / 4 has min -2, max 1.75, so
+    scale = 3.75 / 15 = 1/4 exactly, zero = 8 and q_i = i % 16: every output follows by hand.  Then properties the
+    definition fixes for any group that straddles zero: the minimum quantises to 0 and the maximum to 15, and inside
+    the representable range the reconstruction error is at most half a step."""
+    gs = 128
+    ramp = ((np.arange(2 * gs) % 16 - 8) / 4.0).astype(np.float32)
+    w = np.stack([ramp, -ramp[::-1] * 0 + ramp * 2])          # row 1: the same ramp doubled (scale 1/2)
+    a_q, s_bits, z = awq.fake_quantize_awq_int4_loop(w, gs)
+    nib = awq.l1_unpack_nibbles(a_q)
+    assert np.array_equal(nib[0], np.arange(2 * gs) % 16) and np.array_equal(nib[1], np.arange(2 * gs) % 16)
+    assert s_bits.shape == (2, 2) and z.shape == (2, 2)        # [groups, rows]
+    assert np.array_equal(s_bits[:, 0], [0x3E80, 0x3E80]) and np.array_equal(s_bits[:, 1], [0x3F00, 0x3F00])
+    assert np.all(z == 8)
+    assert a_q[0, 0] == (0 | (1 << 4)) and a_q[0, 7] == (14 | (15 << 4))   # even k in the low nibble
+    # the dequantised ramp is the ramp
+    back = (nib[0].astype(np.float64) - 8) * 0.25
+    assert np.array_equal(back, ramp.astype(np.float64))
+    # random groups straddling zero
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((6, 3 * gs)) * rng.uniform(0.01, 3.0, (6, 1))).astype(np.float32)
+    a_q, s_bits, z = awq.fake_quantize_awq_int4_loop(w, gs)
+    nib = awq.l1_unpack_nibbles(a_q).reshape(6, 3, gs)
+    wg = w.reshape(6, 3, gs)
+    step = ((wg.max(axis=2) - wg.min(axis=2)) / np.float32(15.0)).astype(np.float64)
+    assert np.all(np.take_along_axis(nib, wg.argmin(axis=2)[:, :, None], 2)[:, :, 0] == 0)
+    assert np.all(np.take_along_axis(nib, wg.argmax(axis=2)[:, :, None], 2)[:, :, 0] == 15)
+    recon = (nib - z.T[:, :, None].astype(np.float64)) * step[:, :, None]
+    inside = (nib > 0) & (nib < 15)
+    assert np.all(np.abs(recon - wg)[inside] <= 0.5 * np.broadcast_to(step[:, :, None], wg.shape)[inside] * (1 + 1e-5))
+    # scales leave as bf16 of the float32 step
+    assert np.array_equal(s_bits.T, f32_to_bf16_bits(step.astype(np.float32)))
+    # a constant group: step 1e-7, everything clips to one end
+    a_q, s_bits, z = awq.fake_quantize_awq_int4_loop(np.full((1, gs), 0.5, np.float32), gs)
+    assert s_bits[0, 0] == f32_to_bf16_bits(np.float32([1e-7]))[0] and z[0, 0] == 0 and np.all(awq.l1_unpack_nibbles(a_q) == 15)
+    a_q, s_bits, z = awq.fake_quantize_awq_int4_loop(np.full((1, gs), -0.5, np.float32), gs)
+    assert z[0, 0] == 15 and np.all(awq.l1_unpack_nibbles(a_q) == 0)
+    # an all-positive group: the zero point clips to 0 and the minimum lands above 0
+    a_q, s_bits, z = awq.fake_quantize_awq_int4_loop(np.linspace(1.0, 2.5, gs, dtype=np.float32)[None], gs)
+    assert z[0, 0] == 0 and awq.l1_unpack_nibbles(a_q)[0, 0] == 10 and awq.l1_unpack_nibbles(a_q)[0, -1] == 15
