@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|gemv_awq|dequant|gemm16|gemm64|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|probe|gemv_awq|dequant|gemm16|gemm64|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -31,6 +31,9 @@ CONFIGS = {
     "dequant": dict(M=0, K=4096, N=4096, cfg=0, desc="AWQ dequant K=4096 N=4096 -> bf16"),
     # the weights re-packed once at load time (untimed, as the reference re-packs them) into stream order
     "gemv": dict(M=1, K=4096, N=11008, cfg=1, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128, stream-order weights"),
+    # read-only pass over the same stream-order arena with the GEMV's launch shape and request pattern (no x, no
+    # arithmetic): the floor of any kernel that reads the matrix once; priced with config 1's algorithmic bytes
+    "probe": dict(M=1, K=4096, N=11008, cfg=None, desc="read-only probe of the stream-order matrix of config 1 (K=4096 N=11008), GEMV launch shape"),
     # the same product on the AutoAWQ checkpoint layout (split-K kernel with a workspace)
     "gemv_awq": dict(M=1, K=4096, N=11008, cfg=None, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128, checkpoint-layout weights"),
     "gemm16": dict(M=16, K=4096, N=14336, cfg=2, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128, stream-order weights"),
@@ -57,11 +60,18 @@ CONFIGS = {
 }
 LAYER_HEADS, LAYER_KV, LAYER_HD, LAYER_POS, LAYER_MAXSEQ = 32, 8, 128, 2047, 2048
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
-# scaled by the same counter's reading for a 256 MiB device copy: x2.000 and x1.000); the
-# summaries under profiles/ hold the commands and the raw readings.
-MEASURED_TRAFFIC_BYTES = {"gemv": 24.11e6, "gemm16": 32.83e6, "prefill": 347.4e6, "ffn": 94.07e6,
-                          "gemv_awq": 24.26e6, "gemm16_awq": 41.9e6, "prefill_awq": 351.7e6, "ffn_awq": 94.4e6, "lm_head": 525.9e6}
+
+
+def measured_traffic(name):
+    """HBM bytes per launch of a workload's dominant kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two
+    runs, each scaled by the same counter's reading for a 256 MiB device copy), from profiles/traffic.json: the figure,
+    the commit of the kernel it was measured on and the summary under profiles/ that holds the command and the raw
+    readings.  None for a workload that has no entry."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(name)
+    except OSError:
+        return None
 
 
 def weight_bytes(K, N):
@@ -136,7 +146,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
 
     q4nx = name.startswith("q4nx")
     lm_head = name == "lm_head"
-    stream_order = name in ("gemv", "gemm16", "gemm64", "prefill", "ffn", "block", "layer")     # weights re-packed at load time (untimed)
+    stream_order = name in ("gemv", "probe", "gemm16", "gemm64", "prefill", "ffn", "block", "layer")     # weights re-packed at load time (untimed)
     kind = name[:-4] if name.endswith("_awq") else name
     per_copy = K * N * 2 if lm_head else q4nx_weight_bytes(K, N) if q4nx else weight_bytes(K, N) * (3 if kind in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if kind in ("block", "layer") else 0)
     nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
@@ -164,7 +174,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             gw = torch.Generator(device="cuda")
             gw.manual_seed(100 + i)
             copies.append(((torch.randn((N, K), device="cuda", generator=gw) * 0.05).to(torch.bfloat16),))
-        elif name == "gemv":
+        elif name in ("gemv", "probe"):
             # all copies in one arena, as a loader would place a model's layers
             from air_hip import ops
             w = make_weights(torch, K, N, 100 + i)
@@ -176,7 +186,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             del w
         else:
             copies.append(make_weights(torch, K, N, 100 + i))
-        if stream_order and kind != "gemv":
+        if stream_order and kind not in ("gemv", "probe"):
             from air_hip import ops
             if i == 0:
                 awq0 = copies[0]
@@ -191,6 +201,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         outs = [torch.empty((K,), dtype=torch.bfloat16, device=dev)]
     else:
         outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev)]
+    if name == "probe":
+        probe_out = torch.empty((N,), dtype=torch.int32, device=dev)
     if lm_head:
         outs = [torch.empty((N,), dtype=torch.bfloat16, device=dev)]
         best = torch.empty((1,), dtype=torch.int32, device=dev)
@@ -274,6 +286,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                        best.data_ptr(), N, K, lm_ws.data_ptr(), lm_ws.numel(), st)
         elif name == "gemv":
             rc = lib.w4a16_gemv_stream_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), K, N, 128, st)
+        elif name == "probe":
+            rc = lib.w4a16_probe_stream_read(w[0].data_ptr(), probe_out.data_ptr(), K, N, st)
         elif name in ("gemm16", "gemm64", "prefill"):
             rc = lib.w4a16_gemm_stream_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), M, K, N, 128, st)
         elif name == "q4nx_gemv":
@@ -377,7 +391,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                  "avg": sum(per_launch) / len(per_launch), "max": per_launch[-1]},
     }
 
-    if with_cpu_baseline and kind not in ("block", "layer", "lm_head") and not name.endswith("_awq") and not q4nx:
+    if with_cpu_baseline and kind not in ("block", "layer", "lm_head", "probe") and not name.endswith("_awq") and not q4nx:
         w0 = copies[0][1:] if name == "gemv" else awq0 if awq0 is not None else copies[0]
         res["cpu_baseline"] = cpu_baseline(name, torch, w0, x, outs, launch, stream)
     return res
@@ -760,9 +774,12 @@ def main():
         value = main_res["bytes"] / sec / 1e9
         roof = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": value / HBM_PEAK_GBS, "traffic": None}
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
+    t = measured_traffic(name)
+    roof["traffic"] = t["bytes"] if t else None
+    if t:
+        roof["traffic_measured_at"] = {"commit": t["commit"], "profile": t["profile"]}
     roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_wsp_kernel", "prefill_awq": "gemm_kernel", "lm_head": "lm_head_kernel",
-                      "gemv": "gemv_ws_kernel", "gemm16": "gemm_ws_kernel", "gemm64": "gemm_ws_rows_kernel", "ffn": "gemv_ws_kernel", "block": "gemv_ws_kernel", "layer": "gemv_ws_kernel"}.get(name, "stream_kernel")
+                      "gemv": "gemv_ws_kernel", "probe": "probe_ws_kernel", "gemm16": "gemm_ws_kernel", "gemm64": "gemm_ws_rows_kernel", "ffn": "gemv_ws_kernel", "block": "gemv_ws_kernel", "layer": "gemv_ws_kernel"}.get(name, "stream_kernel")
     roof["algorithmic_per_launch"] = main_res["flops"] if name in ("prefill", "prefill_awq") else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]
 
@@ -818,7 +835,8 @@ def main():
                     "metric": "W4A16 prefill GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "steps": 20, "warmup": 5,
                     "ms_per_step": r["cold_us"] * 1e-3, "config": {"workload": CONFIGS["prefill"]["desc"]},
                     "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                 "frac": tf / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get("prefill"),
+                                 "frac": tf / MFMA_BF16_PEAK_TFLOPS, "traffic": (measured_traffic("prefill") or {}).get("bytes"),
+                                 "traffic_measured_at": {k: (measured_traffic("prefill") or {}).get(k) for k in ("commit", "profile")},
                                  "kernel": "gemm_wsp_kernel", "algorithmic_per_launch": r["flops"], "avg_launch_us": r["cold_us"]},
                     "graph_us_per_step": r["graph_us"]}
                 if "cpu_baseline" in r:

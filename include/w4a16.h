@@ -215,6 +215,12 @@ int w4a16_gemv_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, 
                            void *stream);
 int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual,
                                uint16_t *y, int K, int N, int group, void *stream);
+/* Measurement aid, no counterpart among the reference's kernels (its harness times the kernel alone,
+ * programming_examples/matrix_vector_multiplication/int4_awq/test_packed.cpp:114-150): one read-only pass over a
+ * stream-order matrix with w4a16_gemv_stream_bf16's launch shape and request pattern, everything loaded folded with XOR
+ * into out_words (N words: 16 per 16-column tile, one per wave; the others are not written).  Its time is the floor of
+ * any kernel that reads the matrix once in that order, which bench.py reports beside the GEMV. */
+int w4a16_probe_stream_read(const void *wstream, uint32_t *out_words, int K, int N, void *stream);
 /* Batched decode on a stream-order matrix: y[M, N] = bf16(x[M, K] . W), unrounded weights, fp32 accumulation
  * (matmul_int4_packed.cpu_reference, programming_examples/matrix_multiplication/int4_awq/matmul_int4_packed.py:89-105;
  * device kernel matmul_int4_bf16_packed_f32, mv_int4_bf16.cc:430-448).  Up to 64 rows per launch stream the weights

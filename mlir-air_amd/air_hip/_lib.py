@@ -57,6 +57,7 @@ SYMBOLS = {
     "w4a16_stream_bytes": (_sz, [_ci, _ci]),
     "w4a16_repack_stream": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_gemv_stream_bf16": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
+    "w4a16_probe_stream_read": (_ci, [_vp, _vp, _ci, _ci, _vp]),
     "w4a16_gemm_stream_bf16": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]),
     "w4a16_gemv_add_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_gemv_swiglu_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),

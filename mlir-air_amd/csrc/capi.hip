@@ -460,6 +460,14 @@ int w4a16_repack_stream(const int32_t *qweight, const int32_t *qzeros, const uin
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+int w4a16_probe_stream_read(const void *wstream, uint32_t *out_words, int K, int N, void *stream) {
+    if (!wstream || !out_words) return W4A16_ERR_NULL;
+    if (K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
+    if (misaligned(wstream) || misaligned(out_words)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_probe_ws(wstream, out_words, K, N, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 namespace {
 // One whole-K launch on stream-order weights: argument checks shared by every stream-order entry point.
 int gemv_stream_call(const uint16_t *x, const void *w, const void *w_up, uint16_t *y, int K, int N, int group, void *stream,

@@ -277,6 +277,41 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
     }
 }
 
+// Read-only pass over a stream-order matrix with the GEMV's launch shape and request pattern (one workgroup per tile,
+// a wave per task of CT cells, the block's scale words and the cells requested up front, non-temporal cell loads):
+// everything loaded is folded with XOR into one word per wave.  No x, no arithmetic: what this takes is the floor of
+// any kernel that reads the buffer once in this order.
+template <int CT>
+__global__ void __launch_bounds__(kMaxWaves * 64) probe_ws_kernel(const char *__restrict__ w, uint32_t *__restrict__ out, int G, int NB,
+                                                                  int nwaves) {
+    constexpr int SUB = kWsBlockGroups / CT;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const size_t tile_bytes = (size_t)(NB + G) * kWsCellBytes;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (int task = wave; task < NB * SUB; task += nwaves) {
+        const int b = task / SUB, r0 = (task % SUB) * CT;
+        const int ng = min(kWsBlockGroups, G - kWsBlockGroups * b);
+        if (r0 >= ng) continue;
+        const char *blk = w + (size_t)blockIdx.x * tile_bytes + (size_t)b * ((kWsBlockGroups + 1) * kWsCellBytes);
+        u32x4 cell[CT];
+        const u32x4 md = *(reinterpret_cast<const u32x4 *>(blk) + lane);
+#pragma unroll
+        for (int r = 0; r < CT; ++r) {
+            const int rc = r0 + r < ng ? r0 + r : ng - 1;
+            cell[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(blk + (size_t)(1 + rc) * kWsCellBytes) + lane);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        acc ^= md;
+#pragma unroll
+        for (int r = 0; r < CT; ++r) acc ^= cell[r];
+    }
+    uint32_t v = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v ^= __shfl_xor(v, off);
+    if (lane == 0) out[blockIdx.x * kMaxWaves + wave] = v;
+}
+
 // One thread per dword of the stream-order buffer.
 __global__ void __launch_bounds__(256) repack_ws_kernel(const uint32_t *__restrict__ qweight, const uint32_t *__restrict__ qzeros,
                                                         const uint16_t *__restrict__ scales, uint32_t *__restrict__ out, int G,
@@ -414,6 +449,17 @@ hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, ui
         case 16: return launch_ct<16>(nmat, pl.waves, x, w, w_up, y, K, N, extras, stream);
         default: return launch_ct<8>(nmat, pl.waves, x, w, w_up, y, K, N, extras, stream);
     }
+}
+
+hipError_t launch_probe_ws(const void *w, uint32_t *out, int K, int N, hipStream_t stream) {
+    const GemvWsPlan pl = plan_gemv_ws(K, 1, N, false);
+    const int G = K / kGroup, NB = ws_blocks(K);
+    const dim3 grid(N / kWsTileCols), block(pl.waves * 64);
+    const char *p = static_cast<const char *>(w);
+    if (pl.ct == 16) hipLaunchKernelGGL(probe_ws_kernel<16>, grid, block, 0, stream, p, out, G, NB, pl.waves);
+    else if (pl.ct == 4) hipLaunchKernelGGL(probe_ws_kernel<4>, grid, block, 0, stream, p, out, G, NB, pl.waves);
+    else hipLaunchKernelGGL(probe_ws_kernel<8>, grid, block, 0, stream, p, out, G, NB, pl.waves);
+    return hipGetLastError();
 }
 
 hipError_t launch_repack_ws_q4(const int32_t *qweight, const uint16_t *scales, const uint16_t *mins, void *out, int K, int N,

@@ -119,6 +119,8 @@ GemvWsPlan plan_gemv_ws(int K, int nmat, int N, bool rms);
 // y = bf16(silu(bf16(x.W)) * bf16(x.W_up)).
 hipError_t launch_gemv_ws(const uint16_t *x, const void *w, const void *w_up, uint16_t *y, int K, int N, hipStream_t stream,
                           const GemvWsExtras &extras = GemvWsExtras());
+// Read-only pass over a stream-order matrix in the GEMV's launch shape; `out` takes one word per wave (N / 16 * 16 words).
+hipError_t launch_probe_ws(const void *w, uint32_t *out, int K, int N, hipStream_t stream);
 // y[M, N] = bf16(x[M, K] . W (+ residual [M, N])) with W in stream order, any M >= 2 (launches of up to 64 rows; Q4NX order: 16).
 hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
                           hipStream_t stream, bool q4 = false);   // q4: W in Q4NX order
