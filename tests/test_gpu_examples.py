@@ -227,11 +227,15 @@ def test_backend_runs_the_stream_order_kernels_and_reports_library_errors():
 
 
 @pytest.mark.parametrize("example,argv", [
+    # the shapes the reference's own lit tests run (run_packed*_peano.lit, run_packed_npu2_*.lit, run_int4_npu2_peano.lit)
     ("matvec_int4_packed", ["--m", "2048", "--k", "2048"]),
-    ("matvec_int4_packed_add", ["--m", "1024", "--k", "2048"]),
+    ("matvec_int4_packed", ["--m", "2048", "--k", "8192"]),
+    ("matvec_int4_packed_add", ["--m", "2048", "--k", "2048"]),
+    ("matmul_int4_packed", []),                                                # 64 x 128 x 128
+    ("matmul_int4_packed", ["--m", "32", "--k", "2048", "--n", "2048"]),
+    ("matvec_int4_swiglu_rms", []),                                            # M = 16384 interleaved rows, K = 2048
+    # and the tiled kernel
     ("matmul_int4_packed", ["--m", "2048", "--k", "2048", "--n", "2048"]),
-    ("matmul_int4_packed", []),
-    ("matvec_int4_swiglu_rms", ["--m", "4096", "--k", "2048"]),
     ("o_gemv_ffn_int4", ["--emb-dim", "1024", "--hidden-dim", "4096"]),
     ("dequant_awq", []),
 ])
