@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|probe|gemv_awq|dequant|gemm16|gemm64|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|probe|gemv_awq|dequant|gemm16|gemm64|gemm64_down|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -37,8 +37,10 @@ CONFIGS = {
     # the same product on the AutoAWQ checkpoint layout (split-K kernel with a workspace)
     "gemv_awq": dict(M=1, K=4096, N=11008, cfg=None, desc="decode GEMV W4A16 M=1 K=4096 N=11008 g128, checkpoint-layout weights"),
     "gemm16": dict(M=16, K=4096, N=14336, cfg=2, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128, stream-order weights"),
-    # the same product for a batch of 64 (one launch of four row tiles; no BASELINE config)
+    # the same product for a batch of 64 (split along K, a launch of four row tiles plus the launch that adds the slices;
+    # no BASELINE config)
     "gemm64": dict(M=64, K=4096, N=14336, cfg=None, desc="batched decode GEMM W4A16 M=64 K=4096 N=14336 g128, stream-order weights"),
+    "gemm64_down": dict(M=64, K=14336, N=4096, cfg=None, desc="batched decode GEMM W4A16 M=64 K=14336 N=4096 g128 (down projection), stream-order weights, split along K"),
     "gemm16_awq": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM W4A16 M=16 K=4096 N=14336 g128, checkpoint-layout weights"),
     "prefill": dict(M=2048, K=4096, N=14336, cfg=3, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128, stream-order weights"),
     "prefill_awq": dict(M=2048, K=4096, N=14336, cfg=None, desc="prefill GEMM W4A16 M=2048 K=4096 N=14336 g128, checkpoint-layout weights"),
@@ -146,7 +148,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
 
     q4nx = name.startswith("q4nx")
     lm_head = name == "lm_head"
-    stream_order = name in ("gemv", "probe", "gemm16", "gemm64", "prefill", "ffn", "block", "layer")     # weights re-packed at load time (untimed)
+    stream_order = name in ("gemv", "probe", "gemm16", "gemm64", "gemm64_down", "prefill", "ffn", "block", "layer")     # weights re-packed at load time (untimed)
     kind = name[:-4] if name.endswith("_awq") else name
     per_copy = K * N * 2 if lm_head else q4nx_weight_bytes(K, N) if q4nx else weight_bytes(K, N) * (3 if kind in ("ffn", "block", "layer") else 1) + (weight_bytes(K, K) if kind in ("block", "layer") else 0)
     nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
@@ -190,7 +192,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             from air_hip import ops
             if i == 0:
                 awq0 = copies[0]
-            mats = (copies[i],) if kind in ("gemm16", "gemm64", "prefill") else copies[i]
+            mats = (copies[i],) if kind in ("gemm16", "gemm64", "gemm64_down", "prefill") else copies[i]
             copies[i] = tuple(ops.repack_stream(*m).buf for m in mats)
     gx = torch.Generator(device="cuda")
     gx.manual_seed(7)
@@ -203,6 +205,8 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
         outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev)]
     if name == "probe":
         probe_out = torch.empty((N,), dtype=torch.int32, device=dev)
+    if name in ("gemm16", "gemm64", "gemm64_down", "prefill"):
+        gemm_scratch = torch.empty(max(int(lib.w4a16_gemm_stream_scratch_bytes(M, K, N)), 16), dtype=torch.uint8, device=dev)
     if lm_head:
         outs = [torch.empty((N,), dtype=torch.bfloat16, device=dev)]
         best = torch.empty((1,), dtype=torch.int32, device=dev)
@@ -288,8 +292,10 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
             rc = lib.w4a16_gemv_stream_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), K, N, 128, st)
         elif name == "probe":
             rc = lib.w4a16_probe_stream_read(w[0].data_ptr(), probe_out.data_ptr(), K, N, st)
-        elif name in ("gemm16", "gemm64", "prefill"):
-            rc = lib.w4a16_gemm_stream_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), M, K, N, 128, st)
+        elif name in ("gemm16", "gemm64", "gemm64_down", "prefill"):
+            # (17 .. 128 rows: split along K with plain scratch; other row counts take no scratch)
+            rc = lib.w4a16_gemm_stream_scratch_bf16(x.data_ptr(), w[0].data_ptr(), outs[0].data_ptr(), M, K, N, 128,
+                                                    gemm_scratch.data_ptr(), gemm_scratch.numel(), st)
         elif name == "q4nx_gemv":
             rc = lib.w4a16_q4nx_gemv_stream_bf16(x.data_ptr(), w[0].data_ptr(), None, outs[0].data_ptr(), K, N, st)
         elif name == "q4nx_gemm16":
@@ -813,7 +819,7 @@ def main():
     if t:
         roof["traffic_measured_at"] = {"commit": t["commit"], "profile": t["profile"]}
     roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_wsp_kernel", "prefill_awq": "gemm_kernel", "lm_head": "lm_head_kernel",
-                      "gemv": "gemv_ws_kernel", "probe": "probe_ws_kernel", "gemm16": "gemm_ws_kernel", "gemm64": "gemm_ws_rows_kernel", "ffn": "gemv_ws_kernel", "block": "gemv_ws_kernel", "layer": "gemv_ws_kernel"}.get(name, "stream_kernel")
+                      "gemv": "gemv_ws_kernel", "probe": "probe_ws_kernel", "gemm16": "gemm_ws_kernel", "gemm64": "gemm_ws_rows_kernel", "gemm64_down": "gemm_wsk_kernel", "ffn": "gemv_ws_kernel", "block": "gemv_ws_kernel", "layer": "gemv_ws_kernel"}.get(name, "stream_kernel")
     roof["algorithmic_per_launch"] = main_res["flops"] if name in ("prefill", "prefill_awq") else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]
 

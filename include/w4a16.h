@@ -235,6 +235,20 @@ int w4a16_probe_stream_read(const void *wstream, uint32_t *out_words, int K, int
  * bits for every M keeps M <= 128 per call.  K % 128 == 0, N % 16 == 0. */
 int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int M, int K, int N, int group,
                            void *stream);
+/* w4a16_gemm_stream_bf16 with plain scratch for the shapes where 17 .. 128 rows run faster split along K (same
+ * reference, matmul_int4_packed.py:89-105; the reference's own kernel also walks K in slices, one L1 K-chunk at a
+ * time, and adds them in an fp32 accumulator, matmul_int4_packed.py:179-181, 293-345).  A workgroup takes 256 columns and a slice of K, shares
+ * the x rows of its slice through LDS and writes fp32 partial sums to `scratch`; a second launch adds the slices in
+ * slice order and rounds once.  That pays where the whole-K launches re-read the x rows most: K >= 4096, rows * K / 128
+ * >= 1536 and N < 12800 (K = 14336, N = 4096, 64 rows: 34.6 us against 59.2 us; K = 8192, N = 6144: 26.1 against 63.7);
+ * for every other shape and row count the call is w4a16_gemm_stream_bf16 itself and `scratch` is not touched.
+ * w4a16_gemm_stream_scratch_bytes(M, K, N) is the scratch the call needs (0 where it takes none): no initialisation,
+ * nothing kept between calls, 16-byte aligned; calls that overlap on one GPU need a buffer each.  Same numerics as
+ * w4a16_gemm_stream_bf16 below 129 rows (exact weights, fp32 sums, one rounding); the two differ by the order of the
+ * fp32 additions only. */
+size_t w4a16_gemm_stream_scratch_bytes(int M, int K, int N);
+int w4a16_gemm_stream_scratch_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int M, int K, int N, int group,
+                                   void *scratch, size_t scratch_bytes, void *stream);
 int w4a16_gemv_swiglu_stream_bf16(const uint16_t *x, const void *gate_wstream, const void *up_wstream,
                                   uint16_t *h, int K, int H, int group, void *stream);
 

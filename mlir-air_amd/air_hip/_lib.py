@@ -59,6 +59,8 @@ SYMBOLS = {
     "w4a16_gemv_stream_bf16": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_probe_stream_read": (_ci, [_vp, _vp, _ci, _ci, _vp]),
     "w4a16_gemm_stream_bf16": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]),
+    "w4a16_gemm_stream_scratch_bytes": (_sz, [_ci, _ci, _ci]),
+    "w4a16_gemm_stream_scratch_bf16": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_gemv_add_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_gemv_swiglu_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_rms_gemv_stream_bf16": (_ci, [_vp, _vp, _ci, _vp, _cf, _vp, _vp, _ci, _ci, _ci, _vp]),

@@ -257,8 +257,13 @@ def w4a16_gemv_stream(x, w, residual=None, group=GROUP, out=None):
     return out
 
 
+_gemm_scratch = {}
+
+
 def w4a16_gemm_stream(x, w, group=GROUP, out=None):
-    """y[M, N] = bf16(x[M, K] . W) on a StreamWeight; x may be a vector [K]."""
+    """y[M, N] = bf16(x[M, K] . W) on a StreamWeight; x may be a vector [K].  Batches of 17 to 128 rows run split along
+    K with their partial sums in a scratch buffer of this module (plain scratch per device and stream, grown on
+    demand, nothing kept in it between calls)."""
     lib = _lib.load_library()
     _need_cuda(x, w.buf)
     vec = x.dim() == 1
@@ -268,7 +273,16 @@ def w4a16_gemm_stream(x, w, group=GROUP, out=None):
         raise ValueError(f"x has K={K} but the matrix has {w.K} rows")
     if out is None:
         out = torch.empty((M, w.N), dtype=torch.bfloat16, device=x.device)
-    _lib.check(lib.w4a16_gemm_stream_bf16(_ptr(_bits(x2)), _ptr(w.buf), _ptr(out), M, K, w.N, group, _stream()))
+    need = lib.w4a16_gemm_stream_scratch_bytes(M, K, w.N)
+    if need:
+        key = (x.device.index, _stream())
+        scratch = _gemm_scratch.get(key)
+        if scratch is None or scratch.numel() < need:
+            scratch = _gemm_scratch[key] = torch.empty(int(need), dtype=torch.uint8, device=x.device)
+        _lib.check(lib.w4a16_gemm_stream_scratch_bf16(_ptr(_bits(x2)), _ptr(w.buf), _ptr(out), M, K, w.N, group, _ptr(scratch),
+                                                      scratch.numel(), _stream()))
+    else:
+        _lib.check(lib.w4a16_gemm_stream_bf16(_ptr(_bits(x2)), _ptr(w.buf), _ptr(out), M, K, w.N, group, _stream()))
     return out.squeeze(0) if vec else out
 
 

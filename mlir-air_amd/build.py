@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libw4a16_hip.so")
-SOURCES = ["capi.hip", "dequant.hip", "stream.hip", "gemv_ws.hip", "gemm_ws.hip", "gemm.hip", "attention.hip", "q4nx.hip", "lm_head.hip", "prefill_block.hip", "prefill_attention.hip"]
+SOURCES = ["capi.hip", "dequant.hip", "stream.hip", "gemv_ws.hip", "gemm_ws.hip", "gemm_wsk.hip", "gemm.hip", "attention.hip", "q4nx.hip", "lm_head.hip", "prefill_block.hip", "prefill_attention.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

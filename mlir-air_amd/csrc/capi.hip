@@ -558,6 +558,28 @@ int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, 
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+size_t w4a16_gemm_stream_scratch_bytes(int M, int K, int N) {
+    if (M <= 16 || M > kGemmWsMaxM || K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return 0;
+    return gemm_wsk_pays(M, K, N) ? gemm_wsk_scratch_bytes(M, K, N) : 0;
+}
+
+int w4a16_gemm_stream_scratch_bf16(const uint16_t *x, const void *wstream, uint16_t *y, int M, int K, int N, int group, void *scratch,
+                                   size_t scratch_bytes, void *stream) {
+    // 17 .. 128 rows of a shape where the split along K is the faster one: the split-K kernel; everything else is
+    // w4a16_gemm_stream_bf16
+    const int prefill_min_m = g_gemv_ws_tune.prefill_min_m > 16 ? g_gemv_ws_tune.prefill_min_m : kGemmWsMaxM + 1;
+    const bool shape_ok = K > 0 && N > 0 && K % kGroup == 0 && N % kWsTileCols == 0;
+    if (M <= 16 || M >= prefill_min_m || !shape_ok || !gemm_wsk_pays(M, K, N))
+        return w4a16_gemm_stream_bf16(x, wstream, y, M, K, N, group, stream);
+    if (!x || !wstream || !y) return W4A16_ERR_NULL;
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    if (misaligned(x) || misaligned(wstream) || misaligned(y) || misaligned(scratch)) return W4A16_ERR_ALIGN;
+    const size_t need = gemm_wsk_scratch_bytes(M, K, N);
+    if (need && (!scratch || scratch_bytes < need)) return W4A16_ERR_WORKSPACE;
+    hipError_t e = launch_gemm_wsk(x, wstream, y, nullptr, static_cast<float *>(scratch), M, K, N, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 int w4a16_gemv_add_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int K, int N,
                                int group, void *stream) {
     if (!residual) return W4A16_ERR_NULL;
@@ -961,6 +983,9 @@ int w4a16_tune(const char *key, int value) {
     } else if (!strcmp(key, "prefill_swiglu_split")) {
         if (value != 0 && value != 1) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.prefill_swiglu_split = value;
+    } else if (!strcmp(key, "gemm_splitk")) {
+        if (value < 0 || value > 2) return W4A16_ERR_TUNE;
+        g_gemv_ws_tune.splitk = value;
     } else if (!strcmp(key, "prefill_band")) {
         if (value > 64) return W4A16_ERR_TUNE;
         g_gemv_ws_tune.prefill_band = value;

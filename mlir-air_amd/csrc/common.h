@@ -77,6 +77,19 @@ __device__ __forceinline__ float wave_reduce(float v) {
     return op(v, __shfl_xor(v, 32));
 }
 
+// Sum over the 16 lanes of a DPP row, every lane of the row receiving it (the four in-row steps of wave_reduce).
+__device__ __forceinline__ float row_sum16(float v) {
+    auto dpp = [&](auto ctrl) {
+        constexpr int CTRL = decltype(ctrl)::value;
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+    };
+    dpp(std::integral_constant<int, 0xB1>());    // quad_perm [1, 0, 3, 2]
+    dpp(std::integral_constant<int, 0x4E>());    // quad_perm [2, 3, 0, 1]
+    dpp(std::integral_constant<int, 0x141>());   // row_half_mirror
+    dpp(std::integral_constant<int, 0x140>());   // row_mirror
+    return v;
+}
+
 // silu(g) in the reference's tanh form (matvec_int4_swiglu_rms.py:512-514), fp32
 __device__ __forceinline__ float silu_tanh(float g) { return g * 0.5f * (tanhf(g * 0.5f) + 1.0f); }
 

@@ -108,6 +108,7 @@ struct GemvWsTune {
     int gemm_rows = 0;       // batched kernel: most rows per launch, 16, 32 or 64 (0 = 64)
     int prefill_min_m = 0;   // smallest M that w4a16_gemm_stream_bf16 gives to the prefill kernel (0 = default)
     int prefill_band = 0;    // prefill kernel: row panels per band of the tile order (0 = default)
+    int splitk = 0;          // w4a16_gemm_stream_scratch_bf16 at 17 .. 128 rows: 0 split-K where it pays by shape, 1 always, 2 never
     int prefill_swiglu_split = 0;   // 1: the prompt-pass FFN runs gate and up as two launches instead of one
 };
 extern GemvWsTune g_gemv_ws_tune;
@@ -124,6 +125,12 @@ hipError_t launch_probe_ws(const void *w, uint32_t *out, int K, int N, hipStream
 // y[M, N] = bf16(x[M, K] . W (+ residual [M, N])) with W in stream order, any M >= 2 (launches of up to 64 rows; Q4NX order: 16).
 hipError_t launch_gemm_ws(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, int M, int K, int N,
                           hipStream_t stream, bool q4 = false);   // q4: W in Q4NX order
+// Batched decode split along K (gemm_wsk.hip), 17 <= M: launches of up to 64 rows, each followed by the launch that adds the
+// slices; `scratch`: gemm_wsk_scratch_bytes(M, K, N) bytes of plain scratch (0: not needed, one slice).
+size_t gemm_wsk_scratch_bytes(int M, int K, int N);
+bool gemm_wsk_pays(int M, int K, int N);   // the split is the faster of the two for this shape (or forced by the tune key)
+hipError_t launch_gemm_wsk(const uint16_t *x, const void *w, uint16_t *y, const uint16_t *residual, float *scratch, int M, int K,
+                           int N, hipStream_t stream);
 // Prefill GEMM on stream-order weights (gemm_ws.hip): bf16-rounded weights dequantised in registers, x through LDS.
 bool gemm_prefill_ws_supported(int M, int K, int N);   // K % 256 == 0, N % 64 == 0
 // Epilogues as for launch_gemm_prefill (kEpi*); kEpiRope with heads of 128 needs N % 128 == 0.

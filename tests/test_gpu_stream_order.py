@@ -194,6 +194,75 @@ def test_gemm_stream_more_than_sixteen_rows(ops, M, K, N):
     _gemm_case(ops, M, K, N, seed=M + K + N)
 
 
+@pytest.mark.parametrize("M,K,N", [(17, 256, 64), (32, 1024, 544), (48, 128 * 19, 48), (64, 4096, 6400), (65, 1024, 512),
+                                   (128, 2048, 2048), (30, 128 * 19, 528), (64, 4096, 14336), (20, 14336, 4096), (33, 128, 272)])
+def test_gemm_stream_split_k_against_whole_k(ops, M, K, N):
+    """17 .. 128 rows through ops.w4a16_gemm_stream run split along K where that is the faster way (256-column
+    workgroups, x through LDS, the slices added by a second launch), else as the whole-K launches of
+    w4a16_gemm_stream_bf16; here each way is forced in turn.  Both are within one ulp of the float64 product (checked
+    by _gemm_case) and differ from each other by summation order only.  Shapes: one slice (K = 128), ragged column sets
+    (N = 48, 272, 528, 544), a short last quad of groups (19), two launches of rows (65, 128), both row-tile counts."""
+    try:
+        ops.tune("gemm_splitk", 1)
+        split = bf16_bits_to_f32(_gemm_case(ops, M, K, N, seed=M + K + N)).astype(np.float64)
+        ops.tune("gemm_splitk", 2)
+        whole = bf16_bits_to_f32(_gemm_case(ops, M, K, N, seed=M + K + N)).astype(np.float64)
+    finally:
+        ops.tune("gemm_splitk", 0)
+    assert np.all(np.abs(split - whole) <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(whole), 1e-30))) - 7) + 2e-3)
+    assert np.mean(split != whole) < 0.05
+
+
+def test_gemm_stream_split_k_scratch_contract(ops):
+    """The split-K entry point: scratch size by shape (none below 17 rows, above 128, or for a single slice), a short or
+    missing scratch buffer is refused before any launch, and the result does not depend on what the scratch held."""
+    from air_hip import _lib
+    lib = _lib.load_library()
+    K, N, M = 1024, 512, 40
+    # by shape: long K, enough rows, and not where the whole-K workgroups are 64 columns wide already
+    assert lib.w4a16_gemm_stream_scratch_bytes(64, 14336, 4096) == 7 * 64 * 4096 * 4        # 112 groups in slices of 16
+    assert lib.w4a16_gemm_stream_scratch_bytes(64, 4096, 4096) > 0 and lib.w4a16_gemm_stream_scratch_bytes(32, 4096, 4096) == 0
+    assert lib.w4a16_gemm_stream_scratch_bytes(64, 2048, 8192) == 0 and lib.w4a16_gemm_stream_scratch_bytes(64, 4096, 14336) == 0
+    assert lib.w4a16_gemm_stream_scratch_bytes(M, K, N) == 0
+    ops.tune("gemm_splitk", 1)
+    try:
+        _split_k_scratch_contract(ops, lib, M, K, N)
+    finally:
+        ops.tune("gemm_splitk", 0)
+
+
+def _split_k_scratch_contract(ops, lib, M, K, N):
+    from air_hip import _lib
+    assert lib.w4a16_gemm_stream_scratch_bytes(16, K, N) == 0 and lib.w4a16_gemm_stream_scratch_bytes(129, K, N) == 0
+    assert lib.w4a16_gemm_stream_scratch_bytes(M, 128, N) == 0                 # one group: one slice
+    need = lib.w4a16_gemm_stream_scratch_bytes(M, K, N)
+    assert need == 2 * M * N * 4                                              # 8 groups in slices of 4
+    assert lib.w4a16_gemm_stream_scratch_bytes(128, K, N) == 2 * 64 * N * 4   # launches of 64 rows share it
+    qw, qz, s = make_awq(K, N, seed=91)
+    w = _stream_weight(ops, qw, qz, s)
+    x = dev(make_x((M, K), seed=92))
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    scratch = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")     # NaN patterns: must all be overwritten
+    p = lambda t: t.data_ptr()
+    assert lib.w4a16_gemm_stream_scratch_bf16(p(x), p(w.buf), p(y), M, K, N, 128, None, 0, st) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_gemm_stream_scratch_bf16(p(x), p(w.buf), p(y), M, K, N, 128, p(scratch), need - 1, st) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_gemm_stream_scratch_bf16(p(x), p(w.buf), p(y), M, K, N, 128, p(scratch) + 4, need, st) == _lib.ERR_ALIGN
+    torch.cuda.synchronize()
+    assert not y.any()
+    _lib.check(lib.w4a16_gemm_stream_scratch_bf16(p(x), p(w.buf), p(y), M, K, N, 128, p(scratch), need, st))
+    y2 = ops.w4a16_gemm_stream(x, w)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16)) and torch.isfinite(y.float()).all()
+    # rows outside the split range go to the same launches as w4a16_gemm_stream_bf16, scratch or not
+    x16 = x[:16].contiguous()
+    ya, yb = torch.zeros((16, N), dtype=torch.bfloat16, device="cuda"), torch.zeros((16, N), dtype=torch.bfloat16, device="cuda")
+    _lib.check(lib.w4a16_gemm_stream_scratch_bf16(p(x16), p(w.buf), p(ya), 16, K, N, 128, None, 0, st))
+    _lib.check(lib.w4a16_gemm_stream_bf16(p(x16), p(w.buf), p(yb), 16, K, N, 128, st))
+    torch.cuda.synchronize()
+    assert torch.equal(ya.view(torch.int16), yb.view(torch.int16))
+
+
 @pytest.mark.parametrize("rows", [16, 32])
 def test_gemm_stream_rows_per_launch_agree_up_to_summation_order(ops, rows):
     """The rows a launch takes change only how a column's groups are dealt to the waves: the same sums in another order."""
