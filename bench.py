@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X W4A16 path.  One JSON line on stdout.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|probe|gemv_awq|dequant|gemm16|gemm64|gemm64_down|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemv|probe|gemv_awq|dequant|gemm16|gemm64|gemm64_down|gemm16_awq|prefill|prefill_awq|ffn|ffn_awq|block|block_awq|layer|layer_awq|q4nx_gemv|q4nx_gemm16|q4nx_prefill|lm_head|decode_1b|decode_8b|prefill_block|prefill_block_awq|prefill_1b|prefill_1b_awq|prefill_8b]
 
 Default workload is the decode GEMV (x bf16 [1,4096], W int4 [4096 x 11008], group 128).
 A step is one launch of the hot path on synthetic inputs that are already resident in HBM.
@@ -57,6 +57,7 @@ CONFIGS = {
     # projection shape of Llama-3.1-8B (programming_examples/llms/llama31_8b_q4nx)
     "q4nx_gemv": dict(M=1, K=4096, N=14336, cfg=None, desc="decode GEMV Q4NX M=1 K=4096 N=14336 g32, weights in Q4NX stream order"),
     "q4nx_gemm16": dict(M=16, K=4096, N=14336, cfg=None, desc="batched decode GEMM Q4NX M=16 K=4096 N=14336 g32, weights in Q4NX stream order"),
+    "q4nx_prefill": dict(M=2048, K=4096, N=14336, cfg=None, desc="prefill GEMM Q4NX M=2048 K=4096 N=14336 g32, weights in Q4NX stream order"),
     # the tail of a decode step of Llama-3.2-1B: final RMSNorm + bf16 lm_head GEMV + argmax
     "lm_head": dict(M=1, K=2048, N=128256, cfg=None, desc="decode tail RMSNorm + bf16 lm_head GEMV + argmax E=2048 V=128256"),
 }
@@ -154,7 +155,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
     nqkv = (LAYER_HEADS + 2 * LAYER_KV) * LAYER_HD
     if kind == "layer":
         per_copy += weight_bytes(K, nqkv)
-    if kind == "prefill":
+    if kind in ("prefill", "q4nx_prefill"):
         ncopies = 1
     else:
         ncopies = max(2, -(-(MALL_BYTES + MALL_BYTES // 2) // per_copy))
@@ -298,7 +299,7 @@ def run_workload(name, steps, warmup, with_cpu_baseline):
                                                     gemm_scratch.data_ptr(), gemm_scratch.numel(), st)
         elif name == "q4nx_gemv":
             rc = lib.w4a16_q4nx_gemv_stream_bf16(x.data_ptr(), w[0].data_ptr(), None, outs[0].data_ptr(), K, N, st)
-        elif name == "q4nx_gemm16":
+        elif name in ("q4nx_gemm16", "q4nx_prefill"):
             rc = lib.w4a16_q4nx_gemm_stream_bf16(x.data_ptr(), w[0].data_ptr(), None, outs[0].data_ptr(), M, K, N, st)
         else:
             rc = lib.w4a16_gemm_bf16(x.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
@@ -804,7 +805,7 @@ def main():
     main_res = run_workload(a.workload, a.steps, a.warmup, not a.no_cpu_baseline)
     name = a.workload
     sec = main_res["cold_us"] * 1e-6
-    if name in ("prefill", "prefill_awq"):
+    if name in ("prefill", "prefill_awq", "q4nx_prefill"):
         metric, unit = "W4A16 prefill GEMM TFLOP/s", "TFLOP/s"
         value = main_res["flops"] / sec / 1e12
         roof = {"bound": "mfma", "achieved": value, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -818,9 +819,9 @@ def main():
     roof["traffic"] = t["bytes"] if t else None
     if t:
         roof["traffic_measured_at"] = {"commit": t["commit"], "profile": t["profile"]}
-    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_wsp_kernel", "prefill_awq": "gemm_kernel", "lm_head": "lm_head_kernel",
+    roof["kernel"] = {"dequant": "dequant_kernel", "prefill": "gemm_wsp_kernel", "q4nx_prefill": "gemm_wsp_kernel", "q4nx_gemv": "gemv_ws_kernel", "q4nx_gemm16": "gemm_ws_kernel", "prefill_awq": "gemm_kernel", "lm_head": "lm_head_kernel",
                       "gemv": "gemv_ws_kernel", "probe": "probe_ws_kernel", "gemm16": "gemm_ws_kernel", "gemm64": "gemm_ws_rows_kernel", "gemm64_down": "gemm_wsk_kernel", "ffn": "gemv_ws_kernel", "block": "gemv_ws_kernel", "layer": "gemv_ws_kernel"}.get(name, "stream_kernel")
-    roof["algorithmic_per_launch"] = main_res["flops"] if name in ("prefill", "prefill_awq") else main_res["bytes"]
+    roof["algorithmic_per_launch"] = main_res["flops"] if name in ("prefill", "prefill_awq", "q4nx_prefill") else main_res["bytes"]
     roof["avg_launch_us"] = main_res["cold_us"]
 
     out = {
@@ -845,7 +846,7 @@ def main():
         "per_launch_events_us": main_res["per_launch_events_us"],
         "graph_us_per_step": main_res["graph_us"],
         "hot_cache": {"us_per_step": main_res["hot_us"],
-                      "value": (main_res["flops"] / 1e12 if name in ("prefill", "prefill_awq") else main_res["bytes"] / 1e9) / (main_res["hot_us"] * 1e-6),
+                      "value": (main_res["flops"] / 1e12 if name in ("prefill", "prefill_awq", "q4nx_prefill") else main_res["bytes"] / 1e9) / (main_res["hot_us"] * 1e-6),
                       "note": "same buffers every step (Infinity Cache resident for the decode shapes)"},
     }
     if main_res.get("overlapped_us"):

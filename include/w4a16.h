@@ -539,17 +539,40 @@ int q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t
  * y += s * (sum q x) + min * (sum x) of _qmm_q4k_bf16 (programming_examples/fused_decode/kernels/q4_k.h:39-45: c += (q*b)*scale;
  * c += min*sum(b)): no workspace protocol, no state.  They cover the proj / O / FFN phases of the fused decode dispatch
  * (programming_examples/fused_decode/fused_decode.py: proj_qmm, rms_residual, glu kernels) around w4a16_decode_attention_bf16; the
- * reference runs the prefill of these models as dense bf16 GEMMs on dequantised weights, so there is no large-M kernel for the codec.  `residual` may be NULL; x_sumsq / n_pieces, res1_out, h_out, y_sumsq and the workspace
+ * reference runs the prefill of these models as dense bf16 GEMMs on dequantised weights; the large-M entry points below multiply the same bf16 values without leaving the codec.  `residual` may be NULL; x_sumsq / n_pieces, res1_out, h_out, y_sumsq and the workspace
  * (w4a16_block_stream_workspace_bytes) as in the AWQ entry points of the same names.  K % 128 == 0, N % 16 == 0.
  */
 size_t w4a16_q4nx_stream_bytes(int K, int N);
+/* Blocks of W[M, K] (uint8 [M / 32 * K / 256, 5120], as q4nx_dequant_bf16 takes them) -> the Q4NX order of the [K, N = M]
+ * matrix in one pass: the same bytes as q4nx_repack followed by w4a16_q4nx_repack_stream, without the intermediate
+ * operands; the one load-time re-pack of the reference's packer (programming_examples/fused_decode/proj_qmm_pack.py:61-140).
+ * `wstream`: w4a16_q4nx_stream_bytes(K, M) bytes.  M % 32 == 0, K % 256 == 0, mode as for q4nx_repack. */
+int w4a16_q4nx_blocks_to_stream(const void *blocks, void *wstream, int M, int K, int mode, void *stream);
 int w4a16_q4nx_repack_stream(const int32_t *qweight, const uint16_t *scales, const uint16_t *mins, void *wstream, int K, int N,
                              void *stream);
 int w4a16_q4nx_gemv_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int K, int N,
                                 void *stream);
-/* y[M, N] = bf16(x[M, K] . W + residual [M, N]): the GEMV at M = 1, the batched whole-K kernel in launches of 16 rows else */
+/* y[M, N] = bf16(x[M, K] . W + residual [M, N]): the GEMV at M = 1, the batched whole-K kernel in launches of 16 rows
+ * above (exact weights s q + min', fp32 sums, one rounding).  From M = 65 on, without a residual and with K % 256 == 0,
+ * N % 64 == 0, the tiled MFMA kernel of w4a16_gemm_stream_bf16 runs on the Q4NX order: it dequantises each K-step of a
+ * cell with its own (scale, min') word to W = bf16_rne(s q + min'), the dense dequant's values (q4nx_dequant_bf16,
+ * bit for bit), and multiplies those, which is what the reference's prompt pass of these models computes with its
+ * dense bf16 GEMMs on dequantised weights (programming_examples/llms/llama31_8b_q4nx/README.md:11-15). */
 int w4a16_q4nx_gemm_stream_bf16(const uint16_t *x, const void *wstream, const uint16_t *residual, uint16_t *y, int M, int K, int N,
                                 void *stream);
+/* The two prompt-pass blocks (w4a16_prefill_rms_qkv_rope_stream_bf16, w4a16_prefill_o_ffn_stream_bf16: same arguments
+ * without `group`, same stages, rounding points and workspaces) on matrices in Q4NX order: the reference runs these
+ * stages op by op as bf16 GEMM / RMSNorm / RoPE / SwiGLU on the dequantised weights
+ * (programming_examples/llms/llama31_8b_q4nx/README.md:11-15); here the weights stay at 5 bits and are dequantised in
+ * registers to the same bf16 values. */
+int w4a16_q4nx_prefill_rms_qkv_rope_stream_bf16(const uint16_t *x, const uint16_t *attn_norm_weight, float eps, const void *qkv_wstream,
+                                                const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out, int M,
+                                                int E, int n_heads, int n_kv_heads, int head_dim, void *workspace,
+                                                size_t workspace_bytes, void *stream);
+int w4a16_q4nx_prefill_o_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                                         float eps, const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                         const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
+                                         int H, void *workspace, size_t workspace_bytes, void *stream);
 int w4a16_q4nx_rms_gemv_stream_bf16(const uint16_t *x, const float *x_sumsq, int n_pieces, const uint16_t *norm_weight, float eps,
                                     const void *wstream, uint16_t *y, int K, int N, void *stream);
 int w4a16_q4nx_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
@@ -564,7 +587,7 @@ int w4a16_q4nx_o_gemv_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *
  * "gemv_spin_limit" (reducer poll bound), "gemv_skip_publish" (fault injection for the
  * timeout test: split-K producers do not publish), "gemv_ws_ct", "gemv_ws_waves",
  * "gemm_ws_cb", "gemm_ws_rows" (stream-order GEMV / small-batch shapes; rows: most rows per batched launch, 16, 32 or 64), "prefill_tile" (one tile width only, 1: 256 columns, 2: 192, 3: 128,
- * 4: 64; 5: 256 mixed with 128 in the launches that take that mix; 0: by shape), "prefill_min_m" (smallest M given to the tiled prefill kernel) and "prefill_swiglu_split" (1: the
+ * 4: 64; 5: 256 mixed with 128 in the launches that take that mix; 0: by shape), "prefill_min_m" (smallest M given to the tiled prefill kernel), "prefill_band" (row panels per band of its tile order), "gemm_splitk" (w4a16_gemm_stream_scratch_bf16 at 17 .. 128 rows: 0 split along K by shape, 1 always, 2 never) and "prefill_swiglu_split" (1: the
  * stream-order prompt-pass FFN runs its gate and up projections as two launches instead of one; same bits).  Process-wide.
  */
 int w4a16_tune(const char *key, int value);

@@ -40,6 +40,8 @@ SYMBOLS = {
     "w4a16_prefill_rms_qkv_rope_bf16": (_ci, [_vp, _vp, _cf, _vp, _vp, _vp, _vp, _ci, _ci, _vp] + [_ci] * 6 + [_vp, _sz, _vp]),
     "w4a16_prefill_rms_qkv_rope_stream_bf16": (_ci, [_vp, _vp, _cf, _vp, _vp, _ci, _ci, _vp] + [_ci] * 6 + [_vp, _sz, _vp]),
     "w4a16_prefill_o_ffn_stream_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 7 + [_ci, _ci, _ci, _ci, _vp, _sz, _vp]),
+    "w4a16_q4nx_prefill_rms_qkv_rope_stream_bf16": (_ci, [_vp, _vp, _cf, _vp, _vp, _ci, _ci, _vp] + [_ci] * 5 + [_vp, _sz, _vp]),
+    "w4a16_q4nx_prefill_o_ffn_stream_bf16": (_ci, [_vp, _vp, _vp, _cf] + [_vp] * 7 + [_ci, _ci, _ci, _vp, _sz, _vp]),
     "w4a16_prefill_attention_bf16": (_ci, [_vp, _vp, _ci, _ci, _ci, _ci, _vp]),
     "lm_head_workspace_bytes": (_sz, [_ci]),
     "w4a16_decode_attn_o_gemv_ffn_bf16": (_ci, [_vp] * 5 + [_ci] * 5 + [_vp, _sz, _vp, _vp, _cf] + [_vp] * 12 + [_vp, _vp, _ci, _ci, _ci, _vp, _sz, _vp]),
@@ -49,6 +51,7 @@ SYMBOLS = {
     "q4nx_dequant_bf16": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp]),
     "q4nx_repack": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_q4nx_stream_bytes": (_sz, [_ci, _ci]),
+    "w4a16_q4nx_blocks_to_stream": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp]),
     "w4a16_q4nx_repack_stream": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _vp]),
     "w4a16_q4nx_gemv_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _vp]),
     "w4a16_q4nx_gemm_stream_bf16": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp]),

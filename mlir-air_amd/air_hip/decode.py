@@ -73,8 +73,8 @@ def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda
     """A Q4NX / Q4_0 layer -> DecodeLayer.  `blocks` maps q, k, v, o, gate, up, down to the tensor's
     blocks (uint8 [n_blocks, 5120], numpy or torch) in (row-block, col-block) order as a model.q4nx
     bundle stores them; Q, K, V are fused by concatenating their blocks (whole row-blocks of the output
-    axis), and every matrix is repacked on the GPU into the decode kernels' stream order in two steps (as the
-    reference re-packs the blocks into its cascade order, proj_qmm_pack.py:61-140).
+    axis), and every matrix is re-packed on the GPU, in one pass, into the Q4NX stream order that the decode kernels
+    and the prompt pass read (as the reference re-packs the blocks once into its cascade order, proj_qmm_pack.py:61-140).
     Norm weights are bf16 bit patterns or tensors."""
     E, H = config.emb_dim, config.hidden_dim
     nq, nkv = config.n_heads * config.head_dim, config.kv_dim
@@ -89,14 +89,14 @@ def prepare_layer_q4nx(blocks, attn_norm, ffn_norm, config, mode=0, device="cuda
         return torch.from_numpy(np.ascontiguousarray(np.asarray(a).view(np.int16))).to(device).view(torch.bfloat16)
 
     def repack(t, M, K):
-        return ops.q4nx_repack(t.contiguous(), M, K, mode)
+        return ops.q4nx_blocks_to_stream(t.contiguous(), M, K, mode)
 
     qkv = torch.cat([dev_blocks(blocks[n]) for n in ("q", "k", "v")], dim=0)
-    out = DecodeLayer(attn_norm=dev_vec(attn_norm), ffn_norm=dev_vec(ffn_norm),
-                      wqkv=repack(qkv, nq + 2 * nkv, E), wo=repack(dev_blocks(blocks["o"]), E, nq),
-                      w_gate=repack(dev_blocks(blocks["gate"]), H, E), w_up=repack(dev_blocks(blocks["up"]), H, E),
-                      w_down=repack(dev_blocks(blocks["down"]), E, H), codec="q4nx")
-    return out.with_stream()
+    stream = {"wqkv": repack(qkv, nq + 2 * nkv, E), "wo": repack(dev_blocks(blocks["o"]), E, nq),
+              "w_gate": repack(dev_blocks(blocks["gate"]), H, E), "w_up": repack(dev_blocks(blocks["up"]), H, E),
+              "w_down": repack(dev_blocks(blocks["down"]), E, H)}
+    return DecodeLayer(attn_norm=dev_vec(attn_norm), ffn_norm=dev_vec(ffn_norm), wqkv=None, wo=None, w_gate=None, w_up=None,
+                       w_down=None, codec="q4nx", stream=stream)
 
 
 def prepare_layer(layer: wmod.LayerWeights, device="cuda", stream_order=True, keep_triples=False) -> DecodeLayer:
@@ -190,14 +190,17 @@ def run_prefill_layer(x, layer: DecodeLayer, config, k_cache_layer, v_cache_laye
     RoPE, causal attention, O projection + FFN block; x bf16 [M, emb] -> bf16 [M, emb].  The roped K and V
     rows are written to the caches [n_kv_heads, max_seq, head_dim] at positions 0..M-1, where the decode
     steps that follow expect them."""
-    if layer.codec != "awq":
-        raise ValueError("the prefill kernels take AWQ layers (the reference prefills its Q4NX models in bf16)")
     M = x.shape[0]
     nh, nkv, hd = config.n_heads, config.n_kv_heads, config.head_dim
     # the stream-order copies where the layer has them and the tiled stream-order GEMM takes every matrix
     sw = layer.stream if layer.stream is not None and _stream_covers_prefill(layer.stream) else None
+    if layer.codec != "awq" and sw is None:
+        # (the reference prefills its Q4NX models as dense bf16 GEMMs on dequantised weights; the tiled kernel multiplies
+        # the same bf16 values from the Q4NX order and has no checkpoint-layout twin)
+        raise ValueError("a Q4NX layer is prefilled from its stream-order re-pack: E, H multiples of 256, widths of 64")
     if sw is not None:
-        qkv = ops.prefill_rms_qkv_rope_stream(x, layer.attn_norm, sw["wqkv"], rope_lut, 0, nh, nkv, hd, eps=config.rms_eps)
+        qkv = ops.prefill_rms_qkv_rope_stream(x, layer.attn_norm, sw["wqkv"], rope_lut, 0, nh, nkv, hd, eps=config.rms_eps,
+                                              codec=layer.codec)
     else:
         qkv = ops.prefill_rms_qkv_rope(x, layer.attn_norm, layer.wqkv, rope_lut, 0, nh, nkv, hd, eps=config.rms_eps)
     nq, nk = nh * hd, nkv * hd
@@ -205,7 +208,8 @@ def run_prefill_layer(x, layer: DecodeLayer, config, k_cache_layer, v_cache_laye
     v_cache_layer[:, :M].copy_(qkv[:, nq + nk:].reshape(M, nkv, hd).transpose(0, 1))
     attn_out = ops.prefill_attention(qkv, nh, nkv, hd)
     if sw is not None:
-        return ops.prefill_o_ffn_stream(attn_out, x, layer.ffn_norm, sw["wo"], sw["w_gate"], sw["w_up"], sw["w_down"], eps=config.rms_eps)
+        return ops.prefill_o_ffn_stream(attn_out, x, layer.ffn_norm, sw["wo"], sw["w_gate"], sw["w_up"], sw["w_down"], eps=config.rms_eps,
+                                        codec=layer.codec)
     return ops.prefill_o_ffn(attn_out, x, layer.ffn_norm, layer.wo, layer.w_gate, layer.w_up, layer.w_down, eps=config.rms_eps)
 
 

@@ -217,10 +217,17 @@ class StreamWeight:
     by `repack_stream`: the counterpart of the reference's per-layer packed decode buffers
     (repack_for_gemv, programming_examples/llms/llama32_1b_int4/awq_repacker.py:112-135)."""
 
-    __slots__ = ("buf", "K", "N")
+    __slots__ = ("buf", "K", "N", "order")
 
-    def __init__(self, buf, K, N):
-        self.buf, self.K, self.N = buf, K, N
+    def __init__(self, buf, K, N, order="awq"):
+        self.buf, self.K, self.N, self.order = buf, K, N, order   # order: "awq", or "q4nx" (q4nx_repack_stream)
+
+
+def _need_order(order, *weights):
+    """The two orders are read by different kernels (a Q4NX-order kernel on an AWQ-order buffer would run past its end)."""
+    for w in weights:
+        if w is not None and w.order != order:
+            raise ValueError(f"this op takes StreamWeights in {order} order, got one in {w.order} order")
 
 
 def repack_stream(qweight, qzeros, scales, group=GROUP):
@@ -242,6 +249,7 @@ def w4a16_gemv_stream(x, w, residual=None, group=GROUP, out=None):
     Stateless (no workspace)."""
     lib = _lib.load_library()
     _need_cuda(x, w.buf)
+    _need_order("awq", w)
     if x.numel() != w.K:
         raise ValueError(f"x has K={x.numel()} but the matrix has {w.K} rows")
     if out is None:
@@ -266,6 +274,7 @@ def w4a16_gemm_stream(x, w, group=GROUP, out=None):
     demand, nothing kept in it between calls)."""
     lib = _lib.load_library()
     _need_cuda(x, w.buf)
+    _need_order("awq", w)
     vec = x.dim() == 1
     x2 = x.unsqueeze(0) if vec else x
     M, K = x2.shape
@@ -290,6 +299,7 @@ def w4a16_swiglu_stream(x, gate, up, group=GROUP, out=None):
     """Decode FFN front half on two StreamWeights: h[H] = bf16(silu(bf16(x Wg)) * bf16(x Wu))."""
     lib = _lib.load_library()
     _need_cuda(x, gate.buf, up.buf)
+    _need_order("awq", gate, up)
     if x.numel() != gate.K or (up.K, up.N) != (gate.K, gate.N):
         raise ValueError("w4a16_swiglu_stream: gate and up must both be [K, H]")
     if out is None:
@@ -469,6 +479,7 @@ def w4a16_rms_gemv_stream(x, norm_weight, w, eps=1e-5, group=GROUP, x_sumsq=None
     call that produced x (o_gemv_ffn_stream / decode_attn_o_gemv_ffn_stream with return_sumsq)."""
     lib = _lib.load_library()
     _need_cuda(x, norm_weight, w.buf)
+    _need_order("awq", w)
     if x.numel() != w.K or norm_weight.numel() != w.K:
         raise ValueError("w4a16_rms_gemv_stream: x and norm_weight must have K elements")
     out = torch.empty((w.N,), dtype=torch.bfloat16, device=x.device)
@@ -484,6 +495,7 @@ def w4a16_rms_swiglu_stream(x, norm_weight, gate, up, eps=1e-5, group=GROUP):
     """h[H] = bf16(silu(bf16(n Wg)) * bf16(n Wu)), n = bf16((x * rstd) * norm_weight), on two StreamWeights."""
     lib = _lib.load_library()
     _need_cuda(x, norm_weight, gate.buf, up.buf)
+    _need_order("awq", gate, up)
     if x.numel() != gate.K or (up.K, up.N) != (gate.K, gate.N) or norm_weight.numel() != gate.K:
         raise ValueError("w4a16_rms_swiglu_stream: gate and up must both be [K, H], x and norm_weight [K]")
     h = torch.empty((gate.N,), dtype=torch.bfloat16, device=x.device)
@@ -496,6 +508,7 @@ def ffn_swiglu_stream(x, gate, up, down, group=GROUP, return_h=False):
     """Decode FFN on StreamWeights: y = Wd(silu(x Wg) * (x Wu)); two whole-K launches, no workspace."""
     lib = _lib.load_library()
     _need_cuda(x, gate.buf, up.buf, down.buf)
+    _need_order("awq", gate, up, down)
     K, H = gate.K, gate.N
     if x.numel() != K or (up.K, up.N) != (K, H) or (down.K, down.N) != (H, K):
         raise ValueError("ffn_swiglu_stream: gate/up must be [K, H] and down [H, K]")
@@ -519,6 +532,7 @@ def o_gemv_ffn_stream(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down,
     appended for the next layer's w4a16_rms_gemv_stream."""
     lib = _lib.load_library()
     _need_cuda(attn_out, x_residual, ffn_norm_weight, wo.buf, gate.buf, up.buf, down.buf)
+    _need_order("awq", wo, gate, up, down)
     E, H = wo.K, gate.N
     _check_block_stream(E, H, wo, gate, up, down, attn_out, x_residual, ffn_norm_weight)
     dev = attn_out.device
@@ -543,6 +557,7 @@ def decode_attn_o_gemv_ffn_stream(qkv, rope_lut_row, k_cache, v_cache, pos, n_he
     of squares of y per 16 columns (float32 [E / 16])."""
     lib = _lib.load_library()
     _need_cuda(qkv, rope_lut_row, k_cache, v_cache, x_residual, ffn_norm_weight, wo.buf, gate.buf, up.buf, down.buf)
+    _need_order("awq", wo, gate, up, down)
     n_kv, max_seq, hd = k_cache.shape
     E, H = n_heads * hd, gate.N
     if v_cache.shape != k_cache.shape or qkv.numel() != (n_heads + 2 * n_kv) * hd or rope_lut_row.numel() != hd:
@@ -645,11 +660,14 @@ def prefill_o_ffn(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps
     return (y, res1, h) if return_intermediates else y
 
 
-def prefill_rms_qkv_rope_stream(x, attn_norm_weight, wqkv, rope_lut, pos0, n_heads, n_kv_heads, head_dim, eps=1e-5, group=GROUP):
+def prefill_rms_qkv_rope_stream(x, attn_norm_weight, wqkv, rope_lut, pos0, n_heads, n_kv_heads, head_dim, eps=1e-5, group=GROUP,
+                                codec="awq"):
     """prefill_rms_qkv_rope on a StreamWeight (the re-pack of the concatenated Q|K|V matrix): the tiled stream-order
-    GEMM with the RoPE epilogue in place of the checkpoint-layout GEMM, same rounding points."""
+    GEMM with the RoPE epilogue in place of the checkpoint-layout GEMM, same rounding points.  codec "q4nx": the
+    StreamWeight is in Q4NX order (q4nx_repack_stream)."""
     lib = _lib.load_library()
     _need_cuda(x, attn_norm_weight, rope_lut, wqkv.buf)
+    _need_order(codec, wqkv)
     M, E = x.shape
     N = (n_heads + 2 * n_kv_heads) * head_dim
     if (wqkv.K, wqkv.N) != (E, N):
@@ -660,6 +678,12 @@ def prefill_rms_qkv_rope_stream(x, attn_norm_weight, wqkv, rope_lut, pos0, n_hea
     if ws is None:
         ws = torch.empty(int(lib.w4a16_prefill_qkv_workspace_bytes(M, E)), dtype=torch.uint8, device=x.device)
         _attn_ws[key] = ws
+    if codec == "q4nx":
+        _lib.check(lib.w4a16_q4nx_prefill_rms_qkv_rope_stream_bf16(_ptr(_bits(x)), _ptr(_bits(attn_norm_weight)), float(eps),
+                                                                   _ptr(wqkv.buf), _ptr(_bits(rope_lut)), rope_lut.shape[0], int(pos0),
+                                                                   _ptr(out), M, E, n_heads, n_kv_heads, head_dim, _ptr(ws), ws.numel(),
+                                                                   _stream()))
+        return out
     _lib.check(lib.w4a16_prefill_rms_qkv_rope_stream_bf16(_ptr(_bits(x)), _ptr(_bits(attn_norm_weight)), float(eps), _ptr(wqkv.buf),
                                                           _ptr(_bits(rope_lut)), rope_lut.shape[0], int(pos0), _ptr(out), M, E,
                                                           n_heads, n_kv_heads, head_dim, group, _ptr(ws), ws.numel(), _stream()))
@@ -667,10 +691,12 @@ def prefill_rms_qkv_rope_stream(x, attn_norm_weight, wqkv, rope_lut, pos0, n_hea
 
 
 def prefill_o_ffn_stream(attn_out, x_residual, ffn_norm_weight, wo, gate, up, down, eps=1e-5, group=GROUP,
-                         return_intermediates=False):
-    """prefill_o_ffn on four StreamWeights: bf16 [M, E] -> [M, E]; with return_intermediates also res1 [M, E] and h [M, H]."""
+                         return_intermediates=False, codec="awq"):
+    """prefill_o_ffn on four StreamWeights: bf16 [M, E] -> [M, E]; with return_intermediates also res1 [M, E] and h [M, H].
+    codec "q4nx": the StreamWeights are in Q4NX order (q4nx_repack_stream)."""
     lib = _lib.load_library()
     _need_cuda(attn_out, x_residual, ffn_norm_weight, wo.buf, gate.buf, up.buf, down.buf)
+    _need_order(codec, wo, gate, up, down)
     M, E = attn_out.shape
     H = gate.N
     if (wo.K, wo.N) != (E, E) or (gate.K, up.K, up.N) != (E, E, H) or (down.K, down.N) != (H, E):
@@ -683,10 +709,13 @@ def prefill_o_ffn_stream(attn_out, x_residual, ffn_norm_weight, wo, gate, up, do
     if ws is None:
         ws = torch.empty(int(lib.w4a16_prefill_block_workspace_bytes(M, E, H)), dtype=torch.uint8, device=attn_out.device)
         _attn_ws[key] = ws
-    _lib.check(lib.w4a16_prefill_o_ffn_stream_bf16(_ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)),
-                                                   float(eps), _ptr(wo.buf), _ptr(gate.buf), _ptr(up.buf), _ptr(down.buf), _ptr(y),
-                                                   _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
-                                                   M, E, H, group, _ptr(ws), ws.numel(), _stream()))
+    args = (_ptr(_bits(attn_out)), _ptr(_bits(x_residual)), _ptr(_bits(ffn_norm_weight)), float(eps), _ptr(wo.buf), _ptr(gate.buf),
+            _ptr(up.buf), _ptr(down.buf), _ptr(y), _ptr(res1) if res1 is not None else None, _ptr(h) if h is not None else None,
+            M, E, H)
+    if codec == "q4nx":
+        _lib.check(lib.w4a16_q4nx_prefill_o_ffn_stream_bf16(*args, _ptr(ws), ws.numel(), _stream()))
+    else:
+        _lib.check(lib.w4a16_prefill_o_ffn_stream_bf16(*args, group, _ptr(ws), ws.numel(), _stream()))
     return (y, res1, h) if return_intermediates else y
 
 
@@ -777,13 +806,29 @@ def q4nx_repack_stream(qweight, scales, mins):
         raise ValueError(f"Q4NX stream order needs K % 128 == 0 and N % 16 == 0, got K={K}, N={N}")
     buf = torch.empty(int(nbytes), dtype=torch.uint8, device=qweight.device)
     _lib.check(lib.w4a16_q4nx_repack_stream(_ptr(qweight), _ptr(_bits(scales)), _ptr(_bits(mins)), _ptr(buf), K, N, _stream()))
-    return StreamWeight(buf, K, N)
+    return StreamWeight(buf, K, N, "q4nx")
+
+
+def q4nx_blocks_to_stream(blocks, M, K, mode=0):
+    """Blocks of W[M, K] (uint8 [n_blocks, 5120] on the GPU) -> StreamWeight in Q4NX order of the [K, N = M] matrix, in
+    one pass (the same bytes as q4nx_repack followed by q4nx_repack_stream); once per tensor at load time."""
+    lib = _lib.load_library()
+    _need_cuda(blocks)
+    if blocks.numel() != (M // 32) * (K // 256) * 5120:
+        raise ValueError(f"blocks must hold {(M // 32) * (K // 256)} blocks of 5120 bytes for W[{M}, {K}]")
+    nbytes = lib.w4a16_q4nx_stream_bytes(K, M)
+    if nbytes == 0 or M % 32 or K % 256:
+        raise ValueError(f"Q4NX blocks need M % 32 == 0 and K % 256 == 0, got M={M}, K={K}")
+    buf = torch.empty(int(nbytes), dtype=torch.uint8, device=blocks.device)
+    _lib.check(lib.w4a16_q4nx_blocks_to_stream(_ptr(blocks), _ptr(buf), M, K, int(mode), _stream()))
+    return StreamWeight(buf, K, M, "q4nx")
 
 
 def q4nx_gemv_stream(x, w, residual=None, out=None):
     """y[N] = bf16(x[K] . W (+ residual)) on a Q4NX-order StreamWeight; stateless, no workspace."""
     lib = _lib.load_library()
     _need_cuda(x, w.buf)
+    _need_order("q4nx", w)
     if x.numel() != w.K or (residual is not None and residual.numel() != w.N):
         raise ValueError("q4nx_gemv_stream: x must have K elements, residual N")
     if out is None:
@@ -797,6 +842,7 @@ def q4nx_gemm_stream(x, w, residual=None, out=None):
     """y[M, N] = bf16(x[M, K] . W (+ residual [M, N])) on a Q4NX-order StreamWeight; x may be a vector [K]."""
     lib = _lib.load_library()
     _need_cuda(x, w.buf)
+    _need_order("q4nx", w)
     vec = x.dim() == 1
     x2 = x.unsqueeze(0) if vec else x
     M, K = x2.shape
@@ -813,6 +859,7 @@ def q4nx_rms_gemv_stream(x, norm_weight, w, eps=1e-5, x_sumsq=None):
     """y[N] = bf16(rms_norm(x, norm_weight) . W) on a Q4NX-order StreamWeight (x_sumsq as in w4a16_rms_gemv_stream)."""
     lib = _lib.load_library()
     _need_cuda(x, norm_weight, w.buf)
+    _need_order("q4nx", w)
     if x.numel() != w.K or norm_weight.numel() != w.K:
         raise ValueError("q4nx_rms_gemv_stream: x and norm_weight must have K elements")
     out = torch.empty((w.N,), dtype=torch.bfloat16, device=x.device)
@@ -829,6 +876,7 @@ def q4nx_o_gemv_ffn_stream(attn_out, x_residual, ffn_norm_weight, wo, gate, up, 
     """o_gemv_ffn_stream on Q4NX-order StreamWeights: same stages, outputs and scratch."""
     lib = _lib.load_library()
     _need_cuda(attn_out, x_residual, ffn_norm_weight, wo.buf, gate.buf, up.buf, down.buf)
+    _need_order("q4nx", wo, gate, up, down)
     E, H = wo.K, gate.N
     _check_block_stream(E, H, wo, gate, up, down, attn_out, x_residual, ffn_norm_weight)
     dev = attn_out.device

@@ -757,12 +757,11 @@ int w4a16_prefill_o_ffn_bf16(const uint16_t *attn_out, const uint16_t *x_residua
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
-int w4a16_prefill_rms_qkv_rope_stream_bf16(const uint16_t *x, const uint16_t *attn_norm_weight, float eps, const void *qkv_wstream,
-                                           const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out, int M, int E,
-                                           int n_heads, int n_kv_heads, int head_dim, int group, void *workspace,
-                                           size_t workspace_bytes, void *stream) {
+namespace {
+int prefill_qkv_stream_call(const uint16_t *x, const uint16_t *attn_norm_weight, float eps, const void *qkv_wstream,
+                            const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out, int M, int E, int n_heads,
+                            int n_kv_heads, int head_dim, void *workspace, size_t workspace_bytes, void *stream, bool q4) {
     if (!x || !attn_norm_weight || !qkv_wstream || !rope_lut || !qkv_out) return W4A16_ERR_NULL;
-    if (group != kGroup) return W4A16_ERR_GROUP;
     if (head_dim != 64 && head_dim != 128) return W4A16_ERR_SHAPE;
     if (n_heads <= 0 || n_kv_heads <= 0 || n_heads > 1024 || n_kv_heads > 1024) return W4A16_ERR_SHAPE;
     const int N = (n_heads + 2 * n_kv_heads) * head_dim;
@@ -774,17 +773,16 @@ int w4a16_prefill_rms_qkv_rope_stream_bf16(const uint16_t *x, const uint16_t *at
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
     hipError_t e = launch_prefill_rms_qkv_rope_stream(x, attn_norm_weight, eps, qkv_wstream, rope_lut, pos0, qkv_out, M, E, n_heads,
                                                       n_kv_heads, head_dim, static_cast<uint16_t *>(workspace),
-                                                      static_cast<hipStream_t>(stream));
+                                                      static_cast<hipStream_t>(stream), q4);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
-int w4a16_prefill_o_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
-                                    const void *o_wstream, const void *gate_wstream, const void *up_wstream,
-                                    const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
-                                    int H, int group, void *workspace, size_t workspace_bytes, void *stream) {
+int prefill_o_ffn_stream_call(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                              const void *o_wstream, const void *gate_wstream, const void *up_wstream, const void *down_wstream,
+                              uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E, int H, void *workspace,
+                              size_t workspace_bytes, void *stream, bool q4) {
     if (!attn_out || !x_residual || !ffn_norm_weight || !y || !o_wstream || !gate_wstream || !up_wstream || !down_wstream)
         return W4A16_ERR_NULL;
-    if (group != kGroup) return W4A16_ERR_GROUP;
     if (!prefill_block_stream_supported(M, E, H) || !(eps >= 0.f)) return W4A16_ERR_SHAPE;
     if (misaligned(attn_out) || misaligned(x_residual) || misaligned(ffn_norm_weight) || misaligned(y) || misaligned(o_wstream) ||
         misaligned(gate_wstream) || misaligned(up_wstream) || misaligned(down_wstream) || (res1_out && misaligned(res1_out)) ||
@@ -793,8 +791,43 @@ int w4a16_prefill_o_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_
     if (!workspace || workspace_bytes < w4a16_prefill_block_workspace_bytes(M, E, H)) return W4A16_ERR_WORKSPACE;
     if (misaligned(workspace)) return W4A16_ERR_ALIGN;
     hipError_t e = launch_prefill_o_ffn_stream(attn_out, x_residual, ffn_norm_weight, eps, o_wstream, gate_wstream, up_wstream,
-                                               down_wstream, y, res1_out, h_out, M, E, H, workspace, static_cast<hipStream_t>(stream));
+                                               down_wstream, y, res1_out, h_out, M, E, H, workspace, static_cast<hipStream_t>(stream), q4);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+}  // namespace
+
+int w4a16_prefill_rms_qkv_rope_stream_bf16(const uint16_t *x, const uint16_t *attn_norm_weight, float eps, const void *qkv_wstream,
+                                           const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out, int M, int E,
+                                           int n_heads, int n_kv_heads, int head_dim, int group, void *workspace,
+                                           size_t workspace_bytes, void *stream) {
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    return prefill_qkv_stream_call(x, attn_norm_weight, eps, qkv_wstream, rope_lut, rope_lut_rows, pos0, qkv_out, M, E, n_heads,
+                                   n_kv_heads, head_dim, workspace, workspace_bytes, stream, false);
+}
+
+int w4a16_prefill_o_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight, float eps,
+                                    const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                    const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
+                                    int H, int group, void *workspace, size_t workspace_bytes, void *stream) {
+    if (group != kGroup) return W4A16_ERR_GROUP;
+    return prefill_o_ffn_stream_call(attn_out, x_residual, ffn_norm_weight, eps, o_wstream, gate_wstream, up_wstream, down_wstream, y,
+                                     res1_out, h_out, M, E, H, workspace, workspace_bytes, stream, false);
+}
+
+int w4a16_q4nx_prefill_rms_qkv_rope_stream_bf16(const uint16_t *x, const uint16_t *attn_norm_weight, float eps, const void *qkv_wstream,
+                                                const uint16_t *rope_lut, int rope_lut_rows, int pos0, uint16_t *qkv_out, int M,
+                                                int E, int n_heads, int n_kv_heads, int head_dim, void *workspace,
+                                                size_t workspace_bytes, void *stream) {
+    return prefill_qkv_stream_call(x, attn_norm_weight, eps, qkv_wstream, rope_lut, rope_lut_rows, pos0, qkv_out, M, E, n_heads,
+                                   n_kv_heads, head_dim, workspace, workspace_bytes, stream, true);
+}
+
+int w4a16_q4nx_prefill_o_ffn_stream_bf16(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_weight,
+                                         float eps, const void *o_wstream, const void *gate_wstream, const void *up_wstream,
+                                         const void *down_wstream, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
+                                         int H, void *workspace, size_t workspace_bytes, void *stream) {
+    return prefill_o_ffn_stream_call(attn_out, x_residual, ffn_norm_weight, eps, o_wstream, gate_wstream, up_wstream, down_wstream, y,
+                                     res1_out, h_out, M, E, H, workspace, workspace_bytes, stream, true);
 }
 
 size_t w4a16_attention_workspace_bytes(int n_heads, int head_dim) {
@@ -903,6 +936,14 @@ int q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 
+int w4a16_q4nx_blocks_to_stream(const void *blocks, void *wstream, int M, int K, int mode, void *stream) {
+    if (!blocks || !wstream) return W4A16_ERR_NULL;
+    if (M <= 0 || K <= 0 || M % 32 != 0 || K % 256 != 0 || mode < 0 || mode > 2) return W4A16_ERR_SHAPE;
+    if (misaligned(blocks) || misaligned(wstream)) return W4A16_ERR_ALIGN;
+    hipError_t e = launch_q4nx_blocks_to_stream(blocks, wstream, M, K, mode, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? W4A16_OK : hip_fail(e);
+}
+
 size_t w4a16_q4nx_stream_bytes(int K, int N) {
     if (K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return 0;
     return ws_q4_matrix_bytes(K, N);
@@ -931,7 +972,13 @@ int w4a16_q4nx_gemm_stream_bf16(const uint16_t *x, const void *wstream, const ui
     if (!x || !wstream || !y) return W4A16_ERR_NULL;
     if (M <= 0 || K <= 0 || N <= 0 || K % kGroup != 0 || N % kWsTileCols != 0) return W4A16_ERR_SHAPE;
     if (misaligned(x) || misaligned(wstream) || misaligned(y) || (residual && misaligned(residual))) return W4A16_ERR_ALIGN;
-    hipError_t e = launch_gemm_ws(x, wstream, y, residual, M, K, N, static_cast<hipStream_t>(stream), true);
+    // launches of 16 rows take 13 us each at K = 4096, N = 14336, the tiled kernel ~55 us for up to 256 rows: from 65 rows on
+    // the tiled kernel (bf16-rounded weights, as the dense dequant gives them); a residual stays with the launches of 16
+    // rows, which add it in fp32 before the one rounding
+    const int tiled_min_m = g_gemv_ws_tune.prefill_min_m > 16 ? g_gemv_ws_tune.prefill_min_m : 65;
+    hipError_t e = M >= tiled_min_m && !residual && gemm_prefill_ws_supported(M, K, N)
+                       ? launch_gemm_prefill_ws(x, wstream, y, M, K, N, static_cast<hipStream_t>(stream), kEpiNone, nullptr, nullptr, true)
+                       : launch_gemm_ws(x, wstream, y, residual, M, K, N, static_cast<hipStream_t>(stream), true);
     return e == hipSuccess ? W4A16_OK : hip_fail(e);
 }
 

@@ -137,6 +137,12 @@ __device__ __forceinline__ void mfma_one(floatx4 &acc, const bf16x8 &a, const bf
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
+// Q4NX order: scale word -> scale s and min' (two bf16 halves)
+__device__ __forceinline__ void decode_md_q4(uint32_t md, float &sf, float &c0) {
+    sf = __builtin_bit_cast(float, md << 16);
+    c0 = __builtin_bit_cast(float, md & 0xFFFF0000u);
+}
+
 // A wave-uniform pointer pinned to scalar registers: the loads below then take the form "scalar base + 32-bit lane
 // offset" and the per-lane part stays one loop-invariant VGPR (left alone the compiler folds the lane offset into
 // a 64-bit VGPR base per stream and spends two VGPRs and a 64-bit add on every request).
@@ -180,10 +186,16 @@ struct PfArgs {
     int epi;                // kEpi*, or kEpiSwigluPair
     int rope_cols, rope_hd, rope_pos0;
     int band;               // row panels per band of the tile order (pf_tile_of)
+    bool q4;                // the matrices are in Q4NX order
 };
 
 // One output tile: rows m0 .., columns col0 .. col0 + 64 NCB - 1.
-template <int NCB>
+// Q4: the matrix is in Q4NX order (wstream.h): W = bf16_rne(q s + min') with a (scale, min') word per K-step of a cell
+// (32 rows) instead of one (scale, zero point) word per group; a block carries 4 KiB of such words, KiB t for K-step t,
+// and the operand of K-step t is dequantised with its own word.  Same loop otherwise: four scale-word requests per
+// tile and group instead of one, two more instructions per operand (the word's halves to two fp32 registers) instead
+// of three per group.
+template <int NCB, bool Q4>
 __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int m0, int col0) {
     constexpr int RT = kPfRowTiles, TM = kPfRows, WN = 16 * NCB, TN = 4 * WN;
     constexpr int kStageBytes = TM * 256;
@@ -232,11 +244,12 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     };
 
     // this wave's NCB tiles of the stream-order buffer
-    const size_t tile_bytes = (size_t)(p.NB + G) * kWsCellBytes;
+    constexpr int MDK = Q4 ? kWsQ4MdKiB : 1;   // KiB of scale words in front of a block's cells, words per (group, column)
+    const size_t tile_bytes = (size_t)(MDK * p.NB + G) * kWsCellBytes;
     const bool pair = p.epi == kEpiSwigluPair;
     const char *wt = p.w + (size_t)((pair ? n0 / 2 : n0) / kWsTileCols) * tile_bytes;
     u32x4 cell[2][NCB];
-    uint32_t md[2][NCB];
+    uint32_t md[2][NCB][MDK];
     uint32_t lane16 = (uint32_t)lane * 16, ln16 = (uint32_t)ln * 16;
     // Scale word and cell of tile c for group g: lane 16 (gl / 4) + ln, dword gl % 4 of the block's first KiB, and the
     // (1 + gl)-th KiB of the block.  The tiles' base addresses stay in scalar registers and the group's offset is
@@ -255,13 +268,15 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     };
     auto w_offsets = [&](int g) {
         const int gl = g & 15;
-        const uint32_t blk = (uint32_t)(g >> 4) * (uint32_t)((kWsBlockGroups + 1) * kWsCellBytes);
-        WOffsets o{ln16 + (blk + 256 * (gl >> 2) + 4 * (gl & 3)), lane16 + (blk + (uint32_t)(1 + gl) * (uint32_t)kWsCellBytes)};
+        const uint32_t blk = (uint32_t)(g >> 4) * (uint32_t)((kWsBlockGroups + MDK) * kWsCellBytes);
+        WOffsets o{ln16 + (blk + 256 * (gl >> 2) + 4 * (gl & 3)), lane16 + (blk + (uint32_t)(MDK + gl) * (uint32_t)kWsCellBytes)};
         asm volatile("" : "+v"(o.md), "+v"(o.cell));
         return o;
     };
     auto load_w_tile = [&](int set, const WOffsets &o, int c) {
-        md[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(tile_base[c] + o.md);
+#pragma unroll
+        for (int t = 0; t < MDK; ++t)   // (Q4NX order: the word of K-step t is 1 KiB further on, an immediate offset)
+            md[set][c][t] = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(tile_base[c] + o.md + t * 1024);
         // (a plain load: the workgroups of the same band and column tile on this XCD read the same cells out of its L2)
         cell[set][c] = *reinterpret_cast<const __attribute__((address_space(1))) u32x4 *>(tile_base[c] + o.cell);
     };
@@ -272,7 +287,8 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     auto take_w = [&](int set) {
 #pragma unroll
         for (int c = 0; c < NCB; ++c) {
-            asm volatile("" : "+v"(md[set][c]));
+#pragma unroll
+            for (int t = 0; t < MDK; ++t) asm volatile("" : "+v"(md[set][c][t]));
 #pragma unroll
             for (int t = 0; t < 4; ++t) asm volatile("" : "+v"(cell[set][c][t]));
         }
@@ -345,11 +361,15 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
             for (int c = 0; c < NCB; ++c) {
                 const bool last = t == 3 && c == NCB - 1;
                 const int cn = c + 1 < NCB ? c + 1 : 0, tn = c + 1 < NCB ? t : (t + 1) & 3;
-                if (last) decode_md(md[set ^ 1][0], sf[0], c0[0]);
                 DequantSlots dq;
                 dq.w = last ? cell[set ^ 1][0][0] : cell[set][cn][tn];
-                dq.sf = sf[cn];
-                dq.c0 = c0[cn];
+                if constexpr (Q4) {
+                    decode_md_q4(last ? md[set ^ 1][0][0] : md[set][cn][tn], dq.sf, dq.c0);
+                } else {
+                    if (last) decode_md(md[set ^ 1][0][0], sf[0], c0[0]);
+                    dq.sf = sf[cn];
+                    dq.c0 = c0[cn];
+                }
                 const bf16x8(&ac)[RT] = a[t & 1];
                 // This tile's share of the LDS reads that fetch the next K-step's A operands: operands n0 .. n1 - 1, all of
                 // them issued by the last tile but one, so that one wait at the head of the next K-step (instead of one
@@ -396,9 +416,9 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
                     // ... its cells and scale words (K-step 0) ...
                     if (t == 0 && k == 3) load_w_tile(set ^ 1, wo, c);
                     // ... and the scale words of its other tiles, behind the last MFMA of the group
-                    if (last && k == 3) {
+                    if (!Q4 && last && k == 3) {
 #pragma unroll
-                        for (int n = 1; n < NCB; ++n) decode_md(md[set ^ 1][n], sf[n], c0[n]);
+                        for (int n = 1; n < NCB; ++n) decode_md(md[set ^ 1][n][0], sf[n], c0[n]);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -415,8 +435,12 @@ __device__ __forceinline__ void pf_tile(const PfArgs &p, unsigned char *lds, int
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the x tile copy writes LDS behind the compiler's back
     __syncthreads();
     take_w(0);
+    if constexpr (Q4) {
+        decode_md_q4(md[0][0][0], sf[0], c0[0]);
+    } else {
 #pragma unroll
-    for (int c = 0; c < NCB; ++c) decode_md(md[0][c], sf[c], c0[c]);
+        for (int c = 0; c < NCB; ++c) decode_md(md[0][c][0], sf[c], c0[c]);
+    }
 #pragma unroll
     for (int r = 0; r < RT; ++r) a[0][r] = read_a(0, 0, r);
     b_cur = dequant_operand(cell[0][0][0], sf[0], c0[0]);
@@ -530,7 +554,7 @@ __device__ __forceinline__ void pf_tile_of(int idx, int tiles_m, int n_cols, int
 
 // blockIdx -> tile.  The wide tiles come first in dispatch order, so that the narrow ones fill in behind them.  Each
 // XCD (blockIdx % 8) takes a contiguous range of the tiles of either width in the order of pf_tile_of.
-template <int NW, int NN>
+template <int NW, int NN, bool Q4>
 __global__ void __launch_bounds__(kPfThreads, 1) gemm_wsp_kernel(const PfArgs p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
@@ -541,13 +565,13 @@ __global__ void __launch_bounds__(kPfThreads, 1) gemm_wsp_kernel(const PfArgs p)
         if (tile >= wide_total) return;
         int row, col;
         pf_tile_of(tile, p.tiles_m, p.n_wide, p.band, row, col);
-        pf_tile<NW>(p, lds, row * kPfRows, col * 64 * NW);
+        pf_tile<NW, Q4>(p, lds, row * kPfRows, col * 64 * NW);
     } else if constexpr (NN > 0) {
         const int tile = xcd * narrow_per_xcd + (slot - wide_per_xcd);
         if (tile >= narrow_total) return;
         int row, col;
         pf_tile_of(tile, p.tiles_m, p.n_narrow, p.band, row, col);
-        pf_tile<NN>(p, lds, row * kPfRows, p.n_wide * 64 * NW + col * 64 * NN);
+        pf_tile<NN, Q4>(p, lds, row * kPfRows, p.n_wide * 64 * NW + col * 64 * NN);
     }
 }
 
@@ -630,18 +654,23 @@ int pf_band(int tiles_m) {
     return want < tiles_m ? want : tiles_m;
 }
 
-template <int NW, int NN>
-hipError_t launch_wsp(const PfArgs &p, hipStream_t stream) {
+template <int NW, int NN, bool Q4>
+hipError_t launch_wsp_q(const PfArgs &p, hipStream_t stream) {
     constexpr size_t kStages = 2 * (size_t)kPfRows * 256, kOut = (size_t)kPfRows * (64 * NW + 8) * sizeof(uint16_t);
     constexpr size_t kLds = kStages > kOut ? kStages : kOut;
     static_assert(kLds <= 160 * 1024, "tile does not fit LDS");
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wsp_kernel<NW, NN>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wsp_kernel<NW, NN, Q4>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
     if (e != hipSuccess) return e;
     const int wide_per_xcd = (p.tiles_m * p.n_wide + 7) / 8, narrow_per_xcd = (p.tiles_m * p.n_narrow + 7) / 8;
     const int grid = 8 * (wide_per_xcd + narrow_per_xcd);
-    hipLaunchKernelGGL((gemm_wsp_kernel<NW, NN>), dim3(grid), dim3(kPfThreads), kLds, stream, p);
+    hipLaunchKernelGGL((gemm_wsp_kernel<NW, NN, Q4>), dim3(grid), dim3(kPfThreads), kLds, stream, p);
     return hipGetLastError();
+}
+
+template <int NW, int NN>
+hipError_t launch_wsp(const PfArgs &p, hipStream_t stream) {
+    return p.q4 ? launch_wsp_q<NW, NN, true>(p, stream) : launch_wsp_q<NW, NN, false>(p, stream);
 }
 
 }  // namespace
@@ -649,7 +678,7 @@ hipError_t launch_wsp(const PfArgs &p, hipStream_t stream) {
 bool gemm_prefill_ws_supported(int M, int K, int N) { return M > 0 && K > 0 && K % (2 * kGroup) == 0 && N > 0 && N % 64 == 0; }
 
 hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream, int epi,
-                                  const uint16_t *aux, const GemmRope *rope) {
+                                  const uint16_t *aux, const GemmRope *rope, bool q4) {
     if (!gemm_prefill_ws_supported(M, K, N)) return hipErrorInvalidValue;
     if ((epi != kEpiNone && !aux) || (epi == kEpiRope && (!rope || (rope->head_dim != 64 && rope->head_dim != 128) ||
                                                           rope->cols % rope->head_dim || N % rope->head_dim)))
@@ -660,6 +689,7 @@ hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y,
     p.y = y;
     p.aux = aux;
     p.epi = epi;
+    p.q4 = q4;
     if (epi == kEpiRope) p.rope_cols = rope->cols, p.rope_hd = rope->head_dim, p.rope_pos0 = rope->pos0;
     const bool heads128 = epi == kEpiRope && rope->head_dim == 128;
     p.M = M, p.K = K, p.N = N, p.G = K / kGroup, p.NB = ws_blocks(K);
@@ -689,7 +719,7 @@ hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y,
 // h[M, H] = bf16(silu(bf16(x . W_gate)) * bf16(x . W_up)): both projections in one launch, a tile holding the same
 // 128 (or 64) columns of either; the gate projection never leaves the chip.  H % 64 == 0.
 hipError_t launch_gemm_prefill_ws_swiglu(const uint16_t *x, const void *w_gate, const void *w_up, uint16_t *h, int M, int K, int H,
-                                         hipStream_t stream) {
+                                         hipStream_t stream, bool q4) {
     if (!gemm_prefill_ws_supported(M, K, H) || !w_up) return hipErrorInvalidValue;
     PfArgs p{};
     p.x = x;
@@ -697,6 +727,7 @@ hipError_t launch_gemm_prefill_ws_swiglu(const uint16_t *x, const void *w_gate, 
     p.w_up = static_cast<const char *>(w_up);
     p.y = h;
     p.epi = kEpiSwigluPair;
+    p.q4 = q4;
     p.M = M, p.K = K, p.N = H, p.G = K / kGroup, p.NB = ws_blocks(K);
     p.tiles_m = (M + kPfRows - 1) / kPfRows;
     p.band = pf_band(p.tiles_m);

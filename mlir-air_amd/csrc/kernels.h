@@ -134,12 +134,13 @@ hipError_t launch_gemm_wsk(const uint16_t *x, const void *w, uint16_t *y, const 
 // Prefill GEMM on stream-order weights (gemm_ws.hip): bf16-rounded weights dequantised in registers, x through LDS.
 bool gemm_prefill_ws_supported(int M, int K, int N);   // K % 256 == 0, N % 64 == 0
 // Epilogues as for launch_gemm_prefill (kEpi*); kEpiRope with heads of 128 needs N % 128 == 0.
+// `q4`: the matrix is in Q4NX order (launch_repack_ws_q4), W = bf16_rne(q s + min').
 hipError_t launch_gemm_prefill_ws(const uint16_t *x, const void *w, uint16_t *y, int M, int K, int N, hipStream_t stream,
-                                  int epi = kEpiNone, const uint16_t *aux = nullptr, const GemmRope *rope = nullptr);
+                                  int epi = kEpiNone, const uint16_t *aux = nullptr, const GemmRope *rope = nullptr, bool q4 = false);
 // h[M, H] = bf16(silu(bf16(x . W_gate)) * bf16(x . W_up)) in one launch (H % 64 == 0): bit for bit the gate launch followed
 // by the up launch with kEpiSiluGateMul.
 hipError_t launch_gemm_prefill_ws_swiglu(const uint16_t *x, const void *w_gate, const void *w_up, uint16_t *h, int M, int K, int H,
-                                         hipStream_t stream);
+                                         hipStream_t stream, bool q4 = false);
 // Operands of the affine path (q4nx_repack: qweight [K, N / 8], scales and mins [K / 32, N]) -> Q4NX order
 // (ws_q4_matrix_bytes(K, N) bytes at `out`).
 hipError_t launch_repack_ws_q4(const int32_t *qweight, const uint16_t *scales, const uint16_t *mins, void *out, int K, int N,
@@ -168,20 +169,22 @@ hipError_t launch_prefill_o_ffn(const uint16_t *attn_out, const uint16_t *x_resi
                                 const PrefillLinear &wo, const PrefillLinear &wg, const PrefillLinear &wu,
                                 const PrefillLinear &wd, uint16_t *y, uint16_t *res1_out, uint16_t *h_out, int M, int E,
                                 int H, void *workspace, int cus, hipStream_t stream);
-// The same blocks on stream-order weights (every matrix re-packed with launch_repack_ws).
+// The same blocks on stream-order weights (every matrix re-packed with launch_repack_ws; `q4`: with launch_repack_ws_q4).
 bool prefill_block_stream_supported(int M, int E, int H);
 hipError_t launch_prefill_rms_qkv_rope_stream(const uint16_t *x, const uint16_t *norm_w, float eps, const void *wqkv,
                                               const uint16_t *rope_lut, int pos0, uint16_t *qkv_out, int M, int E, int n_heads,
-                                              int n_kv, int head_dim, uint16_t *normed, hipStream_t stream);
+                                              int n_kv, int head_dim, uint16_t *normed, hipStream_t stream, bool q4 = false);
 hipError_t launch_prefill_o_ffn_stream(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_w, float eps,
                                        const void *wo, const void *wg, const void *wu, const void *wd, uint16_t *y,
                                        uint16_t *res1_out, uint16_t *h_out, int M, int E, int H, void *workspace,
-                                       hipStream_t stream);
+                                       hipStream_t stream, bool q4 = false);
 
 // Q4NX / Q4_0 block codec (q4nx.hip).  mode: 0 w = s q + m, 1 w = s (q - m), 2 signed q, w = s q.
 hipError_t launch_q4nx_dequant(const void *blocks, uint16_t *out, int M, int K, int mode, hipStream_t stream);
 hipError_t launch_q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *scales, uint16_t *mins, int M, int K,
                               int mode, hipStream_t stream);
+// Blocks of W[M, K] -> Q4NX stream order of the [K, N = M] matrix (ws_q4_matrix_bytes(K, M) bytes) in one pass.
+hipError_t launch_q4nx_blocks_to_stream(const void *blocks, void *out, int M, int K, int mode, hipStream_t stream);
 
 // Final RMSNorm + bf16 lm_head GEMV + argmax (lm_head.hip).  The scratch buffer holds one 8-byte
 // argmax key per 16 rows and needs no initialisation.

@@ -146,17 +146,17 @@ bool prefill_block_stream_supported(int M, int E, int H) {
 
 hipError_t launch_prefill_rms_qkv_rope_stream(const uint16_t *x, const uint16_t *norm_w, float eps, const void *wqkv,
                                               const uint16_t *rope_lut, int pos0, uint16_t *qkv_out, int M, int E, int n_heads,
-                                              int n_kv, int head_dim, uint16_t *normed, hipStream_t stream) {
+                                              int n_kv, int head_dim, uint16_t *normed, hipStream_t stream, bool q4) {
     hipError_t e = launch_rmsnorm_rows(x, norm_w, normed, M, E, eps, stream);
     if (e != hipSuccess) return e;
     const GemmRope rope = {(n_heads + n_kv) * head_dim, head_dim, pos0};
-    return launch_gemm_prefill_ws(normed, wqkv, qkv_out, M, E, (n_heads + 2 * n_kv) * head_dim, stream, kEpiRope, rope_lut, &rope);
+    return launch_gemm_prefill_ws(normed, wqkv, qkv_out, M, E, (n_heads + 2 * n_kv) * head_dim, stream, kEpiRope, rope_lut, &rope, q4);
 }
 
 hipError_t launch_prefill_o_ffn_stream(const uint16_t *attn_out, const uint16_t *x_residual, const uint16_t *ffn_norm_w, float eps,
                                        const void *wo, const void *wg, const void *wu, const void *wd, uint16_t *y,
                                        uint16_t *res1_out, uint16_t *h_out, int M, int E, int H, void *workspace,
-                                       hipStream_t stream) {
+                                       hipStream_t stream, bool q4) {
     char *base = static_cast<char *>(workspace);
     uint16_t *res1 = reinterpret_cast<uint16_t *>(base);
     base += round256((size_t)M * E * sizeof(uint16_t));
@@ -167,19 +167,19 @@ hipError_t launch_prefill_o_ffn_stream(const uint16_t *attn_out, const uint16_t 
     uint16_t *h = reinterpret_cast<uint16_t *>(base);
     if (res1_out) res1 = res1_out;
     if (h_out) h = h_out;
-    hipError_t e = launch_gemm_prefill_ws(attn_out, wo, res1, M, E, E, stream, kEpiAddRounded, x_residual);
+    hipError_t e = launch_gemm_prefill_ws(attn_out, wo, res1, M, E, E, stream, kEpiAddRounded, x_residual, nullptr, q4);
     if (e != hipSuccess) return e;
     e = launch_rmsnorm_rows(res1, ffn_norm_w, normed, M, E, eps, stream);
     if (e != hipSuccess) return e;
     if (g_gemv_ws_tune.prefill_swiglu_split) {
-        e = launch_gemm_prefill_ws(normed, wg, gate, M, E, H, stream);
+        e = launch_gemm_prefill_ws(normed, wg, gate, M, E, H, stream, kEpiNone, nullptr, nullptr, q4);
         if (e != hipSuccess) return e;
-        e = launch_gemm_prefill_ws(normed, wu, h, M, E, H, stream, kEpiSiluGateMul, gate);
+        e = launch_gemm_prefill_ws(normed, wu, h, M, E, H, stream, kEpiSiluGateMul, gate, nullptr, q4);
     } else {
-        e = launch_gemm_prefill_ws_swiglu(normed, wg, wu, h, M, E, H, stream);
+        e = launch_gemm_prefill_ws_swiglu(normed, wg, wu, h, M, E, H, stream, q4);
     }
     if (e != hipSuccess) return e;
-    return launch_gemm_prefill_ws(h, wd, y, M, H, E, stream, kEpiAddRounded, res1);
+    return launch_gemm_prefill_ws(h, wd, y, M, H, E, stream, kEpiAddRounded, res1, nullptr, q4);
 }
 
 }  // namespace w4a16

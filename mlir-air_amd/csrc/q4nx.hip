@@ -19,6 +19,7 @@
 // reads (8 output features per word), up to the nibble order inside a word.
 #include "common.h"
 #include "kernels.h"
+#include "wstream.h"
 
 namespace w4a16 {
 
@@ -120,6 +121,66 @@ hipError_t launch_q4nx_repack(const void *blocks, int32_t *qweight, uint16_t *sc
     hipLaunchKernelGGL(q4nx_repack_kernel, dim3(K / kQ4nxCols, M / kQ4nxRows), dim3(256), 0, stream,
                        reinterpret_cast<const uint8_t *>(blocks), reinterpret_cast<uint32_t *>(qweight), scales, mins, M,
                        mode);
+    return hipGetLastError();
+}
+
+// Blocks -> Q4NX stream order (wstream.h) in one pass, the form the whole-K decode kernels and the tiled kernel read:
+// the counterpart of the reference's single load-time re-pack of the bundle's blocks into the order its cores consume
+// (programming_examples/fused_decode/proj_qmm_pack.py:61-140).  Same bytes as q4nx_repack_kernel followed by
+// repack_ws_q4_kernel, without the intermediate operands.  One thread per dword of the buffer.
+//   cell dword (tile, group g, lane (lg, ln), K-step t): nibble p = q[n = 16 tile + ln][k = 128 g + 32 t + 8 lg + order(p)],
+//     i.e. block (tile / 2, g / 2), row group tile % 2, nibble ln of the eight entries of columns
+//     128 (g % 2) + 32 t + 8 lg + 0..7: 64 contiguous bytes, shared by the 16 lanes ln
+//   scale word (tile, block b, K-step t, lane (lg, ln), dword i): group g = 16 b + 4 lg + i, the block's column group
+//     4 (g % 2) + t, row 16 (tile % 2) + ln
+__global__ void __launch_bounds__(256) q4nx_blocks_to_stream_kernel(const uint8_t *__restrict__ blocks, uint32_t *__restrict__ out, int G,
+                                                                   int NB, int tiles, int KB, int mode) {
+    const size_t tile_dwords = (size_t)(kWsQ4MdKiB * NB + G) * (kWsCellBytes / 4);
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= tile_dwords * tiles) return;
+    const int tile = (int)(idx / tile_dwords);
+    const int off = (int)(idx - (size_t)tile * tile_dwords);
+    constexpr int BLOCK_DWORDS = (kWsBlockGroups + kWsQ4MdKiB) * (int)(kWsCellBytes / 4);
+    const int b = min(off / BLOCK_DWORDS, NB - 1);
+    const int within = off - b * BLOCK_DWORDS;
+    const int l = (within & 255) >> 2, sub = within & 3;   // lane and dword of a 1 KiB piece
+    const int lg = l >> 4, ln = l & 15;
+    const int bi = tile >> 1, rg = tile & 1;
+    uint32_t v = 0;
+    if (within < kWsQ4MdKiB * 256) {
+        const int t = within >> 8;
+        const int g = kWsBlockGroups * b + 4 * lg + sub;
+        if (g < G) {
+            const uint8_t *blk = blocks + ((size_t)bi * KB + (g >> 1)) * kQ4nxBlockBytes;
+            const int at = (4 * (g & 1) + t) * kQ4nxRows + 16 * rg + ln;
+            const uint16_t sb = reinterpret_cast<const uint16_t *>(blk)[at];
+            uint16_t mb = reinterpret_cast<const uint16_t *>(blk + 512)[at];
+            const float sc = bf16_bits_to_float(sb);
+            if (mode == 1) mb = float_to_bf16_bits(-(sc * bf16_bits_to_float(mb)));
+            if (mode == 2) mb = float_to_bf16_bits(-8.0f * sc);
+            v = (uint32_t)sb | ((uint32_t)mb << 16);
+        }
+    } else {
+        const int g = kWsBlockGroups * b + (within >> 8) - kWsQ4MdKiB;
+        const uint8_t *blk = blocks + ((size_t)bi * KB + (g >> 1)) * kQ4nxBlockBytes;
+        const int col0 = 128 * (g & 1) + 32 * sub + 8 * lg;
+        const uint32_t *qs = reinterpret_cast<const uint32_t *>(blk + 1024 + ((size_t)rg * kQ4nxCols + col0) * 8);
+        const uint32_t flip = mode == 2 ? 8u : 0u;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const int c = pack_order(p);                              // column col0 + c: entry c, nibble ln of its 16
+            const uint32_t word = qs[2 * c + (ln >> 3)];
+            v |= (((word >> (4 * (ln & 7))) & 0xFu) ^ flip) << (4 * p);
+        }
+    }
+    out[idx] = v;
+}
+
+hipError_t launch_q4nx_blocks_to_stream(const void *blocks, void *out, int M, int K, int mode, hipStream_t stream) {
+    const size_t dwords = ws_q4_matrix_bytes(K, M) / 4;
+    const size_t grid = (dwords + 255) / 256;
+    hipLaunchKernelGGL(q4nx_blocks_to_stream_kernel, dim3((unsigned)grid), dim3(256), 0, stream, reinterpret_cast<const uint8_t *>(blocks),
+                       static_cast<uint32_t *>(out), K / kGroup, ws_blocks(K), M / kWsTileCols, K / kQ4nxCols, mode);
     return hipGetLastError();
 }
 

@@ -290,6 +290,42 @@ def test_decode_block_q4nx_matches_the_oracle_chain(ops):
         vc[:, pos] = dev(vc_ref[:, pos])
 
 
+def test_prefill_layer_q4nx_agrees_with_decode_steps(ops):
+    """A Q4NX layer over a prompt of 70 tokens (run_prefill_layer: the tiled kernel on bf16-rounded weights, causal
+    attention over the prompt) against the same tokens fed one at a time through run_decode_block (exact weights, the
+    cache growing by one position per step): row m of the prompt pass is step m's output up to the roundings of either
+    path, and both leave the same K / V cache."""
+    from air_hip import decode, weights
+
+    cfg = weights.LlamaConfig(n_layers=1, emb_dim=512, n_heads=8, head_dim=64, n_kv_heads=2, hidden_dim=1024, vocab_size=32)
+    E, H, nq, nkv = cfg.emb_dim, cfg.hidden_dim, cfg.n_heads * cfg.head_dim, cfg.kv_dim
+    M, max_seq = 70, 96
+
+    def qw(out, K, seed):
+        rng = np.random.default_rng(seed)
+        q, sc, mn = oq.requant_q4k((rng.standard_normal((out, K)) * 0.02).astype(np.float32))
+        return q, f32_to_bf16_bits(sc), f32_to_bf16_bits(mn)
+
+    w = {"q": qw(nq, E, 11), "k": qw(nkv, E, 12), "v": qw(nkv, E, 13), "o": qw(E, nq, 14),
+         "gate": qw(H, E, 15), "up": qw(H, E, 16), "down": qw(E, H, 17)}
+    layer = decode.prepare_layer_q4nx({k: oq.pack_matrix(*v) for k, v in w.items()}, _norm_w(E, 18), _norm_w(E, 19), cfg)
+    lut = decode.generate_rope_lut(cfg, max_seq)
+    rng = np.random.default_rng(20)
+    x = dev(f32_to_bf16_bits(rng.standard_normal((M, E)).astype(np.float32)))
+    (kc, vc), = decode.new_kv_cache(cfg, max_seq)
+    print("q4nx prefill layer, 70 tokens", flush=True)
+    y = decode.run_prefill_layer(x, layer, cfg, kc, vc, lut)
+    torch.cuda.synchronize()
+    (kc2, vc2), = decode.new_kv_cache(cfg, max_seq)
+    steps = torch.stack([decode.run_decode_block(x[m].contiguous(), layer, cfg, kc2, vc2, m, lut) for m in range(M)])
+    torch.cuda.synchronize()
+    err = (y.double() - steps.double()).abs()
+    assert float(err.max()) <= 8 * 2.0 ** -8 * float(steps.double().abs().max()), float(err.max())
+    for a, b in ((kc, kc2), (vc, vc2)):
+        d = (a[:, :M].double() - b[:, :M].double()).abs()
+        assert float(d.max()) <= 4 * 2.0 ** -8 * float(b[:, :M].double().abs().max()), float(d.max())
+
+
 # ---- the same codec in stream order (Q4NX order): whole-K kernels, no workspace ------------------------------------
 
 def _stream_gemv_case(ops, M, K, seed, mode=oq.ADDITIVE, residual=False):
@@ -357,6 +393,124 @@ def test_stream_gemm_rows(ops, rows, M, K, residual):
     assert np.all(np.abs(a - b) <= bf16_ulp(b) + 1e-3)
 
 
+# From 65 rows on (no residual) the tiled MFMA kernel runs on the Q4NX order: bf16-rounded weights, i.e. the dense
+# dequant's values, as the reference's own prompt pass multiplies them (dense bf16 GEMMs on dequantised weights).
+# Shapes: N = 64 U with U = 3 (64-column tiles), 8 (128), 13 (256 mixed with 192), 16; K of one block, of two blocks with a
+# short one (K = 2304: 18 groups) and of 32 groups; ragged row panels (65, 300) and two full ones (512).
+@pytest.mark.parametrize("rows,M,K,wild", [(65, 192, 256, True), (300, 512, 2304, False), (512, 832, 512, True), (130, 1024, 4096, False)])
+def test_stream_gemm_tiled(ops, rows, M, K, wild):
+    print(f"q4nx tiled stream gemm rows={rows} M={M} K={K} wild={wild}", flush=True)
+    q, s, m = make(M, K, seed=rows + M + K, wild=wild)
+    rng = np.random.default_rng(rows + 3)
+    x = f32_to_bf16_bits(rng.standard_normal((rows, K)).astype(np.float32))
+    blocks = oq.pack_matrix(q, s, m)
+    w = ops.q4nx_repack_stream(*ops.q4nx_repack(dev(blocks), M, K, oq.ADDITIVE))
+    y = ops.q4nx_gemm_stream(dev(x), w)
+    torch.cuda.synchronize()
+    wd = bf16_bits_to_f32(oq.dequant(blocks, M, K, oq.ADDITIVE)).astype(np.float64)     # [M, K], rounded to bf16
+    want = bf16_bits_to_f32(x).astype(np.float64) @ wd.T
+    assert_bf16_close(bits(y), want, ulps=1.0, atol=2e-3, what=f"q4nx tiled gemm rows={rows} M={M} K={K}")
+    # the first 16 rows through the batched whole-K kernel (exact weights): the two agree up to the weights' rounding
+    y16 = bf16_bits_to_f32(bits(ops.q4nx_gemm_stream(dev(x[:16]), w))).astype(np.float64)
+    bound = 2.0 ** -8 * (np.abs(bf16_bits_to_f32(x[:16]).astype(np.float64)) @ np.abs(wd.T)) + 2.0 ** -7 * np.abs(y16) + 2e-3
+    assert np.all(np.abs(bf16_bits_to_f32(bits(y)[:16]).astype(np.float64) - y16) <= bound)
+
+
+def test_stream_gemm_tiled_one_hot_rows_are_the_dense_dequant(ops):
+    """x = the identity (K rows, one-hot): y[k, :] is row k of W^T, one weight each, so the tiled kernel's output is the
+    dense dequant bit for bit; any mix-up of a K-step's scale word with another's shows as a wrong row block of 32."""
+    M, K = 320, 256
+    q, s, m = make(M, K, seed=77, wild=True)
+    blocks = oq.pack_matrix(q, s, m)
+    w = ops.q4nx_repack_stream(*ops.q4nx_repack(dev(blocks), M, K, oq.ADDITIVE))
+    x = f32_to_bf16_bits(np.eye(K, dtype=np.float32))
+    y = ops.q4nx_gemm_stream(dev(x), w)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y), oq.dequant(blocks, M, K, oq.ADDITIVE).T)
+
+
+def _q4_sw(ops, q, s, m):
+    M, K = q.shape
+    return ops.q4nx_repack_stream(*ops.q4nx_repack(dev(oq.pack_matrix(q, s, m)), M, K, oq.ADDITIVE))
+
+
+def _q4_dense(q, s, m):
+    """[K, out] float64 of the dense dequant's bf16 values."""
+    return bf16_bits_to_f32(f32_to_bf16_bits(oq.dequant_values(q, s, m, oq.ADDITIVE))).astype(np.float64).T
+
+
+@pytest.mark.parametrize("rows,E,H", [(70, 256, 512), (300, 512, 1280)])
+def test_prefill_o_ffn_q4nx_stage_by_stage(ops, rows, E, H):
+    """The prompt-pass O + FFN block on Q4NX-order weights: every epilogue against the library's own tiled product bit
+    for bit (the epilogues work on the bf16 product), every product against float64 on the dense dequant's values."""
+    from helpers import bf16_ulp
+    print(f"q4nx prefill o+ffn rows={rows} E={E} H={H}", flush=True)
+    mats = [make(out, K, seed=rows + i) for i, (out, K) in enumerate(((E, E), (H, E), (H, E), (E, H)))]
+    so, sg, su, sd = (_q4_sw(ops, *w) for w in mats)
+    do, dg, du, dd = (_q4_dense(*w) for w in mats)
+    rng = np.random.default_rng(rows)
+    attn = f32_to_bf16_bits(rng.standard_normal((rows, E)).astype(np.float32))
+    xres = f32_to_bf16_bits(rng.standard_normal((rows, E)).astype(np.float32))
+    nw = f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32))
+    y, res1, h = ops.prefill_o_ffn_stream(dev(attn), dev(xres), dev(nw), so, sg, su, sd, return_intermediates=True, codec="q4nx")
+    y2 = ops.prefill_o_ffn_stream(dev(attn), dev(xres), dev(nw), so, sg, su, sd, codec="q4nx")
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+    f = lambda b: bf16_bits_to_f32(b).astype(np.float64)
+    add_rounded = lambda prod, add: (prod.float() + add.float()).to(torch.bfloat16)
+
+    def close_sum(got_bits, prod64, add, what):
+        want = prod64 + add
+        err = np.abs(f(got_bits) - want)
+        tol = bf16_ulp(want) + bf16_ulp(prod64) + 2e-3
+        assert np.all(err <= tol), f"{what}: {np.max(err - tol)}"
+
+    assert torch.equal(res1.view(torch.int16), add_rounded(ops.q4nx_gemm_stream(dev(attn), so), dev(xres)).view(torch.int16))
+    close_sum(bits(res1), f(attn) @ do, f(xres), "res1")
+    normed = ops.rms_norm_rows(res1, dev(nw))
+    gb, ub = f(bits(ops.q4nx_gemm_stream(normed, sg))), f(bits(ops.q4nx_gemm_stream(normed, su)))
+    h_exact = gb / (1.0 + np.exp(-gb)) * ub
+    assert np.all(np.abs(f(bits(h)) - h_exact) <= 0.51 * bf16_ulp(h_exact) + 1e-6 * np.abs(h_exact) + 1e-30)
+    n64 = f(bits(normed))
+    assert_bf16_close(f32_to_bf16_bits(gb.astype(np.float32)), n64 @ dg, ulps=1.0, atol=2e-3, what="gate")
+    assert_bf16_close(f32_to_bf16_bits(ub.astype(np.float32)), n64 @ du, ulps=1.0, atol=2e-3, what="up")
+    assert torch.equal(y.view(torch.int16), add_rounded(ops.q4nx_gemm_stream(h, sd), res1).view(torch.int16))
+    close_sum(bits(y), f(bits(h)) @ dd, f(bits(res1)), "y")
+    # an AWQ-order op refuses a Q4NX-order weight instead of reading it with the wrong kernel, and the other way round
+    with pytest.raises(ValueError):
+        ops.prefill_o_ffn_stream(dev(attn), dev(xres), dev(nw), so, sg, su, sd)
+    with pytest.raises(ValueError):
+        ops.w4a16_gemm_stream(dev(attn), so)
+
+
+@pytest.mark.parametrize("rows,E,nh,nkv,hd,pos0", [(70, 256, 4, 2, 64, 3), (130, 512, 2, 1, 128, 40)])
+def test_prefill_rms_qkv_rope_q4nx(ops, rows, E, nh, nkv, hd, pos0):
+    """RMSNorm + fused Q|K|V product + half-split RoPE on a Q4NX-order matrix: V is the plain tiled product bit for bit, Q
+    and K are the oracle's rotation of that product bit for bit, the product is the float64 one on the dense values."""
+    from oracle import decode as odec
+    print(f"q4nx prefill qkv rope rows={rows} E={E} heads {nh}/{nkv} hd={hd}", flush=True)
+    N = (nh + 2 * nkv) * hd
+    q, s, m = make(N, E, seed=rows + N)
+    sw = _q4_sw(ops, q, s, m)
+    rng = np.random.default_rng(rows + 1)
+    x = f32_to_bf16_bits(rng.standard_normal((rows, E)).astype(np.float32))
+    nw = f32_to_bf16_bits((rng.standard_normal(E) * 0.1 + 1.0).astype(np.float32))
+    lut = odec.generate_rope_lut(hd, 500000.0, pos0 + rows + 2)
+    out = ops.prefill_rms_qkv_rope_stream(dev(x), dev(nw), sw, dev(lut), pos0, nh, nkv, hd, codec="q4nx")
+    normed = ops.rms_norm_rows(dev(x), dev(nw))
+    plain = ops.q4nx_gemm_stream(normed, sw)
+    torch.cuda.synchronize()
+    got, nq, nk = bits(out), nh * hd, nkv * hd
+    assert np.array_equal(got[:, nq + nk:], bits(plain)[:, nq + nk:])
+    rows_lut = lut[pos0:pos0 + rows]
+    for lo, n in ((0, nh), (nq, nkv)):
+        prod = bits(plain)[:, lo:lo + n * hd].reshape(rows * n, hd)
+        want = odec.rope_rows(prod, np.repeat(rows_lut, n, axis=0)).reshape(rows, n * hd)
+        assert np.array_equal(got[:, lo:lo + n * hd], want)
+    assert_bf16_close(bits(plain), bf16_bits_to_f32(bits(normed)).astype(np.float64) @ _q4_dense(q, s, m), ulps=1.0, atol=2e-3,
+                      what="q4nx qkv product")
+
+
 @pytest.mark.parametrize("M,K", [(32, 256), (96, 2304), (1024, 4096)])
 def test_stream_device_repack_equals_host_packer(ops, M, K):
     """w4a16_q4nx_repack_stream on the operands of q4nx_repack against the host packer on the same values."""
@@ -367,6 +521,21 @@ def test_stream_device_repack_equals_host_packer(ops, M, K):
     torch.cuda.synchronize()
     want = awq.repack_stream_q4nx(q.T.copy(), s.T.copy(), m.T.copy())     # [K, N = M] values
     assert np.array_equal(w.buf.cpu().numpy().view(np.uint32).reshape(want.shape), want)
+
+
+@pytest.mark.parametrize("mode", [oq.ADDITIVE, oq.SUBTRACTIVE, oq.Q4_0])
+@pytest.mark.parametrize("M,K", [(32, 256), (96, 2304), (1024, 4096)])
+def test_blocks_to_stream_in_one_pass_equals_the_two_step_repack(ops, M, K, mode):
+    """w4a16_q4nx_blocks_to_stream against q4nx_repack followed by w4a16_q4nx_repack_stream: the same buffer, byte for
+    byte, in all three value conventions (K = 2304: a short last block of groups; M = 96: an odd number of block rows)."""
+    q, s, m = make(M, K, seed=M + K + mode, wild=True)
+    blocks = dev(oq.pack_matrix(q, s, m))
+    two = ops.q4nx_repack_stream(*ops.q4nx_repack(blocks, M, K, mode))
+    one = ops.q4nx_blocks_to_stream(blocks, M, K, mode)
+    torch.cuda.synchronize()
+    assert (one.K, one.N, one.order) == (two.K, two.N, "q4nx") and torch.equal(one.buf, two.buf)
+    with pytest.raises(ValueError):
+        ops.q4nx_blocks_to_stream(blocks[:-1], M, K, mode)
 
 
 def test_stream_gemv_one_hot_x_is_a_dequantised_row(ops):
