@@ -240,7 +240,7 @@ int w4a16_gemm_stream_bf16(const uint16_t *x, const void *wstream, uint16_t *y, 
  * time, and adds them in an fp32 accumulator, matmul_int4_packed.py:179-181, 293-345).  A workgroup takes 256 columns and a slice of K, shares
  * the x rows of its slice through LDS and writes fp32 partial sums to `scratch`; a second launch adds the slices in
  * slice order and rounds once.  That pays where the whole-K launches re-read the x rows most: K >= 4096, rows * K / 128
- * >= 1536 and N < 12800 (K = 14336, N = 4096, 64 rows: 34.6 us against 59.2 us; K = 8192, N = 6144: 26.1 against 63.7);
+ * >= 1536 and N < 12800 (K = 14336, N = 4096, 64 rows: 27.9 us against 59.0 us; K = 4096, N = 6144: 18.1 against 34.2);
  * for every other shape and row count the call is w4a16_gemm_stream_bf16 itself and `scratch` is not touched.
  * w4a16_gemm_stream_scratch_bytes(M, K, N) is the scratch the call needs (0 where it takes none): no initialisation,
  * nothing kept between calls, 16-byte aligned; calls that overlap on one GPU need a buffer each.  Same numerics as

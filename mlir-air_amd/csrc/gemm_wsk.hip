@@ -16,6 +16,8 @@
 //   sum x      = per (row, group), taken while the x tile is written to LDS (16 lanes hold a row: one DPP row sum)
 //   quad       = 4 consecutive groups of a block: their scale words are one 16-byte chunk per (tile, column); the
 //                quad's 8 cells and 2 chunks per lane are requested a quad ahead
+#include <algorithm>
+
 #include "common.h"
 #include "kernels.h"
 #include "wstream.h"
@@ -26,7 +28,7 @@ namespace {
 
 constexpr int kSkWaves = 8;
 constexpr int kSkSetTiles = 16;    // stream tiles (of 16 columns) per workgroup
-constexpr int kSkMaxSlices = 8;
+constexpr int kSkMaxSlices = 16;
 
 __device__ __forceinline__ bf16x8 sk_cell_operand(uint32_t w, uint32_t nib_mask, uint32_t magic) {
     u32x4 b;
@@ -72,18 +74,21 @@ __global__ void __launch_bounds__(kSkWaves * 64) gemm_wsk_kernel(const uint16_t 
 #pragma unroll
         for (int j = 0; j < XL; ++j) {
             const int idx = tid + kSkWaves * 64 * j, row = idx >> 4, chunk = idx & 15;
-            xr[j] = row < M ? *reinterpret_cast<const u32x4 *>(x + (size_t)row * K + (size_t)g * kGroup + chunk * 8) : u32x4{0u, 0u, 0u, 0u};
+            // (requested as it is, a row past M as row M - 1, and zeroed when the registers go to LDS: a select here would
+            // make the wave wait for the request on the spot, and for every older request with it)
+            xr[j] = *reinterpret_cast<const u32x4 *>(x + (size_t)min(row, M - 1) * K + (size_t)g * kGroup + chunk * 8);
         }
     };
     auto store_x = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < XL; ++j) {
             const int idx = tid + kSkWaves * 64 * j, row = idx >> 4, chunk = idx & 15;
-            *reinterpret_cast<u32x4 *>(lds + buf * XT + row * 256 + ((chunk ^ (row & 15)) << 4)) = xr[j];
+            const u32x4 v = row < M ? xr[j] : u32x4{0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4 *>(lds + buf * XT + row * 256 + ((chunk ^ (row & 15)) << 4)) = v;
             float s = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                s += __builtin_bit_cast(float, xr[j][e] << 16) + __builtin_bit_cast(float, xr[j][e] & 0xFFFF0000u);
+                s += __builtin_bit_cast(float, v[e] << 16) + __builtin_bit_cast(float, v[e] & 0xFFFF0000u);
             s = row_sum16(s);   // the 16 lanes of a DPP row hold the 16 chunks of one x row
             if (chunk == 0) xs_lds[buf * ROWS + row] = s;
         }
@@ -114,6 +119,9 @@ __global__ void __launch_bounds__(kSkWaves * 64) gemm_wsk_kernel(const uint16_t 
 
     int buf = 0;
     for (int gq = g_lo; gq < g_hi; gq += 4) {
+        // (the x tile of the next group first: the wait for it then leaves the younger requests, the next quad's cells, in flight)
+        if (gq + 1 < g_hi) load_x(gq + 1);
+        __builtin_amdgcn_sched_barrier(0);
         if (gq + 4 < g_hi) load_quad(gq + 4, nxt);
         // the chunk of the other tile sits in the lane 16 away
         u32x4 other;
@@ -125,7 +133,7 @@ __global__ void __launch_bounds__(kSkWaves * 64) gemm_wsk_kernel(const uint16_t 
             const int g = gq + j;
             if (g >= g_hi) break;   // workgroup-uniform
             const bool more = g + 1 < g_hi;
-            if (more) load_x(g + 1);
+            if (more && j > 0) load_x(g + 1);
             floatx4 acc[RT][2];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) acc[rt][0] = acc[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -164,6 +172,25 @@ __global__ void __launch_bounds__(kSkWaves * 64) gemm_wsk_kernel(const uint16_t 
 
     // ---- this slice's sums: to the scratch buffer, or (one slice) straight to y ----
     const int slices = gridDim.y;
+    if (slices > 1) {
+        // Through LDS, so that a wave stores whole rows of the workgroup's 256 columns (1 KiB per instruction) instead
+        // of four 64-byte pieces: rows padded by 4 floats, which spreads the four lane groups (4 rows apart) over all banks.
+        constexpr int LDP = 16 * kSkSetTiles + 4;
+        float *yt = reinterpret_cast<float *>(lds);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) yt[(16 * rt + 4 * lg + i) * LDP + (2 * wave + c) * kWsTileCols + ln] = Y[rt][c][i];
+        __syncthreads();
+        const int col0 = blockIdx.x * kSkSetTiles * kWsTileCols, ncols = min(kSkSetTiles * kWsTileCols, N - col0);   // a multiple of 16
+        float *dst = partial + (size_t)blockIdx.y * M * N + col0;
+        for (int row = wave; row < M; row += kSkWaves)
+            if (4 * lane < ncols)
+                *reinterpret_cast<floatx4 *>(dst + (size_t)row * N + 4 * lane) = *reinterpret_cast<const floatx4 *>(yt + row * LDP + 4 * lane);
+        return;
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
@@ -222,10 +249,10 @@ int sk_slices(int K, int N, int *gps_out) {
 
 // Where the split pays, measured against the whole-K launches (gemm_ws_rows_kernel) at K 2048 .. 14336, N 2048 .. 14336
 // and 17 .. 128 rows: the whole-K launches re-read the x rows once per 16, 32 or 64 columns, so they lose with long K,
-// many rows and narrow workgroups (K = 8192, N = 6144, 64 rows: 63.7 us whole-K, 26.1 us split; K = 14336, N = 4096,
-// 64 rows: 59.2 / 34.6), and win where the split has only a few groups per slice to spread its fixed costs over (the
-// second launch, the x tile through LDS: K = 2048, any N: 11.0 / 13.8 us at 64 rows) or where their workgroups are 64
-// columns wide already (N >= 12800: K = 4096, N = 14336, 64 rows: 24.5 / 28.2 us).
+// many rows and narrow workgroups (K = 4096, N = 6144, 64 rows: 34.2 us whole-K, 18.1 us split; K = 14336, N = 4096,
+// 64 rows: 59.0 / 27.9), and win where the split has only a few groups per slice to spread its fixed costs over (the
+// second launch, the x tile through LDS: K = 2048, N = 8192: 12.6 / 14.6 us at 64 rows) or where their workgroups are 64
+// columns wide already (N >= 12800: K = 4096, N = 14336, 64 rows: 24.5 / 26.1 us).
 bool gemm_wsk_pays(int M, int K, int N) {
     if (g_gemv_ws_tune.splitk) return g_gemv_ws_tune.splitk == 1;
     const int G = K / kGroup, tiles = N / kWsTileCols, rows = M < 64 ? M : 64;
@@ -255,11 +282,13 @@ hipError_t launch_gemm_wsk(const uint16_t *x, const void *w, uint16_t *y, const 
         uint16_t *yr = y + (size_t)m0 * N;
         const dim3 grid(sets, slices), block(kSkWaves * 64);
         if (rows > 32) {
-            const size_t lds = 2 * (size_t)64 * 256 + 2 * 64 * sizeof(float);
+            const size_t lds = std::max<size_t>(2 * (size_t)64 * 256 + 2 * 64 * sizeof(float), (size_t)64 * (16 * kSkSetTiles + 4) * sizeof(float));
+            hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wsk_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (ea != hipSuccess) return ea;
             hipLaunchKernelGGL((gemm_wsk_kernel<4>), grid, block, lds, stream, xr, static_cast<const char *>(w), scratch, yr, rr, rows, K, N,
                                G, NB, gps);
         } else {
-            const size_t lds = 2 * (size_t)32 * 256 + 2 * 32 * sizeof(float);
+            const size_t lds = std::max<size_t>(2 * (size_t)32 * 256 + 2 * 32 * sizeof(float), (size_t)32 * (16 * kSkSetTiles + 4) * sizeof(float));
             hipLaunchKernelGGL((gemm_wsk_kernel<2>), grid, block, lds, stream, xr, static_cast<const char *>(w), scratch, yr, rr, rows, K, N,
                                G, NB, gps);
         }
