@@ -865,9 +865,10 @@ def main():
                 continue
             # the other headline configs carry the host baseline as well
             with_cpu = not a.no_cpu_baseline and other in ("dequant", "gemm16", "ffn", "prefill")
-            r = run_workload(other, 20 if other.startswith("prefill") else 100, 5, with_cpu)
+            tiled = other.startswith("prefill") or other == "q4nx_prefill"   # the MFMA-bound workloads
+            r = run_workload(other, 20 if tiled else 100, 5, with_cpu)
             s = r["cold_us"] * 1e-6
-            if other.startswith("prefill"):
+            if tiled:
                 extra[other] = {"us": r["cold_us"], "TFLOP/s": r["flops"] / s / 1e12,
                                 "frac_mfma_peak": r["flops"] / s / 1e12 / MFMA_BF16_PEAK_TFLOPS}
             else:
