@@ -83,7 +83,7 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
                                                                  const uint16_t *__restrict__ residual, int G, int NB,
                                                                  int round_before_add, int nwaves, const GemvWsTail tail) {
     constexpr int SUB = kWsBlockGroups / CT;
-    __shared__ float red[NMAT * kMaxWaves * 64];
+    __shared__ float red[NMAT * kMaxWaves * kWsTileCols];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lg = lane >> 4, ln = lane & 15;
@@ -238,19 +238,22 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
         else yv[0] += sum;
     }
 
-    // the 4 lane groups x W waves of every column, added by the first 16 threads
+    // K-reduction: the 4 lane groups of a wave hold different groups of K for the same 16 columns and are added with
+    // wavefront shuffles, (lg 0 + lg 1) + (lg 2 + lg 3); only the waves' sums meet in LDS, added by the first 16 threads
 #pragma unroll
-    for (int m = 0; m < NMAT; ++m) red[(m * kMaxWaves + wave) * 64 + lane] = yv[m];
+    for (int m = 0; m < NMAT; ++m) {
+        float v = yv[m];
+        v += __shfl_xor(v, 16);
+        v += __shfl_xor(v, 32);
+        if (lg == 0) red[(m * kMaxWaves + wave) * kWsTileCols + ln] = v;
+    }
     __syncthreads();
     if (threadIdx.x < kWsTileCols) {
         float tot[NMAT];
 #pragma unroll
         for (int m = 0; m < NMAT; ++m) {
             tot[m] = 0.f;
-            for (int w = 0; w < nwaves; ++w) {
-                const float *src = red + (m * kMaxWaves + w) * 64 + threadIdx.x;
-                tot[m] += (src[0] + src[16]) + (src[32] + src[48]);
-            }
+            for (int w = 0; w < nwaves; ++w) tot[m] += red[(m * kMaxWaves + w) * kWsTileCols + threadIdx.x];
         }
         const int col = tile * kWsTileCols + threadIdx.x;
         float out;
