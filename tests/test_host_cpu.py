@@ -260,6 +260,37 @@ def test_c_abi_rejects_bad_arguments_before_touching_the_gpu():
     assert lib.w4a16_workspace_init(None, 1024, None) == _lib.ERR_NULL
     assert lib.w4a16_workspace_init(P, 16, None) == _lib.ERR_WORKSPACE
     assert lib.w4a16_tune(b"no_such_key", 1) == _lib.ERR_TUNE and lib.w4a16_tune(b"gemv_waves", 0) == 0
+    # the batched GEMM with caller scratch: scratch only where the split along K is the faster way (long K, enough rows, not
+    # the widest matrices), and every argument checked before a launch
+    need = lib.w4a16_gemm_stream_scratch_bytes(64, 14336, 4096)
+    assert need == 14 * 64 * 4096 * 4
+    assert lib.w4a16_gemm_stream_scratch_bytes(64, 4096, 14336) == 0 and lib.w4a16_gemm_stream_scratch_bytes(64, 2048, 4096) == 0
+    assert lib.w4a16_gemm_stream_scratch_bytes(16, 14336, 4096) == 0 and lib.w4a16_gemm_stream_scratch_bytes(129, 14336, 4096) == 0
+    assert lib.w4a16_gemm_stream_scratch_bytes(64, 14336, 4100) == 0
+    big = (P, P, P, 64, 14336, 4096, 128)
+    assert lib.w4a16_gemm_stream_scratch_bf16(*big, None, 0, None) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_gemm_stream_scratch_bf16(*big, P, need - 1, None) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_gemm_stream_scratch_bf16(*big, P + 8, need, None) == _lib.ERR_ALIGN
+    assert lib.w4a16_gemm_stream_scratch_bf16(None, P, P, 64, 14336, 4096, 128, P, need, None) == _lib.ERR_NULL
+    assert lib.w4a16_gemm_stream_scratch_bf16(P, P, P, 64, 14336, 4096, 64, P, need, None) == _lib.ERR_GROUP
+    assert lib.w4a16_gemm_stream_scratch_bf16(P, P, P, 64, 14336, 4100, 128, P, need, None) == _lib.ERR_SHAPE
+    assert lib.w4a16_gemm_stream_scratch_bf16(P, P, None, 64, 4096, 14336, 128, None, 0, None) == _lib.ERR_NULL   # (whole-K route)
+    assert lib.w4a16_tune(b"gemm_splitk", 3) == _lib.ERR_TUNE and lib.w4a16_tune(b"gemm_splitk", 0) == 0
+    # Q4NX order: blocks -> stream order, and the prompt-pass entry points
+    assert lib.w4a16_q4nx_blocks_to_stream(None, P, 32, 256, 0, None) == _lib.ERR_NULL
+    assert lib.w4a16_q4nx_blocks_to_stream(P, P, 48, 256, 0, None) == _lib.ERR_SHAPE      # whole blocks of 32 rows
+    assert lib.w4a16_q4nx_blocks_to_stream(P, P, 32, 128, 0, None) == _lib.ERR_SHAPE      # and of 256 columns
+    assert lib.w4a16_q4nx_blocks_to_stream(P, P, 32, 256, 3, None) == _lib.ERR_SHAPE
+    assert lib.w4a16_q4nx_blocks_to_stream(P, P + 4, 32, 256, 0, None) == _lib.ERR_ALIGN
+    wsq = lib.w4a16_prefill_qkv_workspace_bytes(64, 256)
+    assert lib.w4a16_q4nx_prefill_rms_qkv_rope_stream_bf16(P, P, 1e-5, None, P, 80, 0, P, 64, 256, 4, 2, 64, P, wsq, None) == _lib.ERR_NULL
+    assert lib.w4a16_q4nx_prefill_rms_qkv_rope_stream_bf16(P, P, 1e-5, P, P, 80, 20, P, 64, 256, 4, 2, 64, P, wsq, None) == _lib.ERR_SHAPE
+    assert lib.w4a16_q4nx_prefill_rms_qkv_rope_stream_bf16(P, P, 1e-5, P, P, 80, 0, P, 64, 256, 4, 2, 64, P, wsq - 1, None) == _lib.ERR_WORKSPACE
+    wsb = lib.w4a16_prefill_block_workspace_bytes(64, 256, 512)
+    blk = [P, P, P, 1e-5, P, P, P, P, P, None, None, 64, 256, 512]
+    assert lib.w4a16_q4nx_prefill_o_ffn_stream_bf16(*blk, None, wsb, None) == _lib.ERR_WORKSPACE
+    assert lib.w4a16_q4nx_prefill_o_ffn_stream_bf16(*(blk[:4] + [None] + blk[5:]), P, wsb, None) == _lib.ERR_NULL
+    assert lib.w4a16_q4nx_prefill_o_ffn_stream_bf16(*(blk[:13] + [500]), P, wsb, None) == _lib.ERR_SHAPE
     with pytest.raises(_lib.W4A16Error):
         _lib.check(_lib.ERR_ALIGN)
 
