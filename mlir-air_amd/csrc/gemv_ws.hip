@@ -165,6 +165,9 @@ __global__ void __launch_bounds__(kMaxWaves * 64) gemv_ws_kernel(const uint16_t 
 
         if constexpr (RMS) {
             if (!have_rstd) {   // wave-uniform; the pieces are added in the order a lane walking them would
+                // (taken opaque here: the sum does not depend on the loop, and hoisted in front of it the wait for the
+                // pieces would stand before the task's requests after all)
+                asm volatile("" : "+v"(piece[0]), "+v"(piece[1]), "+v"(piece[2]), "+v"(piece[3]), "+v"(a0), "+v"(a1));
                 a0 += ((piece[0] + piece[1]) + piece[2]) + piece[3];
                 rstd = 1.0f / sqrtf(wave_reduce<false>(a0 + a1) / (float)tail.K + tail.eps);
                 have_rstd = true;
